@@ -1,0 +1,215 @@
+"""ctypes binding of the CPU oracle (oracle/zref.c).
+
+TEST INFRASTRUCTURE ONLY: imported by tests/, the smoke test and the
+benchmark's cpu_baseline leg, never by the zllm_amd package.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+
+F32, F16, Q8_0, Q4_K, BF16 = 0, 1, 8, 12, 30
+
+
+def build() -> None:
+    """Compiles the oracle libraries (gcc, a few seconds)."""
+    subprocess.run(["make", "-C", _HERE, "-B", "all"], check=True, capture_output=True)
+
+
+def _has_avx512() -> bool:
+    try:
+        with open("/proc/cpuinfo") as f:
+            for line in f:
+                if line.startswith("flags"):
+                    flags = line.split()
+                    return all(x in flags for x in ("avx512f", "avx512bw", "avx512vl", "avx512dq", "avx512cd"))
+    except OSError:
+        pass
+    return False
+
+
+def _load() -> C.CDLL:
+    names = ["libzref_avx512.so", "libzref.so"] if _has_avx512() else ["libzref.so"]
+    if not all(os.path.exists(os.path.join(_HERE, n)) for n in names[-1:]):
+        build()
+    for n in names:
+        p = os.path.join(_HERE, n)
+        if os.path.exists(p):
+            return C.CDLL(p)
+    raise OSError("oracle library missing; run make -C oracle")
+
+
+_lib = _load()
+_u8p = C.POINTER(C.c_uint8)
+_f32p = C.POINTER(C.c_float)
+_f64p = C.POINTER(C.c_double)
+
+_lib.zref_half.restype = C.c_float
+_lib.zref_half.argtypes = [C.c_uint16]
+_lib.zref_bf16_round.restype = C.c_float
+_lib.zref_bf16_round.argtypes = [C.c_float]
+_lib.zref_silu.restype = C.c_float
+_lib.zref_silu.argtypes = [C.c_float]
+_lib.zref_layout.restype = C.c_int
+_lib.zref_layout.argtypes = [C.c_int, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
+_lib.zref_scale_min_k4.argtypes = [C.c_uint, _u8p, _u8p, _u8p]
+_lib.zref_pack_scale_min_k4.argtypes = [C.c_uint, _u8p, C.c_uint8, C.c_uint8]
+_lib.zref_dequantize.restype = C.c_int
+_lib.zref_dequantize.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_size_t]
+_lib.zref_rms_norm.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_float]
+_lib.zref_matrix_init.restype = C.c_void_p
+_lib.zref_matrix_init.argtypes = [C.c_int, C.c_void_p, C.c_size_t, C.c_size_t, C.c_uint]
+_lib.zref_matrix_free.argtypes = [C.c_void_p]
+_lib.zref_matrix_row.argtypes = [C.c_void_p, C.c_size_t, C.c_void_p]
+_lib.zref_matmul.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_uint]
+_lib.zref_gate_up_silu.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_uint]
+_lib.zref_argmax.restype = C.c_uint32
+_lib.zref_argmax.argtypes = [C.c_void_p, C.c_size_t]
+_lib.zref_default_threads.restype = C.c_uint
+_lib.zref_row_bytes.restype = C.c_uint64
+_lib.zref_row_bytes.argtypes = [C.c_int, C.c_uint64]
+_lib.zref_repack_q8_0.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t]
+_lib.zref_matmul_slices.argtypes = [C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
+_lib.zref_matmul_f64.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint]
+
+
+def _ptr(a: np.ndarray) -> int:
+    return a.ctypes.data
+
+
+def layout(t: int) -> tuple[int, int]:
+    e, b = C.c_uint32(), C.c_uint32()
+    if not _lib.zref_layout(t, C.byref(e), C.byref(b)):
+        raise ValueError(f"unknown tensor type {t}")
+    return e.value, b.value
+
+
+def half(bits: int) -> float:
+    return _lib.zref_half(bits)
+
+
+def bf16_round(v: float) -> float:
+    return _lib.zref_bf16_round(v)
+
+
+def silu(x: float) -> float:
+    return _lib.zref_silu(x)
+
+
+def scale_min_k4(j: int, q: bytes | np.ndarray) -> tuple[int, int]:
+    buf = (C.c_uint8 * 12)(*bytes(q))
+    sc, m = C.c_uint8(), C.c_uint8()
+    _lib.zref_scale_min_k4(j, buf, C.byref(sc), C.byref(m))
+    return sc.value, m.value
+
+
+def pack_scale_min_k4(scs, ms) -> bytes:
+    """The 12 scale bytes holding (scs[j], ms[j]) for j < 8."""
+    buf = (C.c_uint8 * 12)()
+    for j in range(8):
+        _lib.zref_pack_scale_min_k4(j, buf, int(scs[j]), int(ms[j]))
+    return bytes(buf)
+
+
+def dequantize(t: int, data: np.ndarray, n: int) -> np.ndarray:
+    data = np.ascontiguousarray(data).view(np.uint8)
+    e, b = layout(t)
+    assert n % e == 0 and data.size >= n // e * b
+    out = np.empty(n, dtype=np.float32)
+    if _lib.zref_dequantize(t, _ptr(data), _ptr(out), n) != 0:
+        raise ValueError("UnsupportedTensorType")
+    return out
+
+
+def rms_norm(x: np.ndarray, w: np.ndarray, eps: float) -> np.ndarray:
+    out = np.array(x, dtype=np.float32, copy=True)
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    _lib.zref_rms_norm(_ptr(out), _ptr(w), out.size, eps)
+    return out
+
+
+def default_threads() -> int:
+    return _lib.zref_default_threads()
+
+
+class Matrix:
+    """An n x k weight matrix as the reference's multiply holds it."""
+
+    def __init__(self, t: int, data: np.ndarray, n: int, k: int, threads: int = 1):
+        self.bytes = np.ascontiguousarray(data).view(np.uint8)
+        e, b = layout(t)
+        assert self.bytes.size == n * k // e * b, (self.bytes.size, n, k)
+        self.t, self.n, self.k = t, n, k
+        self.h = _lib.zref_matrix_init(t, _ptr(self.bytes), n, k, threads)
+        if not self.h:
+            raise ValueError("zref_matrix_init failed")
+
+    def row(self, j: int) -> np.ndarray:
+        out = np.empty(self.k, dtype=np.float32)
+        _lib.zref_matrix_row(self.h, j, _ptr(out))
+        return out
+
+    def rows(self) -> np.ndarray:
+        """All weights decoded, n x k."""
+        if self.t in (Q8_0, Q4_K):
+            return dequantize(self.t, self.bytes, self.n * self.k).reshape(self.n, self.k)
+        return np.stack([self.row(j) for j in range(self.n)])
+
+    def __del__(self):
+        if getattr(self, "h", None):
+            _lib.zref_matrix_free(self.h)
+            self.h = None
+
+
+def matmul(x: np.ndarray, w: Matrix, threads: int = 1) -> np.ndarray:
+    """out[t][j] = sum_i x[t][i] w[j][i] in the reference's order of sums."""
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, w.k)
+    out = np.empty((x.shape[0], w.n), dtype=np.float32)
+    _lib.zref_matmul(_ptr(out), _ptr(x), w.h, x.shape[0], threads)
+    return out
+
+
+def gate_up_silu(x: np.ndarray, w: Matrix, half_rows: int, threads: int = 1) -> np.ndarray:
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, w.k)
+    assert w.n == 2 * half_rows
+    out = np.empty((x.shape[0], half_rows), dtype=np.float32)
+    _lib.zref_gate_up_silu(_ptr(out), _ptr(x), w.h, half_rows, x.shape[0], threads)
+    return out
+
+
+def argmax(v: np.ndarray) -> int:
+    v = np.ascontiguousarray(v, dtype=np.float32)
+    return _lib.zref_argmax(_ptr(v), v.size)
+
+
+def row_bytes(t: int, k: int) -> int:
+    return _lib.zref_row_bytes(t, k)
+
+
+def repack_q8_0(raw: np.ndarray, rows: int, k: int) -> np.ndarray:
+    raw = np.ascontiguousarray(raw).view(np.uint8)
+    assert raw.size == rows * k // 32 * 34
+    dst = np.empty(rows * row_bytes(Q8_0, k), dtype=np.uint8)
+    _lib.zref_repack_q8_0(_ptr(raw), _ptr(dst), rows, k)
+    return dst
+
+
+def matmul_slices(n: int, k: int) -> tuple[int, int]:
+    c, s = C.c_uint32(), C.c_uint32()
+    _lib.zref_matmul_slices(n, k, C.byref(c), C.byref(s))
+    return c.value, s.value
+
+
+def matmul_f64(x: np.ndarray, w: np.ndarray, threads: int = 0) -> np.ndarray:
+    """want[t][j] = sum_i x[t][i] w[j][i] in float64 over decoded weights."""
+    w = np.ascontiguousarray(w, dtype=np.float32)
+    n, k = w.shape
+    x = np.ascontiguousarray(x, dtype=np.float32).reshape(-1, k)
+    want = np.empty((x.shape[0], n), dtype=np.float64)
+    _lib.zref_matmul_f64(_ptr(want), _ptr(x), _ptr(w), x.shape[0], n, k, threads or default_threads())
+    return want

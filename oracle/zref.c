@@ -1,0 +1,546 @@
+/* CPU oracle: a plain-C restatement of the reference's src/ref path.
+ * TEST INFRASTRUCTURE ONLY: see zref.h. Build with -ffp-contract=off: the
+ * reference's decoders and microkernel are defined by separately rounded
+ * multiplies, subtracts and adds. */
+#define _GNU_SOURCE
+#include "zref.h"
+
+#include <math.h>
+#include <pthread.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+#include <unistd.h>
+
+/* ---- block geometry: src/gguf/gguf.zig:69-109 ------------------------------ */
+
+int zref_layout(int type, uint32_t *block_elems, uint32_t *block_bytes) {
+    uint32_t e, b;
+    switch (type) {
+    case ZREF_F32: e = 1; b = 4; break;
+    case ZREF_F16: case ZREF_BF16: e = 1; b = 2; break;
+    case ZREF_Q8_0: e = 32; b = 34; break;
+    case ZREF_Q4_K: e = 256; b = 144; break;
+    default: return 0;
+    }
+    if (block_elems) *block_elems = e;
+    if (block_bytes) *block_bytes = b;
+    return 1;
+}
+
+/* ---- scalar conversions ----------------------------------------------------- */
+
+static inline uint16_t rd16(const uint8_t *p) { return (uint16_t)(p[0] | (p[1] << 8)); }
+static inline uint32_t rd32(const uint8_t *p) {
+    return (uint32_t)p[0] | ((uint32_t)p[1] << 8) | ((uint32_t)p[2] << 16) | ((uint32_t)p[3] << 24);
+}
+static inline float bits_f32(uint32_t b) { float f; memcpy(&f, &b, 4); return f; }
+static inline uint32_t f32_bits(float f) { uint32_t b; memcpy(&b, &f, 4); return b; }
+
+/* src/ref/tensor.zig:45-47: the f16 widened to f32, which is exact. */
+float zref_half(uint16_t h) {
+    uint32_t sign = (uint32_t)(h & 0x8000u) << 16;
+    uint32_t exp = (h >> 10) & 0x1f;
+    uint32_t man = h & 0x3ff;
+    if (exp == 0) {
+        if (man == 0) return bits_f32(sign);
+        /* Subnormal: man * 2^-24, exact in f32. */
+        float v = (float)man * 5.9604644775390625e-8f;
+        return sign ? -v : v;
+    }
+    if (exp == 31) return bits_f32(sign | 0x7f800000u | (man << 13));
+    return bits_f32(sign | ((exp + 112) << 23) | (man << 13));
+}
+
+/* src/ref/matmul.zig:250-255. */
+float zref_bf16_round(float v) {
+    uint32_t bits = f32_bits(v);
+    uint32_t r = bits + (0x7fffu + ((bits >> 16) & 1u));
+    return bits_f32(r & 0xffff0000u);
+}
+
+/* src/ref/ops.zig:49-51. */
+float zref_silu(float x) { return x / (1.0f + expf(-x)); }
+
+/* src/ref/ops.zig:25-41: squares rounded to f32, summed and divided in f64,
+ * then an f32 mean, add, sqrt and reciprocal; x * scale, then * w. */
+void zref_rms_norm(float *x, const float *weight, size_t n, float eps) {
+    double sum = 0;
+    for (size_t i = 0; i < n; i++) {
+        float square = x[i] * x[i];
+        sum += square;
+    }
+    float mean = (float)(sum / (double)n);
+    float scale = 1.0f / sqrtf(mean + eps);
+    for (size_t i = 0; i < n; i++) {
+        float t = x[i] * scale;
+        x[i] = t * weight[i];
+    }
+}
+
+/* ---- decoders: src/ref/tensor.zig ------------------------------------------- */
+
+/* src/ref/tensor.zig:94-98. */
+void zref_scale_min_k4(unsigned j, const uint8_t q[12], uint8_t *sc, uint8_t *m) {
+    if (j < 4) {
+        *sc = q[j] & 63;
+        *m = q[j + 4] & 63;
+    } else {
+        *sc = (uint8_t)((q[j + 4] & 0xF) | ((q[j - 4] >> 6) << 4));
+        *m = (uint8_t)((q[j + 4] >> 4) | ((q[j] >> 6) << 4));
+    }
+}
+
+void zref_pack_scale_min_k4(unsigned j, uint8_t q[12], uint8_t sc, uint8_t m) {
+    if (j < 4) {
+        q[j] = (uint8_t)((q[j] & 0xC0) | (sc & 63));
+        q[j + 4] = (uint8_t)((q[j + 4] & 0xC0) | (m & 63));
+    } else {
+        q[j + 4] = (uint8_t)((sc & 0xF) | ((m & 0xF) << 4));
+        q[j - 4] = (uint8_t)((q[j - 4] & 63) | ((sc >> 4) << 6));
+        q[j] = (uint8_t)((q[j] & 63) | ((m >> 4) << 6));
+    }
+}
+
+/* src/ref/tensor.zig:49-53: one f32 multiply per weight. */
+static void q8_0_block(const uint8_t *b, float *y) {
+    float d = zref_half(rd16(b));
+    for (int i = 0; i < 32; i++) y[i] = (float)(int8_t)b[2 + i] * d;
+}
+
+/* src/ref/tensor.zig:100-116: d1 = d*sc, m1 = dmin*m (one rounding each),
+ * then d1*q - m1 as a multiply followed by a subtract. */
+static void q4_k_block(const uint8_t *b, float *y) {
+    float d = zref_half(rd16(b));
+    float min = zref_half(rd16(b + 2));
+    const uint8_t *scales = b + 4;
+    for (unsigned j = 0; j < 4; j++) {
+        const uint8_t *q = b + 16 + 32 * j;
+        uint8_t sc1, mn1, sc2, mn2;
+        zref_scale_min_k4(2 * j, scales, &sc1, &mn1);
+        zref_scale_min_k4(2 * j + 1, scales, &sc2, &mn2);
+        float d1 = d * (float)sc1;
+        float m1 = min * (float)mn1;
+        float d2 = d * (float)sc2;
+        float m2 = min * (float)mn2;
+        for (int l = 0; l < 32; l++) {
+            float p = d1 * (float)(q[l] & 0xF);
+            y[64 * j + l] = p - m1;
+        }
+        for (int l = 0; l < 32; l++) {
+            float p = d2 * (float)(q[l] >> 4);
+            y[64 * j + 32 + l] = p - m2;
+        }
+    }
+}
+
+/* src/ref/tensor.zig:21-43. */
+int zref_dequantize(int type, const uint8_t *bytes, float *out, size_t n) {
+    switch (type) {
+    case ZREF_Q8_0:
+        for (size_t i = 0; i < n / 32; i++) q8_0_block(bytes + i * 34, out + i * 32);
+        return 0;
+    case ZREF_Q4_K:
+        for (size_t i = 0; i < n / 256; i++) q4_k_block(bytes + i * 144, out + i * 256);
+        return 0;
+    case ZREF_F32:
+        for (size_t i = 0; i < n; i++) out[i] = bits_f32(rd32(bytes + 4 * i));
+        return 0;
+    case ZREF_F16:
+        for (size_t i = 0; i < n; i++) out[i] = zref_half(rd16(bytes + 2 * i));
+        return 0;
+    case ZREF_BF16:
+        for (size_t i = 0; i < n; i++) out[i] = bits_f32((uint32_t)rd16(bytes + 2 * i) << 16);
+        return 0;
+    default:
+        return -1;
+    }
+}
+
+/* ---- fork-join pool: src/ref/pool.zig:76-122 --------------------------------
+ * Persistent workers; parallel_for splits [0, n) into contiguous ranges, the
+ * caller taking the range after all workers' ranges. */
+
+typedef void (*range_fn)(void *ctx, size_t first, size_t last);
+
+typedef struct pool {
+    unsigned workers; /* threads besides the caller */
+    pthread_t *threads;
+    pthread_mutex_t mu;
+    pthread_cond_t wake, done;
+    unsigned long generation;
+    unsigned pending;
+    int stop;
+    range_fn fn;
+    void *ctx;
+    size_t n, chunk;
+} pool;
+
+typedef struct { pool *p; unsigned index; } worker_arg;
+
+static void run_range(pool *p, unsigned index) {
+    size_t first = (size_t)index * p->chunk;
+    if (first >= p->n) return;
+    size_t last = first + p->chunk;
+    if (last > p->n) last = p->n;
+    p->fn(p->ctx, first, last);
+}
+
+static void *worker_main(void *argp) {
+    worker_arg *arg = (worker_arg *)argp;
+    pool *p = arg->p;
+    unsigned index = arg->index;
+    free(arg);
+    unsigned long seen = 0;
+    for (;;) {
+        pthread_mutex_lock(&p->mu);
+        while (p->generation == seen && !p->stop) pthread_cond_wait(&p->wake, &p->mu);
+        if (p->stop) { pthread_mutex_unlock(&p->mu); return NULL; }
+        seen = p->generation;
+        pthread_mutex_unlock(&p->mu);
+        run_range(p, index);
+        pthread_mutex_lock(&p->mu);
+        if (--p->pending == 0) pthread_cond_signal(&p->done);
+        pthread_mutex_unlock(&p->mu);
+    }
+}
+
+static pool *pool_create(unsigned threads) {
+    pool *p = (pool *)calloc(1, sizeof *p);
+    p->workers = threads > 0 ? threads - 1 : 0;
+    pthread_mutex_init(&p->mu, NULL);
+    pthread_cond_init(&p->wake, NULL);
+    pthread_cond_init(&p->done, NULL);
+    p->threads = (pthread_t *)calloc(p->workers ? p->workers : 1, sizeof(pthread_t));
+    for (unsigned i = 0; i < p->workers; i++) {
+        worker_arg *a = (worker_arg *)malloc(sizeof *a);
+        a->p = p; a->index = i;
+        pthread_create(&p->threads[i], NULL, worker_main, a);
+    }
+    return p;
+}
+
+/* One cached pool per thread count requested, kept for the process's life as
+ * the reference keeps its pool for the run. */
+static pool *pool_get(unsigned threads) {
+    static pool *cache[8];
+    static unsigned counts[8];
+    static pthread_mutex_t mu = PTHREAD_MUTEX_INITIALIZER;
+    if (threads == 0) threads = 1;
+    pthread_mutex_lock(&mu);
+    pool *found = NULL;
+    for (int i = 0; i < 8; i++) {
+        if (cache[i] && counts[i] == threads) { found = cache[i]; break; }
+    }
+    if (!found) {
+        for (int i = 0; i < 8; i++) {
+            if (!cache[i]) { cache[i] = found = pool_create(threads); counts[i] = threads; break; }
+        }
+    }
+    pthread_mutex_unlock(&mu);
+    if (!found) { fprintf(stderr, "zref: too many distinct pool sizes\n"); abort(); }
+    return found;
+}
+
+/* src/ref/pool.zig:79-101. */
+static void parallel_for(pool *p, size_t n, size_t align_to, size_t min_chunk, void *ctx, range_fn fn) {
+    size_t thread_count = (size_t)p->workers + 1;
+    size_t by_chunk = n / (min_chunk ? min_chunk : 1);
+    size_t parts = thread_count < by_chunk ? thread_count : by_chunk;
+    if (parts < 1) parts = 1;
+    size_t chunk = (n + parts - 1) / parts;
+    chunk = (chunk + align_to - 1) / align_to * align_to;
+    if (parts == 1 || p->workers == 0) { fn(ctx, 0, n); return; }
+    pthread_mutex_lock(&p->mu);
+    p->fn = fn; p->ctx = ctx; p->n = n; p->chunk = chunk;
+    p->pending = p->workers;
+    p->generation++;
+    pthread_cond_broadcast(&p->wake);
+    pthread_mutex_unlock(&p->mu);
+    run_range(p, p->workers);
+    pthread_mutex_lock(&p->mu);
+    while (p->pending != 0) pthread_cond_wait(&p->done, &p->mu);
+    pthread_mutex_unlock(&p->mu);
+}
+
+/* src/main.zig:438-448. */
+unsigned zref_default_threads(void) {
+    const char *env = getenv("ZLLM_THREADS");
+    if (env) {
+        long v = strtol(env, NULL, 10);
+        if (v > 0) return (unsigned)v;
+    }
+    long logical = sysconf(_SC_NPROCESSORS_ONLN);
+    if (logical < 1) logical = 1;
+    FILE *f = fopen("/sys/devices/system/cpu/smt/active", "r");
+    if (!f) return (unsigned)logical;
+    int c = fgetc(f);
+    fclose(f);
+    if (c == '1') return (unsigned)(logical / 2 > 0 ? logical / 2 : 1);
+    return (unsigned)logical;
+}
+
+/* ---- matrix multiply: src/ref/matmul.zig ------------------------------------ */
+
+#define PANEL 32
+#define BLOCK_ROWS 8
+
+struct zref_matrix {
+    float *data; /* packed panels for f32/f16/bf16, NULL for quantized */
+    size_t n, k;
+    int type;
+    const uint8_t *quant; /* raw rows for quantized types */
+};
+
+/* src/ref/matmul.zig:111-133: rows [p*32, p*32+32) decoded k-major, rows past
+ * n zero, decoded in pieces of 256 elements. */
+static void pack_panel(int type, const uint8_t *bytes, size_t n, size_t k, size_t p, float *dst) {
+    uint32_t be, bb;
+    zref_layout(type, &be, &bb);
+    size_t row_bytes = k / be * bb;
+    float buf[256];
+    for (size_t col = 0; col < PANEL; col++) {
+        size_t j = p * PANEL + col;
+        if (j >= n) {
+            for (size_t i = 0; i < k; i++) dst[i * PANEL + col] = 0;
+            continue;
+        }
+        const uint8_t *src = bytes + j * row_bytes;
+        for (size_t start = 0; start < k; start += 256) {
+            size_t len = k - start < 256 ? k - start : 256;
+            size_t b0 = start / be * bb;
+            zref_dequantize(type, src + b0, buf, len);
+            for (size_t i = 0; i < len; i++) dst[(start + i) * PANEL + col] = buf[i];
+        }
+    }
+}
+
+typedef struct { zref_matrix *m; const uint8_t *bytes; } pack_ctx;
+
+static void pack_run(void *ctxp, size_t first, size_t last) {
+    pack_ctx *c = (pack_ctx *)ctxp;
+    for (size_t p = first; p < last; p++)
+        pack_panel(c->m->type, c->bytes, c->m->n, c->m->k, p, c->m->data + p * PANEL * c->m->k);
+}
+
+static size_t panels_of(const zref_matrix *m) { return (m->n + PANEL - 1) / PANEL; }
+
+/* src/ref/matmul.zig:56-82. */
+zref_matrix *zref_matrix_init(int type, const uint8_t *bytes, size_t n, size_t k, unsigned threads) {
+    uint32_t be, bb;
+    if (!zref_layout(type, &be, &bb) || k % be != 0) return NULL;
+    zref_matrix *m = (zref_matrix *)calloc(1, sizeof *m);
+    m->n = n; m->k = k; m->type = type;
+    if (type == ZREF_Q8_0 || type == ZREF_Q4_K) {
+        m->quant = bytes;
+        return m;
+    }
+    size_t n_panels = panels_of(m);
+    if (posix_memalign((void **)&m->data, 64, n_panels * PANEL * k * sizeof(float)) != 0) { free(m); return NULL; }
+    pack_ctx ctx = { m, bytes };
+    parallel_for(pool_get(threads), n_panels, 1, 1, &ctx, pack_run);
+    return m;
+}
+
+void zref_matrix_free(zref_matrix *m) {
+    if (!m) return;
+    free(m->data);
+    free(m);
+}
+
+/* src/ref/matmul.zig:94-106. */
+void zref_matrix_row(const zref_matrix *m, size_t j, float *out) {
+    if (m->quant) {
+        uint32_t be, bb;
+        zref_layout(m->type, &be, &bb);
+        size_t row_bytes = m->k / be * bb;
+        zref_dequantize(m->type, m->quant + j * row_bytes, out, m->k);
+        return;
+    }
+    const float *base = m->data + (j / PANEL) * PANEL * m->k + j % PANEL;
+    for (size_t i = 0; i < m->k; i++) out[i] = base[i * PANEL];
+}
+
+typedef struct {
+    float *out;
+    const float *x;
+    const zref_matrix *w;
+    size_t rows;
+} mm_ctx;
+
+/* src/ref/matmul.zig:262-294: R tokens x 32 outputs; for each i the panel's
+ * 32-wide weight row times one broadcast activation per token, accumulated
+ * with a separate multiply and add; outputs clipped to n. */
+#define MICROKERNEL(R)                                                                     \
+    static void microkernel_##R(const mm_ctx *c, const float *wp, size_t p, size_t t0) {   \
+        size_t k = c->w->k;                                                                \
+        float acc[R][PANEL];                                                               \
+        const float *xp[R];                                                                \
+        for (int a = 0; a < R; a++) {                                                      \
+            xp[a] = c->x + (t0 + a) * k;                                                   \
+            for (int cc = 0; cc < PANEL; cc++) acc[a][cc] = 0;                             \
+        }                                                                                  \
+        for (size_t i = 0; i < k; i++) {                                                   \
+            const float *w = wp + i * PANEL;                                               \
+            for (int a = 0; a < R; a++) {                                                  \
+                float xb = xp[a][i];                                                       \
+                for (int cc = 0; cc < PANEL; cc++) {                                       \
+                    float prod = xb * w[cc];                                               \
+                    acc[a][cc] = acc[a][cc] + prod;                                        \
+                }                                                                          \
+            }                                                                              \
+        }                                                                                  \
+        size_t n = c->w->n;                                                                \
+        size_t j0 = p * PANEL;                                                             \
+        size_t cols = n - j0 < PANEL ? n - j0 : PANEL;                                     \
+        for (int a = 0; a < R; a++) memcpy(c->out + (t0 + a) * n + j0, acc[a], cols * sizeof(float)); \
+    }
+
+MICROKERNEL(1)
+MICROKERNEL(2)
+MICROKERNEL(3)
+MICROKERNEL(4)
+MICROKERNEL(5)
+MICROKERNEL(6)
+MICROKERNEL(7)
+MICROKERNEL(8)
+
+/* src/ref/matmul.zig:135-145: each thread's panel buffer, grown as needed and
+ * kept for the life of the thread. */
+static __thread float *panel_buf;
+static __thread size_t panel_buf_len;
+
+static float *thread_panel(size_t k) {
+    if (panel_buf_len < PANEL * k) {
+        free(panel_buf);
+        if (posix_memalign((void **)&panel_buf, 64, PANEL * k * sizeof(float)) != 0) abort();
+        panel_buf_len = PANEL * k;
+    }
+    return panel_buf;
+}
+
+/* src/ref/matmul.zig:177-192. */
+static void mm_run(void *ctxp, size_t first, size_t last) {
+    const mm_ctx *c = (const mm_ctx *)ctxp;
+    for (size_t p = first; p < last; p++) {
+        const float *wp;
+        if (c->w->quant) {
+            float *buf = thread_panel(c->w->k);
+            pack_panel(c->w->type, c->w->quant, c->w->n, c->w->k, p, buf);
+            wp = buf;
+        } else {
+            wp = c->w->data + p * PANEL * c->w->k;
+        }
+        for (size_t t = 0; t < c->rows; t += BLOCK_ROWS) {
+            size_t r = c->rows - t < BLOCK_ROWS ? c->rows - t : BLOCK_ROWS;
+            switch (r) {
+            case 1: microkernel_1(c, wp, p, t); break;
+            case 2: microkernel_2(c, wp, p, t); break;
+            case 3: microkernel_3(c, wp, p, t); break;
+            case 4: microkernel_4(c, wp, p, t); break;
+            case 5: microkernel_5(c, wp, p, t); break;
+            case 6: microkernel_6(c, wp, p, t); break;
+            case 7: microkernel_7(c, wp, p, t); break;
+            default: microkernel_8(c, wp, p, t); break;
+            }
+        }
+    }
+}
+
+/* src/ref/matmul.zig:160-195 (Activations.f32). */
+void zref_matmul(float *out, const float *x, const zref_matrix *w, size_t rows, unsigned threads) {
+    mm_ctx ctx = { out, x, w, rows };
+    parallel_for(pool_get(threads), panels_of(w), 1, 1, &ctx, mm_run);
+}
+
+typedef struct { float *gate; const float *up; size_t ff; } act_ctx;
+
+static void act_run(void *ctxp, size_t first, size_t last) {
+    act_ctx *c = (act_ctx *)ctxp;
+    for (size_t i = first * c->ff; i < last * c->ff; i++) c->gate[i] = zref_silu(c->gate[i]) * c->up[i];
+}
+
+/* src/ref/dense.zig:179-195: gate and up multiplies, then silu(g)*u split by
+ * token rows across the pool. */
+void zref_gate_up_silu(float *act, const float *x, const zref_matrix *w, size_t half, size_t rows, unsigned threads) {
+    float *gu = (float *)malloc(rows * w->n * sizeof(float));
+    zref_matmul(gu, x, w, rows, threads);
+    float *up = (float *)malloc(rows * half * sizeof(float));
+    for (size_t t = 0; t < rows; t++) {
+        memcpy(act + t * half, gu + t * w->n, half * sizeof(float));
+        memcpy(up + t * half, gu + t * w->n + half, half * sizeof(float));
+    }
+    act_ctx ctx = { act, up, half };
+    parallel_for(pool_get(threads), rows, 1, 1, &ctx, act_run);
+    free(up);
+    free(gu);
+}
+
+/* src/kernels/draft.wgsl:1-4. */
+uint32_t zref_argmax(const float *v, size_t n) {
+    uint32_t at = 0;
+    for (size_t i = 1; i < n; i++)
+        if (v[i] > v[at]) at = (uint32_t)i;
+    return at;
+}
+
+/* ---- GPU-side layouts --------------------------------------------------------- */
+
+/* src/kernels/kernels.zig:144-160. */
+uint64_t zref_row_bytes(int type, uint64_t k) {
+    if (type == ZREF_Q8_0) return (k + k / 16 + 15) & ~(uint64_t)15;
+    uint32_t be, bb;
+    if (!zref_layout(type, &be, &bb)) return 0;
+    return k / be * bb;
+}
+
+/* src/kernels/repack_q8_0.wgsl:26-51. */
+void zref_repack_q8_0(const uint8_t *src, uint8_t *dst, size_t rows, size_t k) {
+    size_t stride = (size_t)zref_row_bytes(ZREF_Q8_0, k);
+    size_t blocks = k / 32;
+    for (size_t r = 0; r < rows; r++) {
+        const uint8_t *raw = src + r * blocks * 34;
+        uint8_t *row = dst + r * stride;
+        memset(row, 0, stride);
+        for (size_t b = 0; b < blocks; b++) {
+            memcpy(row + 32 * b, raw + 34 * b + 2, 32);
+            row[k + 2 * b] = raw[34 * b];
+            row[k + 2 * b + 1] = raw[34 * b + 1];
+        }
+    }
+}
+
+/* src/kernels/kernels.zig:285-295. */
+void zref_matmul_slices(uint32_t n, uint32_t k, uint32_t *count, uint32_t *k_slice) {
+    const uint32_t tile_n = 128, target = 256, min_slice = 512;
+    uint32_t tiles = (n + tile_n - 1) / tile_n;
+    uint32_t want = (target + tiles - 1) / tiles;
+    uint32_t hi = k / min_slice > 1 ? k / min_slice : 1;
+    uint32_t c = want < 1 ? 1 : (want > hi ? hi : want);
+    uint32_t ks = (k + c - 1) / c;
+    ks = (ks + 31) / 32 * 32;
+    *count = (k + ks - 1) / ks;
+    *k_slice = ks;
+}
+
+/* ---- float64 formula checker: src/kernels/check.zig ---------------------------- */
+
+typedef struct { double *want; const float *x; const float *w; size_t rows, n, k; } f64_ctx;
+
+static void f64_run(void *ctxp, size_t first, size_t last) {
+    f64_ctx *c = (f64_ctx *)ctxp;
+    for (size_t j = first; j < last; j++) {
+        const float *wr = c->w + j * c->k;
+        for (size_t t = 0; t < c->rows; t++) {
+            const float *xr = c->x + t * c->k;
+            double s = 0;
+            for (size_t i = 0; i < c->k; i++) s += (double)xr[i] * (double)wr[i];
+            c->want[t * c->n + j] = s;
+        }
+    }
+}
+
+void zref_matmul_f64(double *want, const float *x, const float *w, size_t rows, size_t n, size_t k, unsigned threads) {
+    f64_ctx ctx = { want, x, w, rows, n, k };
+    parallel_for(pool_get(threads), n, 1, 1, &ctx, f64_run);
+}

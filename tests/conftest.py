@@ -1,0 +1,29 @@
+import os
+import sys
+
+import pytest
+
+sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+
+
+def pytest_configure(config):
+    config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
+
+
+@pytest.fixture(scope="session")
+def device():
+    """The one GPU, opened once per test process."""
+    from zllm_amd import Device
+
+    d = Device.open(0)
+    yield d
+    d.deinit()
+
+
+@pytest.fixture()
+def ctx(device):
+    from gpucheck import Ctx
+
+    c = Ctx(device)
+    yield c
+    c.close()

@@ -1,0 +1,366 @@
+"""Kernel checks on the GPU, case for case as the reference's gpu-check runs
+them for this path (src/kernels/check.zig): each kernel on seeded inputs
+through the command stream, against a float64 computation over weights decoded
+by the CPU oracle. Tolerances are the reference's own (1e-5 of the output
+scale; 0 for gathers), written beside each case.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from gpucheck import bound_err, rel_err
+from zllm_amd import kernels as K
+from zllm_amd import synth
+from zllm_amd.kernels import Kernel, TensorType, params as P
+
+pytestmark = pytest.mark.gpu
+
+ORACLE_TYPE = {TensorType.q8_0: oracle.Q8_0, TensorType.q4_k: oracle.Q4_K, TensorType.bf16: oracle.BF16}
+
+
+def quant_rows(c, t: TensorType, rows: int, k: int):
+    """Random blocks with finite super-scales and their oracle-decoded values
+    (src/kernels/check.zig:461-481)."""
+    raw = synth.random_blocks(c.rand, t.name, rows, k)
+    return raw, oracle.dequantize(ORACLE_TYPE[t], raw, rows * k).reshape(rows, k)
+
+
+def random_half(c, n: int, scale: float):
+    """bf16 weights and their f32 values (src/kernels/check.zig randomHalf)."""
+    bits = synth.to_bf16_bits(c.random(n, scale))
+    return bits, synth.bf16_bits_to_f32(bits)
+
+
+def norm_row(x, w, eps):
+    """out = rmsnorm(x) * w in float64 when w is given, else x
+    (src/kernels/check.zig:370-376)."""
+    x = x.astype(np.float64)
+    if w is None:
+        return x
+    scale = 1.0 / np.sqrt(np.sum(x * x) / x.size + eps)
+    return x * scale * w.astype(np.float64)
+
+
+def sigmoid64(x):
+    return 1.0 / (1.0 + np.exp(-x))
+
+
+# ---- half-precision decode multiply: check.zig:327-442 ------------------------------
+
+def matvec_case(c, k, split, fused):
+    rows, n, eps = 3, 100, 1e-6
+    x = c.random(rows * k, 3).reshape(rows, k)
+    nw = c.random(k, 1)
+    bits, values = random_half(c, n * k, 1)
+    bits, values = bits.reshape(n, k), values.reshape(n, k)
+    init = c.random(rows * n, 4 if fused else 0).reshape(rows, n)
+    out, xa, na = c.upload(init), c.upload(x), c.upload(nw)
+    col0 = 0
+    for cols in (split, n - split):
+        wa = c.upload(bits[col0 : col0 + cols])
+        c.launcher().launch(Kernel.matvec_bf16, P.MatvecBf16(n=cols, k=k, col0=col0, out_stride=n, eps=eps, norm=fused, accumulate=fused),
+                            [xa, wa, out, na], (K.div_ceil(cols, K.matvec_rows), rows, 1))
+        col0 += cols
+    got = c.read(out).reshape(rows, n)
+    want = np.stack([norm_row(x[t], nw if fused else None, eps) @ values.astype(np.float64).T for t in range(rows)]) + init
+    return rel_err(got, want)
+
+
+def test_matvec_bf16_two_chunks(ctx):
+    # k = 4000 leaves a partial pass over the lanes; 100 outputs a partial group.
+    assert matvec_case(ctx, 4000, 37, False) <= 1e-5
+
+
+def test_matvec_bf16_norm_accumulate(ctx):
+    assert matvec_case(ctx, 1000, 37, True) <= 1e-5
+
+
+def test_matvec_bf16_silu_pair(ctx):
+    c = ctx
+    rows, ff, k, eps = 3, 100, 1024, 1e-6
+    x = c.random(rows * k, 3).reshape(rows, k)
+    nw = c.random(k, 1)
+    bits, values = random_half(c, 2 * ff * k, 1)
+    values = values.reshape(2 * ff, k).astype(np.float64)
+    out = c.output(rows * ff)
+    c.launcher().launch(Kernel.matvec_bf16, P.MatvecBf16(n=ff, k=k, col0=0, out_stride=ff, eps=eps, norm=True, silu_pair=True, half=ff),
+                        [c.upload(x), c.upload(bits), out, c.upload(nw)], (K.div_ceil(ff, K.matvec_rows), rows, 1))
+    got = c.read(out).reshape(rows, ff)
+    want = np.empty((rows, ff))
+    for t in range(rows):
+        xn = norm_row(x[t], nw, eps)
+        g, u = values[:ff] @ xn, values[ff:] @ xn
+        want[t] = g * sigmoid64(g) * u
+    assert rel_err(got, want) <= 1e-5
+
+
+# ---- quantized decode multiply: check.zig:988-1060 ------------------------------------
+
+def quant_matvec(c, t: TensorType, k: int, pair: bool, variants=None):
+    """3 tokens, 100 outputs, norm prologue and accumulate epilogue, or the
+    SiLU pair over stacked gate and up rows; every variant tuning may pick; each
+    token alone must give the same bits as in the 3-token launch."""
+    rows, n, eps = 3, 100, 1e-6
+    x = c.random(rows * k, 3).reshape(rows, k)
+    nw = c.random(k, 1)
+    raw, values = quant_rows(c, t, 2 * n if pair else n, k)
+    init = c.random(rows * n, 0 if pair else 4).reshape(rows, n)
+    kernel = K.weight_kernel("matvec", t)
+    xa, wa, na = c.upload(x), c.gpu_weights(t, raw, k), c.upload(nw)
+    worst, split_exact = 0.0, True
+    want = np.empty((rows, n))
+    v64 = values.astype(np.float64)
+    for tk in range(rows):
+        xn = norm_row(x[tk], nw, eps)
+        g = v64[:n] @ xn
+        want[tk] = g * sigmoid64(g) * (v64[n:] @ xn) if pair else init[tk] + g
+    for v in variants or K.MatvecVariant.candidates:
+        if not v.suits(t):
+            continue
+        p = lambda: P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, eps=eps, norm=True, accumulate=not pair, silu_pair=pair, half=n if pair else 0)
+        pipeline = c.set.matvec(c.rec, kernel, v)
+        out = c.upload(init)
+        c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, na], (K.div_ceil(n, v.group_rows()), rows, 1))
+        got = c.read(out).reshape(rows, n)
+        for tk in range(rows):
+            single = c.upload(init[tk])
+            c.launcher().launch_pipeline(pipeline, p(), [c.upload(x[tk]), wa, single, na], (K.div_ceil(n, v.group_rows()), 1, 1))
+            split_exact &= got[tk].tobytes() == c.read(single).tobytes()
+        worst = max(worst, rel_err(got, want))
+    return worst, split_exact
+
+
+@pytest.mark.parametrize("t,k,pair", [
+    (TensorType.q8_0, 1024, False),   # "matvec q8_0 norm+="
+    (TensorType.q4_k, 1024, False),   # "matvec q4_k norm+="
+    (TensorType.q4_k, 4096, False),   # "matvec q4_k norm+= (2 tiles)"
+    (TensorType.q8_0, 4160, True),    # "matvec q8_0 norm+silu (tile tail, bitwise splits)"
+    (TensorType.q4_k, 1024, True),    # the SiLU pair on Q4_K (the reference runs it on q3_k)
+])
+def test_quant_matvec(ctx, t, k, pair):
+    worst, split_exact = quant_matvec(ctx, t, k, pair)
+    assert split_exact, "a token's sums differ between a lone launch and a multi-token launch"
+    assert worst <= 1e-5
+
+
+def test_quant_matvec_act_prologue(ctx):
+    """hc_act fused into the multiply after it: each input staged as
+    silu(x / 4), read from rows 264 floats apart (src/kernels/check.zig:1082-1116)."""
+    c = ctx
+    rows, n, k, div = 3, 100, 256, 4
+    stride = k + 8
+    x = c.random(rows * stride, 3).reshape(rows, stride)
+    raw, values = quant_rows(c, TensorType.q8_0, n, k)
+    xa, wa = c.upload(x), c.gpu_weights(TensorType.q8_0, raw, k)
+    v = x[:, :k].astype(np.float64) / div
+    want = (v * sigmoid64(v)) @ values.astype(np.float64).T
+    worst = 0.0
+    for cand in K.MatvecVariant.candidates:
+        var = K.MatvecVariant(cand.wg, cand.lanes, cand.rows, div)
+        out = c.output(rows * n)
+        c.launcher().launch_pipeline(c.set.matvec(c.rec, Kernel.matvec_q8_0, var), P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, x_stride=stride // 4),
+                                     [xa, wa, out, wa], (K.div_ceil(n, var.group_rows()), rows, 1))
+        worst = max(worst, rel_err(c.read(out).reshape(rows, n), want))
+    assert worst <= 1e-5
+
+
+def test_quant_matvec_eight_rows(ctx):
+    """Steps of 5..8 tokens (the HIP backend's extension past the reference's
+    four): every row correct and bitwise equal to its lone launch."""
+    c = ctx
+    n, k, rows = 96, 1024, 8
+    x = c.random(rows * k, 3).reshape(rows, k)
+    raw, values = quant_rows(c, TensorType.q4_k, 2 * n, k)
+    xa, wa = c.upload(x), c.gpu_weights(TensorType.q4_k, raw, k)
+    p = lambda: P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, silu_pair=True, half=n)
+    out = c.output(rows * n)
+    c.launcher().launch(Kernel.matvec_q4_k, p(), [xa, wa, out, wa], (K.div_ceil(n, 8), rows, 1))
+    got = c.read(out).reshape(rows, n)
+    v64 = values.astype(np.float64)
+    g, u = x.astype(np.float64) @ v64[:n].T, x.astype(np.float64) @ v64[n:].T
+    assert rel_err(got, g * sigmoid64(g) * u) <= 1e-5
+    for tk in range(rows):
+        single = c.output(n)
+        c.launcher().launch(Kernel.matvec_q4_k, p(), [c.upload(x[tk]), wa, single, wa], (K.div_ceil(n, 8), 1, 1))
+        assert got[tk].tobytes() == c.read(single)[:n].tobytes()
+
+
+# ---- block decoders bit for bit, through the embedding gathers: check.zig:873-905 -----
+
+@pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q4_k])
+def test_embed_quant_bit_exact(ctx, t):
+    c = ctx
+    vocab, dim, split = 50, 512, 30
+    e, b = K.LAYOUT[t]
+    rb = dim // e * b
+    raw, values = quant_rows(c, t, vocab, dim)
+    raw = raw.reshape(vocab, rb)
+    tokens = np.array([0, 29, 30, 49, 7, 30, 12], dtype=np.uint32)
+    out = c.output(tokens.size * dim)
+    ta = c.upload(tokens)
+    for row0, rows in ((0, split), (split, vocab - split)):
+        wa = c.gpu_weights(t, raw[row0 : row0 + rows], dim)
+        c.launcher().launch(K.weight_kernel("embed", t), P.EmbedBf16(dim=dim, row0=row0, chunk_rows=rows), [ta, wa, out], (tokens.size, 1, 1))
+    got = c.read_words(out).reshape(tokens.size, dim)
+    want = values[tokens].view(np.uint32)
+    assert np.array_equal(got, want), f"{np.count_nonzero(got != want)} decoded weights differ in their bits"
+
+
+def test_embed_q8_0_file_rows(ctx):
+    """Rows laid out as in the GGUF file, `stride` bytes apart
+    (src/kernels/embed_quant.wgsl:4-6)."""
+    c = ctx
+    vocab, dim = 9, 256
+    stride = dim // 32 * 34 + 12
+    raw, values = quant_rows(c, TensorType.q8_0, vocab, dim)
+    table = np.zeros((vocab, stride), dtype=np.uint8)
+    table[:, : dim // 32 * 34] = raw.reshape(vocab, -1)
+    tokens = np.array([8, 0, 3], dtype=np.uint32)
+    out = c.output(tokens.size * dim)
+    c.launcher().launch(Kernel.embed_q8_0, P.EmbedBf16(dim=dim, row0=0, chunk_rows=vocab, stride=stride), [c.upload(tokens), c.upload(table), out], (tokens.size, 1, 1))
+    assert np.array_equal(c.read_words(out).reshape(tokens.size, dim), values[tokens].view(np.uint32))
+
+
+def test_embed_bf16_exact(ctx):
+    c = ctx
+    vocab, dim, split = 50, 64, 30
+    bits, values = random_half(c, vocab * dim, 1)
+    bits, values = bits.reshape(vocab, dim), values.reshape(vocab, dim)
+    tokens = np.array([0, 29, 30, 49, 7, 30, 12], dtype=np.uint32)
+    out = c.output(tokens.size * dim)
+    ta = c.upload(tokens)
+    for row0, rows in ((0, split), (split, vocab - split)):
+        c.launcher().launch(Kernel.embed_bf16, P.EmbedBf16(dim=dim, row0=row0, chunk_rows=rows), [ta, c.upload(bits[row0 : row0 + rows]), out], (tokens.size, 1, 1))
+    assert np.array_equal(c.read(out).reshape(tokens.size, dim), values[tokens])
+
+
+def test_repack_q8_0_matches_split_row_layout(ctx):
+    c = ctx
+    rows, k = 37, 320  # 320 + 20 scale bytes pads to 352
+    raw, _ = quant_rows(c, TensorType.q8_0, rows, k)
+    wa = c.gpu_weights(TensorType.q8_0, raw, k)
+    got = c.read_bytes(wa)[: rows * K.row_bytes(TensorType.q8_0, k)]
+    assert np.array_equal(got, oracle.repack_q8_0(raw, rows, k))
+
+
+def test_repad_pads_blocks(ctx):
+    c = ctx
+    blocks, src_bytes, dst_bytes = 23, 110, 128  # a block size that is not a multiple of 4
+    raw = c.rand.integers(0, 256, size=(blocks, src_bytes), dtype=np.uint8)
+    padded = np.zeros(((raw.size + 15) & ~15), dtype=np.uint8)
+    padded[: raw.size] = raw.reshape(-1)
+    out = c.output(blocks * dst_bytes // 4)
+    c.launcher().launch(Kernel.repad, P.Repad(blocks, src_bytes, dst_bytes), [c.upload(padded), out], K.elementwise(blocks * dst_bytes // 4))
+    got = c.read_bytes(out).reshape(blocks, dst_bytes)
+    assert np.array_equal(got[:, :src_bytes], raw) and not got[:, src_bytes:].any()
+
+
+# ---- prefill multiplies: check.zig:288-325, 752-825 -------------------------------------
+
+def matmul_case(c, rows, n, k, split, accumulate, rung=K.Prefill.scalar_f32):
+    x = c.random(rows * k, 1).reshape(rows, k)
+    bits, values = random_half(c, n * k, 1)
+    bits, values = bits.reshape(n, k), values.reshape(n, k)
+    init = c.random(rows * n, 4 if accumulate else 0).reshape(rows, n)
+    out, xa = c.upload(init), c.upload(x)
+    c.set.select_prefill(c.rec, rung)
+    col0 = 0
+    for cols in (split or n, n - (split or n)):
+        if cols == 0:
+            continue
+        wa = c.upload(bits[col0 : col0 + cols])
+        c.launcher().launch(Kernel.matmul_bf16, P.MatmulBf16(rows=rows, n=cols, k=k, col0=col0, out_stride=n, accumulate=int(accumulate)),
+                            [xa, wa, out], (K.div_ceil(cols, K.matmul_tile_n), K.div_ceil(rows, K.matmul_tile_t), 1))
+        col0 += cols
+    got = c.read(out).reshape(rows, n)
+    c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
+    xs = synth.bf16_round(x) if rung == K.Prefill.bf16_mfma else x
+    want = init + xs.astype(np.float64) @ values.astype(np.float64).T
+    return got, want, values, x
+
+
+def test_matmul_bf16(ctx):
+    # 19 tokens and 100 outputs leave partial tiles in both dimensions.
+    got, want, _, _ = matmul_case(ctx, 19, 100, 1024, None, False)
+    assert rel_err(got, want) <= 1e-5
+
+
+def test_matmul_bf16_chunked_accumulate(ctx):
+    got, want, _, _ = matmul_case(ctx, 33, 150, 96, 70, True)
+    assert rel_err(got, want) <= 1e-5
+
+
+def test_matmul_bf16_mfma_rung(ctx):
+    """The bf16 MFMA rung against its operand contract: x rounded to bf16,
+    weights exact, products summed in float64. The rounded operands are the
+    only difference from the f32 rung, so the bound stays 1e-5."""
+    got, want, values, x = matmul_case(ctx, 19, 100, 1024, None, False, K.Prefill.bf16_mfma)
+    assert rel_err(got, want) <= 1e-5
+    got, want, values, x = matmul_case(ctx, 133, 150, 96, 70, True, K.Prefill.bf16_mfma)
+    assert rel_err(got, want) <= 1e-5
+
+
+def launch_float_q8(c, x, weights, out, rows, accumulate, slices, chunked):
+    """Two weight chunks exercise nonzero col0 and a padded output stride;
+    split-k partials are dense per chunk (src/kernels/check.zig:752-770)."""
+    l = c.launcher()
+    for index, ((start, n), w) in enumerate(zip(((0, 70), (0, 27), (27, 43)), weights)):
+        if (chunked == 0 and index != 0) or (chunked == 1 and index == 0):
+            continue
+        grid = (K.div_ceil(n, 64), K.div_ceil(rows, 16), slices)
+        if slices == 1:
+            l.launch(Kernel.matmul_q8_0_float, P.MatmulQuant(rows=rows, n=n, k=320, col0=3 + start, out_stride=79, accumulate=accumulate, k_slice=320), [x, w, out], grid)
+        else:
+            partial = c.output(slices * rows * n)
+            l.launch(Kernel.matmul_q8_0_float, P.MatmulQuant(rows=rows, n=n, k=320, col0=0, out_stride=n, k_slice=160, slice_stride=rows * n), [x, w, partial], grid)
+            l.launch(Kernel.matmul_reduce, P.MatmulReduce(rows=rows, n=n, slices=slices, col0=3 + start, out_stride=79, accumulate=accumulate, slice_stride=rows * n),
+                     [partial, out], K.elementwise(rows * n))
+
+
+@pytest.mark.parametrize("rung", [K.Prefill.scalar_f32, K.Prefill.bf16_mfma])
+def test_matmul_q8_0_float(ctx, rung):
+    """Unrounded float activations, k = 320, full and partial tiles, weight
+    chunks, padding, accumulate and split-k; within each split-k path token
+    chunking must stay bitwise identical (src/kernels/check.zig:772-825)."""
+    c = ctx
+    rows, n, k, stride = 67, 70, 320, 79
+    x = c.random(rows * k, 1).reshape(rows, k)
+    raw, values = quant_rows(c, TensorType.q8_0, n, k)
+    rb = k // 32 * 34
+    weights = [c.gpu_weights(TensorType.q8_0, raw, k), c.gpu_weights(TensorType.q8_0, raw[: 27 * rb], k), c.gpu_weights(TensorType.q8_0, raw[27 * rb :], k)]
+    xa = c.upload(x)
+    init = c.random(rows * stride, 0.25).reshape(rows, stride)
+    c.set.select_prefill(c.rec, rung)
+    if rung == K.Prefill.bf16_mfma:
+        # The rung's operand contract: both operands rounded to bf16.
+        xs, ws, tol = synth.bf16_round(x), synth.bf16_round(values), 1e-5
+    else:
+        xs, ws, tol = x, values, 1e-5
+    prod = xs.astype(np.float64) @ ws.astype(np.float64).T
+    for accumulate in (0, 1):
+        want = prod + (init[:, 3 : 3 + n] if accumulate else 0)
+        for slices, chunked in ((1, 0), (1, 1), (2, 0), (2, 1)):
+            out = c.upload(init)
+            launch_float_q8(c, xa, weights, out, rows, accumulate, slices, chunked)
+            got = c.read(out).reshape(rows, stride)
+            assert rel_err(got[:, 3 : 3 + n], want) <= tol, (accumulate, slices, chunked)
+            # Nothing outside the output columns is touched.
+            mask = np.ones(stride, dtype=bool)
+            mask[3 : 3 + n] = False
+            assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32))
+            for first, count in ((0, 3), (3, 14), (17, 50)):
+                chunk_out = c.upload(init[first : first + count])
+                launch_float_q8(c, c.upload(x[first : first + count]), weights, chunk_out, count, accumulate, slices, chunked)
+                assert got[first : first + count].tobytes() == c.read(chunk_out).tobytes(), "token chunking changed bits"
+    c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
+
+
+def test_silu_mul(ctx):
+    c = ctx
+    rows, width = 7, 10_001
+    n = rows * width
+    gu = c.random(2 * n, 6).reshape(rows, 2 * width)
+    act = c.output(n)
+    c.launcher().launch(Kernel.silu_mul, P.SiluMul(n, width), [c.upload(gu), act], K.elementwise(n))
+    g = gu[:, :width].astype(np.float64)
+    assert rel_err(c.read(act), g * sigmoid64(g) * gu[:, width:]) <= 1e-6

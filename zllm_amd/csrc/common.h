@@ -1,0 +1,103 @@
+// Internal interface between the command-stream host and the gfx950 kernels.
+#pragma once
+
+#include <hip/hip_runtime_api.h>
+#include <stddef.h>
+#include <stdint.h>
+
+#include "../../include/zllm_hip.h"
+
+namespace zhip {
+
+// Parameter blocks, field for field as src/kernels/kernels.zig:432-505 declares
+// them (extern structs, little-endian, bound at binding 0).
+struct MatvecParams {  // params.MatvecBf16
+    uint32_t n, k, col0, out_stride;
+    float eps;
+    uint32_t flags;
+    uint32_t half;
+    uint32_t x_stride;  // vec4 units between tokens' inputs; 0: k / 4
+};
+enum : uint32_t { FLAG_NORM = 1u, FLAG_ACCUMULATE = 2u, FLAG_SILU_PAIR = 4u };
+
+struct MatmulParams {  // params.MatmulBf16 / params.MatmulQuant
+    uint32_t rows, n, k, col0, out_stride, accumulate;
+    uint32_t k_slice;       // MatmulBf16: padding
+    uint32_t slice_stride;  // MatmulBf16: padding
+};
+
+struct MatmulReduceParams {
+    uint32_t rows, n, slices, col0, out_stride, accumulate, slice_stride, pad;
+};
+
+struct SiluMulParams { uint32_t count, width, pad0, pad1; };
+struct RepackQ80Params { uint32_t rows, k, pad0, pad1; };
+struct RepadParams { uint32_t blocks, src_bytes, dst_bytes, pad; };
+
+static_assert(sizeof(MatvecParams) == 32, "params.MatvecBf16 is 32 bytes");
+static_assert(sizeof(MatmulParams) == 32, "params.MatmulQuant is 32 bytes");
+static_assert(sizeof(MatmulReduceParams) == 32, "params.MatmulReduce is 32 bytes");
+static_assert(sizeof(SiluMulParams) == 16 && sizeof(RepackQ80Params) == 16 && sizeof(RepadParams) == 16, "16-byte blocks");
+
+// A quantized decode multiply's tunables (kernels.MatvecVariant,
+// src/kernels/kernels.zig:319-338), decoded from the create_kernel variant id.
+struct MatvecVariant {
+    uint32_t wg = 256, lanes = 32, rows = 1, act_div = 0;
+    uint32_t groupRows() const { return wg / lanes * rows; }
+};
+
+// Steps of up to this many tokens may use the decode multiplies. The reference
+// caps its kernels at 4 (src/kernels/matvec_quant.wgsl.hbs:64-65); rows 5..8
+// are this backend's extension for speculative-verify widths.
+constexpr uint32_t kMaxDecodeRows = 8;
+
+struct Bind {
+    uint8_t *ptr = nullptr;  // buffer base + binding offset
+    uint64_t size = 0;       // bytes bound
+    bool bound = false;
+};
+
+struct DeviceInfo {
+    int compute_units = 256;
+    int max_lds = 65536;
+};
+
+// One resolved dispatch: binding 0's bytes come from the host's shadow copy of
+// the uniform buffer, so kernels take their parameters by value.
+struct Dispatch {
+    const uint8_t *params = nullptr;
+    size_t params_size = 0;
+    Bind bind[8];
+    uint32_t grid[3] = {0, 0, 0};
+    uint32_t variant = 0;
+    hipStream_t stream = nullptr;
+    const DeviceInfo *dev = nullptr;
+    char *err = nullptr;  // message buffer for a failed launch
+    size_t err_cap = 0;
+};
+
+// Launches one kernel for a dispatch, after checking that the bound ranges
+// cover everything the kernel will touch. Returns ZHIP_OK, ZHIP_E_BAD_COMMAND
+// (with a message) or ZHIP_E_GPU.
+typedef zhip_result (*LaunchFn)(const Dispatch &);
+
+zhip_result launch_matvec_q8_0(const Dispatch &);
+zhip_result launch_matvec_q4_k(const Dispatch &);
+zhip_result launch_matvec_bf16(const Dispatch &);
+zhip_result launch_matmul_reduce(const Dispatch &);
+zhip_result launch_silu_mul(const Dispatch &);
+zhip_result launch_repack_q8_0(const Dispatch &);
+zhip_result launch_repad(const Dispatch &);
+zhip_result launch_embed_q8_0(const Dispatch &);
+zhip_result launch_embed_q4_k(const Dispatch &);
+zhip_result launch_embed_bf16(const Dispatch &);
+
+// Host-side helpers shared by the launchers.
+zhip_result fail(const Dispatch &d, zhip_result code, const char *fmt, ...);
+zhip_result check_launch(const Dispatch &d, const char *kernel);
+
+// Fills `words` 32-bit words at dst with `value` on the stream (clear_buffer;
+// also used instead of memset nodes so a captured stream stays replayable).
+zhip_result launch_fill(hipStream_t stream, void *dst, uint64_t words, uint32_t value);
+
+}  // namespace zhip

@@ -1,0 +1,256 @@
+// Decode multiplies: out[t][col0 + j] (+)= sum_i X(t, i) * w[j][i] for Q8_0,
+// Q4_K and BF16 weights, with the RMSNorm / activation prologues and the
+// accumulate / SiLU-pair epilogues of the reference's matvec kernels
+// (src/kernels/matvec_quant.wgsl.hbs:20-31, src/kernels/matvec_half.wgsl:14-19).
+//
+// General kernel. A workgroup is four wave64s. The step's inputs are staged
+// once per workgroup in LDS (normalised / activated as they are staged), then
+// every wave walks row groups in a grid-stride loop: a group is two weight
+// rows (two outputs, or the gate and up rows of one output with SILU_PAIR).
+// A row's packed weights are split into 16-byte tasks across the 64 lanes, so
+// each load instruction of a wave reads consecutive 16-byte vectors; a lane
+// decodes its task's weights once and multiplies them with every token's
+// inputs; the lanes' partial sums reduce in a fixed butterfly. A token's sums
+// are therefore the same bit for bit whether it runs alone or with others
+// (the reference's split invariant, matvec_quant.wgsl.hbs:14-18).
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "decode.cuh"
+
+namespace zhip {
+
+struct MvArgs {
+    const float *x;
+    const uint8_t *w;
+    float *out;
+    const float *norm_w;
+    uint32_t n, k, col0, out_stride;
+    float eps;
+    uint32_t flags, half;
+    uint32_t xr;         // floats between tokens' inputs
+    uint32_t m;          // tokens
+    uint32_t rows;       // outputs covered by the logical grid
+    uint32_t row_bytes;  // bytes between weight rows
+    float act_div;       // > 0: inputs staged as silu(x / act_div)
+};
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    return v;
+}
+
+__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
+
+template <class D, int MT>
+__global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
+    extern __shared__ float4 xs4[];
+    float *xs = reinterpret_cast<float *>(xs4);
+    __shared__ float red[4];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t gwave = blockIdx.x * 4u + wave, nwaves = gridDim.x * 4u;
+    const bool pair = (a.flags & FLAG_SILU_PAIR) != 0;
+    const uint32_t k4 = a.k / 4u;
+    const uint32_t tasks = a.k / D::E;
+    // Outputs per group: two rows, or one gate/up pair.
+    const uint32_t per_group = pair ? 1u : 2u;
+    const uint32_t groups = (a.rows + per_group - 1u) / per_group;
+
+    for (uint32_t t0 = 0; t0 < a.m; t0 += MT) {
+        const uint32_t mt = min((uint32_t)MT, a.m - t0);
+        __syncthreads();
+        for (uint32_t t = 0; t < (uint32_t)MT; t++) {
+            float4 *dst = xs4 + (size_t)t * k4;
+            if (t >= mt) {
+                for (uint32_t i = tid; i < k4; i += 256u) dst[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                continue;
+            }
+            const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)(t0 + t) * a.xr);
+            float scale = 1.0f;
+            if (a.flags & FLAG_NORM) {
+                float ss = 0.f;
+                for (uint32_t i = tid; i < k4; i += 256u) {
+                    const float4 v = xrow[i];
+                    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                }
+                ss = wave_sum(ss);
+                __syncthreads();
+                if (lane == 0) red[wave] = ss;
+                __syncthreads();
+                ss = (red[0] + red[1]) + (red[2] + red[3]);
+                scale = 1.0f / sqrtf(ss / (float)a.k + a.eps);
+            }
+            const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
+            for (uint32_t i = tid; i < k4; i += 256u) {
+                float4 v = xrow[i];
+                if (a.flags & FLAG_NORM) {
+                    const float4 g = nw[i];
+                    v.x = v.x * scale * g.x; v.y = v.y * scale * g.y;
+                    v.z = v.z * scale * g.z; v.w = v.w * scale * g.w;
+                }
+                if (a.act_div > 0.f) {
+                    v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
+                    v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+                }
+                dst[i] = v;
+            }
+        }
+        __syncthreads();
+
+        for (uint32_t g = gwave; g < groups; g += nwaves) {
+            // The group's two weight rows and whether each exists.
+            const uint32_t j0 = pair ? g : 2u * g;
+            const uint32_t r1 = pair ? a.half + g : j0 + 1u;
+            const bool has1 = pair || r1 < a.rows;
+            const uint8_t *row0 = a.w + (size_t)j0 * a.row_bytes;
+            const uint8_t *row1 = a.w + (size_t)(has1 ? r1 : j0) * a.row_bytes;
+            float acc0[MT], acc1[MT];
+#pragma unroll
+            for (int t = 0; t < MT; t++) acc0[t] = acc1[t] = 0.f;
+
+            for (uint32_t task = lane; task < tasks; task += 64u) {
+                float w0[D::E], w1[D::E];
+                D::decode(row0, a.k, task, w0);
+                D::decode(row1, a.k, task, w1);
+                const uint32_t xo0 = D::xoff(task, 0), xo1 = D::xoff(task, 1);
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    const float *xt = xs + (size_t)t * a.k;
+                    float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                    for (int h = 0; h < 2; h++) {
+                        const float4 *xv = reinterpret_cast<const float4 *>(xt + (h ? xo1 : xo0));
+#pragma unroll
+                        for (int e = 0; e < D::E / 8; e++) {
+                            const float4 v = xv[e];
+                            const int b = h * (D::E / 2) + 4 * e;
+                            s0 = fmaf(w0[b + 0], v.x, s0); s1 = fmaf(w1[b + 0], v.x, s1);
+                            s0 = fmaf(w0[b + 1], v.y, s0); s1 = fmaf(w1[b + 1], v.y, s1);
+                            s0 = fmaf(w0[b + 2], v.z, s0); s1 = fmaf(w1[b + 2], v.z, s1);
+                            s0 = fmaf(w0[b + 3], v.w, s0); s1 = fmaf(w1[b + 3], v.w, s1);
+                        }
+                    }
+                    acc0[t] += s0;
+                    acc1[t] += s1;
+                }
+            }
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                acc0[t] = wave_sum(acc0[t]);
+                acc1[t] = wave_sum(acc1[t]);
+            }
+            if (lane == 0) {
+                for (uint32_t t = 0; t < mt; t++) {
+                    const size_t o = (size_t)(t0 + t) * a.out_stride + a.col0 + j0;
+                    if (pair) {
+                        float v = silu_f(acc0[t]) * acc1[t];
+                        if (a.flags & FLAG_ACCUMULATE) v += a.out[o];
+                        a.out[o] = v;
+                    } else {
+                        float v = acc0[t];
+                        if (a.flags & FLAG_ACCUMULATE) v += a.out[o];
+                        a.out[o] = v;
+                        if (has1) {
+                            float u = acc1[t];
+                            if (a.flags & FLAG_ACCUMULATE) u += a.out[o + 1];
+                            a.out[o + 1] = u;
+                        }
+                    }
+                }
+            }
+        }
+    }
+}
+
+template <class D, int MT>
+static zhip_result run(const Dispatch &d, const MvArgs &a, uint32_t lds_bytes) {
+    static int configured_device = -1;  // dynamic LDS above 64 KiB needs opting in once
+    auto kernel = matvec_kernel<D, MT>;
+    if (lds_bytes > 65536u && configured_device != 1) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(d, ZHIP_E_BAD_COMMAND, "decode multiply: k = %u with %d tokens does not fit workgroup memory", a.k, MT);
+        }
+        configured_device = 1;
+    }
+    const uint32_t per_group = (a.flags & FLAG_SILU_PAIR) ? 1u : 2u;
+    const uint32_t groups = (a.rows + per_group - 1u) / per_group;
+    const uint32_t want = (groups + 3u) / 4u;
+    // Few enough workgroups that staging the inputs stays a small part of each
+    // one's traffic, enough of them to keep every CU's SIMDs busy.
+    const uint32_t cap = (uint32_t)d.dev->compute_units * (lds_bytes > 32768u ? 2u : 4u);
+    const uint32_t blocks = want < cap ? want : cap;
+    hipLaunchKernelGGL((matvec_kernel<D, MT>), dim3(blocks ? blocks : 1), dim3(256), lds_bytes, d.stream, a);
+    return check_launch(d, D::name());
+}
+
+template <class D>
+static zhip_result launch_matvec(const Dispatch &d, bool quant) {
+    if (d.params_size < sizeof(MatvecParams)) return fail(d, ZHIP_E_BAD_COMMAND, "%s: params block of %zu bytes", D::name(), d.params_size);
+    const MatvecParams &p = *reinterpret_cast<const MatvecParams *>(d.params);
+    MatvecVariant v;
+    if (quant && d.variant != 0) {
+        v.wg = (d.variant & 0xffu) * 32u;
+        v.lanes = (d.variant >> 8) & 0xffu;
+        v.rows = (d.variant >> 16) & 0xffu;
+        v.act_div = d.variant >> 24;
+        if (v.wg == 0 || v.lanes == 0 || v.rows == 0 || v.wg % v.lanes != 0)
+            return fail(d, ZHIP_E_BAD_COMMAND, "%s: variant id 0x%08x is not a MatvecVariant", D::name(), d.variant);
+    }
+    // Rows one workgroup of the logical grid covers (kernels.matvec_rows = 8
+    // for the half-precision kernel, groupRows() for the quantized one).
+    const uint32_t group_rows = quant ? v.groupRows() : 8u;
+    if (d.grid[0] == 0 || d.grid[1] == 0 || d.grid[2] == 0) return ZHIP_OK;
+    const uint64_t covered = (uint64_t)d.grid[0] * group_rows;
+    MvArgs a{};
+    a.n = p.n; a.k = p.k; a.col0 = p.col0; a.out_stride = p.out_stride; a.eps = p.eps;
+    a.flags = p.flags; a.half = p.half;
+    a.rows = (uint32_t)(covered < p.n ? covered : p.n);
+    // The quantized kernel runs the first row of workgroups over up to
+    // kMaxDecodeRows tokens; the half-precision one has a grid row per token.
+    a.m = quant ? (d.grid[1] < kMaxDecodeRows ? d.grid[1] : kMaxDecodeRows) : d.grid[1];
+    a.xr = (quant && p.x_stride != 0) ? p.x_stride * 4u : p.k;
+    a.act_div = quant ? (float)v.act_div : 0.f;
+    a.row_bytes = D::row_bytes(p.k);
+    if (p.k == 0 || p.k % D::BLOCK != 0) return fail(d, ZHIP_E_BAD_COMMAND, "%s: k = %u is not a multiple of %u", D::name(), p.k, D::BLOCK);
+    if (p.flags & ~7u) return fail(d, ZHIP_E_BAD_COMMAND, "%s: unknown flags 0x%x", D::name(), p.flags);
+    if (a.rows == 0) return ZHIP_OK;
+    const bool norm = p.flags & FLAG_NORM, pair = p.flags & FLAG_SILU_PAIR;
+    for (int b = 1; b <= (norm ? 4 : 3); b++)
+        if (!d.bind[b].bound) return fail(d, ZHIP_E_BAD_COMMAND, "%s: binding %d is not bound", D::name(), b);
+    const uint64_t x_need = ((uint64_t)(a.m - 1) * a.xr + p.k) * 4u;
+    const uint64_t w_rows = pair ? (uint64_t)p.half + a.rows : a.rows;
+    const uint64_t w_need = w_rows * a.row_bytes;
+    const uint64_t o_need = ((uint64_t)(a.m - 1) * p.out_stride + p.col0 + a.rows) * 4u;
+    if (x_need > d.bind[1].size) return fail(d, ZHIP_E_BAD_COMMAND, "%s: x needs %llu bytes, %llu bound", D::name(), (unsigned long long)x_need, (unsigned long long)d.bind[1].size);
+    if (w_need > d.bind[2].size) return fail(d, ZHIP_E_BAD_COMMAND, "%s: weights need %llu bytes, %llu bound", D::name(), (unsigned long long)w_need, (unsigned long long)d.bind[2].size);
+    if (o_need > d.bind[3].size) return fail(d, ZHIP_E_BAD_COMMAND, "%s: out needs %llu bytes, %llu bound", D::name(), (unsigned long long)o_need, (unsigned long long)d.bind[3].size);
+    if (norm && (uint64_t)p.k * 4u > d.bind[4].size) return fail(d, ZHIP_E_BAD_COMMAND, "%s: norm weights need %u bytes", D::name(), p.k * 4u);
+    if (((uintptr_t)d.bind[1].ptr | (uintptr_t)d.bind[2].ptr | (norm ? (uintptr_t)d.bind[4].ptr : 0)) & 15u)
+        return fail(d, ZHIP_E_BAD_COMMAND, "%s: x, weights and norm weights must be 16-byte aligned", D::name());
+    if (((uintptr_t)d.bind[3].ptr & 3u) || (a.xr & 3u)) return fail(d, ZHIP_E_BAD_COMMAND, "%s: misaligned out or x stride", D::name());
+    a.x = reinterpret_cast<const float *>(d.bind[1].ptr);
+    a.w = d.bind[2].ptr;
+    a.out = reinterpret_cast<float *>(d.bind[3].ptr);
+    a.norm_w = norm ? reinterpret_cast<const float *>(d.bind[4].ptr) : nullptr;
+
+    // Tokens per pass over the weights: as many as fit workgroup memory.
+    const uint64_t row_lds = (uint64_t)p.k * 4u;
+    const uint64_t max_lds = 160u * 1024u - 64u;
+    uint32_t mt = a.m >= 3 ? 4u : a.m;
+    while (mt > 1 && mt * row_lds > 65536u) mt >>= 1;
+    if (mt * row_lds > max_lds) return fail(d, ZHIP_E_BAD_COMMAND, "%s: k = %u does not fit workgroup memory", D::name(), p.k);
+    const uint32_t lds = (uint32_t)(mt * row_lds);
+    switch (mt) {
+    case 1: return run<D, 1>(d, a, lds);
+    case 2: return run<D, 2>(d, a, lds);
+    default: return run<D, 4>(d, a, lds);
+    }
+}
+
+zhip_result launch_matvec_q8_0(const Dispatch &d) { return launch_matvec<DecQ8_0>(d, true); }
+zhip_result launch_matvec_q4_k(const Dispatch &d) { return launch_matvec<DecQ4_K>(d, true); }
+zhip_result launch_matvec_bf16(const Dispatch &d) { return launch_matvec<DecBF16>(d, false); }
+
+}  // namespace zhip
