@@ -1,0 +1,393 @@
+#!/usr/bin/env python3
+"""Benchmark of the quantized linear-layer hot path on one MI355X.
+
+One JSON line. The headline is the decode multiply the metric is quoted on:
+Q4_K weights, M = 1, K = 4096, N = 14336 (Llama-3-8B FFN-up shape). A step is
+one dispatch of matvec_q4_k through the command stream over one copy of the
+weights; steps rotate over enough distinct copies to exceed L2 plus the
+256 MB Infinity Cache, so the rate is HBM's. Inputs are resident in device
+memory before the timed region, which is K back-to-back dispatches in one
+submit bracketed by blocking submits on both sides.
+
+  value      algorithmic bytes per step x steps / wall time of the timed region
+  roofline   algorithmic bytes per launch / mean launch time from HIP events
+             recorded on the host's stream around the same K launches
+  cpu_baseline  the CPU oracle (a C restatement of the reference's src/ref
+             multiply) on the same weights, all physical cores, bounded sample
+
+The other shapes of the path (Q8_0 decode, fused gate/up at M = 1, 4, 8, the
+Q8_0 prefill multiply on bf16 MFMA, the bf16 lm_head) are reported under
+"also" with their own roofline fractions.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+ROTATE_BYTES = 640 << 20    # distinct weight bytes a rotation must exceed (L2 + Infinity Cache, with margin)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=2000)
+    ap.add_argument("--warmup", type=int, default=200)
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c5 for the 'also' section; 'none' skips it")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this path is built and measured on one GPU; --gpus above 1 is not supported "
+              "(more GPUs would each take a share of the output rows)", file=sys.stderr)
+        return 2
+
+    from zllm_amd import Device, Host, cmd, synth
+    from zllm_amd import kernels as K
+    from zllm_amd.kernels import Kernel, TensorType, params as P
+
+    dev = Device.open(0)
+    host = Host(dev)
+    rec = cmd.Recorder()
+    kset = K.Set.create(rec)
+    token = [0]
+
+    def flush():
+        token[0] += 1
+        rec.submit(token[0])
+        done = []
+        host.execute(rec.batch(), done)
+        rec.clear()
+        return done
+
+    flush()
+    storage = cmd.Usage.storage | cmd.Usage.copy_dst | cmd.Usage.copy_src
+
+    def upload(arr) -> K.Arg:
+        arr = np.ascontiguousarray(arr)
+        raw = arr.reshape(-1).view(np.uint8)
+        size = (raw.size + 15) & ~15
+        buf = rec.create_buffer(size, storage)
+        rec.write_buffer(buf, 0, raw if raw.size % 4 == 0 else np.concatenate([raw, np.zeros(size - raw.size, np.uint8)]))
+        flush()
+        return K.Arg(buf, size)
+
+    def output(n_bytes: int) -> K.Arg:
+        buf = rec.create_buffer(n_bytes, storage)
+        return K.Arg(buf, n_bytes)
+
+    def read(arg: K.Arg, dtype=np.float32) -> np.ndarray:
+        dst = np.zeros(arg.size, dtype=np.uint8)
+        rec.read_buffer(0xFFFF0000, arg.buffer, 0, dst)
+        flush()
+        return dst.view(dtype)
+
+    def timed(launches, steps: int, warmup: int):
+        """Runs `warmup` then `steps` dispatches cycling over `launches`; returns
+        (wall seconds, GPU seconds from the host's stream events)."""
+        for n, is_timed in ((warmup, False), (steps, True)):
+            if n == 0:
+                continue
+            for i in range(n):
+                launches[i % len(launches)].record(rec, K.Extent(rows=launches[i % len(launches)].rows))
+            token[0] += 1
+            rec.submit(token[0])
+            words = rec.batch()
+            done = []
+            t0 = time.perf_counter()
+            host.execute(words, done)
+            wall = time.perf_counter() - t0
+            rec.clear()
+            ns, count = host.last_submit()
+            assert count == n
+        return wall, ns * 1e-9
+
+    class L:
+        """A prebuilt launch and the token rows its grid resolves with."""
+
+        def __init__(self, launch, rows):
+            self.launch, self.rows = launch, rows
+
+        def record(self, r, e):
+            self.launch.record(r, e)
+
+    b = K.Builder(rec, kset)
+
+    def rotation(w_bytes: int) -> int:
+        return max(2, -(-ROTATE_BYTES // w_bytes))
+
+    def matvec_workload(t: TensorType, raw_rows: np.ndarray, n_out: int, k: int, m: int, pair: bool, x: np.ndarray):
+        """Uploads a rotation of weight copies and builds one launch per copy."""
+        kernel = K.weight_kernel("matvec", t)
+        rb = K.row_bytes(t, k)
+        w_rows = 2 * n_out if pair else n_out
+        copies = rotation(w_rows * rb)
+        src = upload(raw_rows)
+        xa = upload(x)
+        out = output(4 * m * n_out)
+        launches = []
+        first = None
+        for _ in range(copies):
+            if K.needs_layout(t):
+                wa = output(w_rows * rb)
+                K.Launcher(rec, kset).layout(t, src, wa, w_rows, k)
+            else:
+                buf = rec.create_buffer(src.size, storage)
+                rec.copy_buffer(src.buffer, 0, buf, 0, src.size)
+                wa = K.Arg(buf, src.size)
+            first = first or wa
+            v = K.MatvecVariant()
+            p = P.MatvecBf16(n=n_out, k=k, col0=0, out_stride=n_out, silu_pair=pair, half=n_out if pair else 0)
+            if K.is_half(t):
+                launches.append(L(b.add(kernel, p, [xa, wa, out, wa], K.Grid.rows_y(K.div_ceil(n_out, K.matvec_rows))), m))
+            else:
+                launches.append(L(b.add_matvec(kernel, v, p, [xa, wa, out, wa], K.Grid.rows_y(K.div_ceil(n_out, v.group_rows()))), m))
+        b.finish()
+        flush()
+        return launches, out
+
+    def hbm_entry(name, bytes_per_step, wall, gpu_s, steps, extra=None):
+        e = {
+            "workload": name,
+            "bytes_per_step": bytes_per_step,
+            "us_per_step_wall": round(wall / steps * 1e6, 3),
+            "us_per_launch_gpu": round(gpu_s / steps * 1e6, 3),
+            "GBps_wall": round(bytes_per_step * steps / wall / 1e9, 1),
+            "GBps_gpu": round(bytes_per_step * steps / gpu_s / 1e9, 1),
+            "hbm_frac": round(bytes_per_step * steps / gpu_s / 1e9 / HBM_PEAK_GBPS, 4),
+        }
+        e.update(extra or {})
+        return e
+
+    def check_matvec(got, want_f64, w_rows_f32, x):
+        """(max |err| / (||row|| ||x||), max |err| / max |want|)."""
+        got = got.astype(np.float64)
+        wn = np.linalg.norm(w_rows_f32.astype(np.float64), axis=1)
+        xn = np.linalg.norm(x.astype(np.float64).reshape(got.shape[0], -1), axis=1)
+        err = np.abs(got - want_f64)
+        return float(np.max(err / np.maximum(xn[:, None] * wn[None, :], 1e-30))), float(np.max(err) / max(np.max(np.abs(want_f64)), 1e-30))
+
+    # ---- headline: C2, Q4_K decode multiply M = 1, K = 4096, N = 14336 ----------------------
+    n, k = 14336, 4096
+    g = synth.rng(0xC2)
+    raw = synth.q4_k_rows(g, n, k)
+    x = synth.activations(g, 1, k)
+    launches, out = matvec_workload(TensorType.q4_k, raw, n, k, 1, False, x)
+    c2_bytes = n * K.row_bytes(TensorType.q4_k, k) + 4 * k + 4 * n  # 33,103,872
+    wall, gpu_s = timed(launches, args.steps, args.warmup)
+    got = read(out)[:n].reshape(1, n)
+
+    import oracle  # the checker and the CPU baseline; never the measured path
+
+    w_f32 = oracle.dequantize(oracle.Q4_K, raw, n * k).reshape(n, k)
+    want = oracle.matmul_f64(x, w_f32)
+    bound, rel = check_matvec(got, want, w_f32, x)
+    if not bound <= 1e-3:
+        print(f"bench.py: parity failed on the headline workload: |err| / (||row|| ||x||) = {bound}", file=sys.stderr)
+        return 1
+
+    cpu = None
+    if not args.no_cpu:
+        threads = oracle.default_threads()
+        m = oracle.Matrix(oracle.Q4_K, raw, n, k, threads)
+        oracle.matmul(x, m, threads)  # warm-up
+        times = []
+        t_end = time.perf_counter() + 12.0
+        while len(times) < 5 or (time.perf_counter() < t_end and len(times) < 400):
+            t0 = time.perf_counter()
+            oracle.matmul(x, m, threads)
+            times.append(time.perf_counter() - t0)
+        med = float(np.median(times))
+        cpu = {
+            "value": round(c2_bytes / med / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": f"C restatement of the reference's src/ref multiply (no Zig toolchain), the same C2 weights and input, "
+                      f"median of {len(times)} full multiplies ({med * 1e3:.2f} ms each) after 1 warm-up",
+        }
+
+    result = {
+        "metric": "Q4_K decode matvec GB/s (% HBM peak); Q8_0 prefill matmul TFLOP/s (% MFMA)",
+        "value": round(c2_bytes * args.steps / wall / 1e9, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall / args.steps * 1e3, 6),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {
+            "workload": "C2: Q4_K decode matvec, M=1, K=4096, N=14336 (Llama-3-8B FFN-up), f32 activations, "
+                        f"rotating over {len(launches)} weight copies ({len(launches) * n * K.row_bytes(TensorType.q4_k, k) >> 20} MiB)",
+            "kernel": "matvec_q4_k",
+            "bytes_per_step": c2_bytes,
+        },
+        "roofline": {
+            "bound": "hbm",
+            "achieved": round(c2_bytes * args.steps / gpu_s / 1e9, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(c2_bytes * args.steps / gpu_s / 1e9 / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "us_per_launch": round(gpu_s / args.steps * 1e6, 3),
+        },
+        "cpu_baseline": cpu,
+        "parity": {"max_err_over_row_x_norms": bound, "max_err_over_max_want": rel, "bound": 1e-3},
+    }
+
+    only = [s for s in args.only.split(",") if s]
+    also = {}
+    if "none" not in only:
+        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c5", bench_c5)):
+            if not only or name in only:
+                try:
+                    also[name] = fn(locals())
+                except Exception as e:  # a secondary workload must not lose the headline
+                    also[name] = {"error": f"{type(e).__name__}: {e}"}
+    if also:
+        result["also"] = also
+    print(json.dumps(result))
+    return 0
+
+
+def bench_c1(env):
+    """Q8_0 decode multiply M = 1, K = 1024, N = 3072."""
+    synth, oracle, K, TensorType = env["synth"], env["oracle"], env["K"], env["TensorType"]
+    n, k = 3072, 1024
+    g = synth.rng(0xC1)
+    raw = synth.q8_0_rows(g, n, k)
+    x = synth.activations(g, 1, k)
+    launches, out = env["matvec_workload"](TensorType.q8_0, raw, n, k, 1, False, x)
+    steps = env["args"].steps
+    wall, gpu_s = env["timed"](launches, steps, env["args"].warmup)
+    got = env["read"](out)[:n].reshape(1, n)
+    w = oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k)
+    bound, rel = env["check_matvec"](got, oracle.matmul_f64(x, w), w, x)
+    nbytes = n * k // 32 * 34 + 4 * k + 4 * n  # GGUF bytes: 3,358,720
+    return env["hbm_entry"]("C1: Q8_0 decode matvec M=1 K=1024 N=3072", nbytes, wall, gpu_s, steps,
+                            {"copies": len(launches), "max_err_over_row_x_norms": bound, "max_err_over_max_want": rel})
+
+
+def bench_c3(env):
+    """Fused gate+up Q4_K decode multiply with the SiLU pair epilogue, M in 1, 4, 8."""
+    synth, oracle, K, TensorType = env["synth"], env["oracle"], env["K"], env["TensorType"]
+    n, k = 14336, 4096
+    gate = synth.q4_k_rows(synth.rng(0xC3A), n, k)
+    up = synth.q4_k_rows(synth.rng(0xC3B), n, k)
+    raw = np.concatenate([gate, up])
+    w = oracle.dequantize(oracle.Q4_K, raw, 2 * n * k).reshape(2 * n, k)
+    steps = max(1, env["args"].steps // 2)
+    res = {}
+    for m in (1, 4, 8):
+        x = synth.activations(synth.rng(0xC30 + m), m, k)
+        launches, out = env["matvec_workload"](TensorType.q4_k, raw, n, k, m, True, x)
+        wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 2))
+        got = env["read"](out)[: m * n].reshape(m, n).astype(np.float64)
+        both = oracle.matmul_f64(x, w)
+        gt, u = both[:, :n], both[:, n:]
+        want = gt / (1 + np.exp(-gt)) * u
+        rel = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+        nbytes = 2 * n * K.row_bytes(TensorType.q4_k, k) + m * 4 * k + m * 4 * n
+        res[f"m{m}"] = env["hbm_entry"](f"C3: fused gate+up Q4_K + SiLU*mul, M={m}, K=4096, N=2x14336", nbytes, wall, gpu_s, steps,
+                                        {"copies": len(launches), "max_err_over_max_want": rel})
+    return res
+
+
+def bench_c4(env):
+    """Q8_0 prefill multiply M = 512, K = 4096, N = 4096 on the bf16 MFMA rung."""
+    synth, oracle, K, TensorType, P = env["synth"], env["oracle"], env["K"], env["TensorType"], env["P"]
+    rec, kset, b = env["rec"], env["kset"], env["b"]
+    rows, k, n = 512, 4096, 4096
+    g = synth.rng(0xC4)
+    raw = synth.q8_0_rows(g, n, k)
+    x = synth.activations(g, rows, k, bf16=True)
+    kset.select_prefill(rec, K.Prefill.bf16_mfma)
+    src = env["upload"](raw)
+    xa = env["upload"](x)
+    rb = K.row_bytes(TensorType.q8_0, k)
+    out = env["output"](4 * rows * n)
+    launches = []
+    for _ in range(4):
+        wa = env["output"](n * rb)
+        K.Launcher(rec, kset).layout(TensorType.q8_0, src, wa, n, k)
+        p = P.MatmulQuant(rows=rows, n=n, k=k, col0=0, out_stride=n, k_slice=k)
+        launches.append(env["L"](b.add(K.Kernel.matmul_q8_0_float, p, [xa, wa, out], K.Grid.tiles_y(K.div_ceil(n, 64), 16)), rows))
+    b.finish()
+    env["flush"]()
+    steps = max(1, env["args"].steps // 4)
+    wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 4))
+    got = env["read"](out)[: rows * n].reshape(rows, n).astype(np.float64)
+    kset.select_prefill(rec, K.Prefill.scalar_f32)
+    w = oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k)
+    want = x.astype(np.float64) @ w.astype(np.float64).T
+    wn = np.linalg.norm(w.astype(np.float64), axis=1)
+    xn = np.linalg.norm(x.astype(np.float64), axis=1)
+    bound = float(np.max(np.abs(got - want) / (xn[:, None] * wn[None, :])))
+    flops = 2 * rows * n * k
+    return {
+        "workload": "C4: Q8_0 prefill matmul M=512 K=4096 N=4096, bf16 activations (bound as f32), bf16 MFMA, fp32 accumulate",
+        "flops_per_step": flops,
+        "us_per_step_wall": round(wall / steps * 1e6, 3),
+        "us_per_launch_gpu": round(gpu_s / steps * 1e6, 3),
+        "TFLOPs_wall": round(flops * steps / wall / 1e12, 1),
+        "TFLOPs_gpu": round(flops * steps / gpu_s / 1e12, 1),
+        "mfma_frac": round(flops * steps / gpu_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+        "max_err_over_row_x_norms": bound,
+        "max_err_over_max_want": float(np.max(np.abs(got - want)) / np.max(np.abs(want))),
+    }
+
+
+def bench_c5(env):
+    """bf16 lm_head K = 1024, N = 151936 at M = 1 (decode) and M = 128 (prefill chunk)."""
+    synth, oracle, K, TensorType, P = env["synth"], env["oracle"], env["K"], env["TensorType"], env["P"]
+    rec, kset, b = env["rec"], env["kset"], env["b"]
+    n, k = 151936, 1024
+    g = synth.rng(0xC5)
+    wbits = synth.bf16_matrix(g, n, k, 0.02)
+    w = synth.bf16_bits_to_f32(wbits)
+    res = {}
+    steps = max(1, env["args"].steps // 10)
+    # M = 1: the decode multiply.
+    x = synth.activations(g, 1, k, bf16=True)
+    launches, out = env["matvec_workload"](TensorType.bf16, wbits, n, k, 1, False, x)
+    wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 10))
+    got = env["read"](out)[:n].reshape(1, n)
+    want = oracle.matmul_f64(x, w)
+    bound, rel = env["check_matvec"](got, want, w, x)
+    nbytes = 2 * n * k + 2 * k + 4 * n
+    res["m1"] = env["hbm_entry"]("C5: bf16 lm_head matvec M=1 K=1024 N=151936", nbytes, wall, gpu_s, steps,
+                                 {"copies": len(launches), "max_err_over_row_x_norms": bound, "max_err_over_max_want": rel,
+                                  "argmax_equal": bool(int(np.argmax(got[0])) == oracle.argmax(want[0].astype(np.float32)))})
+    # M = 128: the prefill multiply on the bf16 MFMA rung.
+    rows = 128
+    x = synth.activations(g, rows, k, bf16=True)
+    kset.select_prefill(rec, K.Prefill.bf16_mfma)
+    xa = env["upload"](x)
+    wa = env["upload"](wbits)
+    out = env["output"](4 * rows * n)
+    p = P.MatmulBf16(rows=rows, n=n, k=k, col0=0, out_stride=n)
+    launches = [env["L"](b.add(K.Kernel.matmul_bf16, p, [xa, wa, out], K.Grid.tiles_y(K.div_ceil(n, 64), 16)), rows)]
+    b.finish()
+    env["flush"]()
+    wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 10))
+    got = env["read"](out)[: rows * n].reshape(rows, n)
+    kset.select_prefill(rec, K.Prefill.scalar_f32)
+    want = oracle.matmul_f64(x, w)
+    rel = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+    nbytes = 2 * n * k + 2 * rows * k + 4 * rows * n
+    res["m128"] = env["hbm_entry"]("C5: bf16 lm_head matmul M=128 K=1024 N=151936 (bf16 MFMA)", nbytes, wall, gpu_s, steps,
+                                   {"copies": 1, "max_err_over_max_want": rel,
+                                    "argmax_rows_equal": int(np.count_nonzero(np.argmax(got, axis=1) == np.argmax(want, axis=1))), "rows": rows})
+    return res
+
+
+if __name__ == "__main__":
+    sys.exit(main())
