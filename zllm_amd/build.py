@@ -10,8 +10,8 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libzllm_hip.so")
 
-SOURCES = ["host.cpp", "matvec.hip", "matmul_f32.hip", "matmul_mfma.hip", "elementwise.hip"]
-HEADERS = ["common.h", "decode.cuh", os.path.join("..", "..", "include", "zllm_hip.h")]
+SOURCES = ["host.cpp", "matvec.hip", "matvec_q4k.hip", "matmul_f32.hip", "matmul_mfma.hip", "elementwise.hip"]
+HEADERS = ["common.h", "decode.cuh", "matvec_common.cuh", os.path.join("..", "..", "include", "zllm_hip.h")]
 
 # -packed-fp32-ops off: some packed-FP32 forms have given wrong results on the
 # target machines; ordinary float code must not be turned into them.

@@ -17,31 +17,9 @@
 
 #include "common.h"
 #include "decode.cuh"
+#include "matvec_common.cuh"
 
 namespace zhip {
-
-struct MvArgs {
-    const float *x;
-    const uint8_t *w;
-    float *out;
-    const float *norm_w;
-    uint32_t n, k, col0, out_stride;
-    float eps;
-    uint32_t flags, half;
-    uint32_t xr;         // floats between tokens' inputs
-    uint32_t m;          // tokens
-    uint32_t rows;       // outputs covered by the logical grid
-    uint32_t row_bytes;  // bytes between weight rows
-    float act_div;       // > 0: inputs staged as silu(x / act_div)
-};
-
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
-
-__device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v)); }
 
 template <class D, int MT>
 __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
@@ -66,35 +44,7 @@ __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
                 for (uint32_t i = tid; i < k4; i += 256u) dst[i] = make_float4(0.f, 0.f, 0.f, 0.f);
                 continue;
             }
-            const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)(t0 + t) * a.xr);
-            float scale = 1.0f;
-            if (a.flags & FLAG_NORM) {
-                float ss = 0.f;
-                for (uint32_t i = tid; i < k4; i += 256u) {
-                    const float4 v = xrow[i];
-                    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-                }
-                ss = wave_sum(ss);
-                __syncthreads();
-                if (lane == 0) red[wave] = ss;
-                __syncthreads();
-                ss = (red[0] + red[1]) + (red[2] + red[3]);
-                scale = 1.0f / sqrtf(ss / (float)a.k + a.eps);
-            }
-            const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
-            for (uint32_t i = tid; i < k4; i += 256u) {
-                float4 v = xrow[i];
-                if (a.flags & FLAG_NORM) {
-                    const float4 g = nw[i];
-                    v.x = v.x * scale * g.x; v.y = v.y * scale * g.y;
-                    v.z = v.z * scale * g.z; v.w = v.w * scale * g.w;
-                }
-                if (a.act_div > 0.f) {
-                    v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
-                    v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
-                }
-                dst[i] = v;
-            }
+            stage_token(a, t0 + t, dst, red);
         }
         __syncthreads();
 
@@ -162,6 +112,8 @@ __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
         }
     }
 }
+
+zhip_result launch_matvec_q4k(const Dispatch &d, const MvArgs &a);
 
 template <class D, int MT>
 static zhip_result run(const Dispatch &d, const MvArgs &a, uint32_t lds_bytes) {
@@ -234,6 +186,8 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     a.w = d.bind[2].ptr;
     a.out = reinterpret_cast<float *>(d.bind[3].ptr);
     a.norm_w = norm ? reinterpret_cast<const float *>(d.bind[4].ptr) : nullptr;
+
+    if (D::BLOCK == 256u) return launch_matvec_q4k(d, a);
 
     // Tokens per pass over the weights: as many as fit workgroup memory.
     const uint64_t row_lds = (uint64_t)p.k * 4u;
