@@ -309,9 +309,9 @@ def bench_c4(env):
     g = synth.rng(0xC4)
     raw = synth.q8_0_rows(g, n, k)
     x = synth.activations(g, rows, k, bf16=True)
-    kset.select_prefill(rec, K.Prefill.bf16_mfma)
+    kset.select_prefill(rec, K.Prefill.bf16_mfma_xbf16)
     src = env["upload"](raw)
-    xa = env["upload"](x)
+    xa = env["upload"](synth.to_bf16_bits(x))
     rb = K.row_bytes(TensorType.q8_0, k)
     out = env["output"](4 * rows * n)
     launches = []
@@ -333,7 +333,7 @@ def bench_c4(env):
     bound = float(np.max(np.abs(got - want) / (xn[:, None] * wn[None, :])))
     flops = 2 * rows * n * k
     return {
-        "workload": "C4: Q8_0 prefill matmul M=512 K=4096 N=4096, bf16 activations (bound as f32), bf16 MFMA, fp32 accumulate",
+        "workload": "C4: Q8_0 prefill matmul M=512 K=4096 N=4096, bf16 activations (bound as packed bf16), bf16 MFMA, fp32 accumulate",
         "flops_per_step": flops,
         "us_per_step_wall": round(wall / steps * 1e6, 3),
         "us_per_launch_gpu": round(gpu_s / steps * 1e6, 3),
@@ -369,8 +369,8 @@ def bench_c5(env):
     # M = 128: the prefill multiply on the bf16 MFMA rung.
     rows = 128
     x = synth.activations(g, rows, k, bf16=True)
-    kset.select_prefill(rec, K.Prefill.bf16_mfma)
-    xa = env["upload"](x)
+    kset.select_prefill(rec, K.Prefill.bf16_mfma_xbf16)
+    xa = env["upload"](synth.to_bf16_bits(x))
     wa = env["upload"](wbits)
     out = env["output"](4 * rows * n)
     p = P.MatmulBf16(rows=rows, n=n, k=k, col0=0, out_stride=n)

@@ -262,7 +262,8 @@ def matmul_case(c, rows, n, k, split, accumulate, rung=K.Prefill.scalar_f32):
     bits, values = random_half(c, n * k, 1)
     bits, values = bits.reshape(n, k), values.reshape(n, k)
     init = c.random(rows * n, 4 if accumulate else 0).reshape(rows, n)
-    out, xa = c.upload(init), c.upload(x)
+    packed = rung == K.Prefill.bf16_mfma_xbf16
+    out, xa = c.upload(init), c.upload(synth.to_bf16_bits(x) if packed else x)
     c.set.select_prefill(c.rec, rung)
     col0 = 0
     for cols in (split or n, n - (split or n)):
@@ -274,7 +275,7 @@ def matmul_case(c, rows, n, k, split, accumulate, rung=K.Prefill.scalar_f32):
         col0 += cols
     got = c.read(out).reshape(rows, n)
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
-    xs = synth.bf16_round(x) if rung == K.Prefill.bf16_mfma else x
+    xs = x if rung == K.Prefill.scalar_f32 else synth.bf16_round(x)
     want = init + xs.astype(np.float64) @ values.astype(np.float64).T
     return got, want, values, x
 
@@ -298,6 +299,12 @@ def test_matmul_bf16_mfma_rung(ctx):
     assert rel_err(got, want) <= 1e-5
     got, want, values, x = matmul_case(ctx, 133, 150, 96, 70, True, K.Prefill.bf16_mfma)
     assert rel_err(got, want) <= 1e-5
+    # The same with the activations bound as packed bf16 (an extension of the
+    # contract, which binds f32): identical operands, so identical results.
+    got, want, values, x = matmul_case(ctx, 133, 150, 96, 70, True, K.Prefill.bf16_mfma_xbf16)
+    assert rel_err(got, want) <= 1e-5
+    got, want, values, x = matmul_case(ctx, 300, 4100, 128, None, False, K.Prefill.bf16_mfma_xbf16)  # 128-token tiles
+    assert rel_err(got, want) <= 1e-5
 
 
 def launch_float_q8(c, x, weights, out, rows, accumulate, slices, chunked):
@@ -317,7 +324,7 @@ def launch_float_q8(c, x, weights, out, rows, accumulate, slices, chunked):
                      [partial, out], K.elementwise(rows * n))
 
 
-@pytest.mark.parametrize("rung", [K.Prefill.scalar_f32, K.Prefill.bf16_mfma])
+@pytest.mark.parametrize("rung", [K.Prefill.scalar_f32, K.Prefill.bf16_mfma, K.Prefill.bf16_mfma_xbf16])
 def test_matmul_q8_0_float(ctx, rung):
     """Unrounded float activations, k = 320, full and partial tiles, weight
     chunks, padding, accumulate and split-k; within each split-k path token
@@ -328,10 +335,12 @@ def test_matmul_q8_0_float(ctx, rung):
     raw, values = quant_rows(c, TensorType.q8_0, n, k)
     rb = k // 32 * 34
     weights = [c.gpu_weights(TensorType.q8_0, raw, k), c.gpu_weights(TensorType.q8_0, raw[: 27 * rb], k), c.gpu_weights(TensorType.q8_0, raw[27 * rb :], k)]
-    xa = c.upload(x)
+    packed = rung == K.Prefill.bf16_mfma_xbf16
+    xin = synth.to_bf16_bits(x) if packed else x
+    xa = c.upload(xin)
     init = c.random(rows * stride, 0.25).reshape(rows, stride)
     c.set.select_prefill(c.rec, rung)
-    if rung == K.Prefill.bf16_mfma:
+    if rung != K.Prefill.scalar_f32:
         # The rung's operand contract: both operands rounded to bf16.
         xs, ws, tol = synth.bf16_round(x), synth.bf16_round(values), 1e-5
     else:
@@ -350,7 +359,7 @@ def test_matmul_q8_0_float(ctx, rung):
             assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32))
             for first, count in ((0, 3), (3, 14), (17, 50)):
                 chunk_out = c.upload(init[first : first + count])
-                launch_float_q8(c, c.upload(x[first : first + count]), weights, chunk_out, count, accumulate, slices, chunked)
+                launch_float_q8(c, c.upload(xin[first : first + count]), weights, chunk_out, count, accumulate, slices, chunked)
                 assert got[first : first + count].tobytes() == c.read(chunk_out).tobytes(), "token chunking changed bits"
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
 

@@ -60,7 +60,8 @@ static_assert(kKernelCount == 57, "kernels.Kernel has 57 members");
 // (src/agility/kernels.zig:114-131) and this backend's own rung.
 static constexpr uint32_t kVariantFp16Single = 0xfffc0000u;
 static constexpr uint32_t kVariantFp16Compensated = 0xffff0000u;
-static constexpr uint32_t kVariantBf16 = 0xfffb0000u;
+static constexpr uint32_t kVariantBf16 = 0xfffb0000u;   // bf16 MFMA, f32 activations bound as the contract says
+static constexpr uint32_t kVariantBf16X = 0xfffa0000u;  // bf16 MFMA, activations bound as packed bf16 (an extension)
 
 enum class VariantKind { none, matvec, prefill };
 
@@ -68,6 +69,8 @@ zhip_result launch_matmul_bf16_f32(const Dispatch &);
 zhip_result launch_matmul_q8_0_float_f32(const Dispatch &);
 zhip_result launch_matmul_bf16_mfma(const Dispatch &);
 zhip_result launch_matmul_q8_0_float_mfma(const Dispatch &);
+zhip_result launch_matmul_bf16_mfma_xbf16(const Dispatch &);
+zhip_result launch_matmul_q8_0_float_mfma_xbf16(const Dispatch &);
 
 struct KernelInfo {
     const char *name;
@@ -76,22 +79,23 @@ struct KernelInfo {
     VariantKind variants;
     LaunchFn launch;       // variant 0 / MatvecVariant ids
     LaunchFn launch_bf16;  // the bf16 MFMA rung of a prefill identity
+    LaunchFn launch_bf16x; // the same with packed bf16 activations
     int revision;          // bumped when the implementation changes (plan-cache key)
 };
 
 static const KernelInfo kImplemented[] = {
-    {"matvec_q8_0", 5, 0b01000, VariantKind::matvec, launch_matvec_q8_0, nullptr, 1},
-    {"matvec_q4_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q4_k, nullptr, 1},
-    {"matvec_bf16", 5, 0b01000, VariantKind::none, launch_matvec_bf16, nullptr, 1},
-    {"matmul_bf16", 4, 0b1000, VariantKind::prefill, launch_matmul_bf16_f32, launch_matmul_bf16_mfma, 1},
-    {"matmul_q8_0_float", 4, 0b1000, VariantKind::prefill, launch_matmul_q8_0_float_f32, launch_matmul_q8_0_float_mfma, 1},
-    {"matmul_reduce", 3, 0b100, VariantKind::none, launch_matmul_reduce, nullptr, 1},
-    {"silu_mul", 3, 0b100, VariantKind::none, launch_silu_mul, nullptr, 1},
-    {"repack_q8_0", 3, 0b100, VariantKind::none, launch_repack_q8_0, nullptr, 1},
-    {"repad", 3, 0b100, VariantKind::none, launch_repad, nullptr, 1},
-    {"embed_q8_0", 4, 0b1000, VariantKind::none, launch_embed_q8_0, nullptr, 1},
-    {"embed_q4_k", 4, 0b1000, VariantKind::none, launch_embed_q4_k, nullptr, 1},
-    {"embed_bf16", 4, 0b1000, VariantKind::none, launch_embed_bf16, nullptr, 1},
+    {"matvec_q8_0", 5, 0b01000, VariantKind::matvec, launch_matvec_q8_0, nullptr, nullptr, 1},
+    {"matvec_q4_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q4_k, nullptr, nullptr, 1},
+    {"matvec_bf16", 5, 0b01000, VariantKind::none, launch_matvec_bf16, nullptr, nullptr, 1},
+    {"matmul_bf16", 4, 0b1000, VariantKind::prefill, launch_matmul_bf16_f32, launch_matmul_bf16_mfma, launch_matmul_bf16_mfma_xbf16, 1},
+    {"matmul_q8_0_float", 4, 0b1000, VariantKind::prefill, launch_matmul_q8_0_float_f32, launch_matmul_q8_0_float_mfma, launch_matmul_q8_0_float_mfma_xbf16, 1},
+    {"matmul_reduce", 3, 0b100, VariantKind::none, launch_matmul_reduce, nullptr, nullptr, 1},
+    {"silu_mul", 3, 0b100, VariantKind::none, launch_silu_mul, nullptr, nullptr, 1},
+    {"repack_q8_0", 3, 0b100, VariantKind::none, launch_repack_q8_0, nullptr, nullptr, 1},
+    {"repad", 3, 0b100, VariantKind::none, launch_repad, nullptr, nullptr, 1},
+    {"embed_q8_0", 4, 0b1000, VariantKind::none, launch_embed_q8_0, nullptr, nullptr, 1},
+    {"embed_q4_k", 4, 0b1000, VariantKind::none, launch_embed_q4_k, nullptr, nullptr, 1},
+    {"embed_bf16", 4, 0b1000, VariantKind::none, launch_embed_bf16, nullptr, nullptr, 1},
 };
 
 static const KernelInfo *find_kernel(const char *name, size_t len) {
@@ -456,6 +460,7 @@ zhip_result create_kernel(zhip_context *c, const Command &cmd) {
         if (p.variant == kVariantFp16Single || p.variant == kVariantFp16Compensated)
             return set_error(c, ZHIP_E_UNSUPPORTED_PREFILL, "create_kernel: %s: the fp16 LinAlg rungs are not implemented on HIP", info->name);
         if (p.variant == kVariantBf16) p.launch = info->launch_bf16;
+        else if (p.variant == kVariantBf16X) p.launch = info->launch_bf16x;
         else if (p.variant != 0) return set_error(c, ZHIP_E_BAD_COMMAND, "create_kernel: %s has no variant 0x%08x", info->name, p.variant);
         break;
     }
@@ -712,8 +717,9 @@ zhip_result zhip_get_caps(zhip_context *c, zhip_caps *out) {
 
 int32_t zhip_supports_prefill(zhip_context *c, uint32_t rung) {
     if (!c || c->lost) return 0;
-    // scalar_f32 always; the bf16 MFMA rung is this backend's own (id 3).
-    return rung == ZHIP_PREFILL_SCALAR_F32 || rung == 3u;
+    // scalar_f32 always; the bf16 MFMA rungs are this backend's own (3: f32
+    // activations as bound by the contract, 4: packed bf16 activations).
+    return rung == ZHIP_PREFILL_SCALAR_F32 || rung == 3u || rung == 4u;
 }
 
 zhip_result zhip_set_file(zhip_context *c, const void *bytes, size_t len) {

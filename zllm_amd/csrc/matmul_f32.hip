@@ -124,8 +124,9 @@ __global__ __launch_bounds__(256) void matmul_f32_kernel(MmArgs a) {
 // Checks a prefill multiply's parameters and bound ranges, for either rung.
 // The reference kernels' tile sizes (64 outputs x 16 tokens) give the logical
 // grid its meaning: the outputs and tokens it covers. `*empty` is set when the
-// dispatch has nothing to do.
-zhip_result validate_matmul(const Dispatch &d, const char *name, bool sliced, bool q8_0, bool *empty) {
+// dispatch has nothing to do. `x_bytes` is the size of one activation as bound
+// (4: f32, 2: packed bf16).
+zhip_result validate_matmul(const Dispatch &d, const char *name, bool sliced, bool q8_0, uint32_t x_bytes, bool *empty) {
     *empty = false;
     if (d.params_size < sizeof(MatmulParams)) return fail(d, ZHIP_E_BAD_COMMAND, "%s: params block too small", name);
     const MatmulParams &p = *reinterpret_cast<const MatmulParams *>(d.params);
@@ -146,7 +147,7 @@ zhip_result validate_matmul(const Dispatch &d, const char *name, bool sliced, bo
     }
     if (n == 0 || rows == 0) { *empty = true; return ZHIP_OK; }
     const uint64_t row_bytes = q8_0 ? ((p.k + p.k / 16u + 15u) & ~15u) : 2u * p.k;
-    const uint64_t x_need = rows * p.k * 4u;
+    const uint64_t x_need = rows * p.k * x_bytes;
     const uint64_t w_need = n * row_bytes;
     const uint64_t o_need = ((slices - 1) * slice_stride + (rows - 1) * p.out_stride + p.col0 + n) * 4u;
     if (x_need > d.bind[1].size || w_need > d.bind[2].size || o_need > d.bind[3].size)
@@ -161,7 +162,7 @@ zhip_result validate_matmul(const Dispatch &d, const char *name, bool sliced, bo
 template <class W>
 static zhip_result launch_matmul(const Dispatch &d, const char *name, bool sliced, bool q8_0) {
     bool empty = false;
-    if (zhip_result r = validate_matmul(d, name, sliced, q8_0, &empty)) return r;
+    if (zhip_result r = validate_matmul(d, name, sliced, q8_0, 4u, &empty)) return r;
     if (empty) return ZHIP_OK;
     const MatmulParams &p = *reinterpret_cast<const MatmulParams *>(d.params);
     MmArgs a{};

@@ -176,9 +176,10 @@ class Prefill(enum.IntEnum):
     fp16_single = 1
     fp16_compensated = 2
     bf16_mfma = 3
+    bf16_mfma_xbf16 = 4  # the same with activations bound as packed bf16
 
 
-PREFILL_VARIANT = {Prefill.scalar_f32: 0, Prefill.fp16_single: 0xFFFC0000, Prefill.fp16_compensated: 0xFFFF0000, Prefill.bf16_mfma: 0xFFFB0000}
+PREFILL_VARIANT = {Prefill.scalar_f32: 0, Prefill.fp16_single: 0xFFFC0000, Prefill.fp16_compensated: 0xFFFF0000, Prefill.bf16_mfma: 0xFFFB0000, Prefill.bf16_mfma_xbf16: 0xFFFA0000}
 prefill_kernels = (Kernel.matmul_q8_0_float, Kernel.matmul_bf16)
 
 
