@@ -21,9 +21,13 @@ def device():
 
 
 @pytest.fixture()
-def ctx(device):
+def ctx():
+    """A kernel-check context on a device of its own, so that object ids and
+    failures never leak from one test into the next."""
     from gpucheck import Ctx
+    from zllm_amd import Device
 
-    c = Ctx(device)
+    d = Device.open(0)
+    c = Ctx(d)
     yield c
-    c.close()
+    d.deinit()

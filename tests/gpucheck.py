@@ -40,21 +40,8 @@ class Ctx:
         self.rec = cmd.Recorder()
         self.rand = np.random.Generator(np.random.PCG64(seed))
         self.token = 0
-        self.buffers_from = 0
         self.set = K.Set.create(self.rec)
         self.flush()
-        self.base = [self.rec.created(k) for k in cmd.Kind]
-
-    def close(self):
-        # Release everything this context created on the shared device.
-        for kind in (cmd.Kind.bind_group, cmd.Kind.pipeline, cmd.Kind.buffer):
-            for i in range(self.rec.created(kind)):
-                self.rec.destroy(kind, i)
-        try:
-            self.host.execute(self.rec.batch(), [])
-        except Exception:
-            pass
-        self.rec.clear()
 
     def flush(self) -> list:
         """Submits what is recorded and returns the completions."""

@@ -678,7 +678,8 @@ zhip_result zhip_create(const zhip_options *options, zhip_context **out_context)
     c->caps.memory_bytes = prop.totalGlobalMem;
     c->caps.max_binding = 1ull << 31;
     c->caps.offset_align = 256;
-    snprintf(c->caps.name, sizeof c->caps.name, "%s", prop.name);
+    // Some driver stacks report no marketing name: fall back to the architecture.
+    snprintf(c->caps.name, sizeof c->caps.name, "%s", prop.name[0] ? prop.name : "AMD Instinct (gfx950)");
     snprintf(c->caps.arch, sizeof c->caps.arch, "%s", prop.gcnArchName);
     if (char *colon = strchr(c->caps.arch, ':')) *colon = 0;
     if (hipStreamCreateWithFlags(&c->stream, hipStreamNonBlocking) != hipSuccess ||
