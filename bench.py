@@ -34,6 +34,9 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 ROTATE_BYTES = 640 << 20    # distinct weight bytes a rotation must exceed (L2 + Infinity Cache, with margin)
+# HBM bytes one launch of the headline kernel moves, from rocprofv3 FETCH_SIZE and
+# WRITE_SIZE counter runs scaled by a plain copy of known size (profiles/matvec_q4k_kernel_c2.txt).
+C2_TRAFFIC_BYTES = 33_398_588
 
 
 def main() -> int:
@@ -43,11 +46,23 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c5 for the 'also' section; 'none' skips it")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="first run 4 plain elementwise copies (256 MiB read + 256 MiB written each) so a counter run has a kernel of known traffic to scale by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on one GPU; --gpus above 1 is not supported "
               "(more GPUs would each take a share of the output rows)", file=sys.stderr)
         return 2
+
+    if args.calibrate_copy:
+        import torch
+
+        a = torch.ones(64 << 20, dtype=torch.float32, device="cuda:0")
+        o = torch.empty_like(a)
+        for _ in range(4):
+            torch.add(a, 1.0, out=o)  # one elementwise kernel: reads 256 MiB, writes 256 MiB
+        torch.cuda.synchronize()
+        del a, o
 
     from zllm_amd import Device, Host, cmd, synth
     from zllm_amd import kernels as K
@@ -236,7 +251,7 @@ def main() -> int:
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(c2_bytes * args.steps / gpu_s / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": C2_TRAFFIC_BYTES,
             "us_per_launch": round(gpu_s / args.steps * 1e6, 3),
         },
         "cpu_baseline": cpu,
