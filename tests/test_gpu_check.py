@@ -307,6 +307,47 @@ def test_matmul_bf16_mfma_rung(ctx):
     assert rel_err(got, want) <= 1e-5
 
 
+@pytest.mark.parametrize("rows,n,k", [
+    (40, 200, 128),     # 64-token tiles, one k step
+    (64, 64, 416),      # 64-token tiles, four steps, the last of 32 positions
+    (129, 130, 1056),   # 128-token tiles, nine steps (three groups), ragged
+    (200, 70, 480),     # four steps, the last of 96 positions
+    (257, 100, 512),    # three token tiles, four whole steps
+    (513, 16400, 320),  # 256-token tiling: 3 x 129 tiles fill the CUs; k ragged for its 64-deep tiles
+    (1024, 8192, 256),  # 256-token tiling, whole tiles
+])
+def test_matmul_bf16_mfma_tilings(ctx, rows, n, k):
+    """Every tiling and step-count path of the bf16 rung (64- and 128-token
+    tiles, the 256-token tiling of long steps; whole groups of steps, left-over
+    steps and a ragged last step), with bf16 and Q8_0 weights, f32 and packed
+    bf16 activations, against the rung's operand contract."""
+    c = ctx
+    x = c.random(rows * k, 1).reshape(rows, k)
+    xs = synth.bf16_round(x).astype(np.float64)
+    # bf16 weights
+    bits, values = random_half(c, n * k, 1)
+    for rung in (K.Prefill.bf16_mfma, K.Prefill.bf16_mfma_xbf16):
+        packed = rung == K.Prefill.bf16_mfma_xbf16
+        xa = c.upload(synth.to_bf16_bits(x) if packed else x)
+        c.set.select_prefill(c.rec, rung)
+        out = c.output(rows * n)
+        c.launcher().launch(Kernel.matmul_bf16, P.MatmulBf16(rows=rows, n=n, k=k, col0=0, out_stride=n), [xa, c.upload(bits.reshape(n, k)), out],
+                            (K.div_ceil(n, K.matmul_tile_n), K.div_ceil(rows, K.matmul_tile_t), 1))
+        got = c.read(out).reshape(rows, n)
+        assert rel_err(got, xs @ values.reshape(n, k).astype(np.float64).T) <= 1e-5, rung
+        # Q8_0 weights, accumulating into a strided output at a column offset.
+        raw, wq = quant_rows(c, TensorType.q8_0, n, k)
+        init = c.random(rows * (n + 9), 0.5).reshape(rows, n + 9)
+        out = c.upload(init)
+        c.launcher().launch(Kernel.matmul_q8_0_float, P.MatmulQuant(rows=rows, n=n, k=k, col0=5, out_stride=n + 9, accumulate=1, k_slice=k),
+                            [xa, c.gpu_weights(TensorType.q8_0, raw, k), out], (K.div_ceil(n, 64), K.div_ceil(rows, 16), 1))
+        got = c.read(out).reshape(rows, n + 9)
+        want = init[:, 5 : 5 + n] + xs @ synth.bf16_round(wq).astype(np.float64).T
+        assert rel_err(got[:, 5 : 5 + n], want) <= 1e-5, rung
+        assert np.array_equal(got[:, :5], init[:, :5]) and np.array_equal(got[:, 5 + n :], init[:, 5 + n :]), "columns outside the chunk were written"
+    c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
+
+
 def launch_float_q8(c, x, weights, out, rows, accumulate, slices, chunked):
     """Two weight chunks exercise nonzero col0 and a padded output stride;
     split-k partials are dense per chunk (src/kernels/check.zig:752-770)."""

@@ -62,6 +62,20 @@ struct DeviceInfo {
     int max_lds = 65536;
 };
 
+struct Dispatch;
+
+// Device scratch a launcher may ask for (the bf16 copy of a step's f32
+// activations). Owned by the context, grown on demand, freed with the context.
+// Everything runs on the context's one in-order stream, so consecutive
+// dispatches can share it.
+struct Workspace {
+    uint8_t *data = nullptr;
+    uint64_t bytes = 0;
+    // Makes at least `want` bytes available.
+    zhip_result reserve(const Dispatch &d, uint64_t want);
+    void release();
+};
+
 // One resolved dispatch: binding 0's bytes come from the host's shadow copy of
 // the uniform buffer, so kernels take their parameters by value.
 struct Dispatch {
@@ -72,6 +86,7 @@ struct Dispatch {
     uint32_t variant = 0;
     hipStream_t stream = nullptr;
     const DeviceInfo *dev = nullptr;
+    Workspace *work = nullptr;
     char *err = nullptr;  // message buffer for a failed launch
     size_t err_cap = 0;
 };

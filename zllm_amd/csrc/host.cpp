@@ -193,11 +193,37 @@ struct TimingTotal { uint64_t ns = 0, count = 0; };
 
 using namespace zhip;
 
+// Growing replaces the allocation, so earlier dispatches that may still be
+// running with the old one are waited for first.
+zhip_result Workspace::reserve(const Dispatch &d, uint64_t want) {
+    if (want <= bytes) return ZHIP_OK;
+    const uint64_t size = (want + (8u << 20) - 1) & ~(uint64_t)((8u << 20) - 1);
+    if (hipStreamSynchronize(d.stream) != hipSuccess) return fail(d, ZHIP_E_GPU, "workspace: stream synchronisation failed");
+    if (data) (void)hipFree(data);
+    data = nullptr;
+    bytes = 0;
+    const hipError_t e = hipMalloc(reinterpret_cast<void **>(&data), size);
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        data = nullptr;
+        return fail(d, e == hipErrorOutOfMemory ? ZHIP_E_OUT_OF_MEMORY : ZHIP_E_GPU, "workspace: cannot allocate %llu bytes", (unsigned long long)size);
+    }
+    bytes = size;
+    return ZHIP_OK;
+}
+
+void Workspace::release() {
+    if (data) (void)hipFree(data);
+    data = nullptr;
+    bytes = 0;
+}
+
 struct zhip_context {
     int device = 0;
     hipStream_t stream = nullptr;
     hipEvent_t ev_begin = nullptr, ev_end = nullptr;
     DeviceInfo info;
+    Workspace work;
     zhip_caps caps{};
     bool lost = false;
     std::string message;
@@ -297,6 +323,7 @@ zhip_result run_dispatch(zhip_context *c, const Op &op, size_t &timed) {
     Dispatch d;
     d.stream = c->stream;
     d.dev = &c->info;
+    d.work = &c->work;
     d.variant = pl->variant;
     memcpy(d.grid, op.grid, sizeof d.grid);
     char err[384] = "";
@@ -698,6 +725,7 @@ zhip_result zhip_destroy(zhip_context *c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     for (Buffer &b : c->buffers)
         if (b.alive && b.dev) (void)hipFree(b.dev);
+    c->work.release();
     for (hipEvent_t ev : c->events) (void)hipEventDestroy(ev);
     if (c->download) (void)hipHostFree(c->download);
     if (c->ev_begin) (void)hipEventDestroy(c->ev_begin);

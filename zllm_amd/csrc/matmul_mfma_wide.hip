@@ -1,0 +1,249 @@
+// Prefill multiplies of many tokens on the CDNA4 matrix cores: the bf16 rung of
+// matmul_q8_0_float and matmul_bf16 (src/kernels/matmul_q8_0_float.wgsl,
+// src/kernels/matmul_half.wgsl) for steps of more than 128 tokens whose
+// activations are bound as packed bf16.
+//
+// out[t][col0 + j] (+)= sum_i x[t][i] * bf16(w[j][i]), fp32 accumulate.
+//
+// Why a second tiling: turning a Q8_0 weight into bf16 costs 2.5 VALU
+// operations, and a workgroup does that once per weight of its tile whatever
+// the number of tokens it multiplies them with. 256 tokens per workgroup make
+// the matrix cores, not the conversion, the longer pole (per 64-deep k tile and
+// SIMD: 1024 MFMA cycles against ~330 VALU cycles), and halve the bytes a CU
+// pulls from L2 per flop.
+//
+// Tiling: 512 threads = eight wave64s as 4 (tokens) x 2 (outputs), each wave a
+// 64 x 64 quadrant of the 256 x 128 tile as 4 x 4 MFMA tiles of 16 x 16 x 32:
+// two waves per SIMD, so one wave's LDS waits, conversions and barrier hide
+// behind the other's MFMAs. k tiles are 64 deep and double buffered in LDS
+// (rows padded to 144 bytes: conflict-free 16-byte fragment reads); three k
+// tiles of global loads are kept in flight in registers.
+//
+// The launcher picks this tiling only when its tiles fill the CUs; smaller
+// steps take the 128 x 64 tiling of matmul_mfma.hip.
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "decode.cuh"
+
+namespace zhip {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+
+namespace wide {
+
+constexpr int GM = 256, GN = 128, GK = 64, THREADS = 512;
+constexpr int ROW = GK * 2 + 16;                 // LDS bytes per tile row
+constexpr int XS = GM * ROW, WS = GN * ROW;      // bytes per buffer
+constexpr int LDS_BYTES = 2 * (XS + WS);         // 110,592
+
+struct Args {
+    const uint8_t *x;   // packed bf16 rows
+    const uint8_t *w;
+    float *out;
+    uint32_t rows, n, k, col0, out_stride, accumulate, row_bytes;
+    uint32_t mtiles, ntiles;
+};
+
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    const f32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+}
+
+// A thread stages 16 weights of one row per k tile: row = tid / 4, quarter = tid % 4.
+struct WQ8_0 {
+    struct Regs { u32x4 q; uint32_t d; };
+    __device__ static void load(const uint8_t *row, uint32_t k, uint32_t kpos, Regs &r) {
+        r.q = *reinterpret_cast<const u32x4 *>(row + kpos);
+        r.d = *reinterpret_cast<const uint16_t *>(row + k + 2u * (kpos / 32u));
+    }
+    __device__ static void store(const Regs &r, u32x4 *dst) {
+        const float d = half_bits_to_float(r.d);
+        uint32_t o[8];
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const int32_t word = (int32_t)r.q[e];
+            const float f0 = (float)(int8_t)(word) * d;
+            const float f1 = (float)(int8_t)(word >> 8) * d;
+            const float f2 = (float)(int8_t)(word >> 16) * d;
+            const float f3 = (float)(word >> 24) * d;
+            o[2 * e] = pack_bf16(f0, f1);
+            o[2 * e + 1] = pack_bf16(f2, f3);
+        }
+        dst[0] = u32x4{o[0], o[1], o[2], o[3]};
+        dst[1] = u32x4{o[4], o[5], o[6], o[7]};
+    }
+};
+
+struct WBf16 {
+    struct Regs { u32x4 v[2]; };
+    __device__ static void load(const uint8_t *row, uint32_t, uint32_t kpos, Regs &r) {
+        const u32x4 *src = reinterpret_cast<const u32x4 *>(row + 2u * kpos);
+        r.v[0] = src[0];
+        r.v[1] = src[1];
+    }
+    __device__ static void store(const Regs &r, u32x4 *dst) {
+        dst[0] = r.v[0];
+        dst[1] = r.v[1];
+    }
+};
+
+// Activations: four 16-byte pieces per thread and k tile, rows tid / 8 + 64 i,
+// piece tid % 8 of the row's 128 bytes, so eight lanes read one full line.
+struct XRegs { u32x4 v[4]; };
+
+template <class W, bool RAGGED>
+__global__ __launch_bounds__(THREADS) void matmul_mfma_wide_kernel(Args a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    uint8_t *const xs = lds;            // [2][GM * ROW]
+    uint8_t *const ws = lds + 2 * XS;   // [2][GN * ROW]
+
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    // Workgroups go round-robin over the 8 XCDs: renumber them so that one XCD's
+    // L2 sees neighbours in (token tile, output tile) order, which share one slab
+    // of activations.
+    uint32_t id = blockIdx.x;
+    const uint32_t total = gridDim.x;
+    if (total % 8u == 0) id = (id % 8u) * (total / 8u) + id / 8u;
+    const uint32_t nt = id % a.ntiles, mt = id / a.ntiles;
+    const uint32_t j0 = nt * GN, t0 = mt * GM;
+    const uint32_t kb = 0, ke = a.k;
+    const uint32_t wm = (wave >> 1) * 64u, wn = (wave & 1u) * 64u;
+    const uint32_t lrow = lane & 15u, lk = (lane >> 4) * 16u;
+
+    f32x4 acc[4][4];
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+#pragma unroll
+        for (int j = 0; j < 4; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    // Staging assignments. Rows past the matrix or the step are clamped: their
+    // results are never stored.
+    const uint32_t wrow = tid >> 2, wq = tid & 3u;
+    const uint32_t wj = min(j0 + wrow, a.n - 1u);
+    const uint8_t *wsrc = a.w + (size_t)wj * a.row_bytes;
+    uint8_t *wdst = ws + wrow * ROW + 32u * wq;
+    const uint32_t xr0 = tid >> 3, xpiece = tid & 7u;
+    const uint8_t *xsrc[4];
+#pragma unroll
+    for (int i = 0; i < 4; i++) xsrc[i] = a.x + (size_t)min(t0 + xr0 + 64u * i, a.rows - 1u) * a.k * 2u;
+    uint8_t *xdst = xs + xr0 * ROW + 16u * xpiece;
+    const uint32_t wk_last = ke - 16u, xk_last = ke - 8u;
+
+    // Loads are unconditional (positions clamped into the split) so no branch
+    // separates them from their use; a tile that straddles the end of the split
+    // zeroes its activations instead, which zeroes the products whatever finite
+    // weights the clamped loads brought.
+    auto fetch = [&](uint32_t k0, typename W::Regs &w, XRegs &x) __attribute__((always_inline)) {
+        W::load(wsrc, a.k, min(k0 + 16u * wq, wk_last), w);
+        const uint32_t xk = min(k0 + 8u * xpiece, xk_last);
+#pragma unroll
+        for (int i = 0; i < 4; i++) x.v[i] = *reinterpret_cast<const u32x4 *>(xsrc[i] + 2u * xk);
+    };
+    auto commit = [&](uint32_t b, uint32_t k0, const typename W::Regs &w, XRegs &x) __attribute__((always_inline)) {
+        if (RAGGED && k0 + 8u * xpiece >= ke) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) x.v[i] = u32x4{0u, 0u, 0u, 0u};
+        }
+        W::store(w, reinterpret_cast<u32x4 *>(wdst + b * WS));
+#pragma unroll
+        for (int i = 0; i < 4; i++) *reinterpret_cast<u32x4 *>(xdst + b * XS + i * (64 * ROW)) = x.v[i];
+    };
+    uint32_t cur = 0;
+    auto tile = [&](uint32_t kc, typename W::Regs &wfill, XRegs &xfill, typename W::Regs &wnext, XRegs &xnext) __attribute__((always_inline)) {
+        fetch(kc + 3u * GK, wfill, xfill);
+        const uint8_t *xb = xs + cur * XS + (wm + lrow) * ROW + lk;
+        const uint8_t *wb = ws + cur * WS + (wn + lrow) * ROW + lk;
+#pragma unroll
+        for (int kk = 0; kk < GK / 32; kk++) {
+            bf16x8 af[4], bfr[4];
+#pragma unroll
+            for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const bf16x8 *>(xb + 16 * i * ROW + 64 * kk);
+#pragma unroll
+            for (int j = 0; j < 4; j++) bfr[j] = *reinterpret_cast<const bf16x8 *>(wb + 16 * j * ROW + 64 * kk);
+#pragma unroll
+            for (int i = 0; i < 4; i++)
+#pragma unroll
+                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+        if (kc + GK < ke) commit(cur ^ 1u, kc + GK, wnext, xnext);
+        __syncthreads();
+        cur ^= 1u;
+    };
+
+    typename W::Regs w0, w1, w2;
+    XRegs x0, x1, x2;
+    fetch(kb, w0, x0);
+    fetch(kb + GK, w1, x1);
+    fetch(kb + 2 * GK, w2, x2);
+    commit(0, kb, w0, x0);
+    __syncthreads();
+    // Whole groups of three tiles run without a branch between them, so the
+    // loop has a single back edge and the loads in flight are counted exactly;
+    // the one or two tiles left over follow the loop.
+    uint32_t k0 = kb;
+    for (; k0 + 3 * GK <= ke; k0 += 3 * GK) {
+        tile(k0, w0, x0, w1, x1);
+        tile(k0 + GK, w1, x1, w2, x2);
+        tile(k0 + 2 * GK, w2, x2, w0, x0);
+    }
+    if (k0 < ke) {
+        tile(k0, w0, x0, w1, x1);
+        if (k0 + GK < ke) tile(k0 + GK, w1, x1, w2, x2);
+    }
+
+    // D[token][output]: the lane holds output column lane % 16 and token rows
+    // 4 * (lane / 16) .. + 3 of each 16 x 16 tile.
+#pragma unroll
+    for (int i = 0; i < 4; i++) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t col = j0 + wn + 16 * j + lrow;
+            if (col >= a.n) continue;
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                const uint32_t t = t0 + wm + 16 * i + 4 * (lane >> 4) + r;
+                if (t >= a.rows) continue;
+                const size_t o = (size_t)t * a.out_stride + a.col0 + col;
+                const float v = acc[i][j][r];
+                a.out[o] = a.accumulate ? a.out[o] + v : v;
+            }
+        }
+    }
+}
+
+template <class W>
+static zhip_result launch(const Dispatch &d, const char *name, Args a) {
+    a.mtiles = (a.rows + GM - 1) / GM;
+    a.ntiles = (a.n + GN - 1) / GN;
+    const uint32_t tiles = a.mtiles * a.ntiles;
+    const bool ragged = a.k % GK != 0;
+    auto kernel = ragged ? matmul_mfma_wide_kernel<W, true> : matmul_mfma_wide_kernel<W, false>;
+    static bool configured[2] = {false, false};
+    if (!configured[ragged]) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, LDS_BYTES);
+        }
+        configured[ragged] = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3(tiles), dim3(THREADS), LDS_BYTES, d.stream, a);
+    return check_launch(d, name);
+}
+
+}  // namespace wide
+
+// Called by the bf16-activation rung's launchers once the dispatch is validated.
+zhip_result launch_mfma_wide(const Dispatch &d, const char *name, bool q8_0, const uint8_t *x, const uint8_t *w, float *out,
+    uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, uint32_t row_bytes) {
+    wide::Args a{};
+    a.x = x; a.w = w; a.out = out;
+    a.rows = rows; a.n = n; a.k = k; a.col0 = col0; a.out_stride = out_stride; a.accumulate = accumulate; a.row_bytes = row_bytes;
+    return q8_0 ? wide::launch<wide::WQ8_0>(d, name, a) : wide::launch<wide::WBf16>(d, name, a);
+}
+
+}  // namespace zhip
