@@ -386,7 +386,8 @@ zhip_result launch_matvec_q4k(const Dispatch &d, const MvArgs &a) {
     for (uint32_t t0 = 0; t0 < a.m;) {
         uint32_t left = a.m - t0;
         uint32_t mt = left >= 3u ? 4u : left;
-        while (mt > 1u && mt * tok_lds > 65536u) mt >>= 1;
+        // Two workgroups a CU must fit their staged tokens in the 160 KB of LDS.
+        while (mt > 1u && mt * tok_lds > 80u * 1024u - 64u) mt >>= 1;
         q.t0 = t0;
         q.mt = left < mt ? left : mt;
         const uint32_t lds = (uint32_t)(mt * tok_lds);
