@@ -18,7 +18,8 @@
 //  * LDS moves 128 bytes per clock and CU. Q8_0 weights therefore cross LDS as
 //    the bytes they are stored in and are dequantised after the fragment read,
 //    in the registers of the one wave that multiplies them: half the LDS bytes
-//    of staging bf16, and no weight is converted twice.
+//    of staging bf16, and no weight is converted twice. Rows are unpadded
+//    128-byte lines with their 16-byte chunks permuted against bank conflicts.
 //  * MFMAs and ordinary vector instructions share one issue port per SIMD, and
 //    turning a Q8_0 weight into bf16 takes 2.5 of the latter. The tile is
 //    therefore tall: 128 tokens x 64 matrix rows, so that a converted weight
@@ -39,9 +40,10 @@
 // eight of matrix row l % 16: lane group g = l / 16 owns positions 8 g .. 8 g + 7
 // of the wave's 32.
 //
-// Pipeline: three steps of global loads in flight in registers (buffer loads,
-// so anything past the end of a binding reads as zero), LDS double buffered,
-// fragments read one step ahead of their MFMAs, one barrier per step. Activations bound as f32 are first narrowed to packed bf16
+// Pipeline: buffer loads straight into LDS (no registers, no LDS store
+// instructions; anything past the end of a binding reads as zero), three LDS
+// buffers so that memory runs three steps ahead, fragments read one step ahead
+// of their MFMAs, one barrier per step. Activations bound as f32 are first narrowed to packed bf16
 // in the context's workspace by a small kernel.
 #include <hip/hip_runtime.h>
 
@@ -64,7 +66,6 @@ typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 namespace {
 
 constexpr int BN = 64, BK = 128, THREADS = 512;
-constexpr int XROW = BK * 2 + 16;  // LDS bytes per token row; the padding makes 16-byte fragment reads conflict-free
 
 struct MfmaArgs {
     const uint8_t *x;  // packed bf16 rows
@@ -87,36 +88,62 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const uint8_t *bas
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, (int)bytes, 0x00020000);
 }
 
+typedef __attribute__((address_space(3))) void *lds_ptr;
+
+// A workgroup barrier that leaves loads into LDS in flight. __syncthreads()
+// carries a release fence, which waits for every outstanding memory operation,
+// the loads running steps ahead included; here a wave waits for exactly the
+// loads it must (vmcnt) and for its own LDS instructions, then joins.
+template <int LOADS_LEFT>
+__device__ __forceinline__ void sync_keeping_loads() {
+    asm volatile("s_waitcnt vmcnt(%0) lgkmcnt(0)" ::"n"(LOADS_LEFT) : "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// One wave-wide load of 16 bytes a lane straight into LDS: lane l's bytes land
+// at dst + 16 l, whatever global offset the lane asked for.
+__device__ __forceinline__ void load_lds_b128(__amdgpu_buffer_rsrc_t buf, uint8_t *dst, uint32_t offset) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)dst, 16, offset, 0, 0, 0);
+}
+__device__ __forceinline__ void load_lds_b32(__amdgpu_buffer_rsrc_t buf, uint8_t *dst, uint32_t offset) {
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)dst, 4, offset, 0, 0, 0);
+}
+
+// LDS holds operand rows as 128-byte lines, eight rows to the kilobyte one
+// wave-wide load fills. Unpadded lines would put every other row of a fragment
+// read on the same banks, so the 16-byte chunks of a line are stored permuted:
+// chunk c of row r sits at position c ^ key(r). The loading lane asks for the
+// chunk that belongs at its position; a reader applies the same key. With this
+// key the sixteen rows of a fragment read cover all 64 banks once.
+__device__ __forceinline__ uint32_t line_key(uint32_t row) { return (row & 7u) ^ ((row >> 3) & 1u); }
+
 // ---- weights ------------------------------------------------------------------------
-// LDS holds a step's 64 rows as stored (WROW bytes apart), Q8_0 followed by the
-// rows' four scales. Loader thread tid moves 16-byte chunks so that neighbouring
-// lanes cover whole lines; consumer lane (row, g) of k quarter kq reads its
-// eight weights back.
+// A step's 64 rows as stored, Q8_0 followed by the rows' four scales.
+// Consumer lane (row, g) of k quarter kq reads its eight weights back.
 
 struct WQ8_0 {
-    static constexpr int WROW = BK + 16;
-    static constexpr int SCALES = BN * WROW;  // byte offset of the scales: [row][4] f16
+    static constexpr int SCALES = BN * 128;   // byte offset of the scales: [row][4] f16
     static constexpr int WBUF = SCALES + BN * 8;
-    struct Raw { u32x4 q; uint32_t d; };
+    static constexpr int LOADS = 2;           // wave-wide loads a step issues per wave
     struct Offsets { uint32_t q, d; };
-    // chunk tid % 8 of row tid / 8; scale tid % 4 of row (tid % 256) / 4 (the
-    // upper half of the workgroup loads the same scales and does not store them).
-    __device__ static Offsets offsets(const MfmaArgs &a, uint32_t j0, uint32_t tid) {
-        return {(j0 + (tid >> 3)) * a.row_bytes + 16u * (tid & 7u), (j0 + ((tid & 255u) >> 2)) * a.row_bytes + a.k + 2u * (tid & 3u)};
+    // Wave w loads rows 8 w .. 8 w + 7 (lane l: row l / 8, position l % 8) and,
+    // every wave the same (so that all waves have the same loads in flight),
+    // the 128 scale words: word 64 (w % 2) + l = scales 2 (l % 2), + 1 of row
+    // 32 (w % 2) + l / 2.
+    __device__ static Offsets offsets(const MfmaArgs &a, uint32_t j0, uint32_t wave, uint32_t lane) {
+        const uint32_t row = 8u * wave + (lane >> 3);
+        const uint32_t srow = 32u * (wave & 1u) + (lane >> 1);
+        return {(j0 + row) * a.row_bytes + 16u * ((lane & 7u) ^ line_key(row)), (j0 + srow) * a.row_bytes + a.k + 4u * (lane & 1u)};
     }
-    __device__ static void load(__amdgpu_buffer_rsrc_t w, const Offsets &o, uint32_t tid, uint32_t k0, Raw &r) {
-        r.q = __builtin_amdgcn_raw_buffer_load_b128(w, o.q + k0, 0, 0);
-        r.d = __builtin_amdgcn_raw_buffer_load_b16(w, o.d + (k0 >> 4), 0, 0);
-    }
-    // Scales of blocks from `ke` on are stored as zero: what a load past the
-    // slice brought is not a scale.
-    __device__ static void store(const Raw &r, uint8_t *buf, uint32_t tid, uint32_t k0, uint32_t ke, bool ragged) {
-        *reinterpret_cast<u32x4 *>(buf + (tid >> 3) * WROW + 16u * (tid & 7u)) = r.q;
-        if (tid < 256u) *reinterpret_cast<uint16_t *>(buf + SCALES + 2u * tid) = !ragged || k0 + 32u * (tid & 3u) < ke ? (uint16_t)r.d : (uint16_t)0;
+    __device__ static void load(__amdgpu_buffer_rsrc_t w, const Offsets &o, uint8_t *buf, uint32_t wave, uint32_t k0) {
+        load_lds_b128(w, buf + 1024u * wave, o.q + k0);
+        load_lds_b32(w, buf + SCALES + 256u * (wave & 1u), o.d + (k0 >> 4));
     }
     struct Frag { u32x2 q; uint32_t d; };
-    __device__ static void read(const uint8_t *buf, uint32_t row, uint32_t g, uint32_t kq, Frag &f) {
-        f.q = *reinterpret_cast<const u32x2 *>(buf + row * WROW + 32u * kq + 8u * g);
+    // row: the lane's row of the tile (its key is that of row % 16).
+    __device__ static void read(const uint8_t *buf, uint32_t row, uint32_t key, uint32_t g, uint32_t kq, Frag &f) {
+        f.q = *reinterpret_cast<const u32x2 *>(buf + row * 128u + 16u * ((2u * kq + (g >> 1)) ^ key) + 8u * (g & 1u));
         f.d = *reinterpret_cast<const uint16_t *>(buf + SCALES + 8u * row + 2u * kq);
     }
     // bf16(q * d) of the lane's eight weights.
@@ -133,49 +160,36 @@ struct WQ8_0 {
 };
 
 struct WBf16 {
-    static constexpr int WROW = BK * 2 + 16;
-    static constexpr int WBUF = BN * WROW;
-    struct Raw { u32x4 v[2]; };
+    static constexpr int WBUF = 2 * BN * 128;  // two lines a row: [line][row][128]
+    static constexpr int LOADS = 2;
     struct Offsets { uint32_t q[2]; };
-    // chunk tid % 16 of rows tid / 16 and tid / 16 + 32.
-    __device__ static Offsets offsets(const MfmaArgs &a, uint32_t j0, uint32_t tid) {
-        const uint32_t o = (j0 + (tid >> 4)) * a.row_bytes + 16u * (tid & 15u);
-        return {{o, o + 32u * a.row_bytes}};
+    // Wave w loads both lines of rows 8 w .. 8 w + 7 (lane l: row l / 8, position l % 8).
+    __device__ static Offsets offsets(const MfmaArgs &a, uint32_t j0, uint32_t wave, uint32_t lane) {
+        const uint32_t row = 8u * wave + (lane >> 3);
+        const uint32_t o = (j0 + row) * a.row_bytes + 16u * ((lane & 7u) ^ line_key(row));
+        return {{o, o + 128u}};
     }
-    __device__ static void load(__amdgpu_buffer_rsrc_t w, const Offsets &o, uint32_t, uint32_t k0, Raw &r) {
-        r.v[0] = __builtin_amdgcn_raw_buffer_load_b128(w, o.q[0] + 2u * k0, 0, 0);
-        r.v[1] = __builtin_amdgcn_raw_buffer_load_b128(w, o.q[1] + 2u * k0, 0, 0);
-    }
-    __device__ static void store(const Raw &r, uint8_t *buf, uint32_t tid, uint32_t, uint32_t, bool) {
-#pragma unroll
-        for (int i = 0; i < 2; i++) *reinterpret_cast<u32x4 *>(buf + ((tid >> 4) + 32u * i) * WROW + 16u * (tid & 15u)) = r.v[i];
+    __device__ static void load(__amdgpu_buffer_rsrc_t w, const Offsets &o, uint8_t *buf, uint32_t wave, uint32_t k0) {
+        load_lds_b128(w, buf + 1024u * wave, o.q[0] + 2u * k0);
+        load_lds_b128(w, buf + BN * 128 + 1024u * wave, o.q[1] + 2u * k0);
     }
     struct Frag { u32x4 v; };
-    __device__ static void read(const uint8_t *buf, uint32_t row, uint32_t g, uint32_t kq, Frag &f) {
-        f.v = *reinterpret_cast<const u32x4 *>(buf + row * WROW + 64u * kq + 16u * g);
+    __device__ static void read(const uint8_t *buf, uint32_t row, uint32_t key, uint32_t g, uint32_t kq, Frag &f) {
+        f.v = *reinterpret_cast<const u32x4 *>(buf + (kq >> 1) * (BN * 128) + row * 128u + 16u * ((4u * (kq & 1u) + g) ^ key));
     }
     __device__ static bf16x8 frag(const Frag &f) { return __builtin_bit_cast(bf16x8, f.v); }
 };
 
-// ---- activations --------------------------------------------------------------------
-// 16 MT tokens per tile. Loader thread tid: rows tid / 8 (+ 64), piece tid % 8
-// of both 128-byte lines of the row's step, so eight neighbouring lanes read
-// one whole line.
-
-template <int MT>
-struct XStage {
-    static constexpr int HALVES = MT / 4;  // 64-row groups
-    u32x4 v[2 * HALVES];
-};
-
-template <class W, int MT> constexpr int lds_bytes() { return 2 * (16 * MT * XROW + W::WBUF); }
+template <class W, int MT> constexpr int buf_bytes() { return 16 * MT * 256 + W::WBUF; }
+template <class W, int MT> constexpr int lds_bytes() { return 3 * buf_bytes<W, MT>(); }
 
 template <class W, int MT, bool RAGGED>
 __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    constexpr int BM = 16 * MT, XBUF = BM * XROW;
-    constexpr int BUF = XBUF + W::WBUF;  // one buffer: activations, then weights
-    constexpr int HALVES = MT / 4;
+    constexpr int BM = 16 * MT, XBUF = BM * 256;   // activations: [line][row][128]
+    constexpr int BUF = XBUF + W::WBUF;            // one buffer: activations, then weights
+    constexpr int XLOADS = MT / 2;                 // wave-wide activation loads a step issues per wave
+    constexpr int LOADS = XLOADS + W::LOADS;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t j0 = blockIdx.x * BN, t0 = blockIdx.y * BM, z = blockIdx.z;
     const uint32_t kb = z * a.k_slice, ke = min(a.k, kb + a.k_slice);
@@ -187,97 +201,92 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
 #pragma unroll
         for (int j = 0; j < 2; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    // Loads never branch: the k position is part of the offset the hardware
-    // range-checks, so anything past the end of x or w reads as zero; positions
-    // past the slice but inside the operand read whatever follows, and a step
-    // that straddles the end of the slice (RAGGED) stores zeros for those
-    // activations and scales instead.
+    // Loads go straight from memory into LDS, three steps ahead of their use,
+    // through buffers whose range check covers the k position: anything past
+    // the end of x or w reads as zero, positions past the slice but inside the
+    // operand read whatever follows. The 32 positions of a k quarter belong to
+    // one wave, so a step that straddles the end of the slice (RAGGED) needs no
+    // zeroing in LDS: the waves whose quarter lies past the end multiply zeros.
     const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.x, a.x_bytes), wbuf = make_buffer(a.w, a.w_bytes);
-    const typename W::Offsets woff = W::offsets(a, j0, tid);
-    const uint32_t xoff = (t0 + (tid >> 3)) * a.k * 2u + 16u * (tid & 7u);
-    auto fetch = [&](uint32_t k0, typename W::Raw &w, XStage<MT> &x) __attribute__((always_inline)) {
-        W::load(wbuf, woff, tid, k0, w);
+    const typename W::Offsets woff = W::offsets(a, j0, wave, lane);
+    // Activation block b = wave + 8 i of the step: line b / (BM / 8), rows 8 (b % (BM / 8)) .. + 7.
+    uint32_t xoff[XLOADS], xdst[XLOADS];
 #pragma unroll
-        for (int h = 0; h < HALVES; h++) {
-            const uint32_t o = xoff + h * 64u * a.k * 2u + 2u * k0;
-            x.v[2 * h] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, o, 0, 0);
-            x.v[2 * h + 1] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, o + 128u, 0, 0);
-        }
-    };
-    auto commit = [&](uint32_t buf, uint32_t k0, const typename W::Raw &w, const XStage<MT> &x) __attribute__((always_inline)) {
-        uint8_t *xb = lds + buf * BUF + (tid >> 3) * XROW + 16u * (tid & 7u);
+    for (int i = 0; i < XLOADS; i++) {
+        const uint32_t b = wave + 8u * i, line = b / (BM / 8), row = 8u * (b % (BM / 8)) + (lane >> 3);
+        xoff[i] = (t0 + row) * a.k * 2u + 128u * line + 16u * ((lane & 7u) ^ line_key(row));
+        xdst[i] = line * (BM * 128) + 1024u * (b % (BM / 8));
+    }
+    auto fetch = [&](uint32_t buf, uint32_t k0) __attribute__((always_inline)) {
+        uint8_t *base = lds + buf * BUF;
 #pragma unroll
-        for (int h = 0; h < HALVES; h++)
-#pragma unroll
-            for (int l = 0; l < 2; l++) {
-                const bool keep = !RAGGED || k0 + 64u * l + 8u * (tid & 7u) < ke;
-                *reinterpret_cast<u32x4 *>(xb + h * 64 * XROW + 128 * l) = keep ? x.v[2 * h + l] : u32x4{0u, 0u, 0u, 0u};
-            }
-        W::store(w, lds + buf * BUF + XBUF, tid, k0, ke, RAGGED);
+        for (int i = 0; i < XLOADS; i++) load_lds_b128(xbuf, base + xdst[i], xoff[i] + 2u * k0);
+        W::load(wbuf, woff, base + XBUF, wave, k0);
     };
 
-    // Fragments live in registers one step ahead of the MFMAs: during step s
-    // the wave multiplies the fragments of s, reads those of s + 1 from the
-    // other LDS buffer (each token fragment right after the MFMAs that consumed
-    // its predecessor), and writes the global data of s + 2 into the buffer the
-    // fragments of s came from, so LDS traffic, conversions and MFMAs of one
-    // wave overlap instead of queueing behind the barrier. Three steps of
-    // global loads are in flight in registers.
+    // Fragment addresses: the lane's token row within a 16-row tile and its
+    // eight positions 32 kq + 8 g .. + 7 of the step, i.e. chunk 4 (kq % 2) + g
+    // of line kq / 2.
+    const uint32_t key = line_key(lrow);
+    const uint32_t a_at = (kq >> 1) * (BM * 128) + lrow * 128u + 16u * ((4u * (kq & 1u) + g) ^ key);
     bf16x8 af[MT], bf[2];
-    uint32_t cur = 0;
     auto read_b = [&](uint32_t buf, typename W::Frag (&wf)[2]) __attribute__((always_inline)) {
 #pragma unroll
-        for (int j = 0; j < 2; j++) W::read(lds + buf * BUF + XBUF, 32u * wn + 16u * j + lrow, g, kq, wf[j]);
+        for (int j = 0; j < 2; j++) W::read(lds + buf * BUF + XBUF, 32u * wn + 16u * j + lrow, key, g, kq, wf[j]);
     };
-    auto step = [&](uint32_t kc, typename W::Raw &wfill, XStage<MT> &xfill, const typename W::Raw &wput, const XStage<MT> &xput) __attribute__((always_inline)) {
-        fetch(kc + 4u * BK, wfill, xfill);
-        const uint8_t *xn = lds + (cur ^ 1u) * BUF + lrow * XROW + 64u * kq + 16u * g;
-        typename W::Frag wf[2];
-        read_b(cur ^ 1u, wf);
+    auto convert = [&](const typename W::Frag (&wf)[2], uint32_t k0) __attribute__((always_inline)) {
+        const bool live = !RAGGED || k0 + 32u * kq < ke;
 #pragma unroll
-        for (int i = 0; i < MT; i++) {
-#pragma unroll
-            for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
-            af[i] = *reinterpret_cast<const bf16x8 *>(xn + 16 * i * XROW);
-        }
-#pragma unroll
-        for (int j = 0; j < 2; j++) bf[j] = W::frag(wf[j]);
-        // Unconditional: past the last step it writes a buffer nobody reads,
-        // and the step stays one basic block for the scheduler.
-        commit(cur, kc + 2u * BK, wput, xput);
-        __syncthreads();
-        cur ^= 1u;
+        for (int j = 0; j < 2; j++) bf[j] = live ? W::frag(wf[j]) : __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
     };
 
-    typename W::Raw wa, wb, wc;
-    XStage<MT> xa, xb, xc;
-    fetch(kb, wa, xa);
-    fetch(kb + BK, wb, xb);
-    fetch(kb + 2 * BK, wc, xc);
-    commit(0, kb, wa, xa);
-    if (kb + BK < ke) commit(1, kb + BK, wb, xb);
-    fetch(kb + 3 * BK, wa, xa);
-    __syncthreads();
+    const uint32_t steps = (ke - kb + BK - 1) / BK;
+    fetch(0, kb);
+    fetch(1, kb + BK);
+    fetch(2, kb + 2 * BK);
+    sync_keeping_loads<2 * LOADS>();
     {
         typename W::Frag wf[2];
         read_b(0, wf);
 #pragma unroll
-        for (int i = 0; i < MT; i++) af[i] = *reinterpret_cast<const bf16x8 *>(lds + (16 * i + lrow) * XROW + 64u * kq + 16u * g);
+        for (int i = 0; i < MT; i++) af[i] = *reinterpret_cast<const bf16x8 *>(lds + a_at + 2048 * i);
+        convert(wf, kb);
+    }
+    // Every wave has its fragments of step 0 (buffer 0 may be refilled) and its
+    // loads of step 1, which step 0 reads, have landed.
+    sync_keeping_loads<LOADS>();
+
+    // Step s multiplies the fragments of s from registers while it reads those
+    // of s + 1 from buffer (s + 1) % 3 (each token fragment right after the
+    // MFMAs that consumed its predecessor) and memory fills buffer s % 3, whose
+    // fragments were read a step ago, with step s + 3. Before the barrier a
+    // wave waits for its loads of step s + 2, issued a step ago.
+    uint32_t cur = 0, kc = kb;
+    for (uint32_t s = 0; s < steps; s++, kc += BK) {
+        const uint32_t nxt = cur == 2u ? 0u : cur + 1u;
+        // The waves of k quarters 0 and 1 (one on each SIMD) issue their loads
+        // before their MFMAs, those of quarters 2 and 3 after their
+        // conversions. The load path, LDS and the vector ALU are each saturated
+        // by one phase of a wave's step; with the halves of the workgroup in
+        // different phases they work at the same time (measured: 32 -> 29 us
+        // on 512 x 4096 x 4096).
+        if (kq < 2u) fetch(cur, kc + 3u * BK);
+        const uint8_t *xn = lds + nxt * BUF + a_at;
+        typename W::Frag wf[2];
+        read_b(nxt, wf);
 #pragma unroll
-        for (int j = 0; j < 2; j++) bf[j] = W::frag(wf[j]);
+        for (int i = 0; i < MT; i++) {
+#pragma unroll
+            for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+            af[i] = *reinterpret_cast<const bf16x8 *>(xn + 2048 * i);
+        }
+        convert(wf, kc + BK);
+        if (kq >= 2u) fetch(cur, kc + 3u * BK);
+        sync_keeping_loads<LOADS>();
+        cur = nxt;
     }
-    // Whole groups of three steps run without a branch between them, so the
-    // loop has a single back edge and the loads in flight are counted exactly;
-    // the one or two steps left over follow the loop.
-    const uint32_t steps = (ke - kb + BK - 1) / BK;
-    uint32_t k0 = kb;
-    for (uint32_t group = 0; group < steps / 3u; group++, k0 += 3 * BK) {
-        step(k0, wb, xb, wc, xc);
-        step(k0 + BK, wc, xc, wa, xa);
-        step(k0 + 2 * BK, wa, xa, wb, xb);
-    }
-    if (steps % 3u >= 1u) step(k0, wb, xb, wc, xc);
-    if (steps % 3u == 2u) step(k0 + BK, wc, xc, wa, xa);
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still land in LDS below
+    __syncthreads();
 
     // Add the four k quarters through LDS, in a fixed order whatever the
     // timing: quarters 2 and 3 hand everything to 0 and 1, then 0 and 1 swap
