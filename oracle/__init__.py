@@ -13,7 +13,7 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
-F32, F16, Q8_0, Q4_K, BF16 = 0, 1, 8, 12, 30
+F32, F16, Q8_0, Q4_K, Q5_K, Q6_K, BF16 = 0, 1, 8, 12, 13, 14, 30
 
 
 def build() -> None:
@@ -156,7 +156,7 @@ class Matrix:
 
     def rows(self) -> np.ndarray:
         """All weights decoded, n x k."""
-        if self.t in (Q8_0, Q4_K):
+        if self.t in (Q8_0, Q4_K, Q5_K, Q6_K):
             return dequantize(self.t, self.bytes, self.n * self.k).reshape(self.n, self.k)
         return np.stack([self.row(j) for j in range(self.n)])
 

@@ -21,6 +21,8 @@ int zref_layout(int type, uint32_t *block_elems, uint32_t *block_bytes) {
     case ZREF_F16: case ZREF_BF16: e = 1; b = 2; break;
     case ZREF_Q8_0: e = 32; b = 34; break;
     case ZREF_Q4_K: e = 256; b = 144; break;
+    case ZREF_Q5_K: e = 256; b = 176; break;
+    case ZREF_Q6_K: e = 256; b = 210; break;
     default: return 0;
     }
     if (block_elems) *block_elems = e;
@@ -134,6 +136,58 @@ static void q4_k_block(const uint8_t *b, float *y) {
     }
 }
 
+/* src/ref/tensor.zig:118-138: Q4_K with a fifth bit per weight from qh
+ * (bit 2j of qh[l] for the low sub-block of chunk j, bit 2j + 1 for the high). */
+static void q5_k_block(const uint8_t *b, float *y) {
+    float d = zref_half(rd16(b));
+    float min = zref_half(rd16(b + 2));
+    const uint8_t *scales = b + 4;
+    const uint8_t *qh = b + 16;
+    for (unsigned j = 0; j < 4; j++) {
+        const uint8_t *ql = b + 48 + 32 * j;
+        uint8_t bit_lo = (uint8_t)(1u << (2 * j)), bit_hi = (uint8_t)(2u << (2 * j));
+        uint8_t sc1, mn1, sc2, mn2;
+        zref_scale_min_k4(2 * j, scales, &sc1, &mn1);
+        zref_scale_min_k4(2 * j + 1, scales, &sc2, &mn2);
+        float d1 = d * (float)sc1;
+        float m1 = min * (float)mn1;
+        float d2 = d * (float)sc2;
+        float m2 = min * (float)mn2;
+        for (int l = 0; l < 32; l++) {
+            float p = d1 * (float)((ql[l] & 0xF) + ((qh[l] & bit_lo) ? 16 : 0));
+            y[64 * j + l] = p - m1;
+        }
+        for (int l = 0; l < 32; l++) {
+            float p = d2 * (float)((ql[l] >> 4) + ((qh[l] & bit_hi) ? 16 : 0));
+            y[64 * j + 32 + l] = p - m2;
+        }
+    }
+}
+
+/* src/ref/tensor.zig:140-160: d * sc * q evaluated left to right, two
+ * roundings; q = low nibble | two high bits << 4, minus 32. */
+static void q6_k_block(const uint8_t *b, float *y) {
+    float d = zref_half(rd16(b + 208));
+    for (unsigned n = 0; n < 2; n++) {
+        const uint8_t *ql = b + 64 * n;
+        const uint8_t *qh = b + 128 + 32 * n;
+        const int8_t *sc = (const int8_t *)(b + 192 + 8 * n);
+        float *out = y + 128 * n;
+        for (int l = 0; l < 32; l++) {
+            int is = l / 16;
+            int q1 = (int)((ql[l] & 0xF) | (((qh[l] >> 0) & 3) << 4)) - 32;
+            int q2 = (int)((ql[l + 32] & 0xF) | (((qh[l] >> 2) & 3) << 4)) - 32;
+            int q3 = (int)((ql[l] >> 4) | (((qh[l] >> 4) & 3) << 4)) - 32;
+            int q4 = (int)((ql[l + 32] >> 4) | (((qh[l] >> 6) & 3) << 4)) - 32;
+            float t1 = d * (float)sc[is], t2 = d * (float)sc[is + 2], t3 = d * (float)sc[is + 4], t4 = d * (float)sc[is + 6];
+            out[l] = t1 * (float)q1;
+            out[l + 32] = t2 * (float)q2;
+            out[l + 64] = t3 * (float)q3;
+            out[l + 96] = t4 * (float)q4;
+        }
+    }
+}
+
 /* src/ref/tensor.zig:21-43. */
 int zref_dequantize(int type, const uint8_t *bytes, float *out, size_t n) {
     switch (type) {
@@ -142,6 +196,12 @@ int zref_dequantize(int type, const uint8_t *bytes, float *out, size_t n) {
         return 0;
     case ZREF_Q4_K:
         for (size_t i = 0; i < n / 256; i++) q4_k_block(bytes + i * 144, out + i * 256);
+        return 0;
+    case ZREF_Q5_K:
+        for (size_t i = 0; i < n / 256; i++) q5_k_block(bytes + i * 176, out + i * 256);
+        return 0;
+    case ZREF_Q6_K:
+        for (size_t i = 0; i < n / 256; i++) q6_k_block(bytes + i * 210, out + i * 256);
         return 0;
     case ZREF_F32:
         for (size_t i = 0; i < n; i++) out[i] = bits_f32(rd32(bytes + 4 * i));
@@ -331,7 +391,7 @@ zref_matrix *zref_matrix_init(int type, const uint8_t *bytes, size_t n, size_t k
     if (!zref_layout(type, &be, &bb) || k % be != 0) return NULL;
     zref_matrix *m = (zref_matrix *)calloc(1, sizeof *m);
     m->n = n; m->k = k; m->type = type;
-    if (type == ZREF_Q8_0 || type == ZREF_Q4_K) {
+    if (type == ZREF_Q8_0 || type == ZREF_Q4_K || type == ZREF_Q5_K || type == ZREF_Q6_K) {
         m->quant = bytes;
         return m;
     }
@@ -491,6 +551,7 @@ uint64_t zref_row_bytes(int type, uint64_t k) {
     if (type == ZREF_Q8_0) return (k + k / 16 + 15) & ~(uint64_t)15;
     uint32_t be, bb;
     if (!zref_layout(type, &be, &bb)) return 0;
+    if (type == ZREF_Q6_K) bb = 224;  /* blockStride: padded to 16 bytes by repad */
     return k / be * bb;
 }
 

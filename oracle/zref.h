@@ -18,6 +18,14 @@
  *     Parity with ggml's dequantize_row_q4_K (llama.cpp e09a78a2, what the
  *     reference itself is pinned to by tools/check_dequant.py) is "parity
  *     unpinned" here: that library is not available offline.
+ *   - zref_dequantize (q5_k, q6_k): the reference holds no known answers for
+ *     them (its kernel check compares against its own decoder), so they are
+ *     pinned by what the format fixes: packing known quants and scales into
+ *     blocks by an independent numpy bit map and decoding them back, the
+ *     special cases that make every product exact, and single-bit mutations
+ *     that must move exactly one weight. Agreement with ggml's
+ *     dequantize_row_q5_K / q6_K is "parity unpinned" (library not available
+ *     offline).
  *   - zref_matmul: the reference's tests (src/ref/matmul.zig:296-380): naive
  *     product for every row remainder and pool size, and bit-exact results on
  *     dyadic data; float64 numpy products.
@@ -43,6 +51,8 @@ enum {
     ZREF_F16 = 1,
     ZREF_Q8_0 = 8,
     ZREF_Q4_K = 12,
+    ZREF_Q5_K = 13,
+    ZREF_Q6_K = 14,
     ZREF_BF16 = 30,
 };
 

@@ -15,7 +15,8 @@ from zllm_amd.kernels import Kernel, TensorType, params as P
 
 pytestmark = pytest.mark.gpu
 
-ORACLE_TYPE = {TensorType.q8_0: oracle.Q8_0, TensorType.q4_k: oracle.Q4_K, TensorType.bf16: oracle.BF16}
+ORACLE_TYPE = {TensorType.q8_0: oracle.Q8_0, TensorType.q4_k: oracle.Q4_K, TensorType.q5_k: oracle.Q5_K, TensorType.q6_k: oracle.Q6_K,
+               TensorType.bf16: oracle.BF16}
 
 
 def quant_rows(c, t: TensorType, rows: int, k: int):
@@ -136,6 +137,10 @@ def quant_matvec(c, t: TensorType, k: int, pair: bool, variants=None):
     (TensorType.q4_k, 4096, False),   # "matvec q4_k norm+= (2 tiles)"
     (TensorType.q8_0, 4160, True),    # "matvec q8_0 norm+silu (tile tail, bitwise splits)"
     (TensorType.q4_k, 1024, True),    # the SiLU pair on Q4_K (the reference runs it on q3_k)
+    (TensorType.q5_k, 1024, False),   # "matvec q5_k norm+="
+    (TensorType.q6_k, 1024, False),   # "matvec q6_k norm+="
+    (TensorType.q6_k, 2304, True),    # the SiLU pair on Q6_K, nine blocks a row
+    (TensorType.q5_k, 4096, True),
 ])
 def test_quant_matvec(ctx, t, k, pair):
     worst, split_exact = quant_matvec(ctx, t, k, pair)
@@ -187,7 +192,7 @@ def test_quant_matvec_eight_rows(ctx):
 
 # ---- block decoders bit for bit, through the embedding gathers: check.zig:873-905 -----
 
-@pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q4_k])
+@pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q4_k, TensorType.q5_k, TensorType.q6_k])
 def test_embed_quant_bit_exact(ctx, t):
     c = ctx
     vocab, dim, split = 50, 512, 30

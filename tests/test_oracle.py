@@ -192,6 +192,97 @@ def test_q4_k_is_the_correctly_rounded_exact_value():
     assert np.array_equal(bits(got), bits(exact.astype(np.float32)))
 
 
+# ---- Q5_K and Q6_K: no known answers in the reference; pinned by the format ------------
+
+def pack_q5_k(d, dmin, sc, mn, q):
+    """One Q5_K block from its parts, written from the format's description
+    (not from the decoder): element 64 j + 32 h + l keeps its low four bits in
+    the low (h = 0) or high (h = 1) nibble of qs[32 j + l] and its fifth bit in
+    bit 2 j + h of qh[l]."""
+    b = np.zeros(176, dtype=np.uint8)
+    b[0:4] = np.array([d, dmin], dtype=np.float16).view(np.uint8)
+    b[4:16] = synth.pack_scales_k4(np.array([sc]), np.array([mn]))[0]
+    q = np.asarray(q, dtype=np.uint8).reshape(4, 2, 32)
+    for j in range(4):
+        for h in range(2):
+            b[48 + 32 * j : 80 + 32 * j] |= (q[j, h] & 15) << (4 * h)
+            b[16:48] |= (q[j, h] >> 4) << (2 * j + h)
+    return b
+
+
+def pack_q6_k(d, sc, q):
+    """One Q6_K block: element 128 n + 32 r + l holds v = q + 32 (6 bits): its
+    low four bits in the low (r < 2) or high nibble of ql[64 n + 32 (r % 2) + l],
+    its top two bits at bits 2 r of qh[32 n + l]; scale 8 n + 2 r + l / 16."""
+    b = np.zeros(210, dtype=np.uint8)
+    v = (np.asarray(q, dtype=np.int32) + 32).astype(np.uint8).reshape(2, 4, 32)
+    for n in range(2):
+        for r in range(4):
+            b[64 * n + 32 * (r % 2) : 64 * n + 32 * (r % 2) + 32] |= (v[n, r] & 15) << (4 * (r // 2))
+            b[128 + 32 * n : 160 + 32 * n] |= (v[n, r] >> 4) << (2 * r)
+    b[192:208] = np.asarray(sc, dtype=np.int8).view(np.uint8)
+    b[208:210] = np.array([d], dtype=np.float16).view(np.uint8)
+    return b
+
+
+def test_q5_k_is_the_correctly_rounded_exact_value_of_packed_parts():
+    """d (11 bits) x scale (6) x quant (5) = 22 bits and dmin x min = 17 bits
+    are exact in f32, so y must be d*sc*q - dmin*m rounded once, for blocks
+    packed by an independent bit map."""
+    g = synth.rng(21)
+    for _ in range(40):
+        d, dmin = np.float16(g.uniform(-4, 4)), np.float16(g.uniform(-4, 4))
+        sc, mn = g.integers(0, 64, 8), g.integers(0, 64, 8)
+        q = g.integers(0, 32, 256)
+        y = oracle.dequantize(oracle.Q5_K, pack_q5_k(d, dmin, sc, mn, q), 256)
+        exact = float(d) * np.repeat(sc, 32).astype(np.float64) * q - float(dmin) * np.repeat(mn, 32).astype(np.float64)
+        assert np.array_equal(bits(y), bits(exact.astype(np.float32)))
+
+
+def test_q6_k_is_the_correctly_rounded_exact_value_of_packed_parts():
+    """d (11 bits) x scale (8) is exact in f32 and its product with the quant
+    (6 bits) is rounded once, so y must be d*sc*q rounded once."""
+    g = synth.rng(22)
+    for _ in range(40):
+        d = np.float16(g.uniform(-2, 2))
+        sc = g.integers(-128, 128, 16)
+        q = g.integers(-32, 32, 256)
+        y = oracle.dequantize(oracle.Q6_K, pack_q6_k(d, sc, q), 256)
+        exact = float(d) * np.repeat(sc, 16).astype(np.float64) * q
+        assert np.array_equal(bits(y), bits(exact.astype(np.float32)))
+
+
+@pytest.mark.parametrize("t,size,packer", [(oracle.Q5_K, 176, "q5_k"), (oracle.Q6_K, 210, "q6_k")])
+def test_k_quant_single_bit_mutations_move_exactly_their_weights(t, size, packer):
+    """Flipping one quant bit changes exactly one weight; flipping a scale bit
+    changes exactly one sub-block (32 weights for Q5_K, 16 for Q6_K)."""
+    g = synth.rng(23)
+    raw = synth.random_blocks(g, packer, 1, 256, scale=1.0)
+    base = oracle.dequantize(t, raw, 256)
+    quant_bytes = range(16, 176) if t == oracle.Q5_K else range(0, 192)
+    for byte in list(quant_bytes)[::7]:
+        for bit in range(8):
+            m = raw.copy()
+            m[byte] ^= 1 << bit
+            changed = np.flatnonzero(bits(oracle.dequantize(t, m, 256)) != bits(base))
+            assert changed.size <= 1  # a zero scale hides the change
+    if t == oracle.Q6_K:
+        for byte in range(192, 208):
+            m = raw.copy()
+            m[byte] ^= 1
+            changed = np.flatnonzero(bits(oracle.dequantize(t, m, 256)) != bits(base))
+            n, i = (byte - 192) // 8, (byte - 192) % 8
+            want = 128 * n + 32 * (i // 2) + 16 * (i % 2)
+            assert changed.size <= 16 and np.all((changed >= want) & (changed < want + 16))
+    else:
+        sc = np.array([oracle.scale_min_k4(j, raw[4:16]) for j in range(8)])
+        for j in range(8):
+            m = raw.copy()
+            m[4:16] = synth.pack_scales_k4(np.array([sc[:, 0] ^ (np.arange(8) == j)]), np.array([sc[:, 1]]))[0]
+            changed = np.flatnonzero(bits(oracle.dequantize(t, m, 256)) != bits(base))
+            assert changed.size <= 32 and np.all(changed // 32 == j)
+
+
 # ---- ops: RMSNorm's bitwise known answer (src/ref/ops.zig:139-168), SiLU ---------------
 
 def test_rms_norm_known_answer_bitwise():

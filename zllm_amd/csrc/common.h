@@ -98,6 +98,8 @@ typedef zhip_result (*LaunchFn)(const Dispatch &);
 
 zhip_result launch_matvec_q8_0(const Dispatch &);
 zhip_result launch_matvec_q4_k(const Dispatch &);
+zhip_result launch_matvec_q5_k(const Dispatch &);
+zhip_result launch_matvec_q6_k(const Dispatch &);
 zhip_result launch_matvec_bf16(const Dispatch &);
 zhip_result launch_matmul_reduce(const Dispatch &);
 zhip_result launch_silu_mul(const Dispatch &);
@@ -105,6 +107,8 @@ zhip_result launch_repack_q8_0(const Dispatch &);
 zhip_result launch_repad(const Dispatch &);
 zhip_result launch_embed_q8_0(const Dispatch &);
 zhip_result launch_embed_q4_k(const Dispatch &);
+zhip_result launch_embed_q5_k(const Dispatch &);
+zhip_result launch_embed_q6_k(const Dispatch &);
 zhip_result launch_embed_bf16(const Dispatch &);
 
 // Host-side helpers shared by the launchers.

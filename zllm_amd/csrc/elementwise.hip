@@ -147,7 +147,7 @@ zhip_result launch_repad(const Dispatch &d) {
     return check_launch(d, "repad");
 }
 
-// ---- embed_q8_0 / embed_q4_k / embed_bf16: src/kernels/embed_quant.wgsl, -------
+// ---- embed_q8_0 / embed_q4_k / embed_q5_k / embed_q6_k / embed_bf16: src/kernels/embed_quant.wgsl, -------
 // src/kernels/embed_half.wgsl. out[t] = table[tokens[t] - row0] decoded to f32
 // for tokens whose row lies in [row0, row0 + chunk_rows); one workgroup per
 // token. The decoders are the multiplies' own, so these kernels also show the
@@ -165,10 +165,10 @@ __global__ __launch_bounds__(256) void embed_kernel(EmbedParams p, const uint32_
         float w[D::E];
         D::decode(row, p.dim, task, w);
 #pragma unroll
-        for (int h = 0; h < 2; h++) {
+        for (int h = 0; h < D::RUNS; h++) {
             const uint32_t o = D::xoff(task, h);
 #pragma unroll
-            for (int i = 0; i < D::E / 2; i++) dst[o + i] = w[h * (D::E / 2) + i];
+            for (int i = 0; i < D::E / D::RUNS; i++) dst[o + i] = w[h * (D::E / D::RUNS) + i];
         }
     }
 }
@@ -215,6 +215,8 @@ static zhip_result launch_embed(const Dispatch &d, const char *name) {
 
 zhip_result launch_embed_q8_0(const Dispatch &d) { return launch_embed<DecQ8_0>(d, "embed_q8_0"); }
 zhip_result launch_embed_q4_k(const Dispatch &d) { return launch_embed<DecQ4_K>(d, "embed_q4_k"); }
+zhip_result launch_embed_q5_k(const Dispatch &d) { return launch_embed<DecQ5_K>(d, "embed_q5_k"); }
+zhip_result launch_embed_q6_k(const Dispatch &d) { return launch_embed<DecQ6_K>(d, "embed_q6_k"); }
 zhip_result launch_embed_bf16(const Dispatch &d) { return launch_embed<DecBF16>(d, "embed_bf16"); }
 
 // ---- fill ----------------------------------------------------------------------

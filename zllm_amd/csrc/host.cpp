@@ -86,6 +86,8 @@ struct KernelInfo {
 static const KernelInfo kImplemented[] = {
     {"matvec_q8_0", 5, 0b01000, VariantKind::matvec, launch_matvec_q8_0, nullptr, nullptr, 1},
     {"matvec_q4_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q4_k, nullptr, nullptr, 1},
+    {"matvec_q5_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q5_k, nullptr, nullptr, 1},
+    {"matvec_q6_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q6_k, nullptr, nullptr, 1},
     {"matvec_bf16", 5, 0b01000, VariantKind::none, launch_matvec_bf16, nullptr, nullptr, 1},
     {"matmul_bf16", 4, 0b1000, VariantKind::prefill, launch_matmul_bf16_f32, launch_matmul_bf16_mfma, launch_matmul_bf16_mfma_xbf16, 1},
     {"matmul_q8_0_float", 4, 0b1000, VariantKind::prefill, launch_matmul_q8_0_float_f32, launch_matmul_q8_0_float_mfma, launch_matmul_q8_0_float_mfma_xbf16, 1},
@@ -95,6 +97,8 @@ static const KernelInfo kImplemented[] = {
     {"repad", 3, 0b100, VariantKind::none, launch_repad, nullptr, nullptr, 1},
     {"embed_q8_0", 4, 0b1000, VariantKind::none, launch_embed_q8_0, nullptr, nullptr, 1},
     {"embed_q4_k", 4, 0b1000, VariantKind::none, launch_embed_q4_k, nullptr, nullptr, 1},
+    {"embed_q5_k", 4, 0b1000, VariantKind::none, launch_embed_q5_k, nullptr, nullptr, 1},
+    {"embed_q6_k", 4, 0b1000, VariantKind::none, launch_embed_q6_k, nullptr, nullptr, 1},
     {"embed_bf16", 4, 0b1000, VariantKind::none, launch_embed_bf16, nullptr, nullptr, 1},
 };
 

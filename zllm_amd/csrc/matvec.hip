@@ -1,5 +1,5 @@
 // Decode multiplies: out[t][col0 + j] (+)= sum_i X(t, i) * w[j][i] for Q8_0,
-// Q4_K and BF16 weights, with the RMSNorm / activation prologues and the
+// Q4_K, Q5_K, Q6_K and BF16 weights, with the RMSNorm / activation prologues and the
 // accumulate / SiLU-pair epilogues of the reference's matvec kernels
 // (src/kernels/matvec_quant.wgsl.hbs:20-31, src/kernels/matvec_half.wgsl:14-19).
 //
@@ -63,18 +63,17 @@ __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
                 float w0[D::E], w1[D::E];
                 D::decode(row0, a.k, task, w0);
                 D::decode(row1, a.k, task, w1);
-                const uint32_t xo0 = D::xoff(task, 0), xo1 = D::xoff(task, 1);
 #pragma unroll
                 for (int t = 0; t < MT; t++) {
                     const float *xt = xs + (size_t)t * a.k;
                     float s0 = 0.f, s1 = 0.f;
 #pragma unroll
-                    for (int h = 0; h < 2; h++) {
-                        const float4 *xv = reinterpret_cast<const float4 *>(xt + (h ? xo1 : xo0));
+                    for (int h = 0; h < D::RUNS; h++) {
+                        const float4 *xv = reinterpret_cast<const float4 *>(xt + D::xoff(task, h));
 #pragma unroll
-                        for (int e = 0; e < D::E / 8; e++) {
+                        for (int e = 0; e < D::E / (4 * D::RUNS); e++) {
                             const float4 v = xv[e];
-                            const int b = h * (D::E / 2) + 4 * e;
+                            const int b = h * (D::E / D::RUNS) + 4 * e;
                             s0 = fmaf(w0[b + 0], v.x, s0); s1 = fmaf(w1[b + 0], v.x, s1);
                             s0 = fmaf(w0[b + 1], v.y, s0); s1 = fmaf(w1[b + 1], v.y, s1);
                             s0 = fmaf(w0[b + 2], v.z, s0); s1 = fmaf(w1[b + 2], v.z, s1);
@@ -187,7 +186,7 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     a.out = reinterpret_cast<float *>(d.bind[3].ptr);
     a.norm_w = norm ? reinterpret_cast<const float *>(d.bind[4].ptr) : nullptr;
 
-    if (D::BLOCK == 256u) return launch_matvec_q4k(d, a);
+    if (D::CHUNK_KERNEL) return launch_matvec_q4k(d, a);
 
     // Tokens per pass over the weights: as many as fit workgroup memory.
     const uint64_t row_lds = (uint64_t)p.k * 4u;
@@ -205,6 +204,8 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
 
 zhip_result launch_matvec_q8_0(const Dispatch &d) { return launch_matvec<DecQ8_0>(d, true); }
 zhip_result launch_matvec_q4_k(const Dispatch &d) { return launch_matvec<DecQ4_K>(d, true); }
+zhip_result launch_matvec_q5_k(const Dispatch &d) { return launch_matvec<DecQ5_K>(d, true); }
+zhip_result launch_matvec_q6_k(const Dispatch &d) { return launch_matvec<DecQ6_K>(d, true); }
 zhip_result launch_matvec_bf16(const Dispatch &d) { return launch_matvec<DecBF16>(d, false); }
 
 }  // namespace zhip

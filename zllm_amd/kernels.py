@@ -38,11 +38,14 @@ class TensorType(enum.IntEnum):
     f16 = 1
     q8_0 = 8
     q4_k = 12
+    q5_k = 13
+    q6_k = 14
     bf16 = 30
 
 
 # (block_elems, block_bytes): src/gguf/gguf.zig:69-109.
-LAYOUT = {TensorType.f32: (1, 4), TensorType.f16: (1, 2), TensorType.bf16: (1, 2), TensorType.q8_0: (32, 34), TensorType.q4_k: (256, 144)}
+LAYOUT = {TensorType.f32: (1, 4), TensorType.f16: (1, 2), TensorType.bf16: (1, 2), TensorType.q8_0: (32, 34), TensorType.q4_k: (256, 144),
+          TensorType.q5_k: (256, 176), TensorType.q6_k: (256, 210)}
 
 
 @dataclass(frozen=True)
@@ -62,6 +65,8 @@ class Contract:
 CONTRACTS = {
     Kernel.matvec_q8_0: Contract(5, 0b01000),
     Kernel.matvec_q4_k: Contract(5, 0b01000),
+    Kernel.matvec_q5_k: Contract(5, 0b01000),
+    Kernel.matvec_q6_k: Contract(5, 0b01000),
     Kernel.matvec_bf16: Contract(5, 0b01000),
     Kernel.matmul_bf16: Contract(4, 0b1000),
     Kernel.matmul_q8_0_float: Contract(4, 0b1000),
@@ -71,6 +76,8 @@ CONTRACTS = {
     Kernel.repad: Contract(3, 0b100),
     Kernel.embed_q8_0: Contract(4, 0b1000),
     Kernel.embed_q4_k: Contract(4, 0b1000),
+    Kernel.embed_q5_k: Contract(4, 0b1000),
+    Kernel.embed_q6_k: Contract(4, 0b1000),
     Kernel.embed_bf16: Contract(4, 0b1000),
 }
 
@@ -92,8 +99,9 @@ def weight_kernel(op: str, t: TensorType) -> Kernel:
 
 
 def block_stride(t: TensorType) -> int:
-    """src/kernels/kernels.zig:144-151 (types of this path keep their block size)."""
-    return LAYOUT[t][1]
+    """src/kernels/kernels.zig:144-151: the GGUF block size, padded to a multiple
+    of 16 where it is not one (Q6_K: 210 -> 224, laid out by repad)."""
+    return 224 if t == TensorType.q6_k else LAYOUT[t][1]
 
 
 def row_bytes(t: TensorType, k: int) -> int:
