@@ -13,7 +13,7 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
-F32, F16, Q8_0, Q4_K, Q5_K, Q6_K, BF16 = 0, 1, 8, 12, 13, 14, 30
+F32, F16, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, BF16 = 0, 1, 8, 11, 12, 13, 14, 30
 
 
 def build() -> None:
@@ -74,6 +74,8 @@ _lib.zref_default_threads.restype = C.c_uint
 _lib.zref_row_bytes.restype = C.c_uint64
 _lib.zref_row_bytes.argtypes = [C.c_int, C.c_uint64]
 _lib.zref_repack_q8_0.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t]
+_lib.zref_repack_q3_k.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+_lib.zref_repack_q3_k.restype = None
 _lib.zref_matmul_slices.argtypes = [C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
 _lib.zref_matmul_f64.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint]
 
@@ -156,7 +158,7 @@ class Matrix:
 
     def rows(self) -> np.ndarray:
         """All weights decoded, n x k."""
-        if self.t in (Q8_0, Q4_K, Q5_K, Q6_K):
+        if self.t in (Q8_0, Q3_K, Q4_K, Q5_K, Q6_K):
             return dequantize(self.t, self.bytes, self.n * self.k).reshape(self.n, self.k)
         return np.stack([self.row(j) for j in range(self.n)])
 
@@ -196,6 +198,15 @@ def repack_q8_0(raw: np.ndarray, rows: int, k: int) -> np.ndarray:
     assert raw.size == rows * k // 32 * 34
     dst = np.empty(rows * row_bytes(Q8_0, k), dtype=np.uint8)
     _lib.zref_repack_q8_0(_ptr(raw), _ptr(dst), rows, k)
+    return dst
+
+
+def repack_q3_k(raw: np.ndarray, blocks: int) -> np.ndarray:
+    """src/kernels/repack_q3_k.wgsl: 110-byte blocks into 128-byte repacked ones."""
+    raw = np.ascontiguousarray(raw).view(np.uint8)
+    assert raw.size == blocks * 110
+    dst = np.empty(blocks * 128, dtype=np.uint8)
+    _lib.zref_repack_q3_k(_ptr(raw), _ptr(dst), blocks)
     return dst
 
 

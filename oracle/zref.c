@@ -20,6 +20,7 @@ int zref_layout(int type, uint32_t *block_elems, uint32_t *block_bytes) {
     case ZREF_F32: e = 1; b = 4; break;
     case ZREF_F16: case ZREF_BF16: e = 1; b = 2; break;
     case ZREF_Q8_0: e = 32; b = 34; break;
+    case ZREF_Q3_K: e = 256; b = 110; break;
     case ZREF_Q4_K: e = 256; b = 144; break;
     case ZREF_Q5_K: e = 256; b = 176; break;
     case ZREF_Q6_K: e = 256; b = 210; break;
@@ -136,6 +137,44 @@ static void q4_k_block(const uint8_t *b, float *y) {
     }
 }
 
+/* src/ref/tensor.zig:55-92: sixteen 6-bit scales (low four bits in bytes
+ * 0..7 by nibble, top two in bytes 8..11), dl = d * (scale - 32), weight l of
+ * half n and shift j = dl * (two bits 2j of qs[32n + l], minus 4 unless bit
+ * 4n + j of hmask[l] is set). */
+static void q3_k_block(const uint8_t *b, float *y) {
+    const uint8_t *hm = b;
+    float d_all = zref_half(rd16(b + 108));
+    uint32_t aux[4];
+    for (int i = 0; i < 3; i++) aux[i] = rd32(b + 96 + 4 * i);
+    const uint32_t kmask1 = 0x03030303u, kmask2 = 0x0f0f0f0fu;
+    uint32_t tmp = aux[2];
+    aux[2] = ((aux[0] >> 4) & kmask2) | (((tmp >> 4) & kmask1) << 4);
+    aux[3] = ((aux[1] >> 4) & kmask2) | (((tmp >> 6) & kmask1) << 4);
+    aux[0] = (aux[0] & kmask2) | (((tmp >> 0) & kmask1) << 4);
+    aux[1] = (aux[1] & kmask2) | (((tmp >> 2) & kmask1) << 4);
+    int8_t scales[16];
+    for (int i = 0; i < 16; i++) scales[i] = (int8_t)((aux[i / 4] >> (8 * (i % 4))) & 0xff);
+    size_t out = 0;
+    unsigned is = 0;
+    uint8_t m = 1;
+    for (unsigned n = 0; n < 2; n++) {
+        const uint8_t *q = b + 32 + 32 * n;
+        unsigned shift = 0;
+        for (unsigned j = 0; j < 4; j++) {
+            for (unsigned h = 0; h < 2; h++) {
+                float dl = d_all * (float)((int)scales[is++] - 32);
+                for (unsigned l = 0; l < 16; l++) {
+                    int lo = (q[l + 16 * h] >> shift) & 3;
+                    int v = lo - ((hm[l + 16 * h] & m) ? 0 : 4);
+                    y[out++] = dl * (float)v;
+                }
+            }
+            shift += 2;
+            m = (uint8_t)(m << 1);
+        }
+    }
+}
+
 /* src/ref/tensor.zig:118-138: Q4_K with a fifth bit per weight from qh
  * (bit 2j of qh[l] for the low sub-block of chunk j, bit 2j + 1 for the high). */
 static void q5_k_block(const uint8_t *b, float *y) {
@@ -193,6 +232,9 @@ int zref_dequantize(int type, const uint8_t *bytes, float *out, size_t n) {
     switch (type) {
     case ZREF_Q8_0:
         for (size_t i = 0; i < n / 32; i++) q8_0_block(bytes + i * 34, out + i * 32);
+        return 0;
+    case ZREF_Q3_K:
+        for (size_t i = 0; i < n / 256; i++) q3_k_block(bytes + i * 110, out + i * 256);
         return 0;
     case ZREF_Q4_K:
         for (size_t i = 0; i < n / 256; i++) q4_k_block(bytes + i * 144, out + i * 256);
@@ -391,7 +433,7 @@ zref_matrix *zref_matrix_init(int type, const uint8_t *bytes, size_t n, size_t k
     if (!zref_layout(type, &be, &bb) || k % be != 0) return NULL;
     zref_matrix *m = (zref_matrix *)calloc(1, sizeof *m);
     m->n = n; m->k = k; m->type = type;
-    if (type == ZREF_Q8_0 || type == ZREF_Q4_K || type == ZREF_Q5_K || type == ZREF_Q6_K) {
+    if (type == ZREF_Q8_0 || type == ZREF_Q3_K || type == ZREF_Q4_K || type == ZREF_Q5_K || type == ZREF_Q6_K) {
         m->quant = bytes;
         return m;
     }
@@ -552,7 +594,38 @@ uint64_t zref_row_bytes(int type, uint64_t k) {
     uint32_t be, bb;
     if (!zref_layout(type, &be, &bb)) return 0;
     if (type == ZREF_Q6_K) bb = 224;  /* blockStride: padded to 16 bytes by repad */
+    if (type == ZREF_Q3_K) bb = 128;  /* repacked into eight 16-byte units */
     return k / be * bb;
+}
+
+/* src/kernels/repack_q3_k.wgsl:30-75. */
+static uint32_t q3_scale(const uint8_t *sb, uint32_t i) {
+    uint32_t k = i % 4, g = i / 4;
+    uint32_t low = (sb[4 * (g % 2) + k] >> (4 * (g / 2))) & 0xf;
+    uint32_t high = (sb[8 + k] >> (2 * g)) & 3;
+    return low | (high << 4);
+}
+
+void zref_repack_q3_k(const uint8_t *src, uint8_t *dst, size_t blocks) {
+    for (size_t unit = 0; unit < blocks * 8; unit++) {
+        const uint8_t *b = src + (unit / 8) * 110;
+        uint32_t s = (uint32_t)(unit % 8), half = s / 4, j = s % 4;
+        uint32_t l0 = 0, l1 = 0, hw = 0;
+        for (uint32_t l = 0; l < 32; l++) {
+            uint32_t q = (b[32 + 32 * half + l] >> (2 * j)) & 3;
+            uint32_t h = (b[l] >> (4 * half + j)) & 1;
+            uint32_t e = l / 4, byte = l % 4;
+            if (e < 4) l0 |= q << (8 * byte + 2 * e);
+            else l1 |= q << (8 * byte + 2 * (e - 4));
+            hw |= h << (8 * byte + e);
+        }
+        uint32_t sc0 = (q3_scale(b + 96, 8 * half + 2 * j) + 224) & 0xff;
+        uint32_t sc1 = (q3_scale(b + 96, 8 * half + 2 * j + 1) + 224) & 0xff;
+        uint32_t d = (uint32_t)b[108] | ((uint32_t)b[109] << 8);
+        uint32_t words[4] = { l0, l1, hw, sc0 | (sc1 << 8) | (d << 16) };
+        for (int w = 0; w < 4; w++)
+            for (int i = 0; i < 4; i++) dst[unit * 16 + 4 * w + i] = (uint8_t)(words[w] >> (8 * i));
+    }
 }
 
 /* src/kernels/repack_q8_0.wgsl:26-51. */

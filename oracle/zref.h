@@ -18,14 +18,15 @@
  *     Parity with ggml's dequantize_row_q4_K (llama.cpp e09a78a2, what the
  *     reference itself is pinned to by tools/check_dequant.py) is "parity
  *     unpinned" here: that library is not available offline.
- *   - zref_dequantize (q5_k, q6_k): the reference holds no known answers for
+ *   - zref_dequantize (q3_k, q5_k, q6_k): the reference holds no known answers for
  *     them (its kernel check compares against its own decoder), so they are
  *     pinned by what the format fixes: packing known quants and scales into
  *     blocks by an independent numpy bit map and decoding them back, the
  *     special cases that make every product exact, and single-bit mutations
  *     that must move exactly one weight. Agreement with ggml's
- *     dequantize_row_q5_K / q6_K is "parity unpinned" (library not available
- *     offline).
+ *     dequantize_row_q3_K / q5_K / q6_K is "parity unpinned" (library not
+ *     available offline). zref_repack_q3_k is pinned by decoding its units with
+ *     an independent numpy reader and comparing with zref_dequantize.
  *   - zref_matmul: the reference's tests (src/ref/matmul.zig:296-380): naive
  *     product for every row remainder and pool size, and bit-exact results on
  *     dyadic data; float64 numpy products.
@@ -50,6 +51,7 @@ enum {
     ZREF_F32 = 0,
     ZREF_F16 = 1,
     ZREF_Q8_0 = 8,
+    ZREF_Q3_K = 11,
     ZREF_Q4_K = 12,
     ZREF_Q5_K = 13,
     ZREF_Q6_K = 14,
@@ -119,6 +121,9 @@ uint64_t zref_row_bytes(int type, uint64_t k);
 /* 34-byte file blocks -> split rows: k int8 values, k/32 f16 scales, zero pad
  * to 16 bytes (src/kernels/repack_q8_0.wgsl:26-51). */
 void zref_repack_q8_0(const uint8_t *src, uint8_t *dst, size_t rows, size_t k);
+/* src/kernels/repack_q3_k.wgsl: `blocks` 110-byte Q3_K blocks into eight
+ * self-contained 16-byte units each (128 bytes a block). */
+void zref_repack_q3_k(const uint8_t *src, uint8_t *dst, size_t blocks);
 
 /* Split of a prefill multiply over k (src/kernels/kernels.zig:285-295). */
 void zref_matmul_slices(uint32_t n, uint32_t k, uint32_t *count, uint32_t *k_slice);

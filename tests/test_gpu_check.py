@@ -15,7 +15,7 @@ from zllm_amd.kernels import Kernel, TensorType, params as P
 
 pytestmark = pytest.mark.gpu
 
-ORACLE_TYPE = {TensorType.q8_0: oracle.Q8_0, TensorType.q4_k: oracle.Q4_K, TensorType.q5_k: oracle.Q5_K, TensorType.q6_k: oracle.Q6_K,
+ORACLE_TYPE = {TensorType.q8_0: oracle.Q8_0, TensorType.q3_k: oracle.Q3_K, TensorType.q4_k: oracle.Q4_K, TensorType.q5_k: oracle.Q5_K, TensorType.q6_k: oracle.Q6_K,
                TensorType.bf16: oracle.BF16}
 
 
@@ -137,6 +137,8 @@ def quant_matvec(c, t: TensorType, k: int, pair: bool, variants=None):
     (TensorType.q4_k, 4096, False),   # "matvec q4_k norm+= (2 tiles)"
     (TensorType.q8_0, 4160, True),    # "matvec q8_0 norm+silu (tile tail, bitwise splits)"
     (TensorType.q4_k, 1024, True),    # the SiLU pair on Q4_K (the reference runs it on q3_k)
+    (TensorType.q3_k, 1024, False),   # "matvec q3_k norm+="
+    (TensorType.q3_k, 1024, True),    # "matvec q3_k norm+silu pair"
     (TensorType.q5_k, 1024, False),   # "matvec q5_k norm+="
     (TensorType.q6_k, 1024, False),   # "matvec q6_k norm+="
     (TensorType.q6_k, 2304, True),    # the SiLU pair on Q6_K, nine blocks a row
@@ -192,7 +194,7 @@ def test_quant_matvec_eight_rows(ctx):
 
 # ---- block decoders bit for bit, through the embedding gathers: check.zig:873-905 -----
 
-@pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q4_k, TensorType.q5_k, TensorType.q6_k])
+@pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q3_k, TensorType.q4_k, TensorType.q5_k, TensorType.q6_k])
 def test_embed_quant_bit_exact(ctx, t):
     c = ctx
     vocab, dim, split = 50, 512, 30
@@ -246,6 +248,19 @@ def test_repack_q8_0_matches_split_row_layout(ctx):
     wa = c.gpu_weights(TensorType.q8_0, raw, k)
     got = c.read_bytes(wa)[: rows * K.row_bytes(TensorType.q8_0, k)]
     assert np.array_equal(got, oracle.repack_q8_0(raw, rows, k))
+
+
+def test_repack_q3_k_matches_unit_layout(ctx):
+    """repack_q3_k against the oracle's restatement of the same layout, byte for byte."""
+    c = ctx
+    blocks = 37
+    raw = synth.random_blocks(c.rand, "q3_k", 1, blocks * 256)
+    padded = np.zeros((raw.size + 15) & ~15, dtype=np.uint8)
+    padded[: raw.size] = raw
+    out = c.output(blocks * 128 // 4)
+    c.launcher().launch(Kernel.repack_q3_k, P.RepackQ3K(blocks), [c.upload(padded), out], K.elementwise(blocks * 8))
+    got = c.read_words(out).view(np.uint8)[: blocks * 128]
+    assert np.array_equal(got, oracle.repack_q3_k(raw, blocks))
 
 
 def test_repad_pads_blocks(ctx):

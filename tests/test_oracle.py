@@ -225,6 +225,52 @@ def pack_q6_k(d, sc, q):
     return b
 
 
+def pack_q3_k(d, sc, q):
+    """One Q3_K block: element 128 n + 32 j + l holds v = q + 4 in 0..7: its low
+    two bits at bits 2 j of qs[32 n + l], its third bit at bit 4 n + j of
+    hmask[l]; sixteen 6-bit scales (scale 8 n + 2 j + l / 16, stored + 32): low
+    four bits of scale i in byte i % 8 (low nibble for i < 8, high nibble
+    otherwise), top two bits at bits 2 (i / 4) of byte 8 + i % 4."""
+    b = np.zeros(110, dtype=np.uint8)
+    v = (np.asarray(q, dtype=np.int32) + 4).astype(np.uint8).reshape(2, 4, 32)
+    for n in range(2):
+        for j in range(4):
+            b[32 + 32 * n : 64 + 32 * n] |= (v[n, j] & 3) << (2 * j)
+            b[0:32] |= (v[n, j] >> 2) << (4 * n + j)
+    s = (np.asarray(sc, dtype=np.int32) + 32).astype(np.uint8)
+    for i in range(16):
+        b[96 + i % 8] |= (s[i] & 15) << (4 * (i // 8))
+        b[104 + i % 4] |= (s[i] >> 4) << (2 * (i // 4))
+    b[108:110] = np.array([d], dtype=np.float16).view(np.uint8)
+    return b
+
+
+def test_q3_k_is_the_exact_value_of_packed_parts_and_repacks_losslessly():
+    """d (11 bits) x (scale - 32) (6) x quant (3) = 20 bits: every product is
+    exact, so y = d*(sc-32)*q exactly. The repacked units, read by an
+    independent numpy reader written from the unit layout's description, must
+    give the same weights."""
+    g = synth.rng(24)
+    for _ in range(40):
+        d = np.float16(g.uniform(-2, 2))
+        sc = g.integers(-32, 32, 16)
+        q = g.integers(-4, 4, 256)
+        blk = pack_q3_k(d, sc, q)
+        y = oracle.dequantize(oracle.Q3_K, blk, 256)
+        exact = float(d) * np.repeat(sc, 16).astype(np.float64) * q
+        assert np.array_equal(bits(y), bits(exact.astype(np.float32)))
+        units = oracle.repack_q3_k(blk, 1).view(np.uint32).reshape(8, 4)
+        for s_, (l0, l1, hw, tail) in enumerate(units.tolist()):
+            assert tail >> 16 == int(np.array([d], dtype=np.float16).view(np.uint16)[0])
+            for pos in range(32):
+                e, byte = pos // 4, pos % 4
+                lo = ((l0 if e < 4 else l1) >> (8 * byte + 2 * (e % 4))) & 3
+                h = (hw >> (8 * byte + e)) & 1
+                assert lo + 4 * h - 4 == q[32 * s_ + pos]
+            stored = [(tail & 0xff), (tail >> 8) & 0xff]
+            assert [x - 256 if x > 127 else x for x in stored] == [sc[2 * s_], sc[2 * s_ + 1]]
+
+
 def test_q5_k_is_the_correctly_rounded_exact_value_of_packed_parts():
     """d (11 bits) x scale (6) x quant (5) = 22 bits and dmin x min = 17 bits
     are exact in f32, so y must be d*sc*q - dmin*m rounded once, for blocks
@@ -252,14 +298,14 @@ def test_q6_k_is_the_correctly_rounded_exact_value_of_packed_parts():
         assert np.array_equal(bits(y), bits(exact.astype(np.float32)))
 
 
-@pytest.mark.parametrize("t,size,packer", [(oracle.Q5_K, 176, "q5_k"), (oracle.Q6_K, 210, "q6_k")])
+@pytest.mark.parametrize("t,size,packer", [(oracle.Q3_K, 110, "q3_k"), (oracle.Q5_K, 176, "q5_k"), (oracle.Q6_K, 210, "q6_k")])
 def test_k_quant_single_bit_mutations_move_exactly_their_weights(t, size, packer):
     """Flipping one quant bit changes exactly one weight; flipping a scale bit
     changes exactly one sub-block (32 weights for Q5_K, 16 for Q6_K)."""
     g = synth.rng(23)
     raw = synth.random_blocks(g, packer, 1, 256, scale=1.0)
     base = oracle.dequantize(t, raw, 256)
-    quant_bytes = range(16, 176) if t == oracle.Q5_K else range(0, 192)
+    quant_bytes = {oracle.Q3_K: range(0, 96), oracle.Q5_K: range(16, 176), oracle.Q6_K: range(0, 192)}[t]
     for byte in list(quant_bytes)[::7]:
         for bit in range(8):
             m = raw.copy()
@@ -274,6 +320,12 @@ def test_k_quant_single_bit_mutations_move_exactly_their_weights(t, size, packer
             n, i = (byte - 192) // 8, (byte - 192) % 8
             want = 128 * n + 32 * (i // 2) + 16 * (i % 2)
             assert changed.size <= 16 and np.all((changed >= want) & (changed < want + 16))
+    elif t == oracle.Q3_K:
+        for i in range(16):  # the lowest bit of scale i: byte i % 8, bit 4 (i / 8)
+            m = raw.copy()
+            m[96 + i % 8] ^= 1 << (4 * (i // 8))
+            changed = np.flatnonzero(bits(oracle.dequantize(t, m, 256)) != bits(base))
+            assert changed.size <= 16 and np.all(changed // 16 == i)
     else:
         sc = np.array([oracle.scale_min_k4(j, raw[4:16]) for j in range(8)])
         for j in range(8):

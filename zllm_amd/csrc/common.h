@@ -97,6 +97,7 @@ struct Dispatch {
 typedef zhip_result (*LaunchFn)(const Dispatch &);
 
 zhip_result launch_matvec_q8_0(const Dispatch &);
+zhip_result launch_matvec_q3_k(const Dispatch &);
 zhip_result launch_matvec_q4_k(const Dispatch &);
 zhip_result launch_matvec_q5_k(const Dispatch &);
 zhip_result launch_matvec_q6_k(const Dispatch &);
@@ -104,8 +105,10 @@ zhip_result launch_matvec_bf16(const Dispatch &);
 zhip_result launch_matmul_reduce(const Dispatch &);
 zhip_result launch_silu_mul(const Dispatch &);
 zhip_result launch_repack_q8_0(const Dispatch &);
+zhip_result launch_repack_q3_k(const Dispatch &);
 zhip_result launch_repad(const Dispatch &);
 zhip_result launch_embed_q8_0(const Dispatch &);
+zhip_result launch_embed_q3_k(const Dispatch &);
 zhip_result launch_embed_q4_k(const Dispatch &);
 zhip_result launch_embed_q5_k(const Dispatch &);
 zhip_result launch_embed_q6_k(const Dispatch &);

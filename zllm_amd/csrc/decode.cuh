@@ -3,6 +3,7 @@
 // multiply and subtract rounded on its own (no contraction), so decoded
 // weights equal the reference's bit for bit:
 //   Q8_0  src/ref/tensor.zig:49-53    y = f32(q) * f32(d)
+//   Q3_K  src/ref/tensor.zig:55-92    y = (d * (sc - 32)) * (q - 4 (1 - h))
 //   Q4_K  src/ref/tensor.zig:94-116   y = (d * sc) * q - (dmin * m)
 //   Q5_K  src/ref/tensor.zig:118-138  y = (d * sc) * (q | h << 4) - (dmin * m)
 //   Q6_K  src/ref/tensor.zig:140-160  y = (d * sc) * (q - 32)
@@ -57,6 +58,38 @@ struct DecQ8_0 {
             w[4 * e + 1] = __fmul_rn((float)((v << 16) >> 24), d);
             w[4 * e + 2] = __fmul_rn((float)((v << 8) >> 24), d);
             w[4 * e + 3] = __fmul_rn((float)(v >> 24), d);
+        }
+    }
+};
+
+// Q3_K blocks repacked at load into eight self-contained 16-byte units
+// (src/kernels/repack_q3_k.wgsl, src/kernels/quant/q3_k.wgsl): unit s of a
+// block holds the 32 weights 32 s .. 32 s + 31 as two words of 2-bit values
+// (byte b of word 0: positions b, 4 + b, 8 + b, 12 + b at bit pairs 0, 2, 4,
+// 6; word 1: positions 16 + b, ...), a word of third bits (bit e of byte b:
+// position 4 e + b), then scale - 32 for positions 0..15 and 16..31 as signed
+// bytes and d.
+struct DecQ3_K {
+    static constexpr int RUNS = 1;
+    static constexpr int E = 32;
+    static constexpr uint32_t BLOCK = 256;
+    static constexpr bool CHUNK_KERNEL = false;
+    static const char *name() { return "matvec_q3_k"; }
+    static uint32_t row_bytes(uint32_t k) { return k / 256u * 128u; }
+    __device__ static uint32_t xoff(uint32_t task, int) { return 32u * task; }
+    __device__ static void decode(const uint8_t *row, uint32_t, uint32_t task, float (&w)[E]) {
+        const uint4 u = *reinterpret_cast<const uint4 *>(row + 16u * task);
+        const float d = half_bits_to_float(u.w >> 16);
+        const float dl0 = __fmul_rn(d, (float)(int8_t)(u.w & 0xffu)), dl1 = __fmul_rn(d, (float)(int8_t)((u.w >> 8) & 0xffu));
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            const uint32_t lo = (e < 4 ? u.x : u.y) >> (2 * (e & 3));
+            const uint32_t hi = u.z >> e;
+#pragma unroll
+            for (int b = 0; b < 4; b++) {
+                const int v = (int)((lo >> (8 * b)) & 3u) + 4 * (int)((hi >> (8 * b)) & 1u) - 4;
+                w[4 * e + b] = __fmul_rn(e < 4 ? dl0 : dl1, (float)v);
+            }
         }
     }
 };

@@ -115,6 +115,54 @@ zhip_result launch_repack_q8_0(const Dispatch &d) {
     return check_launch(d, "repack_q8_0");
 }
 
+// ---- repack_q3_k: src/kernels/repack_q3_k.wgsl ---------------------------------
+// One thread per 16-byte unit (32 weights) of the repacked blocks.
+struct RepackQ3KParams { uint32_t blocks, pad0, pad1, pad2; };
+
+__device__ __forceinline__ uint32_t q3_scale(const uint8_t *sb, uint32_t i) {
+    const uint32_t k = i % 4u, g = i / 4u;
+    const uint32_t low = ((uint32_t)sb[4u * (g % 2u) + k] >> (4u * (g / 2u))) & 0xfu;
+    const uint32_t high = ((uint32_t)sb[8u + k] >> (2u * g)) & 3u;
+    return low | (high << 4);
+}
+
+__global__ __launch_bounds__(256) void repack_q3_k_kernel(const uint8_t *src, uint4 *dst, uint64_t units) {
+    for (uint64_t unit = (uint64_t)blockIdx.x * 256u + threadIdx.x; unit < units; unit += (uint64_t)gridDim.x * 256u) {
+        const uint8_t *b = src + (unit / 8u) * 110u;
+        const uint32_t s = (uint32_t)(unit % 8u), half = s / 4u, j = s % 4u;
+        uint32_t l0 = 0, l1 = 0, hw = 0;
+        for (uint32_t l = 0; l < 32u; l++) {
+            const uint32_t q = ((uint32_t)b[32u + 32u * half + l] >> (2u * j)) & 3u;
+            const uint32_t h = ((uint32_t)b[l] >> (4u * half + j)) & 1u;
+            const uint32_t e = l / 4u, byte = l % 4u;
+            if (e < 4u) l0 |= q << (8u * byte + 2u * e);
+            else l1 |= q << (8u * byte + 2u * (e - 4u));
+            hw |= h << (8u * byte + e);
+        }
+        // scale - 32 is in [-32, 31]: as a signed byte, (scale + 224) & 0xff.
+        const uint32_t sc0 = (q3_scale(b + 96, 8u * half + 2u * j) + 224u) & 0xffu;
+        const uint32_t sc1 = (q3_scale(b + 96, 8u * half + 2u * j + 1u) + 224u) & 0xffu;
+        const uint32_t d = (uint32_t)b[108] | ((uint32_t)b[109] << 8);
+        dst[unit] = make_uint4(l0, l1, hw, sc0 | (sc1 << 8) | (d << 16));
+    }
+}
+
+zhip_result launch_repack_q3_k(const Dispatch &d) {
+    if (d.params_size < sizeof(RepackQ3KParams)) return fail(d, ZHIP_E_BAD_COMMAND, "repack_q3_k: params block too small");
+    const RepackQ3KParams &p = *reinterpret_cast<const RepackQ3KParams *>(d.params);
+    if (!d.bind[1].bound || !d.bind[2].bound) return fail(d, ZHIP_E_BAD_COMMAND, "repack_q3_k: bindings 1 and 2 must be bound");
+    uint64_t units = (uint64_t)p.blocks * 8u;
+    const uint64_t cover = elementwise_cover(d);
+    if (cover < units) units = cover;
+    if (units == 0) return ZHIP_OK;
+    const uint64_t blocks_touched = (units + 7u) / 8u;
+    if (blocks_touched * 110u > d.bind[1].size || units * 16u > d.bind[2].size) return fail(d, ZHIP_E_BAD_COMMAND, "repack_q3_k: bound ranges too small");
+    if ((uintptr_t)d.bind[2].ptr & 15u) return fail(d, ZHIP_E_BAD_COMMAND, "repack_q3_k: destination must be 16-byte aligned");
+    hipLaunchKernelGGL(repack_q3_k_kernel, dim3(blocks_for(units, 256, 65536)), dim3(256), 0, d.stream, d.bind[1].ptr,
+        reinterpret_cast<uint4 *>(d.bind[2].ptr), units);
+    return check_launch(d, "repack_q3_k");
+}
+
 // ---- repad: src/kernels/repad.wgsl ---------------------------------------------
 __global__ __launch_bounds__(256) void repad_kernel(RepadParams p, const uint8_t *src, uint32_t *dst, uint64_t count) {
     const uint32_t words = p.dst_bytes / 4u;
@@ -147,7 +195,7 @@ zhip_result launch_repad(const Dispatch &d) {
     return check_launch(d, "repad");
 }
 
-// ---- embed_q8_0 / embed_q4_k / embed_q5_k / embed_q6_k / embed_bf16: src/kernels/embed_quant.wgsl, -------
+// ---- embed_q8_0 / embed_q3_k / embed_q4_k / embed_q5_k / embed_q6_k / embed_bf16: src/kernels/embed_quant.wgsl, -------
 // src/kernels/embed_half.wgsl. out[t] = table[tokens[t] - row0] decoded to f32
 // for tokens whose row lies in [row0, row0 + chunk_rows); one workgroup per
 // token. The decoders are the multiplies' own, so these kernels also show the
@@ -215,6 +263,7 @@ static zhip_result launch_embed(const Dispatch &d, const char *name) {
 
 zhip_result launch_embed_q8_0(const Dispatch &d) { return launch_embed<DecQ8_0>(d, "embed_q8_0"); }
 zhip_result launch_embed_q4_k(const Dispatch &d) { return launch_embed<DecQ4_K>(d, "embed_q4_k"); }
+zhip_result launch_embed_q3_k(const Dispatch &d) { return launch_embed<DecQ3_K>(d, "embed_q3_k"); }
 zhip_result launch_embed_q5_k(const Dispatch &d) { return launch_embed<DecQ5_K>(d, "embed_q5_k"); }
 zhip_result launch_embed_q6_k(const Dispatch &d) { return launch_embed<DecQ6_K>(d, "embed_q6_k"); }
 zhip_result launch_embed_bf16(const Dispatch &d) { return launch_embed<DecBF16>(d, "embed_bf16"); }

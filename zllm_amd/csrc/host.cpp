@@ -85,6 +85,7 @@ struct KernelInfo {
 
 static const KernelInfo kImplemented[] = {
     {"matvec_q8_0", 5, 0b01000, VariantKind::matvec, launch_matvec_q8_0, nullptr, nullptr, 1},
+    {"matvec_q3_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q3_k, nullptr, nullptr, 1},
     {"matvec_q4_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q4_k, nullptr, nullptr, 1},
     {"matvec_q5_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q5_k, nullptr, nullptr, 1},
     {"matvec_q6_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q6_k, nullptr, nullptr, 1},
@@ -94,8 +95,10 @@ static const KernelInfo kImplemented[] = {
     {"matmul_reduce", 3, 0b100, VariantKind::none, launch_matmul_reduce, nullptr, nullptr, 1},
     {"silu_mul", 3, 0b100, VariantKind::none, launch_silu_mul, nullptr, nullptr, 1},
     {"repack_q8_0", 3, 0b100, VariantKind::none, launch_repack_q8_0, nullptr, nullptr, 1},
+    {"repack_q3_k", 3, 0b100, VariantKind::none, launch_repack_q3_k, nullptr, nullptr, 1},
     {"repad", 3, 0b100, VariantKind::none, launch_repad, nullptr, nullptr, 1},
     {"embed_q8_0", 4, 0b1000, VariantKind::none, launch_embed_q8_0, nullptr, nullptr, 1},
+    {"embed_q3_k", 4, 0b1000, VariantKind::none, launch_embed_q3_k, nullptr, nullptr, 1},
     {"embed_q4_k", 4, 0b1000, VariantKind::none, launch_embed_q4_k, nullptr, nullptr, 1},
     {"embed_q5_k", 4, 0b1000, VariantKind::none, launch_embed_q5_k, nullptr, nullptr, 1},
     {"embed_q6_k", 4, 0b1000, VariantKind::none, launch_embed_q6_k, nullptr, nullptr, 1},

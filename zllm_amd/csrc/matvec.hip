@@ -1,5 +1,5 @@
 // Decode multiplies: out[t][col0 + j] (+)= sum_i X(t, i) * w[j][i] for Q8_0,
-// Q4_K, Q5_K, Q6_K and BF16 weights, with the RMSNorm / activation prologues and the
+// Q3_K, Q4_K, Q5_K, Q6_K and BF16 weights, with the RMSNorm / activation prologues and the
 // accumulate / SiLU-pair epilogues of the reference's matvec kernels
 // (src/kernels/matvec_quant.wgsl.hbs:20-31, src/kernels/matvec_half.wgsl:14-19).
 //
@@ -204,6 +204,7 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
 
 zhip_result launch_matvec_q8_0(const Dispatch &d) { return launch_matvec<DecQ8_0>(d, true); }
 zhip_result launch_matvec_q4_k(const Dispatch &d) { return launch_matvec<DecQ4_K>(d, true); }
+zhip_result launch_matvec_q3_k(const Dispatch &d) { return launch_matvec<DecQ3_K>(d, true); }
 zhip_result launch_matvec_q5_k(const Dispatch &d) { return launch_matvec<DecQ5_K>(d, true); }
 zhip_result launch_matvec_q6_k(const Dispatch &d) { return launch_matvec<DecQ6_K>(d, true); }
 zhip_result launch_matvec_bf16(const Dispatch &d) { return launch_matvec<DecBF16>(d, false); }

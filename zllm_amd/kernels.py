@@ -37,6 +37,7 @@ class TensorType(enum.IntEnum):
     f32 = 0
     f16 = 1
     q8_0 = 8
+    q3_k = 11
     q4_k = 12
     q5_k = 13
     q6_k = 14
@@ -44,7 +45,7 @@ class TensorType(enum.IntEnum):
 
 
 # (block_elems, block_bytes): src/gguf/gguf.zig:69-109.
-LAYOUT = {TensorType.f32: (1, 4), TensorType.f16: (1, 2), TensorType.bf16: (1, 2), TensorType.q8_0: (32, 34), TensorType.q4_k: (256, 144),
+LAYOUT = {TensorType.f32: (1, 4), TensorType.f16: (1, 2), TensorType.bf16: (1, 2), TensorType.q8_0: (32, 34), TensorType.q3_k: (256, 110), TensorType.q4_k: (256, 144),
           TensorType.q5_k: (256, 176), TensorType.q6_k: (256, 210)}
 
 
@@ -64,6 +65,7 @@ class Contract:
 # the kernels of this path (src/kernels/*.wgsl; tests: kernels.zig:209-221).
 CONTRACTS = {
     Kernel.matvec_q8_0: Contract(5, 0b01000),
+    Kernel.matvec_q3_k: Contract(5, 0b01000),
     Kernel.matvec_q4_k: Contract(5, 0b01000),
     Kernel.matvec_q5_k: Contract(5, 0b01000),
     Kernel.matvec_q6_k: Contract(5, 0b01000),
@@ -73,8 +75,10 @@ CONTRACTS = {
     Kernel.matmul_reduce: Contract(3, 0b100),
     Kernel.silu_mul: Contract(3, 0b100),
     Kernel.repack_q8_0: Contract(3, 0b100),
+    Kernel.repack_q3_k: Contract(3, 0b100),
     Kernel.repad: Contract(3, 0b100),
     Kernel.embed_q8_0: Contract(4, 0b1000),
+    Kernel.embed_q3_k: Contract(4, 0b1000),
     Kernel.embed_q4_k: Contract(4, 0b1000),
     Kernel.embed_q5_k: Contract(4, 0b1000),
     Kernel.embed_q6_k: Contract(4, 0b1000),
@@ -100,8 +104,9 @@ def weight_kernel(op: str, t: TensorType) -> Kernel:
 
 def block_stride(t: TensorType) -> int:
     """src/kernels/kernels.zig:144-151: the GGUF block size, padded to a multiple
-    of 16 where it is not one (Q6_K: 210 -> 224, laid out by repad)."""
-    return 224 if t == TensorType.q6_k else LAYOUT[t][1]
+    of 16 where it is not one (Q6_K: 210 -> 224, laid out by repad); Q3_K is
+    repacked into eight 16-byte units (repack_q3_k)."""
+    return {TensorType.q6_k: 224, TensorType.q3_k: 128}.get(t, LAYOUT[t][1])
 
 
 def row_bytes(t: TensorType, k: int) -> int:
@@ -268,6 +273,13 @@ class params:
             return struct.pack("<4I", self.rows, self.k, 0, 0)
 
     @dataclass
+    class RepackQ3K:
+        blocks: int
+
+        def pack(self) -> bytes:
+            return struct.pack("<4I", self.blocks, 0, 0, 0)
+
+    @dataclass
     class Repad:
         blocks: int
         src_bytes: int
@@ -401,6 +413,8 @@ class Launcher:
         blocks = rows * k // e
         if t == TensorType.q8_0:
             self.launch(Kernel.repack_q8_0, params.RepackQ80(rows, k), [src, dst], elementwise(rows * row_bytes(t, k) // 4))
+        elif t == TensorType.q3_k:
+            self.launch(Kernel.repack_q3_k, params.RepackQ3K(blocks), [src, dst], elementwise(blocks * 8))
         else:
             stride = block_stride(t)
             self.launch(Kernel.repad, params.Repad(blocks, b, stride), [src, dst], elementwise(blocks * stride // 4))

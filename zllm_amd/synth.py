@@ -82,7 +82,7 @@ def q4_k_rows(g: np.random.Generator, n: int, k: int, std: float = 0.01) -> np.n
 def random_blocks(g: np.random.Generator, t: str, n: int, k: int, scale: float = 0.05) -> np.ndarray:
     """Every byte random except the f16 super-scales, which are finite: the
     reference's own kernel-check generator (src/kernels/check.zig:461-481)."""
-    elems, size, scale_at = {"q8_0": (32, 34, (0,)), "q4_k": (256, 144, (0, 2)), "q5_k": (256, 176, (0, 2)), "q6_k": (256, 210, (208,))}[t]
+    elems, size, scale_at = {"q8_0": (32, 34, (0,)), "q3_k": (256, 110, (108,)), "q4_k": (256, 144, (0, 2)), "q5_k": (256, 176, (0, 2)), "q6_k": (256, 210, (208,))}[t]
     blocks = n * k // elems
     out = g.integers(0, 256, size=(blocks, size), dtype=np.uint8)
     for off in scale_at:
