@@ -78,6 +78,16 @@ _lib.zref_repack_q3_k.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
 _lib.zref_repack_q3_k.restype = None
 _lib.zref_matmul_slices.argtypes = [C.c_uint32, C.c_uint32, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]
 _lib.zref_matmul_f64.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_uint]
+_lib.zref_f16_round.restype = C.c_float
+_lib.zref_f16_round.argtypes = [C.c_float]
+_lib.zref_quantize_q8.restype = C.c_int
+_lib.zref_quantize_q8.argtypes = [C.c_void_p, C.c_size_t, C.c_uint, C.c_void_p, C.c_void_p]
+_lib.zref_round_like_llama.restype = C.c_int
+_lib.zref_round_like_llama.argtypes = [C.c_int, C.c_void_p, C.c_size_t]
+_lib.zref_quantize_q8_rows.restype = C.c_int
+_lib.zref_quantize_q8_rows.argtypes = [C.c_void_p, C.c_size_t, C.c_size_t, C.c_uint, C.c_uint, C.c_float, C.c_void_p, C.c_void_p, C.c_void_p]
+_lib.zref_matmul_q8.restype = C.c_int
+_lib.zref_matmul_q8.argtypes = [C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_size_t, C.c_size_t, C.c_size_t, C.c_void_p]
 
 
 def _ptr(a: np.ndarray) -> int:
@@ -224,3 +234,52 @@ def matmul_f64(x: np.ndarray, w: np.ndarray, threads: int = 0) -> np.ndarray:
     want = np.empty((x.shape[0], n), dtype=np.float64)
     _lib.zref_matmul_f64(_ptr(want), _ptr(x), _ptr(w), x.shape[0], n, k, threads or default_threads())
     return want
+
+
+def f16_round(x: float) -> float:
+    return _lib.zref_f16_round(x)
+
+
+def act_block(t: int) -> int:
+    """Activations per rounding block for weights of type t (src/kernels/kernels.zig:301-303)."""
+    return 32 if t == Q8_0 else 256
+
+
+def quantize_q8(x: np.ndarray, block: int, mode: int = 0, eps: float = 0.0, nw: np.ndarray | None = None):
+    """Rows of x rounded to 8-bit blocks: (q int8 rows x k, d f32 rows x k / block).
+
+    Mode 2 takes rows of gate | up, 2k wide (src/kernels/quantize_q8.wgsl:1-9)."""
+    x = np.ascontiguousarray(x, dtype=np.float32)
+    assert x.ndim == 2
+    rows, width = x.shape
+    k = width // 2 if mode == 2 else width
+    q = np.empty((rows, k), dtype=np.int8)
+    d = np.empty((rows, k // block), dtype=np.float32)
+    if nw is None:
+        nw = np.ones(k, dtype=np.float32)
+    nw = np.ascontiguousarray(nw, dtype=np.float32)
+    if _lib.zref_quantize_q8_rows(_ptr(x), rows, k, block, mode, eps, _ptr(nw), _ptr(q), _ptr(d)) != 0:
+        raise ValueError("quantize_q8: bad block or k")
+    return q, d
+
+
+def round_like_llama(t: int, x: np.ndarray) -> np.ndarray:
+    """src/ref/matmul.zig:197-247, row by row, on a copy."""
+    out = np.array(x, dtype=np.float32, order="C", copy=True)
+    rows = out.reshape(-1, out.shape[-1])
+    for r in rows:
+        if _lib.zref_round_like_llama(t, _ptr(r), r.size) != 0:
+            raise ValueError("round_like_llama: unsupported type")
+    return out
+
+
+def matmul_q8(t: int, raw: np.ndarray, q: np.ndarray, d: np.ndarray, n: int) -> np.ndarray:
+    """The int8 prefill multiply's formula over file-layout rows, in float64."""
+    raw = np.ascontiguousarray(raw).view(np.uint8)
+    q = np.ascontiguousarray(q, dtype=np.int8)
+    d = np.ascontiguousarray(d, dtype=np.float32)
+    rows, k = q.shape
+    out = np.empty((rows, n), dtype=np.float64)
+    if _lib.zref_matmul_q8(t, _ptr(raw), _ptr(q), _ptr(d), rows, n, k, _ptr(out)) != 0:
+        raise ValueError("matmul_q8: unsupported type")
+    return out

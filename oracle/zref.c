@@ -678,3 +678,169 @@ void zref_matmul_f64(double *want, const float *x, const float *w, size_t rows, 
     f64_ctx ctx = { want, x, w, rows, n, k };
     parallel_for(pool_get(threads), n, 1, 1, &ctx, f64_run);
 }
+
+/* ---- activations rounded to 8-bit blocks: the quantized prefill multiply --------- */
+
+/* x >= 0 rounded to binary16 precision (nearest, ties to even) and widened
+ * back, as src/kernels/quantize_q8.wgsl:52-60 does on raw bits. Values above
+ * the f16 range do not occur: x is a block maximum divided by 127. */
+float zref_f16_round(float x) {
+    uint32_t u;
+    memcpy(&u, &x, 4);
+    if (((u >> 23) & 0xffu) < 113u) {
+        /* Below f16's normal range: multiples of 2^-24. */
+        return nearbyintf(x * 16777216.0f) * (1.0f / 16777216.0f);
+    }
+    u = (u + 0xfffu + ((u >> 13) & 1u)) & 0xffffe000u;
+    memcpy(&x, &u, 4);
+    return x;
+}
+
+/* ggml's nearest_int: the f32 addition rounds ties to even
+ * (src/ref/matmul.zig:217-219,240-242). */
+static int32_t nearest_int(float y) {
+    float s = y + 12582912.0f;
+    int32_t bits;
+    memcpy(&bits, &s, 4);
+    return bits - 0x4b400000;
+}
+
+/* src/ref/matmul.zig:197-247 with the integers and block scales kept apart
+ * (src/kernels/quantize_q8.wgsl:11-22): x[i] ~ q[i] * d[i / block]. */
+int zref_quantize_q8(const float *x, size_t n, unsigned block, int8_t *q, float *d) {
+    if ((block != 32 && block != 256) || n % block != 0) return -1;
+    for (size_t b = 0; b < n; b += block) {
+        const float *v = x + b;
+        if (block == 32) {
+            float amax = 0;
+            for (unsigned i = 0; i < 32; i++) {
+                float a = fabsf(v[i]);
+                if (a > amax) amax = a;
+            }
+            float d32 = amax / 127.0f;
+            float id = amax != 0 ? 127.0f / amax : 0.0f;
+            d[b / 32] = zref_f16_round(d32);
+            for (unsigned i = 0; i < 32; i++) {
+                float scaled = v[i] * id;
+                q[b + i] = (int8_t)nearest_int(scaled);
+            }
+        } else {
+            float amax = 0, max = 0;
+            for (unsigned i = 0; i < 256; i++) {
+                float a = fabsf(v[i]);
+                if (a > amax) {
+                    amax = a;
+                    max = v[i];
+                }
+            }
+            if (amax == 0) {
+                d[b / 256] = 0;
+                memset(q + b, 0, 256);
+                continue;
+            }
+            float iscale = -127.0f / max;
+            d[b / 256] = 1.0f / iscale;
+            for (unsigned i = 0; i < 256; i++) {
+                float scaled = iscale * v[i];
+                int32_t r = nearest_int(scaled);
+                q[b + i] = (int8_t)(r < 127 ? r : 127);
+            }
+        }
+    }
+    return 0;
+}
+
+/* src/ref/matmul.zig:197-247: a row rounded as the multiply will see it. */
+int zref_round_like_llama(int type, float *x, size_t n) {
+    if (type == ZREF_Q8_0 || type == ZREF_Q3_K || type == ZREF_Q4_K || type == ZREF_Q5_K || type == ZREF_Q6_K) {
+        unsigned block = type == ZREF_Q8_0 ? 32 : 256;
+        int8_t *q = malloc(n);
+        float *d = malloc((n / block + 1) * sizeof(float));
+        int r = q && d ? zref_quantize_q8(x, n, block, q, d) : -1;
+        if (r == 0)
+            for (size_t i = 0; i < n; i++) x[i] = (float)q[i] * d[i / block];
+        free(q);
+        free(d);
+        return r;
+    }
+    if (type == ZREF_BF16) {
+        for (size_t i = 0; i < n; i++) x[i] = zref_bf16_round(x[i]);
+        return 0;
+    }
+    if (type == ZREF_F16) {
+        for (size_t i = 0; i < n; i++) {
+            float a = zref_f16_round(fabsf(x[i]));
+            x[i] = copysignf(a, x[i]);
+        }
+        return 0;
+    }
+    return type == ZREF_F32 ? 0 : -1;
+}
+
+/* src/kernels/quantize_q8.wgsl:1-9,66-104: rows of k values computed by
+ * `mode` (0: x; 1: RMSNorm(x) * nw; 2: silu(gate) * up over rows of gate | up),
+ * then rounded block by block. */
+int zref_quantize_q8_rows(const float *x, size_t rows, size_t k, unsigned block, unsigned mode, float eps,
+                          const float *nw, int8_t *q, float *d) {
+    float *row = malloc(k * sizeof(float));
+    if (!row) return -1;
+    int r = 0;
+    for (size_t t = 0; t < rows && r == 0; t++) {
+        if (mode == 2) {
+            const float *g = x + t * 2 * k, *u = g + k;
+            for (size_t i = 0; i < k; i++) row[i] = zref_silu(g[i]) * u[i];
+        } else {
+            memcpy(row, x + t * k, k * sizeof(float));
+            if (mode == 1) zref_rms_norm(row, nw, k, eps);
+        }
+        r = zref_quantize_q8(row, k, block, q + t * k, d + t * (k / block));
+    }
+    free(row);
+    return r;
+}
+
+/* out[t][j] = sum over 32-weight units of dx * (s * sum(q * qx) - m * sum(qx))
+ * (src/kernels/matmul_quant.wgsl:1-9,130-160), the integer sums exact and the
+ * scaled terms added in double. Weights are file-layout blocks (Q8_0: 34-byte
+ * blocks; Q4_K: 144-byte blocks); dx has one scale per 32 (Q8_0) or 256 (Q4_K)
+ * activations. */
+int zref_matmul_q8(int type, const uint8_t *w, const int8_t *qx, const float *dx, size_t rows, size_t n, size_t k, double *out) {
+    if (type != ZREF_Q8_0 && type != ZREF_Q4_K) return -1;
+    for (size_t t = 0; t < rows; t++) {
+        const int8_t *xr = qx + t * k;
+        for (size_t j = 0; j < n; j++) {
+            double sum = 0;
+            if (type == ZREF_Q8_0) {
+                const uint8_t *row = w + j * (k / 32) * 34;
+                for (size_t u = 0; u < k / 32; u++) {
+                    const uint8_t *b = row + u * 34;
+                    int32_t dot = 0;
+                    for (unsigned i = 0; i < 32; i++) dot += (int32_t)(int8_t)b[2 + i] * xr[u * 32 + i];
+                    sum += (double)dx[t * (k / 32) + u] * ((double)zref_half(rd16(b)) * dot);
+                }
+            } else {
+                const uint8_t *row = w + j * (k / 256) * 144;
+                for (size_t blk = 0; blk < k / 256; blk++) {
+                    const uint8_t *b = row + blk * 144;
+                    float dd = zref_half(rd16(b)), dmin = zref_half(rd16(b + 2));
+                    for (unsigned sb = 0; sb < 8; sb++) {
+                        uint8_t sc, m;
+                        zref_scale_min_k4(sb, b + 4, &sc, &m);
+                        const uint8_t *qs = b + 16 + 32 * (sb / 2);
+                        int32_t dot = 0, xs = 0;
+                        for (unsigned i = 0; i < 32; i++) {
+                            int32_t qv = sb & 1 ? qs[i] >> 4 : qs[i] & 0xF;
+                            int32_t xv = xr[blk * 256 + sb * 32 + i];
+                            dot += qv * xv;
+                            xs += xv;
+                        }
+                        float s = dd * (float)sc, mn = dmin * (float)m;
+                        sum += (double)dx[t * (k / 256) + blk] * ((double)s * dot - (double)mn * xs);
+                    }
+                }
+            }
+            out[t * n + j] = sum;
+        }
+    }
+    return 0;
+}

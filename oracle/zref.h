@@ -33,6 +33,19 @@
  *   - zref_rms_norm: the reference's 17-value bitwise known answer
  *     (src/ref/ops.zig:139-168).
  *   - zref_bf16_round: torch.bfloat16 round-to-nearest-even.
+ *   - zref_f16_round: numpy's float16 conversion over a sweep of every exponent
+ *     with tie and near-tie mantissas.
+ *   - zref_quantize_q8 / zref_round_like_llama: the cases the reference's own
+ *     check builds (src/kernels/check.zig:516-547: a negative maximum, a +amax /
+ *     -amax tie, a zero row, exact half-integers in blocks whose scale is 1)
+ *     with their answers worked by hand, and a numpy restatement that rounds
+ *     with rint instead of the magic-number addition. Agreement with ggml's
+ *     quantize_row_q8_0 / quantize_row_q8_K_ref is "parity unpinned" (library
+ *     not available offline).
+ *   - zref_matmul_q8: must equal, to double rounding, the float64 product of the
+ *     rounded activations q * d with the decoded weights (zref_dequantize),
+ *     the formulation the reference checks its kernel against
+ *     (src/kernels/check.zig:839-871).
  *   - zref_silu: float64 closed form. Its last-ulp agreement with Zig's @exp is
  *     "parity unpinned" (only an import of the Zig build could pin it).
  */
@@ -132,6 +145,29 @@ void zref_matmul_slices(uint32_t n, uint32_t k, uint32_t *count, uint32_t *k_sli
  * (src/kernels/check.zig:34-83,205-222): want[t][j] = init + sum x*w in
  * double over already decoded weights. */
 void zref_matmul_f64(double *want, const float *x, const float *w, size_t rows, size_t n, size_t k, unsigned threads);
+
+/* ---- activations rounded to 8-bit blocks (the quantized prefill multiply) --- */
+
+/* x >= 0 rounded to binary16 (nearest even) and widened back
+ * (src/kernels/quantize_q8.wgsl:52-60). */
+float zref_f16_round(float x);
+/* x[i] ~ q[i] * d[i / block] as llama.cpp's x86 CPU backend rounds activations:
+ * block 32 = Q8_0 (d = amax / 127 in f16, q = rne(x * (127 / amax))), block 256
+ * = Q8_K (d = -max / 127 for the first value of largest magnitude, q =
+ * min(127, rne(x * -127 / max))) (src/ref/matmul.zig:197-247,
+ * src/kernels/quantize_q8.wgsl:11-22). Returns 0, or -1 for a bad block. */
+int zref_quantize_q8(const float *x, size_t n, unsigned block, int8_t *q, float *d);
+/* A row rounded in place as the multiply with weights of `type` sees it
+ * (src/ref/matmul.zig:197-247). */
+int zref_round_like_llama(int type, float *x, size_t n);
+/* quantize_q8 over rows with its fused producers (src/kernels/quantize_q8.wgsl:1-9):
+ * mode 0 x, 1 RMSNorm(x) * nw, 2 silu(gate) * up over rows of gate | up. */
+int zref_quantize_q8_rows(const float *x, size_t rows, size_t k, unsigned block, unsigned mode, float eps,
+                          const float *nw, int8_t *q, float *d);
+/* The int8 prefill multiply's formula (src/kernels/matmul_quant.wgsl:1-9):
+ * exact integer unit sums, scaled and added in double. `w` is file-layout
+ * Q8_0 or Q4_K rows. */
+int zref_matmul_q8(int type, const uint8_t *w, const int8_t *qx, const float *dx, size_t rows, size_t n, size_t k, double *out);
 
 #ifdef __cplusplus
 }

@@ -425,6 +425,153 @@ def test_matmul_q8_0_float(ctx, rung):
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
 
 
+# ---- activations rounded to 8-bit blocks, and the int8 multiply: check.zig:500-594,839-871 ----
+
+def quantize_x(c, t: TensorType, x, rows: int, k: int, mode: int = 0, eps: float = 0.0, nw=None):
+    """quantize_q8 on an uploaded x: (qx words, dx), as src/kernels/check.zig:504-509."""
+    block = K.act_block(t)
+    qx, dx = c.output(rows * k // 4), c.output(rows * k // block)
+    c.launcher().launch(Kernel.quantize_q8, P.QuantizeQ8(k=k, block=block, mode=mode, eps=eps), [x, qx, dx, nw if nw is not None else x],
+                        (K.div_ceil(k, 256), rows, 1))
+    return qx, dx
+
+
+def read_q8(c, qx, dx, rows: int, k: int):
+    return c.read_bytes(qx).view(np.int8)[: rows * k].reshape(rows, k), c.read(dx).reshape(rows, -1)
+
+
+@pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q4_k])
+def test_quantize_q8_value_for_value(ctx, t):
+    """Random rows, a negative maximum, a +amax / -amax tie, a zero row and exact
+    half-integers (src/kernels/check.zig:511-547); tolerance 0, and the integers
+    and scales themselves must equal the oracle's."""
+    c = ctx
+    rows, k = 6, 512
+    x = c.random(rows * k, 3).reshape(rows, k)
+    x[2, 77] = -9.5
+    x[3, 5] = -7.25
+    x[3, 40] = 7.25
+    x[4] = 0
+    x[5] = (np.arange(k) % 32 - 16).astype(np.float32) + np.float32(0.5)
+    x[5, ::32] = 127
+    block = K.act_block(t)
+    qx, dx = quantize_x(c, t, c.upload(x), rows, k)
+    q, d = read_q8(c, qx, dx, rows, k)
+    d = d[:, : k // block]
+    wq, wd = oracle.quantize_q8(x, block)
+    assert np.array_equal(q, wq)
+    assert np.array_equal(d.view(np.uint32), wd.view(np.uint32))
+    got = q.astype(np.float32) * np.repeat(d, block, axis=1)
+    assert np.array_equal(got, oracle.round_like_llama(ORACLE_TYPE[t], x))
+
+
+@pytest.mark.parametrize("mode", [1, 2])
+def test_quantize_q8_fused(ctx, mode):
+    """quantize_q8 computing its input first (RMSNorm, SiLU pair): every value
+    within half a step of the float64 result, tolerance 1.0001 half-steps
+    (src/kernels/check.zig:549-586)."""
+    c = ctx
+    rows, k, eps = 5, 768, 1e-6
+    width = 2 * k if mode == 2 else k
+    x = c.random(rows * width, 2).reshape(rows, width)
+    nw = c.random(k, 1)
+    qx, dx = quantize_x(c, TensorType.q4_k, c.upload(x), rows, k, mode=mode, eps=eps, nw=c.upload(nw))
+    q, d = read_q8(c, qx, dx, rows, k)
+    d = d[:, : k // 256]
+    if mode == 1:
+        want = np.stack([norm_row(r, nw, eps) for r in x])
+    else:
+        g = x[:, :k].astype(np.float64)
+        want = g * sigmoid64(g) * x[:, k:]
+    step = np.repeat(np.abs(d), 256, axis=1).astype(np.float64)
+    got = q.astype(np.float64) * np.repeat(d, 256, axis=1)
+    assert np.max(np.abs(got - want) / (step / 2)) <= 1.0001
+    if mode == 1:
+        # The normalisation follows ggml's arithmetic step for step, so the
+        # integers equal the oracle's.
+        wq, wd = oracle.quantize_q8(x, 256, mode=1, eps=eps, nw=nw)
+        assert np.array_equal(q, wq) and np.array_equal(d.view(np.uint32), wd.view(np.uint32))
+
+
+def launch_int8(c, t, act, wa, out, rows, n, k, accumulate, slices, col0=0, stride=None):
+    l = c.launcher()
+    stride = stride or n
+    kernel = K.weight_kernel("matmul", t)
+    grid = (K.div_ceil(n, K.matmul_quant_tile_n), K.div_ceil(rows, K.matmul_quant_tile_t), 1)
+    qx, dx = act
+    if slices is None:
+        l.launch(kernel, P.MatmulQuant(rows=rows, n=n, k=k, col0=col0, out_stride=stride, accumulate=accumulate, k_slice=k), [qx, wa, out, dx], grid)
+        return
+    count, k_slice = slices
+    partials = c.output(count * rows * n)
+    l.launch(kernel, P.MatmulQuant(rows=rows, n=n, k=k, col0=0, out_stride=n, k_slice=k_slice, slice_stride=rows * n), [qx, wa, partials, dx], (grid[0], grid[1], count))
+    l.launch(Kernel.matmul_reduce, P.MatmulReduce(rows=rows, n=n, slices=count, col0=col0, out_stride=stride, accumulate=accumulate, slice_stride=rows * n),
+             [partials, out], K.elementwise(rows * n))
+
+
+@pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q4_k])
+def test_matmul_int8_whole_and_split(ctx, t):
+    """The prefill multiply on quantize_q8's output, accumulating, over more than
+    one tile each way: whole, and split over k into partials that matmul_reduce
+    adds up; against float64 over the rounded activations, tolerance 1e-5
+    (src/kernels/check.zig:839-871). The integer unit sums make the result equal
+    the oracle's unit formula far more tightly, and token chunks keep their bits."""
+    c = ctx
+    rows, n, k = 70, 150, 1024
+    s = K.matmul_slices(n, k)
+    assert s.count > 1
+    x = c.random(rows * k, 1).reshape(rows, k)
+    xs = oracle.round_like_llama(ORACLE_TYPE[t], x)
+    act = quantize_x(c, t, c.upload(x), rows, k)
+    raw, values = quant_rows(c, t, n, k)
+    wa = c.gpu_weights(t, raw, k)
+    init = c.random(rows * n, 4).reshape(rows, n)
+    want = init + xs.astype(np.float64) @ values.astype(np.float64).T
+    whole, split, odd = c.upload(init), c.upload(init), c.upload(init)
+    launch_int8(c, t, act, wa, whole, rows, n, k, 1, None)
+    launch_int8(c, t, act, wa, split, rows, n, k, 1, (s.count, s.k_slice))
+    # Slices that cut a 256-weight block and leave a short last one.
+    launch_int8(c, t, act, wa, odd, rows, n, k, 1, (3, 352))
+    for out in (whole, split, odd):
+        assert rel_err(c.read(out).reshape(rows, n), want) <= 1e-5
+    block = K.act_block(t)
+    q, d = oracle.quantize_q8(x, block)
+    formula = init + oracle.matmul_q8(ORACLE_TYPE[t], raw, q, d, n)
+    assert rel_err(c.read(whole).reshape(rows, n), formula) <= 2e-6
+    got = c.read(whole).reshape(rows, n)
+    for first, count in ((0, 3), (3, 30), (33, 37)):
+        chunk = c.upload(init[first : first + count])
+        launch_int8(c, t, quantize_x(c, t, c.upload(x[first : first + count]), count, k), wa, chunk, count, n, k, 1, None)
+        assert got[first : first + count].tobytes() == c.read(chunk).tobytes(), "token chunking changed bits"
+
+
+@pytest.mark.parametrize("t,rows,n,k", [
+    (TensorType.q8_0, 67, 70, 320),    # k not a multiple of the 128-deep step
+    (TensorType.q8_0, 130, 200, 4096),
+    (TensorType.q4_k, 1, 129, 2048),
+    (TensorType.q4_k, 257, 64, 1536),
+])
+def test_matmul_int8_shapes(ctx, t, rows, n, k):
+    """Partial tiles each way, a padded output stride and a nonzero first column;
+    nothing outside the output columns is touched."""
+    c = ctx
+    x = c.random(rows * k, 1).reshape(rows, k)
+    xs = oracle.round_like_llama(ORACLE_TYPE[t], x)
+    act = quantize_x(c, t, c.upload(x), rows, k)
+    raw, values = quant_rows(c, t, n, k)
+    wa = c.gpu_weights(t, raw, k)
+    stride, col0 = n + 9, 5
+    init = c.random(rows * stride, 0.25).reshape(rows, stride)
+    out = c.upload(init)
+    launch_int8(c, t, act, wa, out, rows, n, k, 0, None, col0=col0, stride=stride)
+    got = c.read(out).reshape(rows, stride)
+    want = xs.astype(np.float64) @ values.astype(np.float64).T
+    assert rel_err(got[:, col0 : col0 + n], want) <= 1e-5
+    mask = np.ones(stride, dtype=bool)
+    mask[col0 : col0 + n] = False
+    assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32))
+
+
 def test_silu_mul(ctx):
     c = ctx
     rows, width = 7, 10_001

@@ -1,0 +1,176 @@
+"""Pins the oracle's activation rounding (quantize_q8) and int8 multiply.
+
+The reference rounds activations as llama.cpp's x86 CPU backend does
+(src/ref/matmul.zig:197-247) and checks its kernel on a handful of built cases
+(src/kernels/check.zig:516-547). Those cases are worked by hand here, and the
+rest is pinned by a numpy restatement that shares no code with the oracle: it
+rounds with rint instead of the magic-number addition, finds the leading value
+with argmax, and converts the scale with numpy's float16.
+"""
+import numpy as np
+import pytest
+
+import oracle
+from zllm_amd import synth
+
+
+def test_f16_round_matches_numpy_float16():
+    # Every f16 exponent (and the subnormal range) with mantissas at, just below
+    # and just above the halfway points, plus random values.
+    rng = np.random.default_rng(5)
+    exps = np.arange(-26, 16)
+    fracs = np.array([0, 1, 0x0fff, 0x1000, 0x1001, 0x2fff, 0x3000, 0x3001, 0x7fefff, 0x7ff000, 0x7ff001, 0x7fffff], dtype=np.uint32)
+    bits = ((exps[:, None] + 127).astype(np.uint32) << 23) | fracs[None, :]
+    values = np.concatenate([bits.reshape(-1).view(np.float32), rng.random(5000, dtype=np.float32) * np.float32(3.0), np.float32([0.0])])
+    values = values[values < 65504.0]
+    want = values.astype(np.float16).astype(np.float32)
+    got = np.array([oracle.f16_round(float(v)) for v in values], dtype=np.float32)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+
+
+def numpy_quantize(x: np.ndarray, block: int):
+    """x (rows, k) -> (q, d) by the published rule, vectorised."""
+    x = np.asarray(x, dtype=np.float32)
+    rows, k = x.shape
+    b = x.reshape(rows, k // block, block)
+    mag = np.abs(b)
+    first = np.argmax(mag, axis=2)  # first of the largest
+    lead = np.take_along_axis(b, first[..., None], axis=2)[..., 0]
+    amax = np.abs(lead)
+    with np.errstate(divide="ignore", invalid="ignore"):
+        if block == 32:
+            d = (amax / np.float32(127)).astype(np.float16).astype(np.float32)
+            inv = np.where(amax != 0, np.float32(127) / amax, np.float32(0)).astype(np.float32)
+            q = np.rint(b * inv[..., None])
+        else:
+            iscale = (np.float32(-127) / lead).astype(np.float32)
+            d = np.where(amax != 0, np.float32(1) / iscale, np.float32(0)).astype(np.float32)
+            q = np.minimum(np.rint(iscale[..., None] * b), 127)
+            q = np.where(amax[..., None] != 0, q, 0)
+    return q.reshape(rows, k).astype(np.int8), d.astype(np.float32)
+
+
+def check_rows(k: int = 512) -> np.ndarray:
+    """The rows the reference's check builds (src/kernels/check.zig:521-535)."""
+    rng = np.random.default_rng(17)
+    x = ((rng.random((6, k), dtype=np.float32) * 2 - 1) * np.float32(3)).astype(np.float32)
+    x[2, 77] = -9.5
+    x[3, 5] = -7.25
+    x[3, 40] = 7.25
+    x[4] = 0
+    x[5] = (np.arange(k) % 32 - 16).astype(np.float32) + np.float32(0.5)
+    x[5, ::32] = 127
+    return x
+
+
+@pytest.mark.parametrize("block", [32, 256])
+def test_quantize_hand_worked_cases(block):
+    x = check_rows()
+    q, d = oracle.quantize_q8(x, block)
+    # A negative maximum: the value of largest magnitude maps to -127 whatever its sign.
+    assert q[2, 77] == -127
+    blk = 77 // block
+    assert d[2, blk] > 0
+    if block == 256:
+        assert d[2, blk] == np.float32(1) / (np.float32(-127) / np.float32(-9.5))
+    else:
+        assert d[2, blk] == np.float32(np.float16(np.float32(9.5) / np.float32(127)))
+    # +amax and -amax tie: the first one leads; both ends stay within [-127, 127].
+    assert q[3, 5] == -127 and q[3, 40] == 127
+    # A zero row: zero integers, zero scales.
+    assert not q[4].any() and not d[4].any()
+    # Exact half-integers under a scale of exactly one: ties go to even.
+    halves = (np.arange(512) % 32 - 16).astype(np.float64) + 0.5
+    if block == 32:
+        assert np.all(d[5] == 1.0)
+        want = np.rint(halves)
+        want[::32] = 127
+    else:
+        assert np.all(d[5] == -1.0)
+        want = np.rint(-halves)
+        want[::32] = -127
+    assert np.array_equal(q[5].astype(np.float64), want)
+    # -14.5, 0.5 and 1.5 each sit between an odd and an even integer: the even one wins.
+    if block == 32:
+        assert (q[5, 1], q[5, 16 + 0], q[5, 17]) == (-14, 0, 2)
+    else:
+        assert (q[5, 1], q[5, 16 + 0], q[5, 17]) == (14, 0, -2)
+
+
+@pytest.mark.parametrize("block", [32, 256])
+def test_quantize_matches_numpy_restatement(block):
+    rng = np.random.default_rng(23)
+    x = ((rng.random((40, 1024), dtype=np.float32) * 2 - 1) * np.float32(5)).astype(np.float32)
+    x[:6, :512] = check_rows()
+    x[7] *= np.float32(1e-6)   # tiny values: subnormal f16 scales for block 32
+    x[8] *= np.float32(300.0)
+    x[9, 100:400] = 0
+    q, d = oracle.quantize_q8(x, block)
+    wq, wd = numpy_quantize(x, block)
+    assert np.array_equal(d.view(np.uint32), wd.view(np.uint32))
+    assert np.array_equal(q, wq)
+
+
+@pytest.mark.parametrize("t,block", [(oracle.Q8_0, 32), (oracle.Q4_K, 256), (oracle.Q6_K, 256)])
+def test_round_like_llama_is_q_times_d(t, block):
+    x = check_rows()
+    q, d = numpy_quantize(x, block)
+    want = q.astype(np.float32) * np.repeat(d, block, axis=1)
+    got = oracle.round_like_llama(t, x)
+    assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    # Rounding is within half a step of the input, plus what rounding the scale
+    # itself to f16 moves the largest values by (Q8_0: 127 steps * 2^-11).
+    step = np.repeat(np.abs(d), block, axis=1).astype(np.float64)
+    slack = 127.0 / 2048.0 if block == 32 else 1e-4
+    assert np.all(np.abs(got.astype(np.float64) - x) <= (0.5 + slack) * step + 1e-30)
+
+
+def test_round_like_llama_half_types():
+    rng = np.random.default_rng(3)
+    x = ((rng.random(4096, dtype=np.float32) * 2 - 1) * np.float32(8)).astype(np.float32)
+    assert np.array_equal(oracle.round_like_llama(oracle.BF16, x[None])[0], synth.bf16_round(x))
+    assert np.array_equal(oracle.round_like_llama(oracle.F16, x[None])[0], x.astype(np.float16).astype(np.float32))
+    assert np.array_equal(oracle.round_like_llama(oracle.F32, x[None])[0], x)
+
+
+def test_quantize_fused_modes():
+    rng = np.random.default_rng(11)
+    rows, k, eps = 5, 768, 1e-6
+    x = ((rng.random((rows, k), dtype=np.float32) * 2 - 1) * np.float32(2)).astype(np.float32)
+    nw = (rng.random(k, dtype=np.float32) * 2 - 1).astype(np.float32)
+    # Mode 1 is the pinned RMSNorm followed by the pinned rounding.
+    q, d = oracle.quantize_q8(x, 256, mode=1, eps=eps, nw=nw)
+    normed = np.stack([oracle.rms_norm(r, nw, eps) for r in x])
+    wq, wd = numpy_quantize(normed, 256)
+    assert np.array_equal(q, wq) and np.array_equal(d, wd)
+    # Mode 2 rounds silu(gate) * up: within half a step of the float64 value
+    # (src/kernels/check.zig:549-586).
+    gu = ((rng.random((rows, 2 * k), dtype=np.float32) * 2 - 1) * np.float32(2)).astype(np.float32)
+    q, d = oracle.quantize_q8(gu, 256, mode=2)
+    g = gu[:, :k].astype(np.float64)
+    want = g / (1 + np.exp(-g)) * gu[:, k:]
+    step = np.repeat(np.abs(d), 256, axis=1).astype(np.float64)
+    got = q.astype(np.float64) * np.repeat(d, 256, axis=1)
+    assert np.max(np.abs(got - want) / (step / 2)) <= 1.0001
+
+
+@pytest.mark.parametrize("t,name", [(oracle.Q8_0, "q8_0"), (oracle.Q4_K, "q4_k")])
+def test_matmul_q8_equals_rounded_activations_times_decoded_weights(t, name):
+    """The unit formula dx * (s * sum(q qx) - m * sum(qx)) is algebraically the
+    product of the rounded activations with the decoded weights
+    (src/kernels/check.zig:839-871 checks the kernel against exactly that)."""
+    rng = np.random.default_rng(29)
+    rows, n, k = 9, 21, 1024
+    raw = synth.random_blocks(rng, name, n, k)
+    values = oracle.dequantize(t, raw, n * k).reshape(n, k)
+    x = ((rng.random((rows, k), dtype=np.float32) * 2 - 1)).astype(np.float32)
+    block = oracle.act_block(t)
+    q, d = oracle.quantize_q8(x, block)
+    got = oracle.matmul_q8(t, raw, q, d, n)
+    xs = q.astype(np.float64) * np.repeat(d, block, axis=1).astype(np.float64)
+    want = xs @ values.astype(np.float64).T
+    scale = np.max(np.abs(want))
+    # Q4_K's decoded weight d*sc*q - dmin*m is rounded to f32 by the decoder,
+    # the unit formula keeps the two terms apart: they differ by f32 roundings.
+    tol = 1e-12 if t == oracle.Q8_0 else 2e-7
+    assert np.max(np.abs(got - want)) <= tol * scale

@@ -1,0 +1,296 @@
+// matmul_q8_0 / matmul_q4_k: the prefill multiply on activations rounded to
+// 8-bit blocks (quantize_q8), as src/kernels/matmul_quant.wgsl defines it:
+//   out[t][col0 + j] = sum over 32-weight units of dx * (s * sum(q * qx) - m * sum(qx))
+// with every unit's integer sum exact. Here the unit sums run on the int8 matrix
+// cores (v_mfma_i32_16x16x32_i8: one 32-deep unit of 16 tokens x 16 rows per
+// instruction) and the scales are applied to the integer results in f32.
+//
+// A 256-thread workgroup computes 64 tokens x 64 rows; wave w owns rows
+// 16 w .. 16 w + 15 for all 64 tokens (four accumulator tiles). The tokens'
+// bytes are staged through LDS in padded lines (stride = step + 8 bytes, so the
+// sixteen 8-byte fragment reads of a quarter-wave fall in distinct banks); each
+// lane reads its own row's weight bytes and scales straight from memory, one
+// step ahead of their use. Buffers are range-checked: tokens past `rows` and
+// rows past `n` read zeros, and units outside [kb, ke) are skipped, so partial
+// tiles and split-k slices need no special paths. Every output is summed over k
+// in increasing order by a sequence of operations that does not depend on its
+// position in the tile: token chunking cannot change bits.
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "decode.cuh"
+
+namespace zhip {
+
+typedef int i32x4 __attribute__((ext_vector_type(4)));
+typedef float if32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t iu32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t iu32x2 __attribute__((ext_vector_type(2)));
+
+namespace {
+
+constexpr uint32_t TT = 64;   // tokens per workgroup
+constexpr uint32_t TN = 64;   // rows per workgroup
+
+struct I8Args {
+    const uint8_t *qx;   // rows x k int8, four per word
+    const uint8_t *w;    // GPU-layout weight rows
+    const uint8_t *dx;   // rows x k / ACT f32
+    float *out;
+    uint32_t rows, n, k, col0, out_stride, accumulate, k_slice, slice_stride, row_bytes;
+    uint32_t qx_bytes, w_bytes, dx_bytes;
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const uint8_t *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, (int)bytes, 0x00020000);
+}
+
+__device__ __forceinline__ long as_operand(iu32x2 v) {
+    return (long)(((unsigned long)v.y << 32) | (unsigned long)v.x);
+}
+
+// The accumulators' home: lane (l16, g) holds row n0 + 16 wave + l16 for tokens
+// t0 + 16 mt + 4 g + i.
+__device__ __forceinline__ void store_tile(const I8Args &a, const if32x4 (&acc)[4], uint32_t t0, uint32_t j, uint32_t g) {
+    if (j >= a.n) return;
+    float *out = a.out + (size_t)blockIdx.z * a.slice_stride + a.col0 + j;
+#pragma unroll
+    for (uint32_t mt = 0; mt < 4; mt++) {
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) {
+            const uint32_t t = t0 + 16u * mt + 4u * g + i;
+            if (t >= a.rows) continue;
+            float *o = out + (size_t)t * a.out_stride;
+            *o = a.accumulate ? *o + acc[mt][i] : acc[mt][i];
+        }
+    }
+}
+
+// ---- Q8_0 weights (split rows: k bytes, then k / 32 f16 scales), Q8_0 activations ----
+__global__ __launch_bounds__(256) void matmul_q8_0_i8_kernel(I8Args a) {
+    constexpr uint32_t STEP = 128, LINE = STEP + 8;
+    __shared__ __align__(16) uint8_t lds_q[2][TT * LINE];
+    __shared__ __align__(16) float lds_d[2][4][TT];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+    const uint32_t n0 = blockIdx.x * TN, t0 = blockIdx.y * TT;
+    const uint32_t kb = blockIdx.z * a.k_slice, ke = min(a.k, kb + a.k_slice);
+    const uint32_t k_first = kb & ~(STEP - 1u);
+    const uint32_t steps = (ke - k_first + STEP - 1u) / STEP;
+    const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.qx, a.qx_bytes), wbuf = make_buffer(a.w, a.w_bytes), dbuf = make_buffer(a.dx, a.dx_bytes);
+
+    // Staging: two 16-byte chunks of token lines and one block scale per thread.
+    const uint32_t atok = tid >> 3, achunk = tid & 7u;
+    const uint32_t aoff0 = (t0 + atok) * a.k + 16u * achunk, aoff1 = aoff0 + 32u * a.k;
+    const uint32_t dtok = tid & 63u, dunit = tid >> 6;
+    const uint32_t doff = ((t0 + dtok) * (a.k / 32u) + dunit) * 4u;
+    const uint32_t j = n0 + 16u * wave + l16;
+    const uint32_t wq = j * a.row_bytes + 8u * g, ws = j * a.row_bytes + a.k;
+
+    iu32x4 ra0, ra1;
+    uint32_t rd;
+    iu32x2 bq[4], nq[4], bs, ns;
+    auto fetch = [&](uint32_t k0, iu32x2 (&q)[4], iu32x2 &s) __attribute__((always_inline)) {
+        ra0 = __builtin_amdgcn_raw_buffer_load_b128(xbuf, aoff0 + k0, 0, 0);
+        ra1 = __builtin_amdgcn_raw_buffer_load_b128(xbuf, aoff1 + k0, 0, 0);
+        rd = __builtin_amdgcn_raw_buffer_load_b32(dbuf, doff + k0 / 8u, 0, 0);
+#pragma unroll
+        for (uint32_t u = 0; u < 4; u++) q[u] = __builtin_amdgcn_raw_buffer_load_b64(wbuf, wq + k0 + 32u * u, 0, 0);
+        s = __builtin_amdgcn_raw_buffer_load_b64(wbuf, ws + k0 / 16u, 0, 0);
+    };
+    auto stash = [&](uint32_t buf) __attribute__((always_inline)) {
+        uint8_t *line0 = &lds_q[buf][atok * LINE + 16u * achunk];
+        uint8_t *line1 = line0 + 32u * LINE;
+        *reinterpret_cast<iu32x2 *>(line0) = ra0.xy;
+        *reinterpret_cast<iu32x2 *>(line0 + 8) = ra0.zw;
+        *reinterpret_cast<iu32x2 *>(line1) = ra1.xy;
+        *reinterpret_cast<iu32x2 *>(line1 + 8) = ra1.zw;
+        lds_d[buf][dunit][dtok] = __uint_as_float(rd);
+    };
+
+    if32x4 acc[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++) acc[mt] = if32x4{0.f, 0.f, 0.f, 0.f};
+
+    fetch(k_first, bq, bs);
+    stash(0);
+    __syncthreads();
+    for (uint32_t s = 0; s < steps; s++) {
+        const uint32_t k0 = k_first + s * STEP, buf = s & 1u;
+        const bool more = s + 1u < steps;
+        if (more) fetch(k0 + STEP, nq, ns);
+#pragma unroll
+        for (uint32_t u = 0; u < 4; u++) {
+            const uint32_t kpos = k0 + 32u * u;
+            if (kpos < kb || kpos >= ke) continue;
+            const uint32_t sw = u < 2 ? bs.x : bs.y;
+            const float dw = half_bits_to_float(u & 1u ? sw >> 16 : sw & 0xffffu);
+            const long b = as_operand(bq[u]);
+#pragma unroll
+            for (uint32_t mt = 0; mt < 4; mt++) {
+                const long af = *reinterpret_cast<const long *>(&lds_q[buf][(16u * mt + l16) * LINE + 32u * u + 8u * g]);
+                const i32x4 is = __builtin_amdgcn_mfma_i32_16x16x32_i8(af, b, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                const if32x4 dxv = *reinterpret_cast<const if32x4 *>(&lds_d[buf][u][16u * mt + 4u * g]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) acc[mt][i] = fmaf(dxv[i], dw * (float)is[i], acc[mt][i]);
+            }
+        }
+        if (more) {
+            stash(buf ^ 1u);
+#pragma unroll
+            for (int u = 0; u < 4; u++) bq[u] = nq[u];
+            bs = ns;
+        }
+        __syncthreads();
+    }
+    store_tile(a, acc, t0, j, g);
+}
+
+// ---- Q4_K weights (144-byte super-blocks as in the file), Q8_K activations ----------
+__global__ __launch_bounds__(256) void matmul_q4_k_i8_kernel(I8Args a) {
+    constexpr uint32_t STEP = 256, LINE = STEP + 8;
+    __shared__ __align__(16) uint8_t lds_q[2][TT * LINE];
+    __shared__ __align__(16) float lds_d[2][TT];      // the tokens' block scales
+    __shared__ __align__(16) float lds_s[2][8][TT];   // sum of each sub-block's bytes
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+    const uint32_t n0 = blockIdx.x * TN, t0 = blockIdx.y * TT;
+    const uint32_t kb = blockIdx.z * a.k_slice, ke = min(a.k, kb + a.k_slice);
+    const uint32_t k_first = kb & ~(STEP - 1u);
+    const uint32_t steps = (ke - k_first + STEP - 1u) / STEP;
+    const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.qx, a.qx_bytes), wbuf = make_buffer(a.w, a.w_bytes), dbuf = make_buffer(a.dx, a.dx_bytes);
+
+    // Staging: a quarter (two sub-blocks) of one token's super-block per thread.
+    const uint32_t atok = tid >> 2, aq = tid & 3u;
+    const uint32_t aoff = (t0 + atok) * a.k + 64u * aq;
+    const uint32_t doff = (t0 + atok) * (a.k / 256u) * 4u;
+    const uint32_t j = n0 + 16u * wave + l16;
+    const uint32_t wrow = j * a.row_bytes;
+
+    iu32x4 ra[4];
+    uint32_t rd;
+    iu32x4 bh, nh;       // d, dmin and the twelve scale bytes
+    iu32x2 bq[4], nq[4];  // 8 bytes of each 64-weight chunk: low nibbles sub-block 2c, high 2c + 1
+    auto fetch = [&](uint32_t k0, iu32x4 &h, iu32x2 (&q)[4]) __attribute__((always_inline)) {
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) ra[i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, aoff + k0 + 16u * i, 0, 0);
+        rd = __builtin_amdgcn_raw_buffer_load_b32(dbuf, doff + k0 / 64u, 0, 0);
+        const uint32_t blk = wrow + k0 / 256u * 144u;
+        h = __builtin_amdgcn_raw_buffer_load_b128(wbuf, blk, 0, 0);
+#pragma unroll
+        for (uint32_t c = 0; c < 4; c++) q[c] = __builtin_amdgcn_raw_buffer_load_b64(wbuf, blk + 16u + 32u * c + 8u * g, 0, 0);
+    };
+    auto stash = [&](uint32_t buf) __attribute__((always_inline)) {
+        uint8_t *line = &lds_q[buf][atok * LINE + 64u * aq];
+        int sums[2] = {0, 0};
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) {
+            *reinterpret_cast<iu32x2 *>(line + 16u * i) = ra[i].xy;
+            *reinterpret_cast<iu32x2 *>(line + 16u * i + 8u) = ra[i].zw;
+#pragma unroll
+            for (uint32_t e = 0; e < 4; e++) sums[i >> 1] = __builtin_amdgcn_sdot4((int)ra[i][e], 0x01010101, sums[i >> 1], false);
+        }
+        lds_s[buf][2u * aq][atok] = (float)sums[0];
+        lds_s[buf][2u * aq + 1u][atok] = (float)sums[1];
+        if (aq == 0u) lds_d[buf][atok] = __uint_as_float(rd);
+    };
+
+    if32x4 acc[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++) acc[mt] = if32x4{0.f, 0.f, 0.f, 0.f};
+
+    fetch(k_first, bh, bq);
+    stash(0);
+    __syncthreads();
+    for (uint32_t s = 0; s < steps; s++) {
+        const uint32_t k0 = k_first + s * STEP, buf = s & 1u;
+        const bool more = s + 1u < steps;
+        if (more) fetch(k0 + STEP, nh, nq);
+        const float d = half_bits_to_float(bh.x & 0xffffu), dmin = half_bits_to_float(bh.x >> 16);
+        if32x4 part[4];
+#pragma unroll
+        for (int mt = 0; mt < 4; mt++) part[mt] = if32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (uint32_t sb = 0; sb < 8; sb++) {
+            const uint32_t kpos = k0 + 32u * sb;
+            if (kpos < kb || kpos >= ke) continue;
+            const uint2 sm = scale_min_k4(bh.y, bh.z, bh.w, sb);
+            const float dsc = d * (float)sm.x, dmn = dmin * (float)sm.y;
+            iu32x2 nib = bq[sb >> 1];
+            if (sb & 1u) nib = nib >> 4;
+            nib = nib & 0x0f0f0f0fu;
+            const long b = as_operand(nib);
+#pragma unroll
+            for (uint32_t mt = 0; mt < 4; mt++) {
+                const long af = *reinterpret_cast<const long *>(&lds_q[buf][(16u * mt + l16) * LINE + 32u * sb + 8u * g]);
+                const i32x4 is = __builtin_amdgcn_mfma_i32_16x16x32_i8(af, b, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                const if32x4 xs = *reinterpret_cast<const if32x4 *>(&lds_s[buf][sb][16u * mt + 4u * g]);
+#pragma unroll
+                for (int i = 0; i < 4; i++) part[mt][i] = fmaf(-dmn, xs[i], fmaf(dsc, (float)is[i], part[mt][i]));
+            }
+        }
+#pragma unroll
+        for (uint32_t mt = 0; mt < 4; mt++) {
+            const if32x4 dxv = *reinterpret_cast<const if32x4 *>(&lds_d[buf][16u * mt + 4u * g]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[mt][i] = fmaf(dxv[i], part[mt][i], acc[mt][i]);
+        }
+        if (more) {
+            stash(buf ^ 1u);
+            bh = nh;
+#pragma unroll
+            for (int c = 0; c < 4; c++) bq[c] = nq[c];
+        }
+        __syncthreads();
+    }
+    store_tile(a, acc, t0, j, g);
+}
+
+}  // namespace
+
+// matmul_quant.wgsl's workgroup is 128 outputs x 32 tokens: the grid says how
+// much of the product a dispatch covers, whatever tiling computes it.
+static zhip_result launch_int8(const Dispatch &d, const char *name, bool q4k) {
+    if (d.params_size < sizeof(MatmulParams)) return fail(d, ZHIP_E_BAD_COMMAND, "%s: params block too small", name);
+    const MatmulParams &p = *reinterpret_cast<const MatmulParams *>(d.params);
+    for (int b = 1; b <= 4; b++)
+        if (!d.bind[b].bound) return fail(d, ZHIP_E_BAD_COMMAND, "%s: binding %d is not bound", name, b);
+    if (d.grid[0] == 0 || d.grid[1] == 0 || d.grid[2] == 0) return ZHIP_OK;
+    const uint32_t act = q4k ? 256u : 32u;
+    if (p.k == 0 || p.k % act != 0) return fail(d, ZHIP_E_BAD_COMMAND, "%s: k = %u is not a multiple of %u", name, p.k, act);
+    if (p.k_slice == 0 || p.k_slice % 32u != 0) return fail(d, ZHIP_E_BAD_COMMAND, "%s: k_slice = %u", name, p.k_slice);
+    const uint64_t slices = d.grid[2];
+    if ((slices - 1) * p.k_slice >= p.k) return fail(d, ZHIP_E_BAD_COMMAND, "%s: %u slices of %u exceed k = %u", name, (uint32_t)slices, p.k_slice, p.k);
+    const uint64_t cover_n = (uint64_t)d.grid[0] * 128u, cover_t = (uint64_t)d.grid[1] * 32u;
+    const uint64_t n = cover_n < p.n ? cover_n : p.n, rows = cover_t < p.rows ? cover_t : p.rows;
+    if (n == 0 || rows == 0) return ZHIP_OK;
+    const uint64_t row_bytes = q4k ? (uint64_t)p.k / 256u * 144u : (((uint64_t)p.k + p.k / 16u + 15u) & ~15ull);
+    const uint64_t x_need = rows * p.k, d_need = rows * (p.k / act) * 4u, w_need = n * row_bytes;
+    const uint64_t o_need = ((slices - 1) * p.slice_stride + (rows - 1) * p.out_stride + p.col0 + n) * 4u;
+    if (x_need > d.bind[1].size || w_need > d.bind[2].size || o_need > d.bind[3].size || d_need > d.bind[4].size)
+        return fail(d, ZHIP_E_BAD_COMMAND, "%s: bound ranges too small (qx %llu/%llu, w %llu/%llu, out %llu/%llu, dx %llu/%llu)", name,
+            (unsigned long long)x_need, (unsigned long long)d.bind[1].size, (unsigned long long)w_need, (unsigned long long)d.bind[2].size,
+            (unsigned long long)o_need, (unsigned long long)d.bind[3].size, (unsigned long long)d_need, (unsigned long long)d.bind[4].size);
+    if (((uintptr_t)d.bind[1].ptr | (uintptr_t)d.bind[2].ptr) & 15u) return fail(d, ZHIP_E_BAD_COMMAND, "%s: qx and weights must be 16-byte aligned", name);
+    if (((uintptr_t)d.bind[3].ptr | (uintptr_t)d.bind[4].ptr) & 3u) return fail(d, ZHIP_E_BAD_COMMAND, "%s: out and dx must be 4-byte aligned", name);
+    // The kernels index with 32-bit byte offsets, up to a tile past the last token and row.
+    if ((rows + 2u * TT) * p.k >= (1ull << 32) || (n + 2u * TN) * row_bytes >= (1ull << 32))
+        return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
+    const uint64_t tiles_n = (n + TN - 1) / TN, tiles_t = (rows + TT - 1) / TT;
+    if (tiles_t > 65535u || slices > 65535u) return fail(d, ZHIP_E_BAD_COMMAND, "%s: grid too large", name);
+    I8Args a{};
+    a.qx = d.bind[1].ptr;
+    a.w = d.bind[2].ptr;
+    a.out = reinterpret_cast<float *>(d.bind[3].ptr);
+    a.dx = d.bind[4].ptr;
+    a.rows = (uint32_t)rows; a.n = (uint32_t)n; a.k = p.k; a.col0 = p.col0; a.out_stride = p.out_stride;
+    a.accumulate = p.accumulate; a.k_slice = p.k_slice; a.slice_stride = p.slice_stride; a.row_bytes = (uint32_t)row_bytes;
+    a.qx_bytes = (uint32_t)x_need; a.w_bytes = (uint32_t)w_need; a.dx_bytes = (uint32_t)d_need;
+    const dim3 grid((uint32_t)tiles_n, (uint32_t)tiles_t, (uint32_t)slices);
+    if (q4k) hipLaunchKernelGGL(matmul_q4_k_i8_kernel, grid, dim3(256), 0, d.stream, a);
+    else hipLaunchKernelGGL(matmul_q8_0_i8_kernel, grid, dim3(256), 0, d.stream, a);
+    return check_launch(d, name);
+}
+
+zhip_result launch_matmul_q8_0(const Dispatch &d) { return launch_int8(d, "matmul_q8_0", false); }
+zhip_result launch_matmul_q4_k(const Dispatch &d) { return launch_int8(d, "matmul_q4_k", true); }
+
+}  // namespace zhip

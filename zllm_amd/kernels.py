@@ -72,6 +72,9 @@ CONTRACTS = {
     Kernel.matvec_bf16: Contract(5, 0b01000),
     Kernel.matmul_bf16: Contract(4, 0b1000),
     Kernel.matmul_q8_0_float: Contract(4, 0b1000),
+    Kernel.matmul_q8_0: Contract(5, 0b01000),
+    Kernel.matmul_q4_k: Contract(5, 0b01000),
+    Kernel.quantize_q8: Contract(5, 0b01100),
     Kernel.matmul_reduce: Contract(3, 0b100),
     Kernel.silu_mul: Contract(3, 0b100),
     Kernel.repack_q8_0: Contract(3, 0b100),
@@ -119,6 +122,12 @@ def row_bytes(t: TensorType, k: int) -> int:
 def needs_layout(t: TensorType) -> bool:
     """src/kernels/kernels.zig:164-166."""
     return t == TensorType.q8_0 or block_stride(t) != LAYOUT[t][1]
+
+
+def act_block(t: TensorType) -> int:
+    """Activations per rounding block of the int8 prefill multiply for weights
+    of type t (src/kernels/kernels.zig:301-303)."""
+    return 32 if t == TensorType.q8_0 else 256
 
 
 def is_half(t: TensorType) -> bool:
@@ -242,6 +251,17 @@ class params:
 
         def pack(self) -> bytes:
             return struct.pack("<8I", self.rows, self.n, self.k, self.col0, self.out_stride, self.accumulate, self.k_slice, self.slice_stride)
+
+    @dataclass
+    class QuantizeQ8:
+        """src/kernels/kernels.zig:495-501. mode: 0 x, 1 RMSNorm(x) * w, 2 silu(gate) * up."""
+        k: int
+        block: int
+        mode: int = 0
+        eps: float = 0.0
+
+        def pack(self) -> bytes:
+            return struct.pack("<3If", self.k, self.block, self.mode, self.eps)
 
     @dataclass
     class MatmulReduce:
