@@ -22,6 +22,11 @@ HIPCC_FLAGS = [
     "-Wall", "-Wno-unused-function", "-Wno-unknown-warning-option",
 ]
 
+# Per-file additions. The int8 multiply reads every matrix-core result at once
+# (to scale it): with the results in ordinary VGPRs there is no copy out of the
+# accumulator file in between.
+EXTRA_FLAGS = {"matmul_int8.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form"]}
+
 
 def source_hash() -> str:
     h = hashlib.sha256()
@@ -40,7 +45,7 @@ def build(verbose: bool = False) -> str:
     for name in SOURCES:
         src = os.path.join(CSRC, name)
         obj = os.path.join(CSRC, os.path.splitext(name)[0] + ".o")
-        cmd = [hipcc, *HIPCC_FLAGS, f'-DZHIP_SOURCE_HASH="{digest}"', "-c", src, "-o", obj]
+        cmd = [hipcc, *HIPCC_FLAGS, *EXTRA_FLAGS.get(name, []), f'-DZHIP_SOURCE_HASH="{digest}"', "-c", src, "-o", obj]
         if name.endswith(".cpp"):
             cmd[1:1] = ["-x", "hip"]
         procs.append((name, subprocess.Popen(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)))

@@ -2,19 +2,17 @@
 // 8-bit blocks (quantize_q8), as src/kernels/matmul_quant.wgsl defines it:
 //   out[t][col0 + j] = sum over 32-weight units of dx * (s * sum(q * qx) - m * sum(qx))
 // with every unit's integer sum exact. Here the unit sums run on the int8 matrix
-// cores (v_mfma_i32_16x16x32_i8: one 32-deep unit of 16 tokens x 16 rows per
-// instruction) and the scales are applied to the integer results in f32.
+// cores (v_mfma_i32_16x16x32_i8: one 32-deep unit of 16 x 16 outputs per
+// instruction) and the scales are applied to the integer results in f32, which
+// is what bounds these kernels: three vector operations per output and unit.
 //
-// A 256-thread workgroup computes 64 tokens x 64 rows; wave w owns rows
-// 16 w .. 16 w + 15 for all 64 tokens (four accumulator tiles). The tokens'
-// bytes are staged through LDS in padded lines (stride = step + 8 bytes, so the
-// sixteen 8-byte fragment reads of a quarter-wave fall in distinct banks); each
-// lane reads its own row's weight bytes and scales straight from memory, one
-// step ahead of their use. Buffers are range-checked: tokens past `rows` and
-// rows past `n` read zeros, and units outside [kb, ke) are skipped, so partial
-// tiles and split-k slices need no special paths. Every output is summed over k
-// in increasing order by a sequence of operations that does not depend on its
-// position in the tile: token chunking cannot change bits.
+// A 256-thread workgroup computes 64 tokens x 64 rows in steps of 256 positions;
+// wave w owns rows 16 w .. 16 w + 15 for all 64 tokens (four accumulator tiles).
+// Buffers are range-checked: tokens past `rows` and rows past `n` read zeros,
+// and units outside [kb, ke) contribute nothing, so partial tiles and split-k
+// slices need no special paths. Every output is summed over k in increasing
+// order by a sequence of operations that does not depend on its position in
+// the tile: token chunking cannot change bits.
 #include <hip/hip_runtime.h>
 
 #include "common.h"
@@ -29,8 +27,10 @@ typedef uint32_t iu32x2 __attribute__((ext_vector_type(2)));
 
 namespace {
 
-constexpr uint32_t TT = 64;   // tokens per workgroup
-constexpr uint32_t TN = 64;   // rows per workgroup
+constexpr uint32_t TT = 64;     // tokens per workgroup
+constexpr uint32_t TN = 64;     // rows per workgroup
+constexpr uint32_t STEP = 256;  // positions per step
+constexpr uint32_t LINE = STEP + 8;  // bytes between register-staged token lines in LDS
 
 struct I8Args {
     const uint8_t *qx;   // rows x k int8, four per word
@@ -45,8 +45,175 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const uint8_t *bas
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, (int)bytes, 0x00020000);
 }
 
+typedef __attribute__((address_space(3))) void *lds_ptr;
+
+// One wave-wide load straight into LDS: lane l's 4 (16) bytes land at
+// dst + 4 l (16 l), whatever global offset the lane asked for. The destination
+// reaches the load as a bare LDS address: the compiler then keeps no dependency
+// between these loads and later LDS reads (it would wait for every outstanding
+// load before each read); sync_after_loads() orders them.
+__device__ __forceinline__ void load_lds_b32(__amdgpu_buffer_rsrc_t buf, uint8_t *dst, uint32_t offset) {
+    uint32_t address = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);  // the same for all lanes
+    asm volatile("" : "+s"(address));
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)(uintptr_t)address, 4, offset, 0, 0, 0);
+}
+__device__ __forceinline__ void load_lds_b128(__amdgpu_buffer_rsrc_t buf, uint8_t *dst, uint32_t offset) {
+    uint32_t address = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);
+    asm volatile("" : "+s"(address));
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)(uintptr_t)address, 16, offset, 0, 0, 0);
+}
+
+// Every load of this wave has landed, every wave's LDS traffic is done: the
+// buffer just filled may be read, the one just read may be filled.
+__device__ __forceinline__ void sync_after_loads() {
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 __device__ __forceinline__ long as_operand(iu32x2 v) {
     return (long)(((unsigned long)v.y << 32) | (unsigned long)v.x);
+}
+
+// ---- Q8_0 weights (split rows: k bytes, then k / 32 f16 scales), Q8_0 activations ----
+// The accumulators: lane (l16, g) holds token t0 + 16 mt + l16 for rows
+// n0 + 16 wave + 4 g + i (weights are the matrix cores' first operand), so a
+// lane scales its four results of a product by four row scales and one token
+// scale.
+//
+// Both operands cross LDS. Read straight into the operand layout, adjacent
+// lanes would ask for different rows, and the load unit takes such a load apart
+// one lane a clock; here a wave brings sixteen rows and sixteen token lines in
+// as whole 256-byte runs (buffer_load ... lds, 16 bytes a lane, four lines an
+// instruction) and reads its operands back, 8 bytes a lane. The 16-byte chunks
+// of a weight row are stored permuted (chunk c of row r at position c ^ r),
+// which spreads the sixteen rows of an operand read over all banks two deep,
+// the best 16-byte granularity allows. Two buffers: a step's loads are issued
+// before the previous step's multiply and waited for after it.
+
+// Token lines, which every wave reads four times as often as its weights, get
+// a layout without bank conflicts: each instruction's four lines (1 KiB) are
+// followed by XPAD = 8 bytes, and chunk c of token t sits at position
+// c ^ 2 (t % 4). The sixteen tokens of an operand read then start at sixteen
+// different 8-byte bank pairs: 4 (c / 2 ^ t % 4) + 2 (c % 2) + half + t / 4.
+constexpr uint32_t XPAD = 8;
+__device__ __forceinline__ uint32_t xkey(uint32_t token) { return 2u * (token & 3u); }
+
+template <bool RAGGED>
+__global__ __launch_bounds__(256, 2) void matmul_q8_0_i8_kernel(I8Args a) {
+    constexpr uint32_t DBUF = TT * 32u;          // [token][8 units] f32
+    constexpr uint32_t WBUF = TN * STEP;         // [row][256 bytes], chunks permuted
+    constexpr uint32_t SBUF = TN * 16u;          // [row][8 units] f16
+    constexpr uint32_t XBUF = TT * STEP + TT / 4u * XPAD;  // [token][256 bytes], chunks permuted, XPAD bytes after every four tokens
+    __shared__ __align__(16) uint8_t lds_q[2][XBUF];
+    __shared__ __align__(16) uint8_t lds_d[2][DBUF];
+    __shared__ __align__(16) uint8_t lds_w[2][WBUF];
+    __shared__ __align__(16) uint8_t lds_s[2][SBUF];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+    const uint32_t n0 = blockIdx.x * TN, t0 = blockIdx.y * TT;
+    const uint32_t kb = blockIdx.z * a.k_slice, ke = min(a.k, kb + a.k_slice);
+    const uint32_t k_first = kb & ~(STEP - 1u);
+    const uint32_t steps = (ke - k_first + STEP - 1u) / STEP;
+    const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.qx, a.qx_bytes), wbuf = make_buffer(a.w, a.w_bytes), dbuf = make_buffer(a.dx, a.dx_bytes);
+
+    // Weight loads: instruction i takes rows r = 4 i + lane / 16 of the wave's
+    // sixteen; the lane at position p = lane % 16 fetches chunk p ^ r, the one
+    // that belongs there.
+    const uint32_t wl_row = lane >> 4, wl_pos = lane & 15u;
+    const uint32_t woff = (n0 + 16u * wave + wl_row) * a.row_bytes;
+    // Token loads, the same way: instruction i takes tokens 16 wave + 4 i + lane / 16.
+    const uint32_t xoff = (t0 + 16u * wave + wl_row) * a.k;
+    // Scales: one word a lane, row 16 wave + lane / 4, units 2 (lane % 4), + 1.
+    const uint32_t soff = (n0 + 16u * wave + (lane >> 2)) * a.row_bytes + a.k + 4u * (lane & 3u);
+    // Block scales of tokens 16 wave + 8 i + lane / 8, unit lane % 8.
+    const uint32_t doff = ((t0 + 16u * wave + (lane >> 3)) * (a.k / 32u) + (lane & 7u)) * 4u;
+
+    auto fetch = [&](uint32_t k0, uint32_t buf) __attribute__((always_inline)) {
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++)
+            load_lds_b128(wbuf, lds_w[buf] + (16u * wave + 4u * i) * STEP, woff + 4u * i * a.row_bytes + k0 + 16u * (wl_pos ^ (4u * i | wl_row)));
+        load_lds_b32(wbuf, lds_s[buf] + 16u * wave * 16u, soff + k0 / 16u);
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++)
+            load_lds_b128(xbuf, lds_q[buf] + (4u * wave + i) * (4u * STEP + XPAD), xoff + 4u * i * a.k + k0 + 16u * (wl_pos ^ xkey(4u * i | wl_row)));
+#pragma unroll
+        for (uint32_t i = 0; i < 2; i++)
+            load_lds_b32(dbuf, lds_d[buf] + (16u * wave + 8u * i) * 32u, doff + 8u * i * (a.k / 32u) * 4u + k0 / 8u);
+    };
+
+    if32x4 acc[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; mt++) acc[mt] = if32x4{0.f, 0.f, 0.f, 0.f};
+
+    // One unit's integer sums for the four token tiles, and the tokens' block scales.
+    struct Unit {
+        i32x4 is[4];
+        float dx[4];
+    };
+    // This lane's operand bytes of unit u: row 16 wave + l16, logical chunk
+    // 2 u + g / 2, half g % 2.
+    const uint32_t wkey = l16;  // (16 wave + l16) & 15
+    auto multiply = [&](uint32_t buf, uint32_t u, Unit &r) __attribute__((always_inline)) {
+        const uint32_t chunk = (2u * u + (g >> 1)) ^ wkey;
+        const long wf = *reinterpret_cast<const long *>(&lds_w[buf][(16u * wave + l16) * STEP + 16u * chunk + 8u * (g & 1u)]);
+#pragma unroll
+        for (uint32_t mt = 0; mt < 4; mt++) {
+            const uint32_t xchunk = (2u * u + (g >> 1)) ^ xkey(l16);
+            const long xf = *reinterpret_cast<const long *>(&lds_q[buf][(4u * mt + (l16 >> 2)) * (4u * STEP + XPAD) + (l16 & 3u) * STEP + 16u * xchunk + 8u * (g & 1u)]);
+            r.is[mt] = __builtin_amdgcn_mfma_i32_16x16x32_i8(wf, xf, i32x4{0, 0, 0, 0}, 0, 0, 0);
+            r.dx[mt] = *reinterpret_cast<const float *>(lds_d[buf] + (16u * mt + l16) * 32u + 4u * u);
+        }
+    };
+    auto scale = [&](uint32_t k0, const iu32x4 (&sc)[4], uint32_t u, const Unit &r) __attribute__((always_inline)) {
+        // A unit outside [kb, ke) multiplied whatever bytes lie there: zero its scale.
+        const uint32_t kpos = k0 + 32u * u;
+        const bool live = !RAGGED || (kpos >= kb && kpos < ke);
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) {
+            const uint32_t word = sc[i][u >> 1];
+            const float dw = live ? half_bits_to_float(u & 1u ? word >> 16 : word & 0xffffu) : 0.f;
+#pragma unroll
+            for (uint32_t mt = 0; mt < 4; mt++) acc[mt][i] = fmaf(r.dx[mt], dw * (float)r.is[mt][i], acc[mt][i]);
+        }
+    };
+    // The matrix cores work on unit u + 1 while the vector units scale unit u.
+    auto compute = [&](uint32_t k0, uint32_t buf) __attribute__((always_inline)) {
+        iu32x4 sc[4];  // rows 4 g + i: eight f16 scales
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) sc[i] = *reinterpret_cast<const iu32x4 *>(lds_s[buf] + (16u * wave + 4u * g + i) * 16u);
+        Unit even, odd;
+        multiply(buf, 0, even);
+#pragma unroll
+        for (uint32_t u = 0; u < 8; u += 2) {
+            multiply(buf, u + 1u, odd);
+            scale(k0, sc, u, even);
+            __builtin_amdgcn_sched_barrier(0);
+            if (u + 2u < 8u) multiply(buf, u + 2u, even);
+            scale(k0, sc, u + 1u, odd);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+
+    fetch(k_first, 0);
+    sync_after_loads();
+    for (uint32_t s = 0; s < steps; s++) {
+        const uint32_t k0 = k_first + s * STEP;
+        fetch(k0 + STEP, (s + 1u) & 1u);
+        compute(k0, s & 1u);
+        sync_after_loads();
+    }
+
+    const uint32_t j = n0 + 16u * wave + 4u * g;
+    float *out = a.out + (size_t)blockIdx.z * a.slice_stride + a.col0 + j;
+#pragma unroll
+    for (uint32_t mt = 0; mt < 4; mt++) {
+        const uint32_t t = t0 + 16u * mt + l16;
+        if (t >= a.rows) continue;
+        float *o = out + (size_t)t * a.out_stride;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++)
+            if (j + i < a.n) o[i] = a.accumulate ? o[i] + acc[mt][i] : acc[mt][i];
+    }
 }
 
 // The accumulators' home: lane (l16, g) holds row n0 + 16 wave + l16 for tokens
@@ -66,89 +233,9 @@ __device__ __forceinline__ void store_tile(const I8Args &a, const if32x4 (&acc)[
     }
 }
 
-// ---- Q8_0 weights (split rows: k bytes, then k / 32 f16 scales), Q8_0 activations ----
-__global__ __launch_bounds__(256) void matmul_q8_0_i8_kernel(I8Args a) {
-    constexpr uint32_t STEP = 128, LINE = STEP + 8;
-    __shared__ __align__(16) uint8_t lds_q[2][TT * LINE];
-    __shared__ __align__(16) float lds_d[2][4][TT];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
-    const uint32_t n0 = blockIdx.x * TN, t0 = blockIdx.y * TT;
-    const uint32_t kb = blockIdx.z * a.k_slice, ke = min(a.k, kb + a.k_slice);
-    const uint32_t k_first = kb & ~(STEP - 1u);
-    const uint32_t steps = (ke - k_first + STEP - 1u) / STEP;
-    const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.qx, a.qx_bytes), wbuf = make_buffer(a.w, a.w_bytes), dbuf = make_buffer(a.dx, a.dx_bytes);
-
-    // Staging: two 16-byte chunks of token lines and one block scale per thread.
-    const uint32_t atok = tid >> 3, achunk = tid & 7u;
-    const uint32_t aoff0 = (t0 + atok) * a.k + 16u * achunk, aoff1 = aoff0 + 32u * a.k;
-    const uint32_t dtok = tid & 63u, dunit = tid >> 6;
-    const uint32_t doff = ((t0 + dtok) * (a.k / 32u) + dunit) * 4u;
-    const uint32_t j = n0 + 16u * wave + l16;
-    const uint32_t wq = j * a.row_bytes + 8u * g, ws = j * a.row_bytes + a.k;
-
-    iu32x4 ra0, ra1;
-    uint32_t rd;
-    iu32x2 bq[4], nq[4], bs, ns;
-    auto fetch = [&](uint32_t k0, iu32x2 (&q)[4], iu32x2 &s) __attribute__((always_inline)) {
-        ra0 = __builtin_amdgcn_raw_buffer_load_b128(xbuf, aoff0 + k0, 0, 0);
-        ra1 = __builtin_amdgcn_raw_buffer_load_b128(xbuf, aoff1 + k0, 0, 0);
-        rd = __builtin_amdgcn_raw_buffer_load_b32(dbuf, doff + k0 / 8u, 0, 0);
-#pragma unroll
-        for (uint32_t u = 0; u < 4; u++) q[u] = __builtin_amdgcn_raw_buffer_load_b64(wbuf, wq + k0 + 32u * u, 0, 0);
-        s = __builtin_amdgcn_raw_buffer_load_b64(wbuf, ws + k0 / 16u, 0, 0);
-    };
-    auto stash = [&](uint32_t buf) __attribute__((always_inline)) {
-        uint8_t *line0 = &lds_q[buf][atok * LINE + 16u * achunk];
-        uint8_t *line1 = line0 + 32u * LINE;
-        *reinterpret_cast<iu32x2 *>(line0) = ra0.xy;
-        *reinterpret_cast<iu32x2 *>(line0 + 8) = ra0.zw;
-        *reinterpret_cast<iu32x2 *>(line1) = ra1.xy;
-        *reinterpret_cast<iu32x2 *>(line1 + 8) = ra1.zw;
-        lds_d[buf][dunit][dtok] = __uint_as_float(rd);
-    };
-
-    if32x4 acc[4];
-#pragma unroll
-    for (int mt = 0; mt < 4; mt++) acc[mt] = if32x4{0.f, 0.f, 0.f, 0.f};
-
-    fetch(k_first, bq, bs);
-    stash(0);
-    __syncthreads();
-    for (uint32_t s = 0; s < steps; s++) {
-        const uint32_t k0 = k_first + s * STEP, buf = s & 1u;
-        const bool more = s + 1u < steps;
-        if (more) fetch(k0 + STEP, nq, ns);
-#pragma unroll
-        for (uint32_t u = 0; u < 4; u++) {
-            const uint32_t kpos = k0 + 32u * u;
-            if (kpos < kb || kpos >= ke) continue;
-            const uint32_t sw = u < 2 ? bs.x : bs.y;
-            const float dw = half_bits_to_float(u & 1u ? sw >> 16 : sw & 0xffffu);
-            const long b = as_operand(bq[u]);
-#pragma unroll
-            for (uint32_t mt = 0; mt < 4; mt++) {
-                const long af = *reinterpret_cast<const long *>(&lds_q[buf][(16u * mt + l16) * LINE + 32u * u + 8u * g]);
-                const i32x4 is = __builtin_amdgcn_mfma_i32_16x16x32_i8(af, b, i32x4{0, 0, 0, 0}, 0, 0, 0);
-                const if32x4 dxv = *reinterpret_cast<const if32x4 *>(&lds_d[buf][u][16u * mt + 4u * g]);
-#pragma unroll
-                for (int i = 0; i < 4; i++) acc[mt][i] = fmaf(dxv[i], dw * (float)is[i], acc[mt][i]);
-            }
-        }
-        if (more) {
-            stash(buf ^ 1u);
-#pragma unroll
-            for (int u = 0; u < 4; u++) bq[u] = nq[u];
-            bs = ns;
-        }
-        __syncthreads();
-    }
-    store_tile(a, acc, t0, j, g);
-}
-
 // ---- Q4_K weights (144-byte super-blocks as in the file), Q8_K activations ----------
 __global__ __launch_bounds__(256) void matmul_q4_k_i8_kernel(I8Args a) {
-    constexpr uint32_t STEP = 256, LINE = STEP + 8;
-    __shared__ __align__(16) uint8_t lds_q[2][TT * LINE];
+        __shared__ __align__(16) uint8_t lds_q[2][TT * LINE];
     __shared__ __align__(16) float lds_d[2][TT];      // the tokens' block scales
     __shared__ __align__(16) float lds_s[2][8][TT];   // sum of each sub-block's bytes
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
@@ -285,8 +372,13 @@ static zhip_result launch_int8(const Dispatch &d, const char *name, bool q4k) {
     a.accumulate = p.accumulate; a.k_slice = p.k_slice; a.slice_stride = p.slice_stride; a.row_bytes = (uint32_t)row_bytes;
     a.qx_bytes = (uint32_t)x_need; a.w_bytes = (uint32_t)w_need; a.dx_bytes = (uint32_t)d_need;
     const dim3 grid((uint32_t)tiles_n, (uint32_t)tiles_t, (uint32_t)slices);
-    if (q4k) hipLaunchKernelGGL(matmul_q4_k_i8_kernel, grid, dim3(256), 0, d.stream, a);
-    else hipLaunchKernelGGL(matmul_q8_0_i8_kernel, grid, dim3(256), 0, d.stream, a);
+    const bool ragged = p.k % STEP != 0 || (slices > 1 && p.k_slice % STEP != 0);
+    if (q4k) {
+        hipLaunchKernelGGL(matmul_q4_k_i8_kernel, grid, dim3(256), 0, d.stream, a);
+    } else {
+        if (ragged) hipLaunchKernelGGL(matmul_q8_0_i8_kernel<true>, grid, dim3(256), 0, d.stream, a);
+        else hipLaunchKernelGGL(matmul_q8_0_i8_kernel<false>, grid, dim3(256), 0, d.stream, a);
+    }
     return check_launch(d, name);
 }
 
