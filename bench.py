@@ -33,6 +33,7 @@ sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
 MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
+MFMA_INT8_PEAK_TOPS = 5000.0    # MI355X dense int8, published
 ROTATE_BYTES = 640 << 20    # distinct weight bytes a rotation must exceed (L2 + Infinity Cache, with margin)
 # HBM bytes one launch of the headline kernel moves, from rocprofv3 FETCH_SIZE and
 # WRITE_SIZE counter runs scaled by a plain copy of known size (profiles/matvec_q4k_kernel_c2.txt).
@@ -44,7 +45,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c5 for the 'also' section; 'none' skips it")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,c5 for the 'also' section; 'none' skips it")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run 4 plain elementwise copies (256 MiB read + 256 MiB written each) so a counter run has a kernel of known traffic to scale by")
@@ -104,9 +105,10 @@ def main() -> int:
         flush()
         return dst.view(dtype)
 
-    def timed(launches, steps: int, warmup: int):
-        """Runs `warmup` then `steps` dispatches cycling over `launches`; returns
-        (wall seconds, GPU seconds from the host's stream events)."""
+    def timed(launches, steps: int, warmup: int, per_step: int = 1):
+        """Runs `warmup` then `steps` steps cycling over `launches` (each records
+        `per_step` dispatches); returns (wall seconds, GPU seconds from the
+        host's stream events)."""
         for n, is_timed in ((warmup, False), (steps, True)):
             if n == 0:
                 continue
@@ -121,7 +123,7 @@ def main() -> int:
             wall = time.perf_counter() - t0
             rec.clear()
             ns, count = host.last_submit()
-            assert count == n
+            assert count == n * per_step
         return wall, ns * 1e-9
 
     class L:
@@ -132,6 +134,16 @@ def main() -> int:
 
         def record(self, r, e):
             self.launch.record(r, e)
+
+    class Chain:
+        """Several prebuilt launches recorded as one step."""
+
+        def __init__(self, launches, rows):
+            self.launches, self.rows = launches, rows
+
+        def record(self, r, e):
+            for l in self.launches:
+                l.record(r, e)
 
     b = K.Builder(rec, kset)
 
@@ -261,7 +273,7 @@ def main() -> int:
     only = [s for s in args.only.split(",") if s]
     also = {}
     if "none" not in only:
-        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c5", bench_c5)):
+        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c4_int8", bench_c4_int8), ("c5", bench_c5)):
             if not only or name in only:
                 try:
                     also[name] = fn(locals())
@@ -356,6 +368,49 @@ def bench_c4(env):
         "TFLOPs_gpu": round(flops * steps / gpu_s / 1e12, 1),
         "mfma_frac": round(flops * steps / gpu_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "max_err_over_row_x_norms": bound,
+        "max_err_over_max_want": float(np.max(np.abs(got - want)) / np.max(np.abs(want))),
+    }
+
+
+def bench_c4_int8(env):
+    """The same product as C4 the way the reference's default prefill computes it:
+    quantize_q8 rounds the f32 activations to Q8_0 blocks, matmul_q8_0 multiplies
+    integers on the int8 matrix cores and scales every 32-weight unit."""
+    synth, oracle, K, TensorType, P = env["synth"], env["oracle"], env["K"], env["TensorType"], env["P"]
+    rec, kset, b = env["rec"], env["kset"], env["b"]
+    rows, k, n = 512, 4096, 4096
+    g = synth.rng(0xC4)
+    raw = synth.q8_0_rows(g, n, k)
+    x = synth.activations(g, rows, k)
+    src = env["upload"](raw)
+    xa = env["upload"](x)
+    rb = K.row_bytes(TensorType.q8_0, k)
+    out = env["output"](4 * rows * n)
+    qx, dx = env["output"](rows * k), env["output"](4 * rows * k // 32)
+    launches = []
+    for _ in range(4):
+        wa = env["output"](n * rb)
+        K.Launcher(rec, kset).layout(TensorType.q8_0, src, wa, n, k)
+        quant = b.add(K.Kernel.quantize_q8, P.QuantizeQ8(k=k, block=32), [xa, qx, dx, xa], K.Grid.tiles_y(K.div_ceil(k, 256), 1))
+        p = P.MatmulQuant(rows=rows, n=n, k=k, col0=0, out_stride=n, k_slice=k)
+        mul = b.add(K.Kernel.matmul_q8_0, p, [qx, wa, out, dx], K.Grid.tiles_y(K.div_ceil(n, K.matmul_quant_tile_n), K.matmul_quant_tile_t))
+        launches.append(env["Chain"]([quant, mul], rows))
+    b.finish()
+    env["flush"]()
+    steps = max(1, env["args"].steps // 4)
+    wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 4), per_step=2)
+    got = env["read"](out)[: rows * n].reshape(rows, n).astype(np.float64)
+    w = oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k)
+    xs = oracle.round_like_llama(oracle.Q8_0, x)
+    want = xs.astype(np.float64) @ w.astype(np.float64).T
+    ops = 2 * rows * n * k
+    return {
+        "workload": "C4 shape through quantize_q8 + matmul_q8_0: f32 activations rounded to Q8_0 blocks, int8 MFMA, f32 scaling per 32-weight unit",
+        "ops_per_step": ops,
+        "us_per_step_wall": round(wall / steps * 1e6, 3),
+        "us_per_step_gpu": round(gpu_s / steps * 1e6, 3),
+        "TOPs_gpu": round(ops * steps / gpu_s / 1e12, 1),
+        "int8_mfma_frac": round(ops * steps / gpu_s / 1e12 / MFMA_INT8_PEAK_TOPS, 4),
         "max_err_over_max_want": float(np.max(np.abs(got - want)) / np.max(np.abs(want))),
     }
 

@@ -85,26 +85,27 @@ __device__ __forceinline__ long as_operand(iu32x2 v) {
 // lanes would ask for different rows, and the load unit takes such a load apart
 // one lane a clock; here a wave brings sixteen rows and sixteen token lines in
 // as whole 256-byte runs (buffer_load ... lds, 16 bytes a lane, four lines an
-// instruction) and reads its operands back, 8 bytes a lane. The 16-byte chunks
-// of a weight row are stored permuted (chunk c of row r at position c ^ r),
-// which spreads the sixteen rows of an operand read over all banks two deep,
-// the best 16-byte granularity allows. Two buffers: a step's loads are issued
-// before the previous step's multiply and waited for after it.
-
-// Token lines, which every wave reads four times as often as its weights, get
-// a layout without bank conflicts: each instruction's four lines (1 KiB) are
-// followed by XPAD = 8 bytes, and chunk c of token t sits at position
-// c ^ 2 (t % 4). The sixteen tokens of an operand read then start at sixteen
-// different 8-byte bank pairs: 4 (c / 2 ^ t % 4) + 2 (c % 2) + half + t / 4.
+// instruction) and reads its operands back, 8 bytes a lane. Two buffers: a
+// step's loads are issued before the previous step's multiply and waited for
+// after it.
+//
+// The lines are laid out so that operand reads meet no bank conflicts: each
+// instruction's four lines (1 KiB) are followed by XPAD = 8 bytes, and chunk c
+// of line r sits at position c ^ 2 (r % 4). The sixteen lines of an operand
+// read then start at sixteen different 8-byte bank pairs:
+// 4 (c / 2 ^ r % 4) + 2 (c % 2) + half + r / 4. The tokens' block scales sit
+// eight to a token with unit u at position u ^ (t / 4 % 4), which spreads the
+// sixteen tokens a lane group reads over sixteen banks.
 constexpr uint32_t XPAD = 8;
-__device__ __forceinline__ uint32_t xkey(uint32_t token) { return 2u * (token & 3u); }
+__device__ __forceinline__ uint32_t xkey(uint32_t line) { return 2u * (line & 3u); }
+constexpr uint32_t QUAD = 4u * STEP + XPAD;  // four lines and their padding
 
 template <bool RAGGED>
 __global__ __launch_bounds__(256, 2) void matmul_q8_0_i8_kernel(I8Args a) {
     constexpr uint32_t DBUF = TT * 32u;          // [token][8 units] f32
-    constexpr uint32_t WBUF = TN * STEP;         // [row][256 bytes], chunks permuted
+    constexpr uint32_t WBUF = TN / 4u * QUAD;    // [row][256 bytes], chunks permuted, padded every four rows
     constexpr uint32_t SBUF = TN * 16u;          // [row][8 units] f16
-    constexpr uint32_t XBUF = TT * STEP + TT / 4u * XPAD;  // [token][256 bytes], chunks permuted, XPAD bytes after every four tokens
+    constexpr uint32_t XBUF = TT / 4u * QUAD;    // [token][256 bytes], the same way
     __shared__ __align__(16) uint8_t lds_q[2][XBUF];
     __shared__ __align__(16) uint8_t lds_d[2][DBUF];
     __shared__ __align__(16) uint8_t lds_w[2][WBUF];
@@ -117,28 +118,29 @@ __global__ __launch_bounds__(256, 2) void matmul_q8_0_i8_kernel(I8Args a) {
     const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.qx, a.qx_bytes), wbuf = make_buffer(a.w, a.w_bytes), dbuf = make_buffer(a.dx, a.dx_bytes);
 
     // Weight loads: instruction i takes rows r = 4 i + lane / 16 of the wave's
-    // sixteen; the lane at position p = lane % 16 fetches chunk p ^ r, the one
-    // that belongs there.
+    // sixteen; the lane at position p = lane % 16 fetches chunk p ^ key(r), the
+    // one that belongs there.
     const uint32_t wl_row = lane >> 4, wl_pos = lane & 15u;
     const uint32_t woff = (n0 + 16u * wave + wl_row) * a.row_bytes;
     // Token loads, the same way: instruction i takes tokens 16 wave + 4 i + lane / 16.
     const uint32_t xoff = (t0 + 16u * wave + wl_row) * a.k;
     // Scales: one word a lane, row 16 wave + lane / 4, units 2 (lane % 4), + 1.
     const uint32_t soff = (n0 + 16u * wave + (lane >> 2)) * a.row_bytes + a.k + 4u * (lane & 3u);
-    // Block scales of tokens 16 wave + 8 i + lane / 8, unit lane % 8.
-    const uint32_t doff = ((t0 + 16u * wave + (lane >> 3)) * (a.k / 32u) + (lane & 7u)) * 4u;
+    // Block scales of tokens 16 wave + 8 i + lane / 8: the lane at position
+    // lane % 8 fetches unit (lane % 8) ^ (token / 4 % 4); token / 4 % 4 = 2 i + lane / 32 % 2.
+    const uint32_t doff = (t0 + 16u * wave + (lane >> 3)) * (a.k / 32u) * 4u;
 
     auto fetch = [&](uint32_t k0, uint32_t buf) __attribute__((always_inline)) {
 #pragma unroll
         for (uint32_t i = 0; i < 4; i++)
-            load_lds_b128(wbuf, lds_w[buf] + (16u * wave + 4u * i) * STEP, woff + 4u * i * a.row_bytes + k0 + 16u * (wl_pos ^ (4u * i | wl_row)));
+            load_lds_b128(wbuf, lds_w[buf] + (4u * wave + i) * QUAD, woff + 4u * i * a.row_bytes + k0 + 16u * (wl_pos ^ xkey(wl_row)));
         load_lds_b32(wbuf, lds_s[buf] + 16u * wave * 16u, soff + k0 / 16u);
 #pragma unroll
         for (uint32_t i = 0; i < 4; i++)
-            load_lds_b128(xbuf, lds_q[buf] + (4u * wave + i) * (4u * STEP + XPAD), xoff + 4u * i * a.k + k0 + 16u * (wl_pos ^ xkey(4u * i | wl_row)));
+            load_lds_b128(xbuf, lds_q[buf] + (4u * wave + i) * QUAD, xoff + 4u * i * a.k + k0 + 16u * (wl_pos ^ xkey(wl_row)));
 #pragma unroll
         for (uint32_t i = 0; i < 2; i++)
-            load_lds_b32(dbuf, lds_d[buf] + (16u * wave + 8u * i) * 32u, doff + 8u * i * (a.k / 32u) * 4u + k0 / 8u);
+            load_lds_b32(dbuf, lds_d[buf] + (16u * wave + 8u * i) * 32u, doff + 8u * i * (a.k / 32u) * 4u + k0 / 8u + 4u * ((lane & 7u) ^ (2u * i + ((lane >> 5) & 1u))));
     };
 
     if32x4 acc[4];
@@ -150,18 +152,18 @@ __global__ __launch_bounds__(256, 2) void matmul_q8_0_i8_kernel(I8Args a) {
         i32x4 is[4];
         float dx[4];
     };
-    // This lane's operand bytes of unit u: row 16 wave + l16, logical chunk
-    // 2 u + g / 2, half g % 2.
-    const uint32_t wkey = l16;  // (16 wave + l16) & 15
+    // This lane's operand bytes of unit u: line l16 of its row or token tile,
+    // logical chunk 2 u + g / 2, half g % 2.
+    const uint32_t line = (l16 >> 2) * QUAD + (l16 & 3u) * STEP + 8u * (g & 1u);
+    const uint32_t dkey = (l16 >> 2) & 3u;
     auto multiply = [&](uint32_t buf, uint32_t u, Unit &r) __attribute__((always_inline)) {
-        const uint32_t chunk = (2u * u + (g >> 1)) ^ wkey;
-        const long wf = *reinterpret_cast<const long *>(&lds_w[buf][(16u * wave + l16) * STEP + 16u * chunk + 8u * (g & 1u)]);
+        const uint32_t at = line + 16u * ((2u * u + (g >> 1)) ^ xkey(l16));
+        const long wf = *reinterpret_cast<const long *>(&lds_w[buf][4u * wave * QUAD + at]);
 #pragma unroll
         for (uint32_t mt = 0; mt < 4; mt++) {
-            const uint32_t xchunk = (2u * u + (g >> 1)) ^ xkey(l16);
-            const long xf = *reinterpret_cast<const long *>(&lds_q[buf][(4u * mt + (l16 >> 2)) * (4u * STEP + XPAD) + (l16 & 3u) * STEP + 16u * xchunk + 8u * (g & 1u)]);
+            const long xf = *reinterpret_cast<const long *>(&lds_q[buf][4u * mt * QUAD + at]);
             r.is[mt] = __builtin_amdgcn_mfma_i32_16x16x32_i8(wf, xf, i32x4{0, 0, 0, 0}, 0, 0, 0);
-            r.dx[mt] = *reinterpret_cast<const float *>(lds_d[buf] + (16u * mt + l16) * 32u + 4u * u);
+            r.dx[mt] = *reinterpret_cast<const float *>(lds_d[buf] + (16u * mt + l16) * 32u + 4u * (u ^ dkey));
         }
     };
     auto scale = [&](uint32_t k0, const iu32x4 (&sc)[4], uint32_t u, const Unit &r) __attribute__((always_inline)) {

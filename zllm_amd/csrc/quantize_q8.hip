@@ -1,8 +1,8 @@
 // quantize_q8: rows of activations rounded to 8-bit blocks for the int8 prefill
 // multiply, value for value as llama.cpp's x86 CPU backend rounds them
-// (src/kernels/quantize_q8.wgsl, src/ref/matmul.zig:197-247). A 64-lane
-// workgroup takes 256 values of one row, four per lane: one Q8_K block, or
-// eight Q8_0 blocks of eight lanes each. Every operation whose rounding decides
+// (src/kernels/quantize_q8.wgsl, src/ref/matmul.zig:197-247). A wave takes
+// 256 values of one row, four per lane: one Q8_K block, or eight Q8_0 blocks of
+// eight lanes each; a workgroup is four independent waves. Every operation whose rounding decides
 // a value is spelled as a correctly rounded intrinsic, so the compiler can
 // neither fuse the multiply into the rounding addition nor approximate a
 // division.
@@ -36,9 +36,10 @@ __device__ __forceinline__ Lead better(const Lead &a, const Lead &b) {
     return (b.mag > a.mag || (b.mag == a.mag && b.at < a.at)) ? b : a;
 }
 
-__global__ __launch_bounds__(64) void quantize_q8_kernel(QuantizeQ8Params p, const float *x, uint32_t *qx, float *dx, const float *nw) {
-    const uint32_t lane = threadIdx.x, row = blockIdx.y;
-    const uint32_t at = blockIdx.x * 256u + 4u * lane;  // first of this lane's four positions
+__global__ __launch_bounds__(256) void quantize_q8_kernel(QuantizeQ8Params p, const float *x, uint32_t *qx, float *dx, const float *nw) {
+    const uint32_t lane = threadIdx.x & 63u, row = blockIdx.y;
+    const uint32_t at = (blockIdx.x * 4u + (threadIdx.x >> 6)) * 256u + 4u * lane;  // first of this lane's four positions
+    if (at - 4u * lane >= p.k) return;  // a whole wave past the row's end
     const bool live = at < p.k;
     qf32x4 v = {0.f, 0.f, 0.f, 0.f};
     if (p.mode == 2u) {
@@ -133,7 +134,7 @@ zhip_result launch_quantize_q8(const Dispatch &d) {
         return fail(d, ZHIP_E_BAD_COMMAND, "quantize_q8: bound ranges too small");
     if (((uintptr_t)d.bind[1].ptr | (p.mode == 1u ? (uintptr_t)d.bind[4].ptr : 0)) & 15u) return fail(d, ZHIP_E_BAD_COMMAND, "quantize_q8: x and norm weights must be 16-byte aligned");
     if (((uintptr_t)d.bind[2].ptr | (uintptr_t)d.bind[3].ptr) & 3u) return fail(d, ZHIP_E_BAD_COMMAND, "quantize_q8: outputs must be 4-byte aligned");
-    hipLaunchKernelGGL(quantize_q8_kernel, dim3(d.grid[0], d.grid[1]), dim3(64), 0, d.stream, p,
+    hipLaunchKernelGGL(quantize_q8_kernel, dim3((d.grid[0] + 3u) / 4u, d.grid[1]), dim3(256), 0, d.stream, p,
         reinterpret_cast<const float *>(d.bind[1].ptr), reinterpret_cast<uint32_t *>(d.bind[2].ptr),
         reinterpret_cast<float *>(d.bind[3].ptr), reinterpret_cast<const float *>(d.bind[4].ptr));
     return check_launch(d, "quantize_q8");
