@@ -43,7 +43,7 @@ struct DecQ8_0 {
     static constexpr int RUNS = 2;
     static constexpr int E = 16;
     static constexpr uint32_t BLOCK = 32;
-    static constexpr bool CHUNK_KERNEL = false;
+    static constexpr int CHUNK = 0;
     static const char *name() { return "matvec_q8_0"; }
     static uint32_t row_bytes(uint32_t k) { return (k + k / 16u + 15u) & ~15u; }
     __device__ static uint32_t xoff(uint32_t task, int h) { return 16u * task + 8u * h; }
@@ -73,7 +73,7 @@ struct DecQ3_K {
     static constexpr int RUNS = 1;
     static constexpr int E = 32;
     static constexpr uint32_t BLOCK = 256;
-    static constexpr bool CHUNK_KERNEL = false;
+    static constexpr int CHUNK = 0;
     static const char *name() { return "matvec_q3_k"; }
     static uint32_t row_bytes(uint32_t k) { return k / 256u * 128u; }
     __device__ static uint32_t xoff(uint32_t task, int) { return 32u * task; }
@@ -101,7 +101,7 @@ struct DecQ4_K {
     static constexpr int RUNS = 2;
     static constexpr int E = 32;
     static constexpr uint32_t BLOCK = 256;
-    static constexpr bool CHUNK_KERNEL = true;  // has its own multiply (matvec_q4k.hip)
+    static constexpr int CHUNK = 4;  // has its own multiply (matvec_kquant.hip)
     static const char *name() { return "matvec_q4_k"; }
     static uint32_t row_bytes(uint32_t k) { return k / 256u * 144u; }
     __device__ static uint32_t xoff(uint32_t task, int h) {
@@ -141,7 +141,7 @@ struct DecQ5_K {
     static constexpr int RUNS = 2;
     static constexpr int E = 32;
     static constexpr uint32_t BLOCK = 256;
-    static constexpr bool CHUNK_KERNEL = false;
+    static constexpr int CHUNK = 5;
     static const char *name() { return "matvec_q5_k"; }
     static uint32_t row_bytes(uint32_t k) { return k / 256u * 176u; }
     __device__ static uint32_t xoff(uint32_t task, int h) {
@@ -184,7 +184,7 @@ struct DecQ6_K {
     static constexpr int RUNS = 4;
     static constexpr int E = 64;
     static constexpr uint32_t BLOCK = 256;
-    static constexpr bool CHUNK_KERNEL = false;
+    static constexpr int CHUNK = 6;
     static const char *name() { return "matvec_q6_k"; }
     static uint32_t row_bytes(uint32_t k) { return k / 256u * 224u; }
     __device__ static uint32_t xoff(uint32_t task, int h) {
@@ -228,7 +228,7 @@ struct DecBF16 {
     static constexpr int RUNS = 2;
     static constexpr int E = 8;
     static constexpr uint32_t BLOCK = 8;
-    static constexpr bool CHUNK_KERNEL = false;
+    static constexpr int CHUNK = 0;
     static const char *name() { return "matvec_bf16"; }
     static uint32_t row_bytes(uint32_t k) { return 2u * k; }
     __device__ static uint32_t xoff(uint32_t task, int h) { return 8u * task + 4u * h; }

@@ -33,9 +33,10 @@ __device__ __forceinline__ float silu_f(float v) { return v / (1.0f + expf(-v));
 // Stages token `token`'s k inputs at dst (k / 4 vectors): normalised with the
 // RMSNorm prologue and / or activated as silu(x / act_div) as the flags ask
 // (src/kernels/matvec_quant.wgsl.hbs:73-89,175-198). Every thread of the
-// 256-thread workgroup must call it; `red` is four floats of LDS. With `pad`,
-// one vector of padding follows every 16 (vector i lands at i + i / 16).
-__device__ __forceinline__ void stage_token(const MvArgs &a, uint32_t token, float4 *dst, float *red, bool pad = false) {
+// 256-thread workgroup must call it; `red` is four floats of LDS. Vector i of
+// the token lands at dst[place(i)].
+template <class Place>
+__device__ __forceinline__ void stage_token(const MvArgs &a, uint32_t token, float4 *dst, float *red, Place place) {
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t k4 = a.k / 4u;
     const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)token * a.xr);
@@ -65,8 +66,12 @@ __device__ __forceinline__ void stage_token(const MvArgs &a, uint32_t token, flo
             v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
             v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
         }
-        dst[pad ? i + (i >> 4) : i] = v;
+        dst[place(i)] = v;
     }
+}
+
+__device__ __forceinline__ void stage_token(const MvArgs &a, uint32_t token, float4 *dst, float *red) {
+    stage_token(a, token, dst, red, [](uint32_t i) { return i; });
 }
 
 }  // namespace zhip

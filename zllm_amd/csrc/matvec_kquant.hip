@@ -1,0 +1,579 @@
+// matvec_q4_k / matvec_q5_k / matvec_q6_k: out[t][col0 + j] (+)= sum_i X(t, i) * w[j][i]
+// over K-quant rows, the decode step's multiply (contract of
+// src/kernels/matvec_quant.wgsl.hbs with the decoders of
+// src/kernels/quant/q{4,5,6}_k_dot.wgsl; block formulas of src/ref/tensor.zig:94-160).
+//
+// Layout of the work. A 256-weight block splits into four tasks of 64 weights
+// whose sub-blocks share their scales: for Q4_K and Q5_K a 32-byte chunk of
+// nibbles (sub-block 2c in the low nibbles, 2c + 1 in the high ones), for Q6_K
+// sixteen positions of one half (four runs of sixteen weights, 32 apart). The
+// lane that owns a task loads its vectors and the block's scales, so every byte
+// of the weight stream is loaded by exactly one lane per use and a wave's load
+// instruction falls in one contiguous span of the matrix. A row has k / 64
+// tasks: lane l takes tasks l, l + 64, ...; rows of 1024 or 2048 weights pack
+// four or two to a wave pass so that no lane idles.
+//
+// Arithmetic. Per task and token the lane computes, for each sub-block s of
+// the task, scale_s * sum(q * x) - min_s * sum(x): the block formula with
+// scale and min factored out of the sub-block's sums, so a weight costs one
+// convert (shared by all tokens) and one FMA per token. Q4_K high nibbles are
+// used in place as 16 * q (a mask, no shift) with the factor 1/16 folded into
+// the sub-block scale, which is exact. The sub-block input sums are computed
+// once per workgroup. A lane adds its tasks' values in task order and the lanes
+// reduce with DPP row operations in a fixed order, so a token's result does not
+// depend on how many tokens share the launch or on which variant below runs
+// it: the reference's bitwise split invariant (matvec_quant.wgsl.hbs:14-18).
+//
+// Variants. XREG (one token, at most one task per lane, i.e. k <= 4096): the
+// lane's 64 inputs never change from row to row, so they live in registers and
+// the loop touches nothing but the weight stream. Otherwise inputs are read
+// from a bank-conflict-free padded LDS copy kept in task order, once per task
+// for both rows of a pass (two outputs, or the gate and up rows of one output
+// with SILU_PAIR). In both, the next task's vectors are loaded before the
+// current one is multiplied.
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "decode.cuh"
+#include "matvec_common.cuh"
+
+namespace zhip {
+
+// Byte I of w as a float: v_cvt_f32_ubyte{0..3}, one instruction.
+template <int I>
+__device__ __forceinline__ float cvt_byte(uint32_t w) {
+    return (float)((w >> (8 * I)) & 0xffu);
+}
+
+// Bit masks, passed as kernel arguments: were they literals the compiler would
+// fold mask and byte select into one bit-field extract per weight and then
+// convert, three instructions a weight instead of a mask per word and a convert
+// per weight.
+struct Masks {
+    uint32_t lo, hi, two, one;  // 0x0f0f0f0f, 0xf0f0f0f0, 0x03030303, 0x01010101
+};
+
+struct KScales {
+    float d1, m1, d2, m2;  // d*sc(2c), dmin*m(2c), d*sc(2c+1) (/16 for Q4_K), dmin*m(2c+1)
+};
+
+// The scale and min of sub-blocks 2c and 2c + 1 from a Q4_K / Q5_K header
+// vector (src/ref/tensor.zig:94-98); s16 = 16 * (c & 1), upper = c >= 2.
+template <bool SIXTEENTH>
+__device__ __forceinline__ KScales chunk_scales(const uint4 &h, uint32_t s16, bool upper) {
+    const float d = half_bits_to_float(h.x & 0xffffu);
+    const float dmin = half_bits_to_float(h.x >> 16);
+    const uint32_t a0 = h.y >> s16, a1 = h.z >> s16, a2 = h.w >> s16;
+    const uint32_t sc_lo = a0 & 0x3f3fu, mn_lo = a1 & 0x3f3fu;
+    const uint32_t sc_hi = (a2 & 0x0f0fu) | ((a0 >> 2) & 0x3030u);
+    const uint32_t mn_hi = ((a2 >> 4) & 0x0f0fu) | ((a1 >> 2) & 0x3030u);
+    const uint32_t sc = upper ? sc_hi : sc_lo, mn = upper ? mn_hi : mn_lo;
+    KScales s;
+    s.d1 = d * cvt_byte<0>(sc);
+    s.d2 = SIXTEENTH ? d * cvt_byte<1>(sc) * 0.0625f : d * cvt_byte<1>(sc);
+    s.m1 = dmin * cvt_byte<0>(mn);
+    s.m2 = dmin * cvt_byte<1>(mn);
+    return s;
+}
+
+__device__ __forceinline__ uint32_t word_of(const uint4 &v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
+
+// Four weights (the bytes of `word`) times four inputs, added to `sum`.
+__device__ __forceinline__ float dot_bytes(uint32_t word, const float4 &x, float sum) {
+    sum = fmaf(cvt_byte<0>(word), x.x, sum);
+    sum = fmaf(cvt_byte<1>(word), x.y, sum);
+    sum = fmaf(cvt_byte<2>(word), x.z, sum);
+    sum = fmaf(cvt_byte<3>(word), x.w, sum);
+    return sum;
+}
+
+// ---- the formats ---------------------------------------------------------------------
+// A format names its task's vectors (Raw), loads them, says where a row's
+// inputs go in task order, and multiplies one task of one row (ROWS = 1) or of
+// the two rows of a pass (ROWS = 2) for MT tokens. x(t, v) gives inputs
+// 4v .. 4v + 3 of the task in task order for token t; sums(t, s) the sum of the
+// task's s-th run of 64 / NSUM inputs.
+
+// Q4_K: 144-byte blocks (header vector; 128 bytes of nibbles in four chunks of
+// 32: chunk c holds sub-block 2c in its low nibbles and 2c + 1 in its high
+// ones). Task = chunk: 32 low-nibble weights, then 32 high-nibble ones.
+struct KQ4 {
+    static constexpr uint32_t BLOCK_BYTES = 144;
+    static constexpr int NSUM = 2;
+    static const char *name() { return "matvec_q4_k"; }
+    struct Raw {
+        uint4 h, q0, q1;
+    };
+    __device__ static Raw load(const uint8_t *block, uint32_t c) {
+        Raw r;
+        r.h = *reinterpret_cast<const uint4 *>(block);
+        r.q0 = *reinterpret_cast<const uint4 *>(block + 16u + 32u * c);
+        r.q1 = *reinterpret_cast<const uint4 *>(block + 32u + 32u * c);
+        return r;
+    }
+    __device__ static uint32_t stage_index(uint32_t v) { return v; }
+
+    template <int MT, int ROWS, class XF, class SF>
+    __device__ static void dot(const Raw (&r)[ROWS], uint32_t c, Masks nm, XF x, SF sums, float (&out)[ROWS][MT]) {
+        float s_lo[ROWS][MT], s_hi[ROWS][MT];
+#pragma unroll
+        for (int j = 0; j < ROWS; j++)
+#pragma unroll
+            for (int t = 0; t < MT; t++) s_lo[j][t] = s_hi[j][t] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            uint32_t lo[ROWS], hi[ROWS];
+#pragma unroll
+            for (int j = 0; j < ROWS; j++) {
+                const uint32_t word = word_of(e < 4 ? r[j].q0 : r[j].q1, e & 3);
+                lo[j] = word & nm.lo;
+                hi[j] = word & nm.hi;  // 16 q, the sixteenth is in the scale
+            }
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                const float4 xl = x(t, e), xh = x(t, 8 + e);
+#pragma unroll
+                for (int j = 0; j < ROWS; j++) {
+                    s_lo[j][t] = dot_bytes(lo[j], xl, s_lo[j][t]);
+                    s_hi[j][t] = dot_bytes(hi[j], xh, s_hi[j][t]);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < ROWS; j++) {
+            const KScales s = chunk_scales<true>(r[j].h, 16u * (c & 1u), c >= 2u);
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                float v = s.d1 * s_lo[j][t];
+                v = fmaf(-s.m1, sums(t, 0), v);
+                v = fmaf(s.d2, s_hi[j][t], v);
+                v = fmaf(-s.m2, sums(t, 1), v);
+                out[j][t] = v;
+            }
+        }
+    }
+};
+
+// Q5_K: 176-byte blocks (header vector; qh[32]; qs[128] as Q4_K's nibbles).
+// Weight l of sub-block 2c takes bit 2c of qh[l] as its fifth bit, weight l of
+// sub-block 2c + 1 bit 2c + 1 (src/ref/tensor.zig:118-137). Task = chunk.
+struct KQ5 {
+    static constexpr uint32_t BLOCK_BYTES = 176;
+    static constexpr int NSUM = 2;
+    static const char *name() { return "matvec_q5_k"; }
+    struct Raw {
+        uint4 h, b0, b1, q0, q1;
+    };
+    __device__ static Raw load(const uint8_t *block, uint32_t c) {
+        Raw r;
+        r.h = *reinterpret_cast<const uint4 *>(block);
+        r.b0 = *reinterpret_cast<const uint4 *>(block + 16u);
+        r.b1 = *reinterpret_cast<const uint4 *>(block + 32u);
+        r.q0 = *reinterpret_cast<const uint4 *>(block + 48u + 32u * c);
+        r.q1 = *reinterpret_cast<const uint4 *>(block + 64u + 32u * c);
+        return r;
+    }
+    __device__ static uint32_t stage_index(uint32_t v) { return v; }
+
+    template <int MT, int ROWS, class XF, class SF>
+    __device__ static void dot(const Raw (&r)[ROWS], uint32_t c, Masks nm, XF x, SF sums, float (&out)[ROWS][MT]) {
+        float s_lo[ROWS][MT], s_hi[ROWS][MT];
+#pragma unroll
+        for (int j = 0; j < ROWS; j++)
+#pragma unroll
+            for (int t = 0; t < MT; t++) s_lo[j][t] = s_hi[j][t] = 0.f;
+#pragma unroll
+        for (int e = 0; e < 8; e++) {
+            uint32_t lo[ROWS], hi[ROWS];
+#pragma unroll
+            for (int j = 0; j < ROWS; j++) {
+                const uint32_t word = word_of(e < 4 ? r[j].q0 : r[j].q1, e & 3);
+                const uint32_t bits = word_of(e < 4 ? r[j].b0 : r[j].b1, e & 3) >> (2u * c);
+                lo[j] = ((bits & nm.one) << 4) | (word & nm.lo);
+                hi[j] = (((bits >> 1) & nm.one) << 4) | ((word >> 4) & nm.lo);
+            }
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                const float4 xl = x(t, e), xh = x(t, 8 + e);
+#pragma unroll
+                for (int j = 0; j < ROWS; j++) {
+                    s_lo[j][t] = dot_bytes(lo[j], xl, s_lo[j][t]);
+                    s_hi[j][t] = dot_bytes(hi[j], xh, s_hi[j][t]);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < ROWS; j++) {
+            const KScales s = chunk_scales<false>(r[j].h, 16u * (c & 1u), c >= 2u);
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                float v = s.d1 * s_lo[j][t];
+                v = fmaf(-s.m1, sums(t, 0), v);
+                v = fmaf(s.d2, s_hi[j][t], v);
+                v = fmaf(-s.m2, sums(t, 1), v);
+                out[j][t] = v;
+            }
+        }
+    }
+};
+
+// Q6_K: blocks padded from 210 to 224 bytes (ql[128], qh[64], sixteen signed
+// scales, d; src/ref/tensor.zig:139-160). Task p of a block takes positions
+// l = 16 (p % 2) .. + 15 of half n = p / 2: four runs of sixteen weights at
+// 128 n + l + {0, 32, 64, 96}, run r from the low (r < 2) or high nibbles of
+// ql[64 n + 32 (r % 2) + l] and bits 2r, 2r + 1 of qh[32 n + l], with scale
+// 8 n + p % 2 + 2 r; a weight is d * scale * (q - 32).
+struct KQ6 {
+    static constexpr uint32_t BLOCK_BYTES = 224;
+    static constexpr int NSUM = 4;
+    static const char *name() { return "matvec_q6_k"; }
+    struct Raw {
+        uint4 l0, l1, hv;
+        uint2 sc;
+        uint32_t d;
+    };
+    __device__ static Raw load(const uint8_t *block, uint32_t p) {
+        const uint32_t n = p >> 1, lh = p & 1u;
+        Raw r;
+        r.l0 = *reinterpret_cast<const uint4 *>(block + 64u * n + 16u * lh);
+        r.l1 = *reinterpret_cast<const uint4 *>(block + 64u * n + 32u + 16u * lh);
+        r.hv = *reinterpret_cast<const uint4 *>(block + 128u + 32u * n + 16u * lh);
+        r.sc = *reinterpret_cast<const uint2 *>(block + 192u + 8u * n);
+        r.d = *reinterpret_cast<const uint32_t *>(block + 208u);
+        return r;
+    }
+    // Vector v of a row (inputs 4v ..) is vector q of run r of task 4 blk + 2 n + lh.
+    __device__ static uint32_t stage_index(uint32_t v) {
+        const uint32_t blk = v >> 6, n = (v >> 5) & 1u, run = (v >> 3) & 3u, lh = (v >> 2) & 1u, q = v & 3u;
+        return 64u * blk + 32u * n + 16u * lh + 4u * run + q;
+    }
+
+    template <int MT, int ROWS, class XF, class SF>
+    __device__ static void dot(const Raw (&r)[ROWS], uint32_t p, Masks nm, XF x, SF sums, float (&out)[ROWS][MT]) {
+        float s[ROWS][MT][4];
+#pragma unroll
+        for (int j = 0; j < ROWS; j++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int run = 0; run < 4; run++) s[j][t][run] = 0.f;
+#pragma unroll
+        for (int run = 0; run < 4; run++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                uint32_t q[ROWS];
+#pragma unroll
+                for (int j = 0; j < ROWS; j++) {
+                    const uint32_t lw = word_of(run & 1 ? r[j].l1 : r[j].l0, i);
+                    const uint32_t nib = run < 2 ? lw & nm.lo : (lw >> 4) & nm.lo;
+                    const uint32_t two = (word_of(r[j].hv, i) >> (2 * run)) & nm.two;
+                    q[j] = (two << 4) | nib;
+                }
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    const float4 xv = x(t, 4 * run + i);
+#pragma unroll
+                    for (int j = 0; j < ROWS; j++) s[j][t][run] = dot_bytes(q[j], xv, s[j][t][run]);
+                }
+            }
+        }
+        const uint32_t lh = p & 1u;
+#pragma unroll
+        for (int j = 0; j < ROWS; j++) {
+            const float d = half_bits_to_float(r[j].d & 0xffffu);
+            // Scales lh, lh + 2 of the half's eight are bytes lh, lh + 2 of sc.x; lh + 4, lh + 6 of sc.y.
+            const uint32_t s01 = r[j].sc.x >> (8u * lh), s23 = r[j].sc.y >> (8u * lh);
+            const float scale[4] = {d * (float)(int8_t)(s01 & 0xffu), d * (float)(int8_t)((s01 >> 16) & 0xffu),
+                                    d * (float)(int8_t)(s23 & 0xffu), d * (float)(int8_t)((s23 >> 16) & 0xffu)};
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                float v = 0.f;
+#pragma unroll
+                for (int run = 0; run < 4; run++) v = fmaf(scale[run], fmaf(-32.f, sums(t, run), s[j][t][run]), v);
+                out[j][t] = v;
+            }
+        }
+    }
+};
+
+template <int CTRL, int ROW_MASK>
+__device__ __forceinline__ float dpp_add(float v) {
+    const int t = __builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, ROW_MASK, 0xF, true);
+    return v + __int_as_float(t);
+}
+
+// Sums v over each segment of 2^seg_log2 lanes (16, 32 or 64) in a fixed
+// order; the segment's last lane holds the total.
+__device__ __forceinline__ float segment_sum(float v, uint32_t seg_log2) {
+    v = dpp_add<0xB1, 0xF>(v);   // quad_perm [1,0,3,2]
+    v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
+    v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
+    v = dpp_add<0x140, 0xF>(v);  // row_mirror: every lane holds its row of 16's sum
+    if (seg_log2 >= 5) v = dpp_add<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
+    if (seg_log2 >= 6) v = dpp_add<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
+    return v;
+}
+
+// Floats per task in the padded LDS copy: 64 inputs and one vector of padding,
+// so lanes reading the same offset of consecutive tasks hit different banks.
+constexpr uint32_t kTaskStride = 68;
+
+struct KArgs {
+    MvArgs a;
+    uint32_t t0;        // first token of this pass
+    uint32_t mt;        // tokens in this pass (<= MT)
+    uint32_t seg_log2;  // lanes per row: 4, 5 or 6
+    uint32_t tasks;     // k / 64
+    Masks nm;
+};
+
+template <class P, int MT, bool PAIR, bool XREG>
+__global__ __launch_bounds__(256) void matvec_kquant_kernel(KArgs q) {
+    const MvArgs &a = q.a;
+    extern __shared__ float4 lds4[];
+    __shared__ float red[4];
+    constexpr int NSUM = P::NSUM, RUN = 64 / NSUM;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t tasks = q.tasks;
+    const uint32_t tok_stride4 = tasks * (kTaskStride / 4u);  // float4s per token
+    float *sums_lds = reinterpret_cast<float *>(lds4 + (size_t)MT * tok_stride4);
+
+    // Rows a pass takes: the gate and up rows of an output, or two outputs so
+    // that one read of the inputs from LDS serves both; with the inputs in
+    // registers a pass is a single row.
+    constexpr int kRows = (PAIR || !XREG) ? 2 : 1;
+    const uint32_t gwave = blockIdx.x * 4u + wave, nwaves = gridDim.x * 4u;
+    const uint32_t seg = 1u << q.seg_log2;
+    const uint32_t tsub = lane & (seg - 1u), rsub = lane >> q.seg_log2, rpi = 64u >> q.seg_log2;
+    const uint32_t iters = (tasks + seg - 1u) >> q.seg_log2;
+    const uint32_t per_unit = PAIR ? rpi : rpi * kRows;
+    const uint32_t units = (a.rows + per_unit - 1u) / per_unit;
+    const bool writer = tsub == seg - 1u;
+
+    // A position in the wave's walk over (unit, 64-task slice) pairs, and the
+    // weight rows it reads there: output j0 (and j0 + 1), or the gate row j0
+    // and the up row half + j0. Rows past the end are clamped for the loads
+    // and skipped at the store.
+    struct Cursor {
+        uint32_t u, i, j0, ra, rb;
+    };
+    auto place = [&](Cursor &c) {
+        const uint32_t unit = c.u < units ? c.u : units - 1u;
+        c.j0 = PAIR ? unit * rpi + rsub : (unit * rpi + rsub) * kRows;
+        c.ra = c.j0 < a.rows ? c.j0 : 0u;
+        if (PAIR) c.rb = a.half + c.ra;
+        else c.rb = c.j0 + 1u < a.rows ? c.j0 + 1u : c.ra;
+    };
+    auto advance = [&](Cursor &c) {
+        if (c.i + 1u < iters) {
+            c.i++;
+        } else {
+            c.i = 0;
+            c.u += nwaves;
+            place(c);
+        }
+    };
+    // Past the wave's last position the cursor is clamped to a valid one, so
+    // loads need no branch around them (their results are not used).
+    auto load_at = [&](const Cursor &c, typename P::Raw (&dst)[kRows]) {
+        const uint32_t task = tsub + c.i * seg;
+        const uint32_t tk = task < tasks ? task : 0u;
+        const uint32_t blk = tk >> 2, ch = tk & 3u;
+        dst[0] = P::load(a.w + (size_t)c.ra * a.row_bytes + (size_t)blk * P::BLOCK_BYTES, ch);
+        if (kRows == 2) dst[kRows - 1] = P::load(a.w + (size_t)c.rb * a.row_bytes + (size_t)blk * P::BLOCK_BYTES, ch);
+    };
+
+    // Weights do not depend on the inputs: start loading the first positions
+    // before anything else, so the stream is already flowing while the inputs
+    // are fetched. kDepth positions stay in flight ahead of the one multiplied
+    // (deeper queues cost registers, hence occupancy, and measured no faster).
+    constexpr int kDepth = 1;
+    typename P::Raw buf[kDepth + 1][kRows];
+    Cursor cc{gwave < units ? gwave : 0u, 0u, 0u, 0u, 0u};
+    place(cc);
+    Cursor lc = cc;
+#pragma unroll
+    for (int dpt = 0; dpt < kDepth; dpt++) {
+        load_at(lc, buf[dpt]);
+        advance(lc);
+    }
+
+    float xr[64];
+    float xsum[NSUM];
+    // Stage the pass's tokens in task order, padded per task (coalesced loads;
+    // a lane's own 64 inputs are 256 bytes apart from its neighbour's).
+    for (uint32_t t = 0; t < (uint32_t)MT; t++) {
+        float4 *dst = lds4 + (size_t)t * tok_stride4;
+        if (t < q.mt) {
+            stage_token(a, q.t0 + t, dst, red, [](uint32_t v) { const uint32_t i = P::stage_index(v); return i + (i >> 4); });
+        } else {
+            for (uint32_t e = tid; e < tok_stride4; e += 256u) dst[e] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+    __syncthreads();
+    if (XREG) {
+        // The lane's one task's inputs into registers, and their run sums in
+        // the same order the LDS pass below adds them.
+        if (gwave >= units) return;
+        const uint32_t task = tsub < tasks ? tsub : 0u;
+        const float4 *src = lds4 + task * (kTaskStride / 4u);
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const float4 f = src[v];
+            xr[4 * v] = f.x; xr[4 * v + 1] = f.y; xr[4 * v + 2] = f.z; xr[4 * v + 3] = f.w;
+        }
+#pragma unroll
+        for (int s = 0; s < NSUM; s++) {
+            xsum[s] = 0.f;
+#pragma unroll
+            for (int e = 0; e < RUN; e++) xsum[s] += xr[s * RUN + e];
+        }
+    } else {
+        for (uint32_t idx = tid; idx < (uint32_t)MT * tasks * NSUM; idx += 256u) {
+            const uint32_t t = idx / (tasks * NSUM), rem = idx % (tasks * NSUM);
+            const float *src = reinterpret_cast<const float *>(lds4 + (size_t)t * tok_stride4) + (rem / NSUM) * kTaskStride + (rem % NSUM) * RUN;
+            float sum = 0.f;
+#pragma unroll
+            for (int e = 0; e < RUN; e++) sum += src[e];
+            sums_lds[idx] = sum;
+        }
+        __syncthreads();
+        if (gwave >= units) return;
+    }
+
+    float acc[kRows][MT];
+#pragma unroll
+    for (int j = 0; j < kRows; j++)
+#pragma unroll
+        for (int t = 0; t < MT; t++) acc[j][t] = 0.f;
+
+    // Multiplies the position `c` from `cur`; at a unit's last slice reduces
+    // and stores its outputs.
+    auto compute = [&](const Cursor &c, const typename P::Raw (&cur)[kRows]) {
+        const uint32_t task = tsub + c.i * seg;
+        if (task < tasks) {
+            const uint32_t ch = task & 3u;
+            float v[kRows][MT];
+            if (XREG) {
+                P::template dot<MT, kRows>(cur, ch, q.nm,
+                    [&](int, int vi) { return make_float4(xr[4 * vi], xr[4 * vi + 1], xr[4 * vi + 2], xr[4 * vi + 3]); },
+                    [&](int, int s) { return xsum[s]; }, v);
+            } else {
+                const float4 *xt = lds4 + task * (kTaskStride / 4u);
+                const float *st = sums_lds + NSUM * task;
+                P::template dot<MT, kRows>(cur, ch, q.nm,
+                    [&](int t, int vi) { return xt[(size_t)t * tok_stride4 + vi]; },
+                    [&](int t, int s) { return st[(size_t)t * tasks * NSUM + s]; }, v);
+            }
+#pragma unroll
+            for (int j = 0; j < kRows; j++)
+#pragma unroll
+                for (int t = 0; t < MT; t++) acc[j][t] += v[j][t];
+        }
+        if (c.i + 1u == iters) {
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                const float s0 = segment_sum(acc[0][t], q.seg_log2);
+                const float s1 = kRows == 2 ? segment_sum(acc[kRows - 1][t], q.seg_log2) : 0.f;
+                acc[0][t] = acc[kRows - 1][t] = 0.f;
+                if (writer && (uint32_t)t < q.mt && c.j0 < a.rows) {
+                    const size_t o = (size_t)(q.t0 + t) * a.out_stride + a.col0 + c.j0;
+                    if (PAIR) {
+                        float r = silu_f(s0) * s1;
+                        if (a.flags & FLAG_ACCUMULATE) r += a.out[o];
+                        a.out[o] = r;
+                    } else {
+                        float r = s0;
+                        if (a.flags & FLAG_ACCUMULATE) r += a.out[o];
+                        a.out[o] = r;
+                        if (kRows == 2 && c.j0 + 1u < a.rows) {
+                            float r1 = s1;
+                            if (a.flags & FLAG_ACCUMULATE) r1 += a.out[o + 1];
+                            a.out[o + 1] = r1;
+                        }
+                    }
+                }
+            }
+        }
+    };
+
+    // The buffers rotate by position, so every index below is a constant.
+    bool done = false;
+    while (!done) {
+#pragma unroll
+        for (int ph = 0; ph <= kDepth; ph++) {
+            if (done) break;
+            load_at(lc, buf[(ph + kDepth) % (kDepth + 1)]);
+            advance(lc);
+            compute(cc, buf[ph]);
+            advance(cc);
+            done = cc.u >= units;
+        }
+    }
+}
+
+template <class P, int MT, bool PAIR, bool XREG>
+static zhip_result run_kquant(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
+    static bool configured = false;  // dynamic LDS above 64 KiB needs opting in once
+    if (lds > 65536u && !configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_kquant_kernel<P, MT, PAIR, XREG>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(d, ZHIP_E_BAD_COMMAND, "%s: k = %u with %d tokens does not fit workgroup memory", P::name(), q.a.k, MT);
+        }
+        configured = true;
+    }
+    hipLaunchKernelGGL((matvec_kquant_kernel<P, MT, PAIR, XREG>), dim3(blocks), dim3(256), lds, d.stream, q);
+    return check_launch(d, P::name());
+}
+
+// Launches the multiply for validated arguments: one pass per group of up to
+// four tokens.
+template <class P>
+static zhip_result launch_kquant(const Dispatch &d, const MvArgs &a) {
+    KArgs q{};
+    q.a = a;
+    q.tasks = a.k / 64u;
+    q.seg_log2 = q.tasks == 16u ? 4u : q.tasks == 32u ? 5u : 6u;
+    q.nm = Masks{0x0f0f0f0fu, 0xf0f0f0f0u, 0x03030303u, 0x01010101u};
+    const bool pair = a.flags & FLAG_SILU_PAIR;
+    const uint32_t rpi = 64u >> q.seg_log2;
+    const uint64_t tok_lds = (uint64_t)q.tasks * kTaskStride * 4u + (uint64_t)q.tasks * P::NSUM * 4u;
+    const uint64_t max_lds = 160u * 1024u - 64u;
+    if (tok_lds > max_lds) return fail(d, ZHIP_E_BAD_COMMAND, "%s: k = %u does not fit workgroup memory", P::name(), a.k);
+    for (uint32_t t0 = 0; t0 < a.m;) {
+        uint32_t left = a.m - t0;
+        uint32_t mt = left >= 3u ? 4u : left;
+        // Two workgroups a CU must fit their staged tokens in the 160 KB of LDS.
+        while (mt > 1u && mt * tok_lds > 80u * 1024u - 64u) mt >>= 1;
+        q.t0 = t0;
+        q.mt = left < mt ? left : mt;
+        const uint32_t lds = (uint32_t)(mt * tok_lds);
+        const bool xreg = a.m == 1u && q.tasks <= 64u;
+        const uint32_t per_unit = pair ? rpi : rpi * (xreg ? 1u : 2u);
+        const uint32_t units = (a.rows + per_unit - 1u) / per_unit;
+        const uint32_t want = (units + 3u) / 4u;
+        // Three workgroups a CU measured best for the 4096 x 14336 multiply:
+        // more of them repeat the input staging, fewer leave too few loads in flight.
+        const uint32_t cap = (uint32_t)d.dev->compute_units * (xreg ? 3u : 2u);
+        const uint32_t blocks = want < cap ? want : cap;
+        zhip_result r;
+        if (xreg) r = pair ? run_kquant<P, 1, true, true>(d, q, lds, blocks) : run_kquant<P, 1, false, true>(d, q, lds, blocks);
+        else if (mt == 1u) r = pair ? run_kquant<P, 1, true, false>(d, q, lds, blocks) : run_kquant<P, 1, false, false>(d, q, lds, blocks);
+        else if (mt == 2u) r = pair ? run_kquant<P, 2, true, false>(d, q, lds, blocks) : run_kquant<P, 2, false, false>(d, q, lds, blocks);
+        else r = pair ? run_kquant<P, 4, true, false>(d, q, lds, blocks) : run_kquant<P, 4, false, false>(d, q, lds, blocks);
+        if (r != ZHIP_OK) return r;
+        t0 += q.mt;
+    }
+    return ZHIP_OK;
+}
+
+zhip_result launch_matvec_kquant(const Dispatch &d, const MvArgs &a, int type) {
+    switch (type) {
+    case 4: return launch_kquant<KQ4>(d, a);
+    case 5: return launch_kquant<KQ5>(d, a);
+    case 6: return launch_kquant<KQ6>(d, a);
+    default: return fail(d, ZHIP_E_BAD_COMMAND, "decode multiply: no K-quant kernel for type %d", type);
+    }
+}
+
+}  // namespace zhip
