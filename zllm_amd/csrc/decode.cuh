@@ -43,7 +43,7 @@ struct DecQ8_0 {
     static constexpr int RUNS = 2;
     static constexpr int E = 16;
     static constexpr uint32_t BLOCK = 32;
-    static constexpr int CHUNK = 0;
+    static constexpr int CHUNK = 8;
     static const char *name() { return "matvec_q8_0"; }
     static uint32_t row_bytes(uint32_t k) { return (k + k / 16u + 15u) & ~15u; }
     __device__ static uint32_t xoff(uint32_t task, int h) { return 16u * task + 8u * h; }
@@ -73,7 +73,7 @@ struct DecQ3_K {
     static constexpr int RUNS = 1;
     static constexpr int E = 32;
     static constexpr uint32_t BLOCK = 256;
-    static constexpr int CHUNK = 0;
+    static constexpr int CHUNK = 3;
     static const char *name() { return "matvec_q3_k"; }
     static uint32_t row_bytes(uint32_t k) { return k / 256u * 128u; }
     __device__ static uint32_t xoff(uint32_t task, int) { return 32u * task; }
@@ -101,7 +101,7 @@ struct DecQ4_K {
     static constexpr int RUNS = 2;
     static constexpr int E = 32;
     static constexpr uint32_t BLOCK = 256;
-    static constexpr int CHUNK = 4;  // has its own multiply (matvec_kquant.hip)
+    static constexpr int CHUNK = 4;  // has its own multiply (matvec_quant.hip)
     static const char *name() { return "matvec_q4_k"; }
     static uint32_t row_bytes(uint32_t k) { return k / 256u * 144u; }
     __device__ static uint32_t xoff(uint32_t task, int h) {

@@ -112,8 +112,8 @@ __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
     }
 }
 
-// The tuned K-quant multiply (matvec_kquant.hip): type 4, 5 or 6.
-zhip_result launch_matvec_kquant(const Dispatch &d, const MvArgs &a, int type);
+// The tuned multiply (matvec_quant.hip): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
+zhip_result launch_matvec_quant(const Dispatch &d, const MvArgs &a, int type);
 
 template <class D, int MT>
 static zhip_result run(const Dispatch &d, const MvArgs &a, uint32_t lds_bytes) {
@@ -187,7 +187,8 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     a.out = reinterpret_cast<float *>(d.bind[3].ptr);
     a.norm_w = norm ? reinterpret_cast<const float *>(d.bind[4].ptr) : nullptr;
 
-    if (D::CHUNK != 0) return launch_matvec_kquant(d, a, D::CHUNK);
+    // The tuned kernel takes rows of whole 64-weight tasks.
+    if (D::CHUNK != 0 && p.k % 64u == 0) return launch_matvec_quant(d, a, D::CHUNK);
 
     // Tokens per pass over the weights: as many as fit workgroup memory.
     const uint64_t row_lds = (uint64_t)p.k * 4u;

@@ -1,12 +1,15 @@
-// matvec_q4_k / matvec_q5_k / matvec_q6_k: out[t][col0 + j] (+)= sum_i X(t, i) * w[j][i]
-// over K-quant rows, the decode step's multiply (contract of
-// src/kernels/matvec_quant.wgsl.hbs with the decoders of
-// src/kernels/quant/q{4,5,6}_k_dot.wgsl; block formulas of src/ref/tensor.zig:94-160).
+// matvec_q8_0 / matvec_q3_k / matvec_q4_k / matvec_q5_k / matvec_q6_k:
+// out[t][col0 + j] (+)= sum_i X(t, i) * w[j][i] over quantized rows, the decode
+// step's multiply (contract of src/kernels/matvec_quant.wgsl.hbs with the
+// decoders of src/kernels/quant/*_dot.wgsl; block formulas of
+// src/ref/tensor.zig:49-160).
 //
-// Layout of the work. A 256-weight block splits into four tasks of 64 weights
-// whose sub-blocks share their scales: for Q4_K and Q5_K a 32-byte chunk of
+// Layout of the work. A row splits into tasks of 64 weights whose sub-blocks
+// share their scales (four to a 256-weight K-quant block; two 32-weight blocks
+// for Q8_0): for Q4_K and Q5_K a 32-byte chunk of
 // nibbles (sub-block 2c in the low nibbles, 2c + 1 in the high ones), for Q6_K
-// sixteen positions of one half (four runs of sixteen weights, 32 apart). The
+// sixteen positions of one half (four runs of sixteen weights, 32 apart), for
+// Q3_K two of the repacked 16-byte units. The
 // lane that owns a task loads its vectors and the block's scales, so every byte
 // of the weight stream is loaded by exactly one lane per use and a wave's load
 // instruction falls in one contiguous span of the matrix. A row has k / 64
@@ -94,6 +97,131 @@ __device__ __forceinline__ float dot_bytes(uint32_t word, const float4 &x, float
 // 4v .. 4v + 3 of the task in task order for token t; sums(t, s) the sum of the
 // task's s-th run of 64 / NSUM inputs.
 
+// Q8_0 split rows (src/kernels/repack_q8_0.wgsl): k signed bytes, then k / 32
+// f16 scales. Task = 64 consecutive weights, two blocks of 32 with a scale each;
+// no minimum, so the input sums go unused.
+struct KQ8 {
+    static constexpr int NSUM = 2;
+    static const char *name() { return "matvec_q8_0"; }
+    struct Raw {
+        uint4 q[4];
+        uint32_t d;  // the two blocks' scales
+    };
+    __device__ static Raw load(const uint8_t *row, uint32_t k, uint32_t task) {
+        Raw r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) r.q[i] = *reinterpret_cast<const uint4 *>(row + 64u * task + 16u * i);
+        r.d = *reinterpret_cast<const uint32_t *>(row + k + 4u * task);
+        return r;
+    }
+    __device__ static uint32_t stage_index(uint32_t v) { return v; }
+
+    template <int MT, int ROWS, class XF, class SF>
+    __device__ static void dot(const Raw (&r)[ROWS], uint32_t, Masks, XF x, SF, float (&out)[ROWS][MT]) {
+        float s[ROWS][MT][2];
+#pragma unroll
+        for (int j = 0; j < ROWS; j++)
+#pragma unroll
+            for (int t = 0; t < MT; t++) s[j][t][0] = s[j][t][1] = 0.f;
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                const float4 xv = x(t, v);
+#pragma unroll
+                for (int j = 0; j < ROWS; j++) {
+                    const uint32_t word = word_of(r[j].q[v >> 2], v & 3);
+                    float sum = s[j][t][v >> 3];
+                    sum = fmaf((float)(int8_t)(word & 0xffu), xv.x, sum);
+                    sum = fmaf((float)(int8_t)((word >> 8) & 0xffu), xv.y, sum);
+                    sum = fmaf((float)(int8_t)((word >> 16) & 0xffu), xv.z, sum);
+                    sum = fmaf((float)(int8_t)(word >> 24), xv.w, sum);
+                    s[j][t][v >> 3] = sum;
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < ROWS; j++) {
+            const float d0 = half_bits_to_float(r[j].d & 0xffffu), d1 = half_bits_to_float(r[j].d >> 16);
+#pragma unroll
+            for (int t = 0; t < MT; t++) out[j][t] = fmaf(d1, s[j][t][1], d0 * s[j][t][0]);
+        }
+    }
+};
+
+// Q3_K: blocks repacked at load into eight self-contained 16-byte units of 32
+// weights (src/kernels/repack_q3_k.wgsl; the layout is spelled out at DecQ3_K):
+// two words of 2-bit values, a word of third bits, scale - 32 for each half as
+// signed bytes, d. A weight is d * (scale - 32) * (q - 4) with q = low bits +
+// 4 * third bit. Task = two consecutive units: four runs of sixteen weights.
+struct KQ3 {
+    static constexpr uint32_t BLOCK_BYTES = 128;
+    static constexpr int NSUM = 4;
+    static const char *name() { return "matvec_q3_k"; }
+    struct Raw {
+        uint4 u[2];
+    };
+    __device__ static Raw load(const uint8_t *row, uint32_t, uint32_t task) {
+        const uint8_t *block = row + (size_t)(task >> 2) * BLOCK_BYTES;
+        const uint32_t c = task & 3u;
+        Raw r;
+        r.u[0] = *reinterpret_cast<const uint4 *>(block + 32u * c);
+        r.u[1] = *reinterpret_cast<const uint4 *>(block + 32u * c + 16u);
+        return r;
+    }
+    __device__ static uint32_t stage_index(uint32_t v) { return v; }
+
+    template <int MT, int ROWS, class XF, class SF>
+    __device__ static void dot(const Raw (&r)[ROWS], uint32_t, Masks nm, XF x, SF sums, float (&out)[ROWS][MT]) {
+        float s[ROWS][MT][4];
+#pragma unroll
+        for (int j = 0; j < ROWS; j++)
+#pragma unroll
+            for (int t = 0; t < MT; t++)
+#pragma unroll
+                for (int run = 0; run < 4; run++) s[j][t][run] = 0.f;
+#pragma unroll
+        for (int unit = 0; unit < 2; unit++) {
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                uint32_t q[ROWS];
+#pragma unroll
+                for (int j = 0; j < ROWS; j++) {
+                    const uint4 &u = r[j].u[unit];
+                    const uint32_t low = ((e < 4 ? u.x : u.y) >> (2 * (e & 3))) & nm.two;
+                    const uint32_t third = (u.z >> e) & nm.one;
+                    q[j] = (third << 2) | low;
+                }
+                const int run = 2 * unit + (e >> 2);
+#pragma unroll
+                for (int t = 0; t < MT; t++) {
+                    const float4 xv = x(t, 8 * unit + e);
+#pragma unroll
+                    for (int j = 0; j < ROWS; j++) s[j][t][run] = dot_bytes(q[j], xv, s[j][t][run]);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < ROWS; j++) {
+            float scale[4];
+#pragma unroll
+            for (int unit = 0; unit < 2; unit++) {
+                const uint32_t tail = r[j].u[unit].w;
+                const float d = half_bits_to_float(tail >> 16);
+                scale[2 * unit] = d * (float)(int8_t)(tail & 0xffu);
+                scale[2 * unit + 1] = d * (float)(int8_t)((tail >> 8) & 0xffu);
+            }
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                float v = 0.f;
+#pragma unroll
+                for (int run = 0; run < 4; run++) v = fmaf(scale[run], fmaf(-4.f, sums(t, run), s[j][t][run]), v);
+                out[j][t] = v;
+            }
+        }
+    }
+};
+
 // Q4_K: 144-byte blocks (header vector; 128 bytes of nibbles in four chunks of
 // 32: chunk c holds sub-block 2c in its low nibbles and 2c + 1 in its high
 // ones). Task = chunk: 32 low-nibble weights, then 32 high-nibble ones.
@@ -104,7 +232,9 @@ struct KQ4 {
     struct Raw {
         uint4 h, q0, q1;
     };
-    __device__ static Raw load(const uint8_t *block, uint32_t c) {
+    __device__ static Raw load(const uint8_t *row, uint32_t, uint32_t task) {
+        const uint8_t *block = row + (size_t)(task >> 2) * BLOCK_BYTES;
+        const uint32_t c = task & 3u;
         Raw r;
         r.h = *reinterpret_cast<const uint4 *>(block);
         r.q0 = *reinterpret_cast<const uint4 *>(block + 16u + 32u * c);
@@ -164,7 +294,9 @@ struct KQ5 {
     struct Raw {
         uint4 h, b0, b1, q0, q1;
     };
-    __device__ static Raw load(const uint8_t *block, uint32_t c) {
+    __device__ static Raw load(const uint8_t *row, uint32_t, uint32_t task) {
+        const uint8_t *block = row + (size_t)(task >> 2) * BLOCK_BYTES;
+        const uint32_t c = task & 3u;
         Raw r;
         r.h = *reinterpret_cast<const uint4 *>(block);
         r.b0 = *reinterpret_cast<const uint4 *>(block + 16u);
@@ -232,8 +364,9 @@ struct KQ6 {
         uint2 sc;
         uint32_t d;
     };
-    __device__ static Raw load(const uint8_t *block, uint32_t p) {
-        const uint32_t n = p >> 1, lh = p & 1u;
+    __device__ static Raw load(const uint8_t *row, uint32_t, uint32_t task) {
+        const uint8_t *block = row + (size_t)(task >> 2) * BLOCK_BYTES;
+        const uint32_t n = (task >> 1) & 1u, lh = task & 1u;
         Raw r;
         r.l0 = *reinterpret_cast<const uint4 *>(block + 64u * n + 16u * lh);
         r.l1 = *reinterpret_cast<const uint4 *>(block + 64u * n + 32u + 16u * lh);
@@ -328,7 +461,7 @@ struct KArgs {
 };
 
 template <class P, int MT, bool PAIR, bool XREG>
-__global__ __launch_bounds__(256) void matvec_kquant_kernel(KArgs q) {
+__global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     const MvArgs &a = q.a;
     extern __shared__ float4 lds4[];
     __shared__ float red[4];
@@ -378,9 +511,8 @@ __global__ __launch_bounds__(256) void matvec_kquant_kernel(KArgs q) {
     auto load_at = [&](const Cursor &c, typename P::Raw (&dst)[kRows]) {
         const uint32_t task = tsub + c.i * seg;
         const uint32_t tk = task < tasks ? task : 0u;
-        const uint32_t blk = tk >> 2, ch = tk & 3u;
-        dst[0] = P::load(a.w + (size_t)c.ra * a.row_bytes + (size_t)blk * P::BLOCK_BYTES, ch);
-        if (kRows == 2) dst[kRows - 1] = P::load(a.w + (size_t)c.rb * a.row_bytes + (size_t)blk * P::BLOCK_BYTES, ch);
+        dst[0] = P::load(a.w + (size_t)c.ra * a.row_bytes, a.k, tk);
+        if (kRows == 2) dst[kRows - 1] = P::load(a.w + (size_t)c.rb * a.row_bytes, a.k, tk);
     };
 
     // Weights do not depend on the inputs: start loading the first positions
@@ -513,23 +645,23 @@ __global__ __launch_bounds__(256) void matvec_kquant_kernel(KArgs q) {
 }
 
 template <class P, int MT, bool PAIR, bool XREG>
-static zhip_result run_kquant(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
+static zhip_result run_quant(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
     static bool configured = false;  // dynamic LDS above 64 KiB needs opting in once
     if (lds > 65536u && !configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_kquant_kernel<P, MT, PAIR, XREG>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_quant_kernel<P, MT, PAIR, XREG>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
             (void)hipGetLastError();
             return fail(d, ZHIP_E_BAD_COMMAND, "%s: k = %u with %d tokens does not fit workgroup memory", P::name(), q.a.k, MT);
         }
         configured = true;
     }
-    hipLaunchKernelGGL((matvec_kquant_kernel<P, MT, PAIR, XREG>), dim3(blocks), dim3(256), lds, d.stream, q);
+    hipLaunchKernelGGL((matvec_quant_kernel<P, MT, PAIR, XREG>), dim3(blocks), dim3(256), lds, d.stream, q);
     return check_launch(d, P::name());
 }
 
 // Launches the multiply for validated arguments: one pass per group of up to
 // four tokens.
 template <class P>
-static zhip_result launch_kquant(const Dispatch &d, const MvArgs &a) {
+static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
     KArgs q{};
     q.a = a;
     q.tasks = a.k / 64u;
@@ -557,22 +689,24 @@ static zhip_result launch_kquant(const Dispatch &d, const MvArgs &a) {
         const uint32_t cap = (uint32_t)d.dev->compute_units * (xreg ? 3u : 2u);
         const uint32_t blocks = want < cap ? want : cap;
         zhip_result r;
-        if (xreg) r = pair ? run_kquant<P, 1, true, true>(d, q, lds, blocks) : run_kquant<P, 1, false, true>(d, q, lds, blocks);
-        else if (mt == 1u) r = pair ? run_kquant<P, 1, true, false>(d, q, lds, blocks) : run_kquant<P, 1, false, false>(d, q, lds, blocks);
-        else if (mt == 2u) r = pair ? run_kquant<P, 2, true, false>(d, q, lds, blocks) : run_kquant<P, 2, false, false>(d, q, lds, blocks);
-        else r = pair ? run_kquant<P, 4, true, false>(d, q, lds, blocks) : run_kquant<P, 4, false, false>(d, q, lds, blocks);
+        if (xreg) r = pair ? run_quant<P, 1, true, true>(d, q, lds, blocks) : run_quant<P, 1, false, true>(d, q, lds, blocks);
+        else if (mt == 1u) r = pair ? run_quant<P, 1, true, false>(d, q, lds, blocks) : run_quant<P, 1, false, false>(d, q, lds, blocks);
+        else if (mt == 2u) r = pair ? run_quant<P, 2, true, false>(d, q, lds, blocks) : run_quant<P, 2, false, false>(d, q, lds, blocks);
+        else r = pair ? run_quant<P, 4, true, false>(d, q, lds, blocks) : run_quant<P, 4, false, false>(d, q, lds, blocks);
         if (r != ZHIP_OK) return r;
         t0 += q.mt;
     }
     return ZHIP_OK;
 }
 
-zhip_result launch_matvec_kquant(const Dispatch &d, const MvArgs &a, int type) {
+zhip_result launch_matvec_quant(const Dispatch &d, const MvArgs &a, int type) {
     switch (type) {
-    case 4: return launch_kquant<KQ4>(d, a);
-    case 5: return launch_kquant<KQ5>(d, a);
-    case 6: return launch_kquant<KQ6>(d, a);
-    default: return fail(d, ZHIP_E_BAD_COMMAND, "decode multiply: no K-quant kernel for type %d", type);
+    case 8: return launch_quant<KQ8>(d, a);
+    case 3: return launch_quant<KQ3>(d, a);
+    case 4: return launch_quant<KQ4>(d, a);
+    case 5: return launch_quant<KQ5>(d, a);
+    case 6: return launch_quant<KQ6>(d, a);
+    default: return fail(d, ZHIP_E_BAD_COMMAND, "decode multiply: no tuned kernel for type %d", type);
     }
 }
 
