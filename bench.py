@@ -45,7 +45,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,c5 for the 'also' section; 'none' skips it")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,c5,formats for the 'also' section; 'none' skips it")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run 4 plain elementwise copies (256 MiB read + 256 MiB written each) so a counter run has a kernel of known traffic to scale by")
@@ -273,7 +273,7 @@ def main() -> int:
     only = [s for s in args.only.split(",") if s]
     also = {}
     if "none" not in only:
-        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c4_int8", bench_c4_int8), ("c5", bench_c5)):
+        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c4_int8", bench_c4_int8), ("c5", bench_c5), ("formats", bench_formats)):
             if not only or name in only:
                 try:
                     also[name] = fn(locals())
@@ -301,6 +301,29 @@ def bench_c1(env):
     nbytes = n * k // 32 * 34 + 4 * k + 4 * n  # GGUF bytes: 3,358,720
     return env["hbm_entry"]("C1: Q8_0 decode matvec M=1 K=1024 N=3072", nbytes, wall, gpu_s, steps,
                             {"copies": len(launches), "max_err_over_row_x_norms": bound, "max_err_over_max_want": rel})
+
+
+def bench_formats(env):
+    """The decode multiply at C2's shape (M = 1, K = 4096, N = 14336) for the other
+    GGUF formats the kernel reads: algorithmic bytes are the file's bytes per row."""
+    synth, oracle, K, TensorType = env["synth"], env["oracle"], env["K"], env["TensorType"]
+    n, k = 14336, 4096
+    x = synth.activations(synth.rng(0xF0), 1, k)
+    steps = max(1, env["args"].steps // 2)
+    res = {}
+    for name, ot in (("q8_0", oracle.Q8_0), ("q6_k", oracle.Q6_K), ("q5_k", oracle.Q5_K), ("q3_k", oracle.Q3_K)):
+        t = TensorType[name]
+        raw = synth.random_blocks(synth.rng(0xF1), name, n, k)
+        launches, out = env["matvec_workload"](t, raw, n, k, 1, False, x)
+        wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 2))
+        got = env["read"](out)[:n].reshape(1, n)
+        w = oracle.dequantize(ot, raw, n * k).reshape(n, k)
+        bound, rel = env["check_matvec"](got, oracle.matmul_f64(x, w), w, x)
+        e, bb = K.LAYOUT[t]
+        nbytes = n * (k // e) * bb + 4 * k + 4 * n
+        res[name] = env["hbm_entry"](f"{name} decode matvec M=1 K={k} N={n}", nbytes, wall, gpu_s, steps,
+                                     {"copies": len(launches), "max_err_over_row_x_norms": bound, "max_err_over_max_want": rel})
+    return res
 
 
 def bench_c3(env):
