@@ -150,7 +150,7 @@ def main() -> int:
     def rotation(w_bytes: int) -> int:
         return max(2, -(-ROTATE_BYTES // w_bytes))
 
-    def matvec_workload(t: TensorType, raw_rows: np.ndarray, n_out: int, k: int, m: int, pair: bool, x: np.ndarray):
+    def matvec_workload(t: TensorType, raw_rows: np.ndarray, n_out: int, k: int, m: int, pair: bool, x: np.ndarray, variant=None):
         """Uploads a rotation of weight copies and builds one launch per copy."""
         kernel = K.weight_kernel("matvec", t)
         rb = K.row_bytes(t, k)
@@ -170,7 +170,7 @@ def main() -> int:
                 rec.copy_buffer(src.buffer, 0, buf, 0, src.size)
                 wa = K.Arg(buf, src.size)
             first = first or wa
-            v = K.MatvecVariant()
+            v = variant or K.MatvecVariant()
             p = P.MatvecBf16(n=n_out, k=k, col0=0, out_stride=n_out, silu_pair=pair, half=n_out if pair else 0)
             if K.is_half(t):
                 launches.append(L(b.add(kernel, p, [xa, wa, out, wa], K.Grid.rows_y(K.div_ceil(n_out, K.matvec_rows))), m))
@@ -336,9 +336,13 @@ def bench_c3(env):
     w = oracle.dequantize(oracle.Q4_K, raw, 2 * n * k).reshape(2 * n, k)
     steps = max(1, env["args"].steps // 2)
     res = {}
-    for m in (1, 4, 8):
+    # The default variant, and for the multi-token steps the matrix-core variant
+    # (MatvecVariant wg 512, lanes 64, rows 16) a tuner would pick for them.
+    for m, variant, tag in ((1, None, "m1"), (4, None, "m4"), (8, None, "m8"),
+                            (4, K.MatvecVariant(wg=512, lanes=64, rows=16), "m4_matrix_cores"),
+                            (8, K.MatvecVariant(wg=512, lanes=64, rows=16), "m8_matrix_cores")):
         x = synth.activations(synth.rng(0xC30 + m), m, k)
-        launches, out = env["matvec_workload"](TensorType.q4_k, raw, n, k, m, True, x)
+        launches, out = env["matvec_workload"](TensorType.q4_k, raw, n, k, m, True, x, variant)
         wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 2))
         got = env["read"](out)[: m * n].reshape(m, n).astype(np.float64)
         both = oracle.matmul_f64(x, w)
@@ -346,8 +350,8 @@ def bench_c3(env):
         want = gt / (1 + np.exp(-gt)) * u
         rel = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
         nbytes = 2 * n * K.row_bytes(TensorType.q4_k, k) + m * 4 * k + m * 4 * n
-        res[f"m{m}"] = env["hbm_entry"](f"C3: fused gate+up Q4_K + SiLU*mul, M={m}, K=4096, N=2x14336", nbytes, wall, gpu_s, steps,
-                                        {"copies": len(launches), "max_err_over_max_want": rel})
+        name = f"C3: fused gate+up Q4_K + SiLU*mul, M={m}, K=4096, N=2x14336" + (", matrix-core variant" if variant else "")
+        res[tag] = env["hbm_entry"](name, nbytes, wall, gpu_s, steps, {"copies": len(launches), "max_err_over_max_want": rel})
     return res
 
 

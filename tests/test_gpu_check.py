@@ -192,6 +192,51 @@ def test_quant_matvec_eight_rows(ctx):
         assert got[tk].tobytes() == c.read(single)[:n].tobytes()
 
 
+MFMA_VARIANT = K.MatvecVariant(wg=512, lanes=64, rows=16)
+
+
+@pytest.mark.parametrize("pair,rows,n,k", [
+    (True, 8, 200, 1024),     # partial last tile, one slab
+    (True, 5, 96, 4096),      # four slabs
+    (False, 3, 100, 2048),    # accumulate epilogue, an odd token count
+    (False, 1, 530, 1024),    # one token, more than one workgroup
+])
+def test_quant_matvec_mfma_variant(ctx, pair, rows, n, k):
+    """The matrix-core variant of matvec_q4_k (a wave per sixteen rows): every
+    row within 1e-5 of float64 over the decoded weights, each token bitwise
+    equal to its lone launch, and nothing outside the outputs touched."""
+    c = ctx
+    x = c.random(rows * k, 3).reshape(rows, k)
+    x[0] *= np.float32(1e-4)          # tokens of very different magnitudes
+    x[rows - 1] *= np.float32(300.0)
+    raw, values = quant_rows(c, TensorType.q4_k, 2 * n if pair else n, k)
+    stride = n + 7
+    init = c.random(rows * stride, 2).reshape(rows, stride)
+    xa, wa = c.upload(x), c.gpu_weights(TensorType.q4_k, raw, k)
+    v64, x64 = values.astype(np.float64), x.astype(np.float64)
+    if pair:
+        g, u = x64 @ v64[:n].T, x64 @ v64[n:].T
+        want = g * sigmoid64(g) * u
+    else:
+        want = init[:, 3 : 3 + n] + x64 @ v64.T
+    p = lambda: P.MatvecBf16(n=n, k=k, col0=3, out_stride=stride, accumulate=not pair, silu_pair=pair, half=n if pair else 0)
+    pipeline = c.set.matvec(c.rec, Kernel.matvec_q4_k, MFMA_VARIANT)
+    grid_x = K.div_ceil(n, MFMA_VARIANT.group_rows())
+    out = c.upload(init)
+    c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, wa], (grid_x, rows, 1))
+    got = c.read(out).reshape(rows, stride)
+    # Row by row: each token against its own output scale.
+    for tk in range(rows):
+        assert rel_err(got[tk, 3 : 3 + n], want[tk]) <= 1e-5, tk
+    mask = np.ones(stride, dtype=bool)
+    mask[3 : 3 + n] = False
+    assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32))
+    for tk in range(rows):
+        single = c.upload(init[tk])
+        c.launcher().launch_pipeline(pipeline, p(), [c.upload(x[tk]), wa, single, wa], (grid_x, 1, 1))
+        assert got[tk].tobytes() == c.read(single)[:stride].tobytes(), "a token's sums differ between a lone launch and a multi-token launch"
+
+
 # ---- block decoders bit for bit, through the embedding gathers: check.zig:873-905 -----
 
 @pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q3_k, TensorType.q4_k, TensorType.q5_k, TensorType.q6_k])

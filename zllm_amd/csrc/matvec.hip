@@ -112,6 +112,9 @@ __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
     }
 }
 
+// The matrix-core variant of matvec_q4_k (matvec_mfma.hip).
+bool matvec_q4k_mfma_accepts(const MvArgs &a);
+zhip_result launch_matvec_q4k_mfma(const Dispatch &d, const MvArgs &a, uint64_t x_bytes, uint64_t w_bytes);
 // The tuned multiply (matvec_quant.hip): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
 zhip_result launch_matvec_quant(const Dispatch &d, const MvArgs &a, int type);
 
@@ -187,6 +190,9 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     a.out = reinterpret_cast<float *>(d.bind[3].ptr);
     a.norm_w = norm ? reinterpret_cast<const float *>(d.bind[4].ptr) : nullptr;
 
+    // MatvecVariant (wg 512, lanes 64, rows 16) names the matrix-core variant: a wave per sixteen rows.
+    if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && v.act_div == 0u && matvec_q4k_mfma_accepts(a))
+        return launch_matvec_q4k_mfma(d, a, d.bind[1].size, d.bind[2].size);
     // The tuned kernel takes rows of whole 64-weight tasks.
     if (D::CHUNK != 0 && p.k % 64u == 0) return launch_matvec_quant(d, a, D::CHUNK);
 
