@@ -141,9 +141,7 @@ static void q4_k_block(const uint8_t *b, float *y) {
  * 0..7 by nibble, top two in bytes 8..11), dl = d * (scale - 32), weight l of
  * half n and shift j = dl * (two bits 2j of qs[32n + l], minus 4 unless bit
  * 4n + j of hmask[l] is set). */
-static void q3_k_block(const uint8_t *b, float *y) {
-    const uint8_t *hm = b;
-    float d_all = zref_half(rd16(b + 108));
+static void q3_k_scales(const uint8_t *b, int8_t scales[16]) {
     uint32_t aux[4];
     for (int i = 0; i < 3; i++) aux[i] = rd32(b + 96 + 4 * i);
     const uint32_t kmask1 = 0x03030303u, kmask2 = 0x0f0f0f0fu;
@@ -152,8 +150,14 @@ static void q3_k_block(const uint8_t *b, float *y) {
     aux[3] = ((aux[1] >> 4) & kmask2) | (((tmp >> 6) & kmask1) << 4);
     aux[0] = (aux[0] & kmask2) | (((tmp >> 0) & kmask1) << 4);
     aux[1] = (aux[1] & kmask2) | (((tmp >> 2) & kmask1) << 4);
-    int8_t scales[16];
     for (int i = 0; i < 16; i++) scales[i] = (int8_t)((aux[i / 4] >> (8 * (i % 4))) & 0xff);
+}
+
+static void q3_k_block(const uint8_t *b, float *y) {
+    const uint8_t *hm = b;
+    float d_all = zref_half(rd16(b + 108));
+    int8_t scales[16];
+    q3_k_scales(b, scales);
     size_t out = 0;
     unsigned is = 0;
     uint8_t m = 1;
@@ -799,43 +803,87 @@ int zref_quantize_q8_rows(const float *x, size_t rows, size_t k, unsigned block,
     return r;
 }
 
-/* out[t][j] = sum over 32-weight units of dx * (s * sum(q * qx) - m * sum(qx))
+/* Unit u (32 weights) of a 256-weight block as the int8 prefill multiply sees
+ * it: signed integers q, a scale for each half of sixteen and a minimum
+ * (src/kernels/quant/q3_k.wgsl, q4_k.wgsl, q5_k.wgsl, q6_k.wgsl: head, scales,
+ * quad_i8). b is the block as the file stores it. */
+static void kquant_unit(int type, const uint8_t *b, unsigned u, int32_t q[32], float *s0, float *s1, float *mn) {
+    if (type == ZREF_Q4_K || type == ZREF_Q5_K) {
+        float d = zref_half(rd16(b)), dmin = zref_half(rd16(b + 2));
+        uint8_t sc, m;
+        zref_scale_min_k4(u, b + 4, &sc, &m);
+        const uint8_t *qs = b + (type == ZREF_Q4_K ? 16 : 48) + 32 * (u / 2);
+        for (unsigned i = 0; i < 32; i++) {
+            q[i] = u & 1 ? qs[i] >> 4 : qs[i] & 0xF;
+            if (type == ZREF_Q5_K) q[i] += ((b[16 + i] >> u) & 1) << 4;
+        }
+        *s0 = *s1 = d * (float)sc;
+        *mn = dmin * (float)m;
+    } else if (type == ZREF_Q6_K) {
+        unsigned n = u / 4, c = u % 4;
+        float d = zref_half(rd16(b + 208));
+        const uint8_t *ql = b + 64 * n + 32 * (c % 2), *qh = b + 128 + 32 * n;
+        const int8_t *sc = (const int8_t *)(b + 192 + 8 * n + 2 * c);
+        for (unsigned i = 0; i < 32; i++)
+            q[i] = (int32_t)(((ql[i] >> (4 * (c / 2))) & 0xF) | (((qh[i] >> (2 * c)) & 3) << 4)) - 32;
+        *s0 = d * (float)sc[0];
+        *s1 = d * (float)sc[1];
+        *mn = 0.f;
+    } else {  /* ZREF_Q3_K */
+        unsigned n = u / 4, j = u % 4;
+        float d = zref_half(rd16(b + 108));
+        int8_t scales[16];
+        q3_k_scales(b, scales);
+        for (unsigned i = 0; i < 32; i++)
+            q[i] = (int32_t)((b[32 + 32 * n + i] >> (2 * j)) & 3) - (((b[i] >> (4 * n + j)) & 1) ? 0 : 4);
+        *s0 = d * (float)((int)scales[8 * n + 2 * j] - 32);
+        *s1 = d * (float)((int)scales[8 * n + 2 * j + 1] - 32);
+        *mn = 0.f;
+    }
+}
+
+/* out[t][j] = sum over 32-weight units of dx * (s0 * sum(q * qx) over the first
+ * sixteen + s1 * the same over the second sixteen - m * sum(qx))
  * (src/kernels/matmul_quant.wgsl:1-9,130-160), the integer sums exact and the
- * scaled terms added in double. Weights are file-layout blocks (Q8_0: 34-byte
- * blocks; Q4_K: 144-byte blocks); dx has one scale per 32 (Q8_0) or 256 (Q4_K)
- * activations. */
+ * scaled terms added in double. Weights are file-layout blocks (Q8_0: 34
+ * bytes; Q3_K 110; Q4_K 144; Q5_K 176; Q6_K 210); dx has one scale per 32
+ * (Q8_0) or 256 (the K formats) activations. */
 int zref_matmul_q8(int type, const uint8_t *w, const int8_t *qx, const float *dx, size_t rows, size_t n, size_t k, double *out) {
-    if (type != ZREF_Q8_0 && type != ZREF_Q4_K) return -1;
+    size_t bb;
+    switch (type) {
+    case ZREF_Q8_0: bb = 34; break;
+    case ZREF_Q3_K: bb = 110; break;
+    case ZREF_Q4_K: bb = 144; break;
+    case ZREF_Q5_K: bb = 176; break;
+    case ZREF_Q6_K: bb = 210; break;
+    default: return -1;
+    }
     for (size_t t = 0; t < rows; t++) {
         const int8_t *xr = qx + t * k;
         for (size_t j = 0; j < n; j++) {
             double sum = 0;
             if (type == ZREF_Q8_0) {
-                const uint8_t *row = w + j * (k / 32) * 34;
+                const uint8_t *row = w + j * (k / 32) * bb;
                 for (size_t u = 0; u < k / 32; u++) {
-                    const uint8_t *b = row + u * 34;
+                    const uint8_t *b = row + u * bb;
                     int32_t dot = 0;
                     for (unsigned i = 0; i < 32; i++) dot += (int32_t)(int8_t)b[2 + i] * xr[u * 32 + i];
                     sum += (double)dx[t * (k / 32) + u] * ((double)zref_half(rd16(b)) * dot);
                 }
             } else {
-                const uint8_t *row = w + j * (k / 256) * 144;
+                const uint8_t *row = w + j * (k / 256) * bb;
                 for (size_t blk = 0; blk < k / 256; blk++) {
-                    const uint8_t *b = row + blk * 144;
-                    float dd = zref_half(rd16(b)), dmin = zref_half(rd16(b + 2));
-                    for (unsigned sb = 0; sb < 8; sb++) {
-                        uint8_t sc, m;
-                        zref_scale_min_k4(sb, b + 4, &sc, &m);
-                        const uint8_t *qs = b + 16 + 32 * (sb / 2);
-                        int32_t dot = 0, xs = 0;
+                    for (unsigned u = 0; u < 8; u++) {
+                        int32_t q[32], dot0 = 0, dot1 = 0, xs = 0;
+                        float s0, s1, mn;
+                        kquant_unit(type, row + blk * bb, u, q, &s0, &s1, &mn);
                         for (unsigned i = 0; i < 32; i++) {
-                            int32_t qv = sb & 1 ? qs[i] >> 4 : qs[i] & 0xF;
-                            int32_t xv = xr[blk * 256 + sb * 32 + i];
-                            dot += qv * xv;
+                            int32_t xv = xr[blk * 256 + u * 32 + i];
+                            if (i < 16) dot0 += q[i] * xv;
+                            else dot1 += q[i] * xv;
                             xs += xv;
                         }
-                        float s = dd * (float)sc, mn = dmin * (float)m;
-                        sum += (double)dx[t * (k / 256) + blk] * ((double)s * dot - (double)mn * xs);
+                        sum += (double)dx[t * (k / 256) + blk] * ((double)s0 * dot0 + (double)s1 * dot1 - (double)mn * xs);
                     }
                 }
             }

@@ -166,7 +166,7 @@ int zref_quantize_q8_rows(const float *x, size_t rows, size_t k, unsigned block,
                           const float *nw, int8_t *q, float *d);
 /* The int8 prefill multiply's formula (src/kernels/matmul_quant.wgsl:1-9):
  * exact integer unit sums, scaled and added in double. `w` is file-layout
- * Q8_0 or Q4_K rows. */
+ * Q8_0, Q3_K, Q4_K, Q5_K or Q6_K rows. */
 int zref_matmul_q8(int type, const uint8_t *w, const int8_t *qx, const float *dx, size_t rows, size_t n, size_t k, double *out);
 
 #ifdef __cplusplus

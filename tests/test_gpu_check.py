@@ -554,7 +554,7 @@ def launch_int8(c, t, act, wa, out, rows, n, k, accumulate, slices, col0=0, stri
              [partials, out], K.elementwise(rows * n))
 
 
-@pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q4_k])
+@pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q4_k, TensorType.q5_k, TensorType.q6_k, TensorType.q3_k])
 def test_matmul_int8_whole_and_split(ctx, t):
     """The prefill multiply on quantize_q8's output, accumulating, over more than
     one tile each way: whole, and split over k into partials that matmul_reduce
@@ -595,6 +595,9 @@ def test_matmul_int8_whole_and_split(ctx, t):
     (TensorType.q8_0, 130, 200, 4096),
     (TensorType.q4_k, 1, 129, 2048),
     (TensorType.q4_k, 257, 64, 1536),
+    (TensorType.q5_k, 65, 129, 768),
+    (TensorType.q6_k, 129, 65, 1280),
+    (TensorType.q3_k, 3, 200, 512),
 ])
 def test_matmul_int8_shapes(ctx, t, rows, n, k):
     """Partial tiles each way, a padded output stride and a nonzero first column;

@@ -154,7 +154,7 @@ def test_quantize_fused_modes():
     assert np.max(np.abs(got - want) / (step / 2)) <= 1.0001
 
 
-@pytest.mark.parametrize("t,name", [(oracle.Q8_0, "q8_0"), (oracle.Q4_K, "q4_k")])
+@pytest.mark.parametrize("t,name", [(oracle.Q8_0, "q8_0"), (oracle.Q4_K, "q4_k"), (oracle.Q5_K, "q5_k"), (oracle.Q6_K, "q6_k"), (oracle.Q3_K, "q3_k")])
 def test_matmul_q8_equals_rounded_activations_times_decoded_weights(t, name):
     """The unit formula dx * (s * sum(q qx) - m * sum(qx)) is algebraically the
     product of the rounded activations with the decoded weights
@@ -170,7 +170,8 @@ def test_matmul_q8_equals_rounded_activations_times_decoded_weights(t, name):
     xs = q.astype(np.float64) * np.repeat(d, block, axis=1).astype(np.float64)
     want = xs @ values.astype(np.float64).T
     scale = np.max(np.abs(want))
-    # Q4_K's decoded weight d*sc*q - dmin*m is rounded to f32 by the decoder,
-    # the unit formula keeps the two terms apart: they differ by f32 roundings.
+    # A K format's decoded weight (d*sc*q - dmin*m, d*sc*(q - 32) ...) is rounded to
+    # f32 by the decoder, the unit formula keeps the integer sums exact: they
+    # differ by f32 roundings.
     tol = 1e-12 if t == oracle.Q8_0 else 2e-7
     assert np.max(np.abs(got - want)) <= tol * scale

@@ -105,7 +105,10 @@ zhip_result launch_matvec_bf16(const Dispatch &);
 zhip_result launch_matmul_reduce(const Dispatch &);
 zhip_result launch_quantize_q8(const Dispatch &);
 zhip_result launch_matmul_q8_0(const Dispatch &);
+zhip_result launch_matmul_q3_k(const Dispatch &);
 zhip_result launch_matmul_q4_k(const Dispatch &);
+zhip_result launch_matmul_q5_k(const Dispatch &);
+zhip_result launch_matmul_q6_k(const Dispatch &);
 zhip_result launch_silu_mul(const Dispatch &);
 zhip_result launch_repack_q8_0(const Dispatch &);
 zhip_result launch_repack_q3_k(const Dispatch &);

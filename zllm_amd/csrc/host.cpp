@@ -93,7 +93,10 @@ static const KernelInfo kImplemented[] = {
     {"matmul_bf16", 4, 0b1000, VariantKind::prefill, launch_matmul_bf16_f32, launch_matmul_bf16_mfma, launch_matmul_bf16_mfma_xbf16, 1},
     {"matmul_q8_0_float", 4, 0b1000, VariantKind::prefill, launch_matmul_q8_0_float_f32, launch_matmul_q8_0_float_mfma, launch_matmul_q8_0_float_mfma_xbf16, 1},
     {"matmul_q8_0", 5, 0b01000, VariantKind::none, launch_matmul_q8_0, nullptr, nullptr, 1},
+    {"matmul_q3_k", 5, 0b01000, VariantKind::none, launch_matmul_q3_k, nullptr, nullptr, 1},
     {"matmul_q4_k", 5, 0b01000, VariantKind::none, launch_matmul_q4_k, nullptr, nullptr, 1},
+    {"matmul_q5_k", 5, 0b01000, VariantKind::none, launch_matmul_q5_k, nullptr, nullptr, 1},
+    {"matmul_q6_k", 5, 0b01000, VariantKind::none, launch_matmul_q6_k, nullptr, nullptr, 1},
     {"quantize_q8", 5, 0b01100, VariantKind::none, launch_quantize_q8, nullptr, nullptr, 1},
     {"matmul_reduce", 3, 0b100, VariantKind::none, launch_matmul_reduce, nullptr, nullptr, 1},
     {"silu_mul", 3, 0b100, VariantKind::none, launch_silu_mul, nullptr, nullptr, 1},

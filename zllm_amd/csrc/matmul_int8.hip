@@ -1,4 +1,4 @@
-// matmul_q8_0 / matmul_q4_k: the prefill multiply on activations rounded to
+// matmul_q8_0 / matmul_q3_k / matmul_q4_k / matmul_q5_k / matmul_q6_k: the prefill multiply on activations rounded to
 // 8-bit blocks (quantize_q8), as src/kernels/matmul_quant.wgsl defines it:
 //   out[t][col0 + j] = sum over 32-weight units of dx * (s * sum(q * qx) - m * sum(qx))
 // with every unit's integer sum exact. Here the unit sums run on the int8 matrix
@@ -235,11 +235,121 @@ __device__ __forceinline__ void store_tile(const I8Args &a, const if32x4 (&acc)[
     }
 }
 
-// ---- Q4_K weights (144-byte super-blocks as in the file), Q8_K activations ----------
-__global__ __launch_bounds__(256) void matmul_q4_k_i8_kernel(I8Args a) {
-        __shared__ __align__(16) uint8_t lds_q[2][TT * LINE];
+// ---- K formats (256-weight blocks), Q8_K activations ---------------------------------
+// A format gives the bytes a lane loads for one block of its row (Raw, load) and
+// unit u's operand: the eight signed integers at positions 8 g .. 8 g + 7 of the
+// unit with the scales of the unit's two halves of sixteen and its minimum
+// (src/kernels/quant/q3_k.wgsl, q4_k.wgsl, q5_k.wgsl, q6_k.wgsl: head, scales, quad_i8).
+// HALVES: the two halves' scales differ, so a unit takes two instructions, each
+// with the other half's lanes feeding zeros.
+
+__device__ __forceinline__ int sbyte(uint32_t word, uint32_t i) { return (int)(word << (24u - 8u * i)) >> 24; }
+
+struct I8Q4 {
+    static constexpr uint32_t BLOCK = 144;
+    static constexpr bool HAS_MIN = true, HALVES = false;
+    struct Raw {
+        iu32x4 h;       // d, dmin and the twelve scale bytes
+        iu32x2 q[4];    // 8 bytes of each 64-weight chunk: low nibbles unit 2c, high 2c + 1
+    };
+    static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t w, uint32_t blk, uint32_t g, Raw &r) {
+        r.h = __builtin_amdgcn_raw_buffer_load_b128(w, blk, 0, 0);
+#pragma unroll
+        for (uint32_t c = 0; c < 4; c++) r.q[c] = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 16u + 32u * c + 8u * g, 0, 0);
+    }
+    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t, iu32x2 &b, float &s0, float &s1, float &mn) {
+        const float d = half_bits_to_float(r.h.x & 0xffffu), dmin = half_bits_to_float(r.h.x >> 16);
+        const uint2 sm = scale_min_k4(r.h.y, r.h.z, r.h.w, u);
+        s0 = s1 = d * (float)sm.x;
+        mn = dmin * (float)sm.y;
+        b = r.q[u >> 1];
+        if (u & 1u) b = b >> 4;
+        b = b & 0x0f0f0f0fu;
+    }
+};
+
+struct I8Q5 {
+    static constexpr uint32_t BLOCK = 176;
+    static constexpr bool HAS_MIN = true, HALVES = false;
+    struct Raw {
+        iu32x4 h;
+        iu32x2 qh;      // the fifth bits of positions 8 g .. 8 g + 7, bit u for unit u
+        iu32x2 q[4];
+    };
+    static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t w, uint32_t blk, uint32_t g, Raw &r) {
+        r.h = __builtin_amdgcn_raw_buffer_load_b128(w, blk, 0, 0);
+        r.qh = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 16u + 8u * g, 0, 0);
+#pragma unroll
+        for (uint32_t c = 0; c < 4; c++) r.q[c] = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 48u + 32u * c + 8u * g, 0, 0);
+    }
+    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t, iu32x2 &b, float &s0, float &s1, float &mn) {
+        const float d = half_bits_to_float(r.h.x & 0xffffu), dmin = half_bits_to_float(r.h.x >> 16);
+        const uint2 sm = scale_min_k4(r.h.y, r.h.z, r.h.w, u);
+        s0 = s1 = d * (float)sm.x;
+        mn = dmin * (float)sm.y;
+        b = r.q[u >> 1];
+        if (u & 1u) b = b >> 4;
+        b = (b & 0x0f0f0f0fu) | (((r.qh >> u) & 0x01010101u) << 4);
+    }
+};
+
+struct I8Q6 {
+    static constexpr uint32_t BLOCK = 224;  // padded from 210 at load
+    static constexpr bool HAS_MIN = false, HALVES = true;
+    struct Raw {
+        iu32x2 ql[4];   // [2 n + c % 2]: low nibbles unit 4 n + c % 2, high nibbles that + 2
+        iu32x2 qh[2];   // [n]: bits 2 c of unit 4 n + c
+        iu32x4 sc;      // sixteen signed scales
+        uint32_t d;
+    };
+    static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t w, uint32_t blk, uint32_t g, Raw &r) {
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) r.ql[i] = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 32u * i + 8u * g, 0, 0);
+#pragma unroll
+        for (uint32_t n = 0; n < 2; n++) r.qh[n] = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 128u + 32u * n + 8u * g, 0, 0);
+        r.sc = __builtin_amdgcn_raw_buffer_load_b128(w, blk + 192u, 0, 0);
+        r.d = __builtin_amdgcn_raw_buffer_load_b32(w, blk + 208u, 0, 0);
+    }
+    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t, iu32x2 &b, float &s0, float &s1, float &mn) {
+        const uint32_t n = u >> 2, c = u & 3u;
+        const float d = half_bits_to_float(r.d & 0xffffu);
+        const uint32_t pair = r.sc[(8u * n + 2u * c) >> 2] >> (16u * (c & 1u));  // scales 8 n + 2 c and the next
+        s0 = d * (float)sbyte(pair, 0);
+        s1 = d * (float)sbyte(pair, 1);
+        mn = 0.f;
+        const iu32x2 q = ((r.ql[2u * n + (c & 1u)] >> (4u * (c >> 1))) & 0x0f0f0f0fu) | (((r.qh[n] >> (2u * c)) & 0x03030303u) << 4);
+        b = (q + 0x60606060u) ^ 0x80808080u;  // minus 32 a byte, no borrows
+    }
+};
+
+struct I8Q3 {
+    static constexpr uint32_t BLOCK = 128;  // repacked at load: eight 16-byte units
+    static constexpr bool HAS_MIN = false, HALVES = true;
+    struct Raw {
+        iu32x4 u[8];  // two words of 2-bit values, the high bits, scales - 32 and d
+    };
+    static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t w, uint32_t blk, uint32_t, Raw &r) {
+#pragma unroll
+        for (uint32_t i = 0; i < 8; i++) r.u[i] = __builtin_amdgcn_raw_buffer_load_b128(w, blk + 16u * i, 0, 0);
+    }
+    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t g, iu32x2 &b, float &s0, float &s1, float &mn) {
+        const iu32x4 v = r.u[u];
+        const float d = half_bits_to_float(v.w >> 16);
+        s0 = d * (float)sbyte(v.w, 0);
+        s1 = d * (float)sbyte(v.w, 1);
+        mn = 0.f;
+        // Position 4 e + i: bits 2 (e % 4) of byte i of word e / 4, high bit 8 i + e.
+        const uint32_t l = (g < 2u ? v.x : v.y) >> (4u * (g & 1u)), hb = v.z >> (2u * g);
+        const iu32x2 c = {(l & 0x03030303u) | ((hb & 0x01010101u) << 2), ((l >> 2) & 0x03030303u) | (((hb >> 1) & 0x01010101u) << 2)};
+        b = (c + 0x7c7c7c7cu) ^ 0x80808080u;  // minus 4 a byte, no borrows
+    }
+};
+
+template <class P>
+__global__ __launch_bounds__(256) void matmul_kquant_i8_kernel(I8Args a) {
+    __shared__ __align__(16) uint8_t lds_q[2][TT * LINE];
     __shared__ __align__(16) float lds_d[2][TT];      // the tokens' block scales
-    __shared__ __align__(16) float lds_s[2][8][TT];   // sum of each sub-block's bytes
+    __shared__ __align__(16) float lds_s[2][8][TT];   // sum of each unit's bytes
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
     const uint32_t n0 = blockIdx.x * TN, t0 = blockIdx.y * TT;
     const uint32_t kb = blockIdx.z * a.k_slice, ke = min(a.k, kb + a.k_slice);
@@ -247,7 +357,7 @@ __global__ __launch_bounds__(256) void matmul_q4_k_i8_kernel(I8Args a) {
     const uint32_t steps = (ke - k_first + STEP - 1u) / STEP;
     const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.qx, a.qx_bytes), wbuf = make_buffer(a.w, a.w_bytes), dbuf = make_buffer(a.dx, a.dx_bytes);
 
-    // Staging: a quarter (two sub-blocks) of one token's super-block per thread.
+    // Staging: a quarter (two units) of one token's block per thread.
     const uint32_t atok = tid >> 2, aq = tid & 3u;
     const uint32_t aoff = (t0 + atok) * a.k + 64u * aq;
     const uint32_t doff = (t0 + atok) * (a.k / 256u) * 4u;
@@ -256,16 +366,12 @@ __global__ __launch_bounds__(256) void matmul_q4_k_i8_kernel(I8Args a) {
 
     iu32x4 ra[4];
     uint32_t rd;
-    iu32x4 bh, nh;       // d, dmin and the twelve scale bytes
-    iu32x2 bq[4], nq[4];  // 8 bytes of each 64-weight chunk: low nibbles sub-block 2c, high 2c + 1
-    auto fetch = [&](uint32_t k0, iu32x4 &h, iu32x2 (&q)[4]) __attribute__((always_inline)) {
+    typename P::Raw cur, next;
+    auto fetch = [&](uint32_t k0, typename P::Raw &r) __attribute__((always_inline)) {
 #pragma unroll
         for (uint32_t i = 0; i < 4; i++) ra[i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, aoff + k0 + 16u * i, 0, 0);
         rd = __builtin_amdgcn_raw_buffer_load_b32(dbuf, doff + k0 / 64u, 0, 0);
-        const uint32_t blk = wrow + k0 / 256u * 144u;
-        h = __builtin_amdgcn_raw_buffer_load_b128(wbuf, blk, 0, 0);
-#pragma unroll
-        for (uint32_t c = 0; c < 4; c++) q[c] = __builtin_amdgcn_raw_buffer_load_b64(wbuf, blk + 16u + 32u * c + 8u * g, 0, 0);
+        P::load(wbuf, wrow + k0 / 256u * P::BLOCK, g, r);
     };
     auto stash = [&](uint32_t buf) __attribute__((always_inline)) {
         uint8_t *line = &lds_q[buf][atok * LINE + 64u * aq];
@@ -274,11 +380,15 @@ __global__ __launch_bounds__(256) void matmul_q4_k_i8_kernel(I8Args a) {
         for (uint32_t i = 0; i < 4; i++) {
             *reinterpret_cast<iu32x2 *>(line + 16u * i) = ra[i].xy;
             *reinterpret_cast<iu32x2 *>(line + 16u * i + 8u) = ra[i].zw;
+            if (P::HAS_MIN) {
 #pragma unroll
-            for (uint32_t e = 0; e < 4; e++) sums[i >> 1] = __builtin_amdgcn_sdot4((int)ra[i][e], 0x01010101, sums[i >> 1], false);
+                for (uint32_t e = 0; e < 4; e++) sums[i >> 1] = __builtin_amdgcn_sdot4((int)ra[i][e], 0x01010101, sums[i >> 1], false);
+            }
         }
-        lds_s[buf][2u * aq][atok] = (float)sums[0];
-        lds_s[buf][2u * aq + 1u][atok] = (float)sums[1];
+        if (P::HAS_MIN) {
+            lds_s[buf][2u * aq][atok] = (float)sums[0];
+            lds_s[buf][2u * aq + 1u][atok] = (float)sums[1];
+        }
         if (aq == 0u) lds_d[buf][atok] = __uint_as_float(rd);
     };
 
@@ -286,34 +396,42 @@ __global__ __launch_bounds__(256) void matmul_q4_k_i8_kernel(I8Args a) {
 #pragma unroll
     for (int mt = 0; mt < 4; mt++) acc[mt] = if32x4{0.f, 0.f, 0.f, 0.f};
 
-    fetch(k_first, bh, bq);
+    fetch(k_first, cur);
     stash(0);
     __syncthreads();
     for (uint32_t s = 0; s < steps; s++) {
         const uint32_t k0 = k_first + s * STEP, buf = s & 1u;
         const bool more = s + 1u < steps;
-        if (more) fetch(k0 + STEP, nh, nq);
-        const float d = half_bits_to_float(bh.x & 0xffffu), dmin = half_bits_to_float(bh.x >> 16);
+        if (more) fetch(k0 + STEP, next);
         if32x4 part[4];
 #pragma unroll
         for (int mt = 0; mt < 4; mt++) part[mt] = if32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (uint32_t sb = 0; sb < 8; sb++) {
-            const uint32_t kpos = k0 + 32u * sb;
+        for (uint32_t u = 0; u < 8; u++) {
+            const uint32_t kpos = k0 + 32u * u;
             if (kpos < kb || kpos >= ke) continue;
-            const uint2 sm = scale_min_k4(bh.y, bh.z, bh.w, sb);
-            const float dsc = d * (float)sm.x, dmn = dmin * (float)sm.y;
-            iu32x2 nib = bq[sb >> 1];
-            if (sb & 1u) nib = nib >> 4;
-            nib = nib & 0x0f0f0f0fu;
-            const long b = as_operand(nib);
+            iu32x2 w8;
+            float s0, s1, mn;
+            P::unit(cur, u, g, w8, s0, s1, mn);
+            const iu32x2 zero = {0u, 0u};
+            const long b0 = as_operand(P::HALVES ? (g < 2u ? w8 : zero) : w8);
+            const long b1 = as_operand(g < 2u ? zero : w8);
 #pragma unroll
             for (uint32_t mt = 0; mt < 4; mt++) {
-                const long af = *reinterpret_cast<const long *>(&lds_q[buf][(16u * mt + l16) * LINE + 32u * sb + 8u * g]);
-                const i32x4 is = __builtin_amdgcn_mfma_i32_16x16x32_i8(af, b, i32x4{0, 0, 0, 0}, 0, 0, 0);
-                const if32x4 xs = *reinterpret_cast<const if32x4 *>(&lds_s[buf][sb][16u * mt + 4u * g]);
+                const long af = *reinterpret_cast<const long *>(&lds_q[buf][(16u * mt + l16) * LINE + 32u * u + 8u * g]);
+                const i32x4 is = __builtin_amdgcn_mfma_i32_16x16x32_i8(af, b0, i32x4{0, 0, 0, 0}, 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 4; i++) part[mt][i] = fmaf(-dmn, xs[i], fmaf(dsc, (float)is[i], part[mt][i]));
+                for (int i = 0; i < 4; i++) part[mt][i] = fmaf(s0, (float)is[i], part[mt][i]);
+                if (P::HALVES) {
+                    const i32x4 is1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(af, b1, i32x4{0, 0, 0, 0}, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) part[mt][i] = fmaf(s1, (float)is1[i], part[mt][i]);
+                }
+                if (P::HAS_MIN) {
+                    const if32x4 xs = *reinterpret_cast<const if32x4 *>(&lds_s[buf][u][16u * mt + 4u * g]);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) part[mt][i] = fmaf(-mn, xs[i], part[mt][i]);
+                }
             }
         }
 #pragma unroll
@@ -324,9 +442,7 @@ __global__ __launch_bounds__(256) void matmul_q4_k_i8_kernel(I8Args a) {
         }
         if (more) {
             stash(buf ^ 1u);
-            bh = nh;
-#pragma unroll
-            for (int c = 0; c < 4; c++) bq[c] = nq[c];
+            cur = next;
         }
         __syncthreads();
     }
@@ -337,13 +453,13 @@ __global__ __launch_bounds__(256) void matmul_q4_k_i8_kernel(I8Args a) {
 
 // matmul_quant.wgsl's workgroup is 128 outputs x 32 tokens: the grid says how
 // much of the product a dispatch covers, whatever tiling computes it.
-static zhip_result launch_int8(const Dispatch &d, const char *name, bool q4k) {
+static zhip_result launch_int8(const Dispatch &d, const char *name, int type) {
     if (d.params_size < sizeof(MatmulParams)) return fail(d, ZHIP_E_BAD_COMMAND, "%s: params block too small", name);
     const MatmulParams &p = *reinterpret_cast<const MatmulParams *>(d.params);
     for (int b = 1; b <= 4; b++)
         if (!d.bind[b].bound) return fail(d, ZHIP_E_BAD_COMMAND, "%s: binding %d is not bound", name, b);
     if (d.grid[0] == 0 || d.grid[1] == 0 || d.grid[2] == 0) return ZHIP_OK;
-    const uint32_t act = q4k ? 256u : 32u;
+    const uint32_t act = type == 8 ? 32u : 256u;
     if (p.k == 0 || p.k % act != 0) return fail(d, ZHIP_E_BAD_COMMAND, "%s: k = %u is not a multiple of %u", name, p.k, act);
     if (p.k_slice == 0 || p.k_slice % 32u != 0) return fail(d, ZHIP_E_BAD_COMMAND, "%s: k_slice = %u", name, p.k_slice);
     const uint64_t slices = d.grid[2];
@@ -351,7 +467,8 @@ static zhip_result launch_int8(const Dispatch &d, const char *name, bool q4k) {
     const uint64_t cover_n = (uint64_t)d.grid[0] * 128u, cover_t = (uint64_t)d.grid[1] * 32u;
     const uint64_t n = cover_n < p.n ? cover_n : p.n, rows = cover_t < p.rows ? cover_t : p.rows;
     if (n == 0 || rows == 0) return ZHIP_OK;
-    const uint64_t row_bytes = q4k ? (uint64_t)p.k / 256u * 144u : (((uint64_t)p.k + p.k / 16u + 15u) & ~15ull);
+    const uint32_t block = type == 3 ? I8Q3::BLOCK : type == 4 ? I8Q4::BLOCK : type == 5 ? I8Q5::BLOCK : I8Q6::BLOCK;
+    const uint64_t row_bytes = type == 8 ? (((uint64_t)p.k + p.k / 16u + 15u) & ~15ull) : (uint64_t)p.k / 256u * block;
     const uint64_t x_need = rows * p.k, d_need = rows * (p.k / act) * 4u, w_need = n * row_bytes;
     const uint64_t o_need = ((slices - 1) * p.slice_stride + (rows - 1) * p.out_stride + p.col0 + n) * 4u;
     if (x_need > d.bind[1].size || w_need > d.bind[2].size || o_need > d.bind[3].size || d_need > d.bind[4].size)
@@ -375,8 +492,14 @@ static zhip_result launch_int8(const Dispatch &d, const char *name, bool q4k) {
     a.qx_bytes = (uint32_t)x_need; a.w_bytes = (uint32_t)w_need; a.dx_bytes = (uint32_t)d_need;
     const dim3 grid((uint32_t)tiles_n, (uint32_t)tiles_t, (uint32_t)slices);
     const bool ragged = p.k % STEP != 0 || (slices > 1 && p.k_slice % STEP != 0);
-    if (q4k) {
-        hipLaunchKernelGGL(matmul_q4_k_i8_kernel, grid, dim3(256), 0, d.stream, a);
+    if (type == 3) {
+        hipLaunchKernelGGL(matmul_kquant_i8_kernel<I8Q3>, grid, dim3(256), 0, d.stream, a);
+    } else if (type == 4) {
+        hipLaunchKernelGGL(matmul_kquant_i8_kernel<I8Q4>, grid, dim3(256), 0, d.stream, a);
+    } else if (type == 5) {
+        hipLaunchKernelGGL(matmul_kquant_i8_kernel<I8Q5>, grid, dim3(256), 0, d.stream, a);
+    } else if (type == 6) {
+        hipLaunchKernelGGL(matmul_kquant_i8_kernel<I8Q6>, grid, dim3(256), 0, d.stream, a);
     } else {
         if (ragged) hipLaunchKernelGGL(matmul_q8_0_i8_kernel<true>, grid, dim3(256), 0, d.stream, a);
         else hipLaunchKernelGGL(matmul_q8_0_i8_kernel<false>, grid, dim3(256), 0, d.stream, a);
@@ -384,7 +507,10 @@ static zhip_result launch_int8(const Dispatch &d, const char *name, bool q4k) {
     return check_launch(d, name);
 }
 
-zhip_result launch_matmul_q8_0(const Dispatch &d) { return launch_int8(d, "matmul_q8_0", false); }
-zhip_result launch_matmul_q4_k(const Dispatch &d) { return launch_int8(d, "matmul_q4_k", true); }
+zhip_result launch_matmul_q8_0(const Dispatch &d) { return launch_int8(d, "matmul_q8_0", 8); }
+zhip_result launch_matmul_q3_k(const Dispatch &d) { return launch_int8(d, "matmul_q3_k", 3); }
+zhip_result launch_matmul_q4_k(const Dispatch &d) { return launch_int8(d, "matmul_q4_k", 4); }
+zhip_result launch_matmul_q5_k(const Dispatch &d) { return launch_int8(d, "matmul_q5_k", 5); }
+zhip_result launch_matmul_q6_k(const Dispatch &d) { return launch_int8(d, "matmul_q6_k", 6); }
 
 }  // namespace zhip

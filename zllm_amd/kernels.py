@@ -73,7 +73,10 @@ CONTRACTS = {
     Kernel.matmul_bf16: Contract(4, 0b1000),
     Kernel.matmul_q8_0_float: Contract(4, 0b1000),
     Kernel.matmul_q8_0: Contract(5, 0b01000),
+    Kernel.matmul_q3_k: Contract(5, 0b01000),
     Kernel.matmul_q4_k: Contract(5, 0b01000),
+    Kernel.matmul_q5_k: Contract(5, 0b01000),
+    Kernel.matmul_q6_k: Contract(5, 0b01000),
     Kernel.quantize_q8: Contract(5, 0b01100),
     Kernel.matmul_reduce: Contract(3, 0b100),
     Kernel.silu_mul: Contract(3, 0b100),
