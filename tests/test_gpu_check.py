@@ -26,10 +26,17 @@ def quant_rows(c, t: TensorType, rows: int, k: int):
     return raw, oracle.dequantize(ORACLE_TYPE[t], raw, rows * k).reshape(rows, k)
 
 
-def random_half(c, n: int, scale: float):
-    """bf16 weights and their f32 values (src/kernels/check.zig randomHalf)."""
+def random_half(c, n: int, scale: float, half: str = "bf16"):
+    """bf16 or f16 weights and their f32 values (src/kernels/check.zig randomHalf);
+    numpy's float16 is the f16 conversion."""
+    if half == "f16":
+        h = c.random(n, scale).astype(np.float16)
+        return h.view(np.uint16), h.astype(np.float32)
     bits = synth.to_bf16_bits(c.random(n, scale))
     return bits, synth.bf16_bits_to_f32(bits)
+
+
+HALVES = ["bf16", "f16"]
 
 
 def norm_row(x, w, eps):
@@ -48,18 +55,18 @@ def sigmoid64(x):
 
 # ---- half-precision decode multiply: check.zig:327-442 ------------------------------
 
-def matvec_case(c, k, split, fused):
+def matvec_case(c, k, split, fused, half="bf16"):
     rows, n, eps = 3, 100, 1e-6
     x = c.random(rows * k, 3).reshape(rows, k)
     nw = c.random(k, 1)
-    bits, values = random_half(c, n * k, 1)
+    bits, values = random_half(c, n * k, 1, half)
     bits, values = bits.reshape(n, k), values.reshape(n, k)
     init = c.random(rows * n, 4 if fused else 0).reshape(rows, n)
     out, xa, na = c.upload(init), c.upload(x), c.upload(nw)
     col0 = 0
     for cols in (split, n - split):
         wa = c.upload(bits[col0 : col0 + cols])
-        c.launcher().launch(Kernel.matvec_bf16, P.MatvecBf16(n=cols, k=k, col0=col0, out_stride=n, eps=eps, norm=fused, accumulate=fused),
+        c.launcher().launch(Kernel["matvec_" + half], P.MatvecBf16(n=cols, k=k, col0=col0, out_stride=n, eps=eps, norm=fused, accumulate=fused),
                             [xa, wa, out, na], (K.div_ceil(cols, K.matvec_rows), rows, 1))
         col0 += cols
     got = c.read(out).reshape(rows, n)
@@ -67,24 +74,27 @@ def matvec_case(c, k, split, fused):
     return rel_err(got, want)
 
 
-def test_matvec_bf16_two_chunks(ctx):
+@pytest.mark.parametrize("half", HALVES)
+def test_matvec_bf16_two_chunks(ctx, half):
     # k = 4000 leaves a partial pass over the lanes; 100 outputs a partial group.
-    assert matvec_case(ctx, 4000, 37, False) <= 1e-5
+    assert matvec_case(ctx, 4000, 37, False, half) <= 1e-5
 
 
-def test_matvec_bf16_norm_accumulate(ctx):
-    assert matvec_case(ctx, 1000, 37, True) <= 1e-5
+@pytest.mark.parametrize("half", HALVES)
+def test_matvec_bf16_norm_accumulate(ctx, half):
+    assert matvec_case(ctx, 1000, 37, True, half) <= 1e-5
 
 
-def test_matvec_bf16_silu_pair(ctx):
+@pytest.mark.parametrize("half", HALVES)
+def test_matvec_bf16_silu_pair(ctx, half):
     c = ctx
     rows, ff, k, eps = 3, 100, 1024, 1e-6
     x = c.random(rows * k, 3).reshape(rows, k)
     nw = c.random(k, 1)
-    bits, values = random_half(c, 2 * ff * k, 1)
+    bits, values = random_half(c, 2 * ff * k, 1, half)
     values = values.reshape(2 * ff, k).astype(np.float64)
     out = c.output(rows * ff)
-    c.launcher().launch(Kernel.matvec_bf16, P.MatvecBf16(n=ff, k=k, col0=0, out_stride=ff, eps=eps, norm=True, silu_pair=True, half=ff),
+    c.launcher().launch(Kernel["matvec_" + half], P.MatvecBf16(n=ff, k=k, col0=0, out_stride=ff, eps=eps, norm=True, silu_pair=True, half=ff),
                         [c.upload(x), c.upload(bits), out, c.upload(nw)], (K.div_ceil(ff, K.matvec_rows), rows, 1))
     got = c.read(out).reshape(rows, ff)
     want = np.empty((rows, ff))
@@ -273,16 +283,17 @@ def test_embed_q8_0_file_rows(ctx):
     assert np.array_equal(c.read_words(out).reshape(tokens.size, dim), values[tokens].view(np.uint32))
 
 
-def test_embed_bf16_exact(ctx):
+@pytest.mark.parametrize("half", HALVES)
+def test_embed_bf16_exact(ctx, half):
     c = ctx
     vocab, dim, split = 50, 64, 30
-    bits, values = random_half(c, vocab * dim, 1)
+    bits, values = random_half(c, vocab * dim, 1, half)
     bits, values = bits.reshape(vocab, dim), values.reshape(vocab, dim)
     tokens = np.array([0, 29, 30, 49, 7, 30, 12], dtype=np.uint32)
     out = c.output(tokens.size * dim)
     ta = c.upload(tokens)
     for row0, rows in ((0, split), (split, vocab - split)):
-        c.launcher().launch(Kernel.embed_bf16, P.EmbedBf16(dim=dim, row0=row0, chunk_rows=rows), [ta, c.upload(bits[row0 : row0 + rows]), out], (tokens.size, 1, 1))
+        c.launcher().launch(Kernel["embed_" + half], P.EmbedBf16(dim=dim, row0=row0, chunk_rows=rows), [ta, c.upload(bits[row0 : row0 + rows]), out], (tokens.size, 1, 1))
     assert np.array_equal(c.read(out).reshape(tokens.size, dim), values[tokens])
 
 
@@ -322,9 +333,9 @@ def test_repad_pads_blocks(ctx):
 
 # ---- prefill multiplies: check.zig:288-325, 752-825 -------------------------------------
 
-def matmul_case(c, rows, n, k, split, accumulate, rung=K.Prefill.scalar_f32):
+def matmul_case(c, rows, n, k, split, accumulate, rung=K.Prefill.scalar_f32, half="bf16"):
     x = c.random(rows * k, 1).reshape(rows, k)
-    bits, values = random_half(c, n * k, 1)
+    bits, values = random_half(c, n * k, 1, half)
     bits, values = bits.reshape(n, k), values.reshape(n, k)
     init = c.random(rows * n, 4 if accumulate else 0).reshape(rows, n)
     packed = rung == K.Prefill.bf16_mfma_xbf16
@@ -335,7 +346,7 @@ def matmul_case(c, rows, n, k, split, accumulate, rung=K.Prefill.scalar_f32):
         if cols == 0:
             continue
         wa = c.upload(bits[col0 : col0 + cols])
-        c.launcher().launch(Kernel.matmul_bf16, P.MatmulBf16(rows=rows, n=cols, k=k, col0=col0, out_stride=n, accumulate=int(accumulate)),
+        c.launcher().launch(Kernel["matmul_" + half], P.MatmulBf16(rows=rows, n=cols, k=k, col0=col0, out_stride=n, accumulate=int(accumulate)),
                             [xa, wa, out], (K.div_ceil(cols, K.matmul_tile_n), K.div_ceil(rows, K.matmul_tile_t), 1))
         col0 += cols
     got = c.read(out).reshape(rows, n)
@@ -345,14 +356,16 @@ def matmul_case(c, rows, n, k, split, accumulate, rung=K.Prefill.scalar_f32):
     return got, want, values, x
 
 
-def test_matmul_bf16(ctx):
+@pytest.mark.parametrize("half", HALVES)
+def test_matmul_bf16(ctx, half):
     # 19 tokens and 100 outputs leave partial tiles in both dimensions.
-    got, want, _, _ = matmul_case(ctx, 19, 100, 1024, None, False)
+    got, want, _, _ = matmul_case(ctx, 19, 100, 1024, None, False, half=half)
     assert rel_err(got, want) <= 1e-5
 
 
-def test_matmul_bf16_chunked_accumulate(ctx):
-    got, want, _, _ = matmul_case(ctx, 33, 150, 96, 70, True)
+@pytest.mark.parametrize("half", HALVES)
+def test_matmul_bf16_chunked_accumulate(ctx, half):
+    got, want, _, _ = matmul_case(ctx, 33, 150, 96, 70, True, half=half)
     assert rel_err(got, want) <= 1e-5
 
 

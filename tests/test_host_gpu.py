@@ -217,6 +217,8 @@ def test_create_kernel_rejects_what_it_does_not_implement(ctx):
     writes = K.contract(Kernel.matmul_bf16).writes
     for rung in (K.Prefill.fp16_single, K.Prefill.fp16_compensated):
         expect(c, host.UnsupportedPrefill, lambda: c.rec.create_kernel(int(Kernel.matmul_bf16), K.PREFILL_VARIANT[rung], writes, K.artifact(Kernel.matmul_bf16)))
+    # matmul_f16 has only the exact f32 rung.
+    expect(c, host.UnsupportedPrefill, lambda: c.rec.create_kernel(int(Kernel.matmul_f16), K.PREFILL_VARIANT[K.Prefill.bf16_mfma], writes, K.artifact(Kernel.matmul_f16, K.PREFILL_VARIANT[K.Prefill.bf16_mfma])))
     expect(c, host.BadCommand, lambda: c.rec.create_kernel(int(Kernel.matmul_bf16), 0, writes, b"@compute fn main() {}"))           # another backend's artifact
     expect(c, host.BadCommand, lambda: c.rec.create_kernel(int(Kernel.matmul_bf16), 0, 0b10, K.artifact(Kernel.matmul_bf16)))      # contract mismatch
     expect(c, host.BadCommand, lambda: c.rec.create_kernel(int(Kernel.silu_mul), 5, K.contract(Kernel.silu_mul).writes, K.artifact(Kernel.silu_mul)))

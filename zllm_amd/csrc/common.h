@@ -102,6 +102,7 @@ zhip_result launch_matvec_q4_k(const Dispatch &);
 zhip_result launch_matvec_q5_k(const Dispatch &);
 zhip_result launch_matvec_q6_k(const Dispatch &);
 zhip_result launch_matvec_bf16(const Dispatch &);
+zhip_result launch_matvec_f16(const Dispatch &);
 zhip_result launch_matmul_reduce(const Dispatch &);
 zhip_result launch_quantize_q8(const Dispatch &);
 zhip_result launch_matmul_q8_0(const Dispatch &);
@@ -119,6 +120,7 @@ zhip_result launch_embed_q4_k(const Dispatch &);
 zhip_result launch_embed_q5_k(const Dispatch &);
 zhip_result launch_embed_q6_k(const Dispatch &);
 zhip_result launch_embed_bf16(const Dispatch &);
+zhip_result launch_embed_f16(const Dispatch &);
 
 // Host-side helpers shared by the launchers.
 zhip_result fail(const Dispatch &d, zhip_result code, const char *fmt, ...);

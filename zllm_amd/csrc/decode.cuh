@@ -243,4 +243,25 @@ struct DecBF16 {
     }
 };
 
+// F16 rows: two values per word, the low half first
+// (src/kernels/half/f16.wgsl:3-9); every f16 value is exact in f32.
+struct DecF16 {
+    static constexpr int RUNS = 2;
+    static constexpr int E = 8;
+    static constexpr uint32_t BLOCK = 8;
+    static constexpr int CHUNK = 0;
+    static const char *name() { return "matvec_f16"; }
+    static uint32_t row_bytes(uint32_t k) { return 2u * k; }
+    __device__ static uint32_t xoff(uint32_t task, int h) { return 8u * task + 4u * h; }
+    __device__ static void decode(const uint8_t *row, uint32_t, uint32_t task, float (&w)[E]) {
+        const uint4 q = *reinterpret_cast<const uint4 *>(row + 16u * task);
+        const uint32_t words[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            w[2 * e + 0] = half_bits_to_float(words[e] & 0xffffu);
+            w[2 * e + 1] = half_bits_to_float(words[e] >> 16);
+        }
+    }
+};
+
 }  // namespace zhip

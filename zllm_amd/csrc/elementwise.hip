@@ -195,7 +195,7 @@ zhip_result launch_repad(const Dispatch &d) {
     return check_launch(d, "repad");
 }
 
-// ---- embed_q8_0 / embed_q3_k / embed_q4_k / embed_q5_k / embed_q6_k / embed_bf16: src/kernels/embed_quant.wgsl, -------
+// ---- embed_q8_0 / embed_q3_k / embed_q4_k / embed_q5_k / embed_q6_k / embed_bf16 / embed_f16: src/kernels/embed_quant.wgsl, -------
 // src/kernels/embed_half.wgsl. out[t] = table[tokens[t] - row0] decoded to f32
 // for tokens whose row lies in [row0, row0 + chunk_rows); one workgroup per
 // token. The decoders are the multiplies' own, so these kernels also show the
@@ -267,6 +267,7 @@ zhip_result launch_embed_q3_k(const Dispatch &d) { return launch_embed<DecQ3_K>(
 zhip_result launch_embed_q5_k(const Dispatch &d) { return launch_embed<DecQ5_K>(d, "embed_q5_k"); }
 zhip_result launch_embed_q6_k(const Dispatch &d) { return launch_embed<DecQ6_K>(d, "embed_q6_k"); }
 zhip_result launch_embed_bf16(const Dispatch &d) { return launch_embed<DecBF16>(d, "embed_bf16"); }
+zhip_result launch_embed_f16(const Dispatch &d) { return launch_embed<DecF16>(d, "embed_f16"); }
 
 // ---- fill ----------------------------------------------------------------------
 __global__ __launch_bounds__(256) void fill_kernel(uint32_t *dst, uint64_t words, uint32_t value) {

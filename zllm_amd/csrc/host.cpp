@@ -66,6 +66,7 @@ static constexpr uint32_t kVariantBf16X = 0xfffa0000u;  // bf16 MFMA, activation
 enum class VariantKind { none, matvec, prefill };
 
 zhip_result launch_matmul_bf16_f32(const Dispatch &);
+zhip_result launch_matmul_f16_f32(const Dispatch &);
 zhip_result launch_matmul_q8_0_float_f32(const Dispatch &);
 zhip_result launch_matmul_bf16_mfma(const Dispatch &);
 zhip_result launch_matmul_q8_0_float_mfma(const Dispatch &);
@@ -90,6 +91,8 @@ static const KernelInfo kImplemented[] = {
     {"matvec_q5_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q5_k, nullptr, nullptr, 1},
     {"matvec_q6_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q6_k, nullptr, nullptr, 1},
     {"matvec_bf16", 5, 0b01000, VariantKind::none, launch_matvec_bf16, nullptr, nullptr, 1},
+    {"matvec_f16", 5, 0b01000, VariantKind::none, launch_matvec_f16, nullptr, nullptr, 1},
+    {"matmul_f16", 4, 0b1000, VariantKind::prefill, launch_matmul_f16_f32, nullptr, nullptr, 1},
     {"matmul_bf16", 4, 0b1000, VariantKind::prefill, launch_matmul_bf16_f32, launch_matmul_bf16_mfma, launch_matmul_bf16_mfma_xbf16, 1},
     {"matmul_q8_0_float", 4, 0b1000, VariantKind::prefill, launch_matmul_q8_0_float_f32, launch_matmul_q8_0_float_mfma, launch_matmul_q8_0_float_mfma_xbf16, 1},
     {"matmul_q8_0", 5, 0b01000, VariantKind::none, launch_matmul_q8_0, nullptr, nullptr, 1},
@@ -109,6 +112,7 @@ static const KernelInfo kImplemented[] = {
     {"embed_q5_k", 4, 0b1000, VariantKind::none, launch_embed_q5_k, nullptr, nullptr, 1},
     {"embed_q6_k", 4, 0b1000, VariantKind::none, launch_embed_q6_k, nullptr, nullptr, 1},
     {"embed_bf16", 4, 0b1000, VariantKind::none, launch_embed_bf16, nullptr, nullptr, 1},
+    {"embed_f16", 4, 0b1000, VariantKind::none, launch_embed_f16, nullptr, nullptr, 1},
 };
 
 static const KernelInfo *find_kernel(const char *name, size_t len) {
@@ -502,6 +506,7 @@ zhip_result create_kernel(zhip_context *c, const Command &cmd) {
         if (p.variant == kVariantBf16) p.launch = info->launch_bf16;
         else if (p.variant == kVariantBf16X) p.launch = info->launch_bf16x;
         else if (p.variant != 0) return set_error(c, ZHIP_E_BAD_COMMAND, "create_kernel: %s has no variant 0x%08x", info->name, p.variant);
+        if (!p.launch) return set_error(c, ZHIP_E_UNSUPPORTED_PREFILL, "create_kernel: %s has only the f32 rung", info->name);
         break;
     }
     return put(c, c->pipelines, a[0], std::move(p));

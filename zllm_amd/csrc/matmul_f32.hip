@@ -37,6 +37,18 @@ struct WBf16 {
     }
 };
 
+struct WF16 {
+    __device__ static void load8(const uint8_t *row, uint32_t, uint32_t k0, uint32_t c8, float (&w)[8]) {
+        const uint4 q = *reinterpret_cast<const uint4 *>(row + 2u * (k0 + 8u * c8));
+        const uint32_t words[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            w[2 * e] = half_bits_to_float(words[e] & 0xffffu);
+            w[2 * e + 1] = half_bits_to_float(words[e] >> 16);
+        }
+    }
+};
+
 struct WQ8_0 {
     __device__ static void load8(const uint8_t *row, uint32_t k, uint32_t k0, uint32_t c8, float (&w)[8]) {
         const uint2 q = *reinterpret_cast<const uint2 *>(row + k0 + 8u * c8);
@@ -182,6 +194,7 @@ static zhip_result launch_matmul(const Dispatch &d, const char *name, bool slice
 }
 
 zhip_result launch_matmul_bf16_f32(const Dispatch &d) { return launch_matmul<WBf16>(d, "matmul_bf16", false, false); }
+zhip_result launch_matmul_f16_f32(const Dispatch &d) { return launch_matmul<WF16>(d, "matmul_f16", false, false); }
 zhip_result launch_matmul_q8_0_float_f32(const Dispatch &d) { return launch_matmul<WQ8_0>(d, "matmul_q8_0_float", true, true); }
 
 }  // namespace zhip

@@ -216,5 +216,6 @@ zhip_result launch_matvec_q3_k(const Dispatch &d) { return launch_matvec<DecQ3_K
 zhip_result launch_matvec_q5_k(const Dispatch &d) { return launch_matvec<DecQ5_K>(d, true); }
 zhip_result launch_matvec_q6_k(const Dispatch &d) { return launch_matvec<DecQ6_K>(d, true); }
 zhip_result launch_matvec_bf16(const Dispatch &d) { return launch_matvec<DecBF16>(d, false); }
+zhip_result launch_matvec_f16(const Dispatch &d) { return launch_matvec<DecF16>(d, false); }
 
 }  // namespace zhip

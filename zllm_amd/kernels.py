@@ -70,7 +70,9 @@ CONTRACTS = {
     Kernel.matvec_q5_k: Contract(5, 0b01000),
     Kernel.matvec_q6_k: Contract(5, 0b01000),
     Kernel.matvec_bf16: Contract(5, 0b01000),
+    Kernel.matvec_f16: Contract(5, 0b01000),
     Kernel.matmul_bf16: Contract(4, 0b1000),
+    Kernel.matmul_f16: Contract(4, 0b1000),
     Kernel.matmul_q8_0_float: Contract(4, 0b1000),
     Kernel.matmul_q8_0: Contract(5, 0b01000),
     Kernel.matmul_q3_k: Contract(5, 0b01000),
@@ -89,6 +91,7 @@ CONTRACTS = {
     Kernel.embed_q5_k: Contract(4, 0b1000),
     Kernel.embed_q6_k: Contract(4, 0b1000),
     Kernel.embed_bf16: Contract(4, 0b1000),
+    Kernel.embed_f16: Contract(4, 0b1000),
 }
 
 
