@@ -13,7 +13,7 @@ import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
 
-F32, F16, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, BF16 = 0, 1, 8, 11, 12, 13, 14, 30
+F32, F16, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K, IQ4_XS, BF16 = 0, 1, 8, 11, 12, 13, 14, 23, 30
 
 
 def build() -> None:

@@ -24,6 +24,7 @@ int zref_layout(int type, uint32_t *block_elems, uint32_t *block_bytes) {
     case ZREF_Q4_K: e = 256; b = 144; break;
     case ZREF_Q5_K: e = 256; b = 176; break;
     case ZREF_Q6_K: e = 256; b = 210; break;
+    case ZREF_IQ4_XS: e = 256; b = 136; break;
     default: return 0;
     }
     if (block_elems) *block_elems = e;
@@ -231,6 +232,26 @@ static void q6_k_block(const uint8_t *b, float *y) {
     }
 }
 
+/* src/ref/tensor.zig:162-181: d (f16), scales_h (u16), scales_l[4], qs[128]; each
+ * group of 32 has a signed six-bit scale biased by 32 and sixteen bytes of
+ * indices into a nonlinear table, low nibbles first, then high nibbles. */
+static void iq4_xs_block(const uint8_t *b, float *y) {
+    static const int8_t values[16] = { -127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113 };
+    float d = zref_half(rd16(b));
+    uint32_t scales_h = rd16(b + 2);
+    for (unsigned group = 0; group < 8; group++) {
+        uint32_t low = (b[4 + group / 2] >> (4 * (group % 2))) & 15;
+        uint32_t high = (scales_h >> (2 * group)) & 3;
+        int scale = (int)(low | (high << 4)) - 32;
+        float dl = d * (float)scale;
+        const uint8_t *qs = b + 8 + 16 * group;
+        for (unsigned j = 0; j < 16; j++) {
+            y[32 * group + j] = dl * (float)values[qs[j] & 15];
+            y[32 * group + 16 + j] = dl * (float)values[qs[j] >> 4];
+        }
+    }
+}
+
 /* src/ref/tensor.zig:21-43. */
 int zref_dequantize(int type, const uint8_t *bytes, float *out, size_t n) {
     switch (type) {
@@ -248,6 +269,10 @@ int zref_dequantize(int type, const uint8_t *bytes, float *out, size_t n) {
         return 0;
     case ZREF_Q6_K:
         for (size_t i = 0; i < n / 256; i++) q6_k_block(bytes + i * 210, out + i * 256);
+        return 0;
+    case ZREF_IQ4_XS:
+        if (n % 256) return -1;
+        for (size_t i = 0; i < n / 256; i++) iq4_xs_block(bytes + i * 136, out + i * 256);
         return 0;
     case ZREF_F32:
         for (size_t i = 0; i < n; i++) out[i] = bits_f32(rd32(bytes + 4 * i));
@@ -598,6 +623,7 @@ uint64_t zref_row_bytes(int type, uint64_t k) {
     uint32_t be, bb;
     if (!zref_layout(type, &be, &bb)) return 0;
     if (type == ZREF_Q6_K) bb = 224;  /* blockStride: padded to 16 bytes by repad */
+    if (type == ZREF_IQ4_XS) bb = 144;
     if (type == ZREF_Q3_K) bb = 128;  /* repacked into eight 16-byte units */
     return k / be * bb;
 }

@@ -68,6 +68,7 @@ enum {
     ZREF_Q4_K = 12,
     ZREF_Q5_K = 13,
     ZREF_Q6_K = 14,
+    ZREF_IQ4_XS = 23,
     ZREF_BF16 = 30,
 };
 

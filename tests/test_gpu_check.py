@@ -16,7 +16,7 @@ from zllm_amd.kernels import Kernel, TensorType, params as P
 pytestmark = pytest.mark.gpu
 
 ORACLE_TYPE = {TensorType.q8_0: oracle.Q8_0, TensorType.q3_k: oracle.Q3_K, TensorType.q4_k: oracle.Q4_K, TensorType.q5_k: oracle.Q5_K, TensorType.q6_k: oracle.Q6_K,
-               TensorType.bf16: oracle.BF16}
+               TensorType.bf16: oracle.BF16, TensorType.iq4_xs: oracle.IQ4_XS}
 
 
 def quant_rows(c, t: TensorType, rows: int, k: int):
@@ -281,6 +281,50 @@ def test_embed_q8_0_file_rows(ctx):
     out = c.output(tokens.size * dim)
     c.launcher().launch(Kernel.embed_q8_0, P.EmbedBf16(dim=dim, row0=0, chunk_rows=vocab, stride=stride), [c.upload(tokens), c.upload(table), out], (tokens.size, 1, 1))
     assert np.array_equal(c.read_words(out).reshape(tokens.size, dim), values[tokens].view(np.uint32))
+
+
+def test_embed_iq4_xs_exact(ctx):
+    """The reference's kernel check (src/kernels/check.zig:925-985): scale codes,
+    indices and five super-scales cycling over the blocks, two row chunks, a
+    token out of range left untouched; once from the padded layout, once from
+    file rows an unaligned stride apart. Bit for bit against the decoder."""
+    c = ctx
+    vocab, dim, split = 8, 8448, 3
+    per_row = dim // 256
+    row_bytes = per_row * 136
+    raw = np.zeros((vocab * per_row, 136), dtype=np.uint8)
+    ds = np.array([0.0078125, -0.01171875, 0.009765625, 0, -0.00390625], dtype=np.float16)
+    i = np.arange(16)
+    for b in range(vocab * per_row):
+        raw[b, 0:2] = ds[b % 5 : b % 5 + 1].view(np.uint8)
+        high = 0
+        for s in range(8):
+            scale = (b * 8 + s) % 64
+            raw[b, 4 + s // 2] |= (scale & 15) << (4 * (s % 2))
+            high |= (scale >> 4) << (2 * s)
+            raw[b, 8 + 16 * s : 24 + 16 * s] = ((i + 3 * s + b) % 16) | (((15 - i + 5 * s + 3 * b) % 16) << 4)
+        raw[b, 2], raw[b, 3] = high & 0xFF, high >> 8
+    raw = raw.reshape(vocab, row_bytes)
+    values = oracle.dequantize(oracle.IQ4_XS, raw, vocab * dim).reshape(vocab, dim)
+    tokens = np.array([7, 0, 2, 3, 4, 7, 1, 8], dtype=np.uint32)
+    ta = c.upload(tokens)
+    want = np.full((tokens.size, dim), -9999, dtype=np.float32)
+    want[:7] = values[tokens[:7]]
+    for strided in (False, True):
+        out = c.upload(np.full(tokens.size * dim, -9999, dtype=np.float32))
+        for row0, rows in ((0, split), (split, vocab - split)):
+            if strided:
+                stride = row_bytes + 4
+                spaced = np.full((rows * stride + 15) & ~15, 0xA5, dtype=np.uint8)
+                for r in range(rows):
+                    spaced[r * stride : r * stride + row_bytes] = raw[row0 + r]
+                wa = c.upload(spaced)
+            else:
+                stride = 0
+                wa = c.gpu_weights(TensorType.iq4_xs, raw[row0 : row0 + rows], dim)
+            c.launcher().launch(Kernel.embed_iq4_xs, P.EmbedBf16(dim=dim, row0=row0, chunk_rows=rows, stride=stride), [ta, wa, out], (tokens.size, 1, 1))
+        got = c.read_words(out).reshape(tokens.size, dim)
+        assert np.array_equal(got, want.view(np.uint32)), f"strided={strided}: {np.count_nonzero(got != want.view(np.uint32))} values differ"
 
 
 @pytest.mark.parametrize("half", HALVES)

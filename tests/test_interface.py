@@ -62,7 +62,7 @@ def test_artifacts_name_the_kernel_and_missing_kernels_are_empty():
                    Kernel.silu_mul, Kernel.repack_q8_0, Kernel.repad, Kernel.embed_q8_0, Kernel.embed_q4_k, Kernel.embed_bf16,
                    Kernel.matvec_q3_k, Kernel.matvec_q5_k, Kernel.matvec_q6_k, Kernel.embed_q3_k, Kernel.embed_q5_k, Kernel.embed_q6_k,
                    Kernel.repack_q3_k, Kernel.quantize_q8, Kernel.matmul_q8_0, Kernel.matmul_q3_k, Kernel.matmul_q4_k, Kernel.matmul_q5_k, Kernel.matmul_q6_k,
-                   Kernel.matvec_f16, Kernel.matmul_f16, Kernel.embed_f16}
+                   Kernel.matvec_f16, Kernel.matmul_f16, Kernel.embed_f16, Kernel.embed_iq4_xs}
     assert set(Kernel) - s.missing == implemented
     with pytest.raises(K.UnsupportedKernel):
         s.require_all()

@@ -337,6 +337,61 @@ def test_k_quant_single_bit_mutations_move_exactly_their_weights(t, size, packer
 
 # ---- ops: RMSNorm's bitwise known answer (src/ref/ops.zig:139-168), SiLU ---------------
 
+IQ4_VALUES = np.array([-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113], dtype=np.float32)
+
+
+def test_iq4_xs_every_code_scale_and_block_boundary():
+    """The reference's known-answer test (src/ref/tensor.zig:211-245): two blocks
+    with d = 1.5 and -0.25, group g's scale code (code + 7 g) % 64 for every code,
+    byte j of a group holding indices j (low) and 15 - j (high); each value must
+    be the bits of (d * scale) * table[index]."""
+    assert oracle.layout(oracle.IQ4_XS) == (256, 136)
+    for code in range(64):
+        raw = np.zeros(2 * 136, dtype=np.uint8)
+        ds = np.array([1.5, -0.25], dtype=np.float16)
+        for block in range(2):
+            b = raw[136 * block : 136 * (block + 1)]
+            b[0:2] = ds[block : block + 1].view(np.uint8)
+            high = 0
+            for group in range(8):
+                sc = (code + 7 * group) % 64
+                b[4 + group // 2] |= (sc & 15) << (4 * (group % 2))
+                high |= (sc >> 4) << (2 * group)
+                b[8 + 16 * group : 24 + 16 * group] = np.arange(16) | ((15 - np.arange(16)) << 4)
+            b[2], b[3] = high & 0xFF, high >> 8
+        out = oracle.dequantize(oracle.IQ4_XS, raw, 512).reshape(2, 8, 32)
+        for block in range(2):
+            for group in range(8):
+                dl = np.float32(ds[block]) * np.float32((code + 7 * group) % 64 - 32)
+                order = np.concatenate([np.arange(16), 15 - np.arange(16)])
+                want = (dl * IQ4_VALUES[order]).astype(np.float32)
+                assert out[block, group].tobytes() == want.tobytes()
+
+
+def test_iq4_xs_single_bit_mutations_move_their_group_or_lane():
+    """src/ref/tensor.zig:247-275: d = 0.5, every scale code 33 (+1), every index 8
+    (+1): all values 0.5; flipping one bit of the scales changes exactly its group
+    of 32, one bit of an index exactly one weight."""
+    base = np.full(136, 0x88, dtype=np.uint8)
+    base[0:8] = [0, 0x38, 0xAA, 0xAA, 0x11, 0x11, 0x11, 0x11]
+    assert np.all(oracle.dequantize(oracle.IQ4_XS, base, 256) == 0.5)
+    for byte in range(2, 136):
+        for bit in range(8):
+            m = base.copy()
+            m[byte] ^= 1 << bit
+            changed = np.flatnonzero(oracle.dequantize(oracle.IQ4_XS, m, 256) != 0.5)
+            if byte < 4:
+                group = ((byte - 2) * 8 + bit) // 2
+            elif byte < 8:
+                group = (byte - 4) * 2 + bit // 4
+            else:
+                group = (byte - 8) // 16
+            if byte < 8:
+                assert np.array_equal(changed, np.arange(32 * group, 32 * group + 32))
+            else:
+                assert np.array_equal(changed, [32 * group + (byte - 8) % 16 + (bit // 4) * 16])
+
+
 def test_rms_norm_known_answer_bitwise():
     with open(os.path.join(GOLDEN, "rmsnorm_kat.json")) as f:
         kat = json.load(f)

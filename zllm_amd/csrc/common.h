@@ -121,6 +121,7 @@ zhip_result launch_embed_q5_k(const Dispatch &);
 zhip_result launch_embed_q6_k(const Dispatch &);
 zhip_result launch_embed_bf16(const Dispatch &);
 zhip_result launch_embed_f16(const Dispatch &);
+zhip_result launch_embed_iq4_xs(const Dispatch &);
 
 // Host-side helpers shared by the launchers.
 zhip_result fail(const Dispatch &d, zhip_result code, const char *fmt, ...);

@@ -269,6 +269,61 @@ zhip_result launch_embed_q6_k(const Dispatch &d) { return launch_embed<DecQ6_K>(
 zhip_result launch_embed_bf16(const Dispatch &d) { return launch_embed<DecBF16>(d, "embed_bf16"); }
 zhip_result launch_embed_f16(const Dispatch &d) { return launch_embed<DecF16>(d, "embed_f16"); }
 
+// ---- embed_iq4_xs: src/kernels/quant/iq4_xs.wgsl through embed_quant.wgsl ----------
+// Blocks of 256: d (f16), scales_h (u16), scales_l[4], qs[128]; a 32-weight group
+// has a signed six-bit scale biased by 32 and sixteen bytes of indices into a
+// nonlinear table, low nibbles first (src/ref/tensor.zig:162-181). Rows come as
+// the loader lays them out (136-byte blocks padded to 144) or, with a stride, as
+// the file stores them. A thread decodes one index byte: two weights, each
+// (d * scale) * table[index] with both products rounded to nearest.
+__global__ __launch_bounds__(256) void embed_iq4_xs_kernel(EmbedParams p, const uint32_t *tokens, const uint8_t *table, float *out, uint32_t row_bytes, uint32_t block_bytes) {
+    const int values[16] = {-127, -104, -83, -65, -49, -35, -22, -10, 1, 13, 25, 38, 53, 69, 89, 113};
+    const uint32_t t = blockIdx.x;
+    const uint32_t tok = tokens[t];
+    if (tok < p.row0 || tok >= p.row0 + p.chunk_rows) return;
+    const uint8_t *row = table + (size_t)(tok - p.row0) * row_bytes;
+    float *dst = out + (size_t)t * p.dim;
+    for (uint32_t i = threadIdx.x; i < p.dim / 2u; i += 256u) {
+        const uint8_t *b = row + (size_t)(i / 128u) * block_bytes;
+        const uint32_t group = (i / 16u) % 8u, j = i % 16u;
+        const float d = half_bits_to_float((uint32_t)b[0] | ((uint32_t)b[1] << 8));
+        const uint32_t scales_h = (uint32_t)b[2] | ((uint32_t)b[3] << 8);
+        const uint32_t low = (b[4u + group / 2u] >> (4u * (group % 2u))) & 15u, high = (scales_h >> (2u * group)) & 3u;
+        const float dl = __fmul_rn(d, (float)((int)(low | (high << 4)) - 32));
+        const uint32_t q = b[8u + 16u * group + j];
+        int lo = 0, hi = 0;
+#pragma unroll
+        for (uint32_t v = 0; v < 16; v++) {  // a table in registers: selects, not memory
+            lo = (q & 15u) == v ? values[v] : lo;
+            hi = (q >> 4) == v ? values[v] : hi;
+        }
+        float *o = dst + 256u * (i / 128u) + 32u * group + j;
+        o[0] = __fmul_rn(dl, (float)lo);
+        o[16] = __fmul_rn(dl, (float)hi);
+    }
+}
+
+zhip_result launch_embed_iq4_xs(const Dispatch &d) {
+    const char *name = "embed_iq4_xs";
+    if (d.params_size < sizeof(EmbedParams)) return fail(d, ZHIP_E_BAD_COMMAND, "%s: params block too small", name);
+    const EmbedParams &p = *reinterpret_cast<const EmbedParams *>(d.params);
+    for (int b = 1; b <= 3; b++)
+        if (!d.bind[b].bound) return fail(d, ZHIP_E_BAD_COMMAND, "%s: binding %d is not bound", name, b);
+    const uint32_t tokens = d.grid[0];
+    if (tokens == 0 || p.dim == 0) return ZHIP_OK;
+    if (p.dim % 256u != 0) return fail(d, ZHIP_E_BAD_COMMAND, "%s: dim = %u is not a multiple of 256", name, p.dim);
+    const uint32_t block_bytes = p.stride != 0 ? 136u : 144u;
+    const uint64_t min_row = (uint64_t)p.dim / 256u * block_bytes;
+    const uint64_t row_bytes = p.stride != 0 ? p.stride : min_row;
+    if (row_bytes < min_row || row_bytes > 0xffffffffull) return fail(d, ZHIP_E_BAD_COMMAND, "%s: stride %llu against a row of %llu bytes", name, (unsigned long long)row_bytes, (unsigned long long)min_row);
+    if ((uint64_t)tokens * 4u > d.bind[1].size || (p.chunk_rows ? (uint64_t)(p.chunk_rows - 1) * row_bytes + min_row : 0) > d.bind[2].size ||
+        (uint64_t)tokens * p.dim * 4u > d.bind[3].size)
+        return fail(d, ZHIP_E_BAD_COMMAND, "%s: bound ranges too small", name);
+    hipLaunchKernelGGL(embed_iq4_xs_kernel, dim3(tokens), dim3(256), 0, d.stream, p, reinterpret_cast<const uint32_t *>(d.bind[1].ptr), d.bind[2].ptr,
+                       reinterpret_cast<float *>(d.bind[3].ptr), (uint32_t)row_bytes, block_bytes);
+    return check_launch(d, name);
+}
+
 // ---- fill ----------------------------------------------------------------------
 __global__ __launch_bounds__(256) void fill_kernel(uint32_t *dst, uint64_t words, uint32_t value) {
     for (uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x; i < words; i += (uint64_t)gridDim.x * 256u) dst[i] = value;

@@ -113,6 +113,7 @@ static const KernelInfo kImplemented[] = {
     {"embed_q6_k", 4, 0b1000, VariantKind::none, launch_embed_q6_k, nullptr, nullptr, 1},
     {"embed_bf16", 4, 0b1000, VariantKind::none, launch_embed_bf16, nullptr, nullptr, 1},
     {"embed_f16", 4, 0b1000, VariantKind::none, launch_embed_f16, nullptr, nullptr, 1},
+    {"embed_iq4_xs", 4, 0b1000, VariantKind::none, launch_embed_iq4_xs, nullptr, nullptr, 1},
 };
 
 static const KernelInfo *find_kernel(const char *name, size_t len) {

@@ -41,12 +41,13 @@ class TensorType(enum.IntEnum):
     q4_k = 12
     q5_k = 13
     q6_k = 14
+    iq4_xs = 23
     bf16 = 30
 
 
 # (block_elems, block_bytes): src/gguf/gguf.zig:69-109.
 LAYOUT = {TensorType.f32: (1, 4), TensorType.f16: (1, 2), TensorType.bf16: (1, 2), TensorType.q8_0: (32, 34), TensorType.q3_k: (256, 110), TensorType.q4_k: (256, 144),
-          TensorType.q5_k: (256, 176), TensorType.q6_k: (256, 210)}
+          TensorType.q5_k: (256, 176), TensorType.q6_k: (256, 210), TensorType.iq4_xs: (256, 136)}
 
 
 @dataclass(frozen=True)
@@ -92,6 +93,7 @@ CONTRACTS = {
     Kernel.embed_q6_k: Contract(4, 0b1000),
     Kernel.embed_bf16: Contract(4, 0b1000),
     Kernel.embed_f16: Contract(4, 0b1000),
+    Kernel.embed_iq4_xs: Contract(4, 0b1000),
 }
 
 
@@ -113,9 +115,9 @@ def weight_kernel(op: str, t: TensorType) -> Kernel:
 
 def block_stride(t: TensorType) -> int:
     """src/kernels/kernels.zig:144-151: the GGUF block size, padded to a multiple
-    of 16 where it is not one (Q6_K: 210 -> 224, laid out by repad); Q3_K is
-    repacked into eight 16-byte units (repack_q3_k)."""
-    return {TensorType.q6_k: 224, TensorType.q3_k: 128}.get(t, LAYOUT[t][1])
+    of 16 where it is not one (Q6_K: 210 -> 224, IQ4_XS: 136 -> 144, laid out by
+    repad); Q3_K is repacked into eight 16-byte units (repack_q3_k)."""
+    return {TensorType.q6_k: 224, TensorType.q3_k: 128, TensorType.iq4_xs: 144}.get(t, LAYOUT[t][1])
 
 
 def row_bytes(t: TensorType, k: int) -> int:
