@@ -470,6 +470,44 @@ def test_matmul_bf16_mfma_tilings(ctx, rows, n, k):
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
 
 
+@pytest.mark.parametrize("rows,n,k,col0,pad,accumulate,packed", [
+    (128, 16400, 1024, 0, 0, False, True),    # whole token tiles, vector stores
+    (70, 16389, 768, 5, 9, True, False),      # ragged last weight tile, unaligned output: scalar stores
+    (17, 16400, 256, 4, 4, True, True),       # 64-token kernel, one chunk of k a wave
+    (1, 20000, 512, 0, 0, False, False),
+])
+def test_matmul_bf16_streamed_chunk(ctx, rows, n, k, col0, pad, accumulate, packed):
+    """A chunk of up to 128 tokens against a tall bf16 matrix with k <= 1024 (the
+    vocabulary projection of a prefill chunk) takes the kernel that streams the
+    weights into registers: against the rung's operand contract, columns
+    outside the chunk untouched, and every token's bits the same whether it runs
+    in the chunk or alone."""
+    c = ctx
+    rung = K.Prefill.bf16_mfma_xbf16 if packed else K.Prefill.bf16_mfma
+    x = c.random(rows * k, 1).reshape(rows, k)
+    xs = synth.bf16_round(x).astype(np.float64)
+    bits, values = random_half(c, n * k, 1)
+    wa = c.upload(bits.reshape(n, k))
+    stride = n + pad
+    init = c.random(rows * stride, 0.5).reshape(rows, stride)
+    c.set.select_prefill(c.rec, rung)
+
+    def run(first, count):
+        xa = c.upload(synth.to_bf16_bits(x[first : first + count]) if packed else x[first : first + count])
+        out = c.upload(init[first : first + count])
+        c.launcher().launch(Kernel.matmul_bf16, P.MatmulBf16(rows=count, n=n, k=k, col0=col0, out_stride=stride, accumulate=int(accumulate)), [xa, wa, out],
+                            (K.div_ceil(n, K.matmul_tile_n), K.div_ceil(count, K.matmul_tile_t), 1))
+        return c.read(out).reshape(count, stride)
+
+    got = run(0, rows)
+    want = xs @ values.reshape(n, k).astype(np.float64).T + (init[:, col0 : col0 + n] if accumulate else 0)
+    assert rel_err(got[:, col0 : col0 + n], want) <= 1e-5
+    assert np.array_equal(got[:, :col0], init[:, :col0]) and np.array_equal(got[:, col0 + n :], init[:, col0 + n :]), "columns outside the chunk were written"
+    for first, count in ((0, 1), (rows // 2, 1), (rows - 1, 1), (rows // 3, min(20, rows - rows // 3))):
+        assert run(first, count).tobytes() == got[first : first + count].tobytes(), "a token's bits depend on its chunk"
+    c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
+
+
 def launch_float_q8(c, x, weights, out, rows, accumulate, slices, chunked):
     """Two weight chunks exercise nonzero col0 and a padded output stride;
     split-k partials are dense per chunk (src/kernels/check.zig:752-770)."""

@@ -1,0 +1,258 @@
+// matmul_bf16 on the matrix cores for steps of up to 128 tokens over a short k
+// (up to 1024) and many matrix rows: the vocabulary projection of a prefill
+// chunk (src/kernels/matmul_half.wgsl's contract, the bf16 rung's operands).
+// Such a step is bound by the one pass over the weights, like a decode
+// multiply, so the kernel is built like one: the weights stream from memory
+// straight into the registers of the wave that multiplies them, each byte
+// loaded once by one wave, and nothing but results crosses LDS.
+//
+// A 512-thread workgroup is eight waves that split k eight ways. A wave keeps
+// its k range of every token in registers for the whole kernel, as matrix-core
+// operands (up to 128 tokens x 128 positions = 128 VGPRs), and walks over
+// sixteen-row weight tiles: a tile's operand is the lane's own row and eight
+// positions (16 bytes; the four lane groups cover 64 contiguous bytes of a row,
+// so a load touches 16 half lines, which costs what 8 whole lines cost), loaded
+// DEPTH - 1 tiles ahead. v_mfma_f32_16x16x32_bf16 takes the weights as its first
+// operand, so a lane ends up with four neighbouring outputs of one token; the
+// eight waves' partial sums meet in LDS (one 16-byte write a lane and token
+// tile) and thread i adds the eight partial vectors i, always in the order of
+// the k ranges, while the matrix cores are already on the next tile. The sums
+// of two neighbouring tiles are stored together, eight lanes to a token's 128
+// bytes: a store that fills whole cache lines spares L2 from fetching them
+// first (a plain copy with this write pattern takes 10 us longer over 78 MB in
+// 64-byte pieces than in 128-byte ones). Workgroups are persistent: workgroup
+// b of G takes the pairs of tiles b, b + G, b + 2 G ...
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+
+namespace zhip {
+
+typedef __bf16 sbf16x8 __attribute__((ext_vector_type(8)));
+typedef float sf32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t su32x4 __attribute__((ext_vector_type(4)));
+
+namespace {
+
+constexpr uint32_t THREADS = 512, WAVES = 8;
+constexpr int DEPTH = 2;  // weight tiles in registers a wave: one multiplied, the others in flight
+
+struct StreamArgs {
+    const uint8_t *x;  // packed bf16 rows
+    const uint8_t *w;
+    float *out;
+    uint32_t rows, n, k, col0, out_stride, accumulate;
+    uint32_t x_bytes, w_bytes;
+    uint32_t tiles;     // sixteen-row weight tiles
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const uint8_t *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, (int)bytes, 0x00020000);
+}
+
+// A barrier that waits for this wave's LDS traffic only: the weight loads of the
+// tiles ahead stay in flight.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+// Stores 16 bytes without the compiler's wait-count bookkeeping seeing a store. Loads
+// and stores complete out of order with each other, so with a store pending the
+// compiler makes every wait for a load a wait for all outstanding memory
+// operations, which would drain the weight tiles in flight once per tile. A wait
+// that counts only the loads issued after the awaited one is still sufficient
+// while a store is outstanding (loads complete in order among themselves; the
+// store only makes the wait stricter). The two idle cycles keep a following
+// instruction from overwriting the data registers before the store has read them.
+__device__ __forceinline__ void store_apart(sf32x4 *at, sf32x4 v) {
+    asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" ::"v"(at), "v"(v) : "memory");
+}
+
+// Each lane's vector of the lane whose number times four is `from`.
+__device__ __forceinline__ sf32x4 from_lane(sf32x4 v, uint32_t from) {
+    sf32x4 r;
+    r.x = __int_as_float(__builtin_amdgcn_ds_bpermute((int)from, __float_as_int(v.x)));
+    r.y = __int_as_float(__builtin_amdgcn_ds_bpermute((int)from, __float_as_int(v.y)));
+    r.z = __int_as_float(__builtin_amdgcn_ds_bpermute((int)from, __float_as_int(v.z)));
+    r.w = __int_as_float(__builtin_amdgcn_ds_bpermute((int)from, __float_as_int(v.w)));
+    return r;
+}
+
+// MT: token tiles of sixteen (rows <= 16 MT); KC: 32-position chunks of a wave's
+// k range (k = 256 KC).
+template <int MT, int KC>
+__global__ __launch_bounds__(THREADS) void matmul_bf16_stream_kernel(StreamArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [2][wave][MT * 64 lanes] partial vectors
+    constexpr uint32_t PART = MT * 64u * 16u;                       // bytes a wave writes per tile
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+    const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.x, a.x_bytes), wbuf = make_buffer(a.w, a.w_bytes);
+    // The lane's eight positions of chunk c: k = 32 KC wave + 32 c + 8 g.
+    const uint32_t kbyte = 2u * (32u * KC * wave + 8u * g);
+
+    // This wave's part of every token (tokens past `rows` lie past the buffer: zeros).
+    sbf16x8 xf[MT][KC];
+#pragma unroll
+    for (int i = 0; i < MT; i++)
+#pragma unroll
+        for (int c = 0; c < KC; c++)
+            xf[i][c] = __builtin_bit_cast(sbf16x8, __builtin_amdgcn_raw_buffer_load_b128(xbuf, (16u * i + l16) * a.k * 2u + kbyte + 64u * c, 0, 0));
+
+    // This workgroup's tiles, in pairs (a pair's outputs fill whole 128-byte lines): pairs
+    // b, b + G, b + 2 G ... of the G workgroups, so that at any time the chip reads one
+    // contiguous stretch of the matrix. Tile p of the run:
+    const uint32_t pairs = (a.tiles + 1u) / 2u;
+    auto tile_of = [&](uint32_t p) { return 2u * (blockIdx.x + (p >> 1) * gridDim.x) + (p & 1u); };
+    uint32_t count = 0;  // tiles of the run
+    if (blockIdx.x < pairs) {
+        const uint32_t mine = (pairs - 1u - blockIdx.x) / gridDim.x + 1u;
+        count = 2u * mine - (tile_of(2u * mine - 1u) >= a.tiles ? 1u : 0u);
+    }
+    // Row 16 tile + l16 of the matrix: the lane's part of the offset never changes, the
+    // tile's part is uniform and travels in a scalar register (which the buffer's range
+    // check does not see: n is a multiple of sixteen here, every row of a tile exists).
+    // Past the workgroup's last tile the loads still run, so that every wait counts the same
+    // loads on every path, but fetch the matrix's first tile again (from cache; unused).
+    const uint32_t wlane = l16 * a.k * 2u + kbyte, tile_bytes = 32u * a.k;
+    auto load_tile = [&](uint32_t p, su32x4 (&b)[KC]) __attribute__((always_inline)) {
+        const uint32_t base = (p < count ? tile_of(p) : 0u) * tile_bytes;
+#pragma unroll
+        for (int c = 0; c < KC; c++) b[c] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, wlane + 64u * c, base, 0);
+    };
+    // Tile q of the run: its matrix-core instructions, with the reads of tile q - 1's eight
+    // partial vectors in between (the matrix cores work while LDS answers), then the sum and
+    // store of tile q - 1, then this tile's partial sums into LDS buffer q % 2 and the
+    // barrier that publishes them. Buffer (q - 1) % 2 is written again in step q + 1, after
+    // that barrier, which every wave passes only when it has read what it needs.
+    static_assert(MT <= (int)WAVES, "one partial vector is read per token tile's instructions");
+    sf32x4 held = {0.f, 0.f, 0.f, 0.f};
+    auto step = [&](uint32_t q, const su32x4 (&b)[KC]) __attribute__((always_inline)) {
+        // (the four vectors of a token are stored permuted, see below)
+        const uint8_t *prev = lds + ((q & 1u) ^ 1u) * (WAVES * PART) + ((tid & (MT * 64u - 1u)) ^ ((tid >> 4) & 3u)) * 16u;
+        constexpr int PER = WAVES / MT;  // partial vectors read per token tile's instructions
+        // acc[i][r]: matrix row 16 tile + 4 g + r, token 16 i + l16: vector (i, token, g), stored
+        // at g ^ (token / 4) within the token's four so that the lanes of one lane group, whose
+        // vectors lie 64 bytes apart, fall into sixteen different bank groups. A token tile's
+        // sums leave for LDS while the next one's instructions run: two accumulators suffice.
+        uint8_t *mine = lds + (q & 1u) * (WAVES * PART) + wave * PART + (l16 * 4u + (g ^ (l16 >> 2))) * 16u;
+        sf32x4 acc[2], got[PER], sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int i = 0; i < MT; i++) {
+            acc[i & 1] = sf32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int c = 0; c < KC; c++) acc[i & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sbf16x8, b[c]), xf[i][c], acc[i & 1], 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            if (i > 0) {
+                *reinterpret_cast<sf32x4 *>(mine + (i - 1) * 1024u) = acc[(i - 1) & 1];
+                // The vectors read a group of instructions ago are added, in the order of the k ranges.
+#pragma unroll
+                for (int e = 0; e < PER; e++) sum = (i == 1 && e == 0) ? got[0] : sum + got[e];
+            }
+#pragma unroll
+            for (int e = 0; e < PER; e++) got[e] = *reinterpret_cast<const sf32x4 *>(prev + (i * PER + e) * PART);
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        *reinterpret_cast<sf32x4 *>(mine + (MT - 1) * 1024u) = acc[(MT - 1) & 1];
+#pragma unroll
+        for (int e = 0; e < PER; e++) sum = (MT == 1 && e == 0) ? got[0] : sum + got[e];
+        if (q > 0u && tid < MT * 64u) {
+            // Vector tid of tile p = q - 1 of the run: token tile tid / 64 (this wave's lanes
+            // hold all of it), token lane / 4, outputs 4 (lane % 4) .. + 3 of the tile's 16.
+            const uint32_t p = q - 1u, ttile = 16u * (tid >> 6);
+            if (!(p & 1u) && p + 1u < count) {
+                held = sum;  // waits for its neighbour: a pair fills whole 128-byte lines
+            } else if (p & 1u) {
+                // Two stores of eight tokens: lanes 8 u .. 8 u + 7 write token u's 32 outputs.
+#pragma unroll
+                for (uint32_t half8 = 0; half8 < 2; half8++) {
+                    const uint32_t tt = 8u * half8 + (lane >> 3), from = 4u * (4u * tt + (lane & 3u));
+                    // Both gathers run in every lane (a lane's source may sit in the other half).
+                    const sf32x4 first = from_lane(held, from), second = from_lane(sum, from);
+                    const sf32x4 v = (lane & 4u) ? second : first;
+                    const uint32_t t = ttile + tt, j = 16u * tile_of(p - 1u) + 4u * (lane & 7u);
+                    if (t < a.rows) {
+                        sf32x4 *o = reinterpret_cast<sf32x4 *>(a.out + (size_t)t * a.out_stride + a.col0 + j);
+                        store_apart(o, a.accumulate ? v + *o : v);
+                    }
+                }
+            } else {
+                const uint32_t t = ttile + (lane >> 2), j = 16u * tile_of(p) + 4u * (lane & 3u);
+                if (t < a.rows) {
+                    sf32x4 *o = reinterpret_cast<sf32x4 *>(a.out + (size_t)t * a.out_stride + a.col0 + j);
+                    if (a.accumulate) sum += *o;
+                    store_apart(o, sum);
+                }
+            }
+        }
+        lds_barrier();
+    };
+
+    // DEPTH register sets in rotation: DEPTH - 1 tiles in flight behind the one multiplied.
+    // Every wave of the workgroup runs the same steps (the barrier inside); one step past
+    // the last tile sums and stores that tile (its own instructions multiply stale registers
+    // into partial sums nobody reads).
+    su32x4 b[DEPTH][KC];
+#pragma unroll
+    for (int s = 0; s < DEPTH - 1; s++) load_tile(s, b[s]);
+    const uint32_t rounds = count ? count + 1u : 0u;
+    for (uint32_t r = 0; r < rounds; r += DEPTH) {
+#pragma unroll
+        for (int s = 0; s < DEPTH; s++) {
+            load_tile(r + s + (DEPTH - 1), b[(s + DEPTH - 1) % DEPTH]);
+            if (r + s < rounds) step(r + s, b[s]);
+        }
+    }
+}
+
+template <int MT, int KC>
+static zhip_result launch(const Dispatch &d, const char *name, const StreamArgs &a, uint32_t groups) {
+    auto kernel = matmul_bf16_stream_kernel<MT, KC>;
+    constexpr int bytes = 2 * WAVES * MT * 64 * 16;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
+        }
+        configured = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3(groups), dim3(THREADS), bytes, d.stream, a);
+    return check_launch(d, name);
+}
+
+template <int MT>
+static zhip_result launch_k(const Dispatch &d, const char *name, const StreamArgs &a, uint32_t groups) {
+    switch (a.k / 256u) {
+    case 1: return launch<MT, 1>(d, name, a, groups);
+    case 2: return launch<MT, 2>(d, name, a, groups);
+    case 3: return launch<MT, 3>(d, name, a, groups);
+    default: return launch<MT, 4>(d, name, a, groups);
+    }
+}
+
+}  // namespace
+
+// Whether the streaming kernel suits a (validated) bf16 step: few tokens, a short
+// k in whole chunks, enough whole weight tiles to occupy every CU several times,
+// and outputs that can be stored 16 bytes at a time.
+bool matmul_bf16_stream_accepts(const Dispatch &d, const float *out, uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride) {
+    return rows >= 1 && rows <= 128 && k >= 256 && k <= 1024 && k % 256u == 0 && (n + 15u) / 16u >= 4u * (uint32_t)d.dev->compute_units &&
+           (uintptr_t)out % 16u == 0 && out_stride % 4u == 0 && col0 % 4u == 0 && n % 16u == 0;
+}
+
+zhip_result launch_matmul_bf16_stream(const Dispatch &d, const char *name, const uint8_t *x, const uint8_t *w, float *out,
+    uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate) {
+    const uint64_t x_bytes = (uint64_t)rows * k * 2u, w_bytes = (uint64_t)n * k * 2u;
+    // 32-bit byte offsets, up to a tile of sixteen past the last token and row.
+    if (w_bytes + 32ull * k >= 0xfffffff0ull - 256u) return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
+    StreamArgs a{};
+    a.x = x; a.w = w; a.out = out;
+    a.rows = rows; a.n = n; a.k = k; a.col0 = col0; a.out_stride = out_stride; a.accumulate = accumulate;
+    a.x_bytes = (uint32_t)x_bytes; a.w_bytes = (uint32_t)w_bytes;
+    a.tiles = (n + 15u) / 16u;
+    const uint32_t groups = a.tiles < (uint32_t)d.dev->compute_units ? a.tiles : (uint32_t)d.dev->compute_units;
+    return rows <= 64u ? launch_k<4>(d, name, a, groups) : launch_k<8>(d, name, a, groups);
+}
+
+}  // namespace zhip
