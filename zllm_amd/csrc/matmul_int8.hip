@@ -3,8 +3,11 @@
 //   out[t][col0 + j] = sum over 32-weight units of dx * (s * sum(q * qx) - m * sum(qx))
 // with every unit's integer sum exact. Here the unit sums run on the int8 matrix
 // cores (v_mfma_i32_16x16x32_i8: one 32-deep unit of 16 x 16 outputs per
-// instruction) and the scales are applied to the integer results in f32, which
-// is what bounds these kernels: three vector operations per output and unit.
+// instruction). Q8_0's f16 unit scales are applied to the integer results in
+// f32 (three vector operations per output and unit, which bounds that kernel);
+// the K formats' 6- and 8-bit integer scales are applied in integers (one
+// 24-bit multiply-add per output and unit), their minimums by one more matrix
+// instruction per unit, and a block's two f32 scales once per 256 positions.
 //
 // A 256-thread workgroup computes 64 tokens x 64 rows in steps of 256 positions;
 // wave w owns rows 16 w .. 16 w + 15 for all 64 tokens (four accumulator tiles).
@@ -31,6 +34,7 @@ constexpr uint32_t TT = 64;     // tokens per workgroup
 constexpr uint32_t TN = 64;     // rows per workgroup
 constexpr uint32_t STEP = 256;  // positions per step
 constexpr uint32_t LINE = STEP + 8;  // bytes between register-staged token lines in LDS
+constexpr uint32_t UNITS = 1;  // units the K-format kernel schedules together (2 and 4 measured no faster)
 
 struct I8Args {
     const uint8_t *qx;   // rows x k int8, four per word
@@ -257,11 +261,14 @@ struct I8Q4 {
 #pragma unroll
         for (uint32_t c = 0; c < 4; c++) r.q[c] = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 16u + 32u * c + 8u * g, 0, 0);
     }
-    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t, iu32x2 &b, float &s0, float &s1, float &mn) {
-        const float d = half_bits_to_float(r.h.x & 0xffffu), dmin = half_bits_to_float(r.h.x >> 16);
+    static __device__ __forceinline__ void block(const Raw &r, float &d, float &dmin) {
+        d = half_bits_to_float(r.h.x & 0xffffu);
+        dmin = half_bits_to_float(r.h.x >> 16);
+    }
+    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t, iu32x2 &b, int &s0, int &s1, int &mn) {
         const uint2 sm = scale_min_k4(r.h.y, r.h.z, r.h.w, u);
-        s0 = s1 = d * (float)sm.x;
-        mn = dmin * (float)sm.y;
+        s0 = s1 = (int)sm.x;
+        mn = (int)sm.y;
         b = r.q[u >> 1];
         if (u & 1u) b = b >> 4;
         b = b & 0x0f0f0f0fu;
@@ -282,11 +289,14 @@ struct I8Q5 {
 #pragma unroll
         for (uint32_t c = 0; c < 4; c++) r.q[c] = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 48u + 32u * c + 8u * g, 0, 0);
     }
-    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t, iu32x2 &b, float &s0, float &s1, float &mn) {
-        const float d = half_bits_to_float(r.h.x & 0xffffu), dmin = half_bits_to_float(r.h.x >> 16);
+    static __device__ __forceinline__ void block(const Raw &r, float &d, float &dmin) {
+        d = half_bits_to_float(r.h.x & 0xffffu);
+        dmin = half_bits_to_float(r.h.x >> 16);
+    }
+    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t, iu32x2 &b, int &s0, int &s1, int &mn) {
         const uint2 sm = scale_min_k4(r.h.y, r.h.z, r.h.w, u);
-        s0 = s1 = d * (float)sm.x;
-        mn = dmin * (float)sm.y;
+        s0 = s1 = (int)sm.x;
+        mn = (int)sm.y;
         b = r.q[u >> 1];
         if (u & 1u) b = b >> 4;
         b = (b & 0x0f0f0f0fu) | (((r.qh >> u) & 0x01010101u) << 4);
@@ -310,13 +320,16 @@ struct I8Q6 {
         r.sc = __builtin_amdgcn_raw_buffer_load_b128(w, blk + 192u, 0, 0);
         r.d = __builtin_amdgcn_raw_buffer_load_b32(w, blk + 208u, 0, 0);
     }
-    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t, iu32x2 &b, float &s0, float &s1, float &mn) {
+    static __device__ __forceinline__ void block(const Raw &r, float &d, float &dmin) {
+        d = half_bits_to_float(r.d & 0xffffu);
+        dmin = 0.f;
+    }
+    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t, iu32x2 &b, int &s0, int &s1, int &mn) {
         const uint32_t n = u >> 2, c = u & 3u;
-        const float d = half_bits_to_float(r.d & 0xffffu);
         const uint32_t pair = r.sc[(8u * n + 2u * c) >> 2] >> (16u * (c & 1u));  // scales 8 n + 2 c and the next
-        s0 = d * (float)sbyte(pair, 0);
-        s1 = d * (float)sbyte(pair, 1);
-        mn = 0.f;
+        s0 = sbyte(pair, 0);
+        s1 = sbyte(pair, 1);
+        mn = 0;
         const iu32x2 q = ((r.ql[2u * n + (c & 1u)] >> (4u * (c >> 1))) & 0x0f0f0f0fu) | (((r.qh[n] >> (2u * c)) & 0x03030303u) << 4);
         b = (q + 0x60606060u) ^ 0x80808080u;  // minus 32 a byte, no borrows
     }
@@ -332,12 +345,15 @@ struct I8Q3 {
 #pragma unroll
         for (uint32_t i = 0; i < 8; i++) r.u[i] = __builtin_amdgcn_raw_buffer_load_b128(w, blk + 16u * i, 0, 0);
     }
-    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t g, iu32x2 &b, float &s0, float &s1, float &mn) {
+    static __device__ __forceinline__ void block(const Raw &r, float &d, float &dmin) {
+        d = half_bits_to_float(r.u[0].w >> 16);  // every unit of a block carries the block's d
+        dmin = 0.f;
+    }
+    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t g, iu32x2 &b, int &s0, int &s1, int &mn) {
         const iu32x4 v = r.u[u];
-        const float d = half_bits_to_float(v.w >> 16);
-        s0 = d * (float)sbyte(v.w, 0);
-        s1 = d * (float)sbyte(v.w, 1);
-        mn = 0.f;
+        s0 = sbyte(v.w, 0);
+        s1 = sbyte(v.w, 1);
+        mn = 0;
         // Position 4 e + i: bits 2 (e % 4) of byte i of word e / 4, high bit 8 i + e.
         const uint32_t l = (g < 2u ? v.x : v.y) >> (4u * (g & 1u)), hb = v.z >> (2u * g);
         const iu32x2 c = {(l & 0x03030303u) | ((hb & 0x01010101u) << 2), ((l >> 2) & 0x03030303u) | (((hb >> 1) & 0x01010101u) << 2)};
@@ -346,10 +362,9 @@ struct I8Q3 {
 };
 
 template <class P>
-__global__ __launch_bounds__(256) void matmul_kquant_i8_kernel(I8Args a) {
+__global__ __launch_bounds__(256, 2) void matmul_kquant_i8_kernel(I8Args a) {
     __shared__ __align__(16) uint8_t lds_q[2][TT * LINE];
     __shared__ __align__(16) float lds_d[2][TT];      // the tokens' block scales
-    __shared__ __align__(16) float lds_s[2][8][TT];   // sum of each unit's bytes
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
     const uint32_t n0 = blockIdx.x * TN, t0 = blockIdx.y * TT;
     const uint32_t kb = blockIdx.z * a.k_slice, ke = min(a.k, kb + a.k_slice);
@@ -375,19 +390,10 @@ __global__ __launch_bounds__(256) void matmul_kquant_i8_kernel(I8Args a) {
     };
     auto stash = [&](uint32_t buf) __attribute__((always_inline)) {
         uint8_t *line = &lds_q[buf][atok * LINE + 64u * aq];
-        int sums[2] = {0, 0};
 #pragma unroll
         for (uint32_t i = 0; i < 4; i++) {
             *reinterpret_cast<iu32x2 *>(line + 16u * i) = ra[i].xy;
             *reinterpret_cast<iu32x2 *>(line + 16u * i + 8u) = ra[i].zw;
-            if (P::HAS_MIN) {
-#pragma unroll
-                for (uint32_t e = 0; e < 4; e++) sums[i >> 1] = __builtin_amdgcn_sdot4((int)ra[i][e], 0x01010101, sums[i >> 1], false);
-            }
-        }
-        if (P::HAS_MIN) {
-            lds_s[buf][2u * aq][atok] = (float)sums[0];
-            lds_s[buf][2u * aq + 1u][atok] = (float)sums[1];
         }
         if (aq == 0u) lds_d[buf][atok] = __uint_as_float(rd);
     };
@@ -403,42 +409,70 @@ __global__ __launch_bounds__(256) void matmul_kquant_i8_kernel(I8Args a) {
         const uint32_t k0 = k_first + s * STEP, buf = s & 1u;
         const bool more = s + 1u < steps;
         if (more) fetch(k0 + STEP, next);
-        if32x4 part[4];
+        // A block's units are summed in integers: a unit's exact sum times its 6- or 8-bit
+        // scale (one 24-bit multiply-add a result), the minimums as one more matrix
+        // instruction a unit whose second operand is the unit's minimum in all 32 positions,
+        // accumulated by the matrix cores. The block's two f32 scales are applied once.
+        i32x4 isum[4], msum[4];
 #pragma unroll
-        for (int mt = 0; mt < 4; mt++) part[mt] = if32x4{0.f, 0.f, 0.f, 0.f};
+        for (int mt = 0; mt < 4; mt++) isum[mt] = msum[mt] = i32x4{0, 0, 0, 0};
 #pragma unroll
-        for (uint32_t u = 0; u < 8; u++) {
-            const uint32_t kpos = k0 + 32u * u;
-            if (kpos < kb || kpos >= ke) continue;
-            iu32x2 w8;
-            float s0, s1, mn;
-            P::unit(cur, u, g, w8, s0, s1, mn);
-            const iu32x2 zero = {0u, 0u};
-            const long b0 = as_operand(P::HALVES ? (g < 2u ? w8 : zero) : w8);
-            const long b1 = as_operand(g < 2u ? zero : w8);
+        for (uint32_t u = 0; u < 8; u += UNITS) {
+            // UNITS units at a time, behind a branch that skips units outside the slice [kb, ke)
+            // and keeps the groups apart (scheduled all together they need hundreds of
+            // registers); a group's units overlap each other's LDS and matrix-core latencies.
+            bool live[UNITS], any = false;
+#pragma unroll
+            for (uint32_t e = 0; e < UNITS; e++) {
+                const uint32_t kpos = k0 + 32u * (u + e);
+                live[e] = kpos >= kb && kpos < ke;
+                any = any || live[e];
+            }
+            if (!any) continue;
+            long b0[UNITS], b1[UNITS], bm[UNITS];
+            int s0[UNITS], s1[UNITS];
+#pragma unroll
+            for (uint32_t e = 0; e < UNITS; e++) {
+                iu32x2 w8;
+                int mn;
+                P::unit(cur, u + e, g, w8, s0[e], s1[e], mn);
+                s0[e] = live[e] ? s0[e] : 0;
+                s1[e] = live[e] ? s1[e] : 0;
+                mn = live[e] ? mn : 0;
+                const iu32x2 zero = {0u, 0u};
+                b0[e] = as_operand(P::HALVES ? (g < 2u ? w8 : zero) : w8);
+                b1[e] = as_operand(g < 2u ? zero : w8);
+                const uint32_t m4 = (uint32_t)mn * 0x01010101u;
+                bm[e] = as_operand(iu32x2{m4, m4});
+            }
 #pragma unroll
             for (uint32_t mt = 0; mt < 4; mt++) {
-                const long af = *reinterpret_cast<const long *>(&lds_q[buf][(16u * mt + l16) * LINE + 32u * u + 8u * g]);
-                const i32x4 is = __builtin_amdgcn_mfma_i32_16x16x32_i8(af, b0, i32x4{0, 0, 0, 0}, 0, 0, 0);
 #pragma unroll
-                for (int i = 0; i < 4; i++) part[mt][i] = fmaf(s0, (float)is[i], part[mt][i]);
-                if (P::HALVES) {
-                    const i32x4 is1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(af, b1, i32x4{0, 0, 0, 0}, 0, 0, 0);
+                for (uint32_t e = 0; e < UNITS; e++) {
+                    const long af = *reinterpret_cast<const long *>(&lds_q[buf][(16u * mt + l16) * LINE + 32u * (u + e) + 8u * g]);
+                    const i32x4 is = __builtin_amdgcn_mfma_i32_16x16x32_i8(af, b0[e], i32x4{0, 0, 0, 0}, 0, 0, 0);
 #pragma unroll
-                    for (int i = 0; i < 4; i++) part[mt][i] = fmaf(s1, (float)is1[i], part[mt][i]);
-                }
-                if (P::HAS_MIN) {
-                    const if32x4 xs = *reinterpret_cast<const if32x4 *>(&lds_s[buf][u][16u * mt + 4u * g]);
+                    for (int i = 0; i < 4; i++) isum[mt][i] = __mul24(s0[e], is[i]) + isum[mt][i];
+                    if (P::HALVES) {
+                        const i32x4 is1 = __builtin_amdgcn_mfma_i32_16x16x32_i8(af, b1[e], i32x4{0, 0, 0, 0}, 0, 0, 0);
 #pragma unroll
-                    for (int i = 0; i < 4; i++) part[mt][i] = fmaf(-mn, xs[i], part[mt][i]);
+                        for (int i = 0; i < 4; i++) isum[mt][i] = __mul24(s1[e], is1[i]) + isum[mt][i];
+                    }
+                    if (P::HAS_MIN) msum[mt] = __builtin_amdgcn_mfma_i32_16x16x32_i8(af, bm[e], msum[mt], 0, 0, 0);
                 }
             }
         }
+        float d, dmin;
+        P::block(cur, d, dmin);
 #pragma unroll
         for (uint32_t mt = 0; mt < 4; mt++) {
             const if32x4 dxv = *reinterpret_cast<const if32x4 *>(&lds_d[buf][16u * mt + 4u * g]);
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[mt][i] = fmaf(dxv[i], part[mt][i], acc[mt][i]);
+            for (int i = 0; i < 4; i++) {
+                float part = d * (float)isum[mt][i];
+                if (P::HAS_MIN) part = fmaf(-dmin, (float)msum[mt][i], part);
+                acc[mt][i] = fmaf(dxv[i], part, acc[mt][i]);
+            }
         }
         if (more) {
             stash(buf ^ 1u);
