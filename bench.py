@@ -402,44 +402,58 @@ def bench_c4(env):
 def bench_c4_int8(env):
     """The same product as C4 the way the reference's default prefill computes it:
     quantize_q8 rounds the f32 activations to Q8_0 blocks, matmul_q8_0 multiplies
-    integers on the int8 matrix cores and scales every 32-weight unit."""
+    integers on the int8 matrix cores and scales every 32-weight unit. The K
+    formats' multiplies (Q8_K activations) on the same shape ride along."""
     synth, oracle, K, TensorType, P = env["synth"], env["oracle"], env["K"], env["TensorType"], env["P"]
     rec, kset, b = env["rec"], env["kset"], env["b"]
     rows, k, n = 512, 4096, 4096
     g = synth.rng(0xC4)
-    raw = synth.q8_0_rows(g, n, k)
     x = synth.activations(g, rows, k)
-    src = env["upload"](raw)
     xa = env["upload"](x)
-    rb = K.row_bytes(TensorType.q8_0, k)
     out = env["output"](4 * rows * n)
-    qx, dx = env["output"](rows * k), env["output"](4 * rows * k // 32)
-    launches = []
-    for _ in range(4):
-        wa = env["output"](n * rb)
-        K.Launcher(rec, kset).layout(TensorType.q8_0, src, wa, n, k)
-        quant = b.add(K.Kernel.quantize_q8, P.QuantizeQ8(k=k, block=32), [xa, qx, dx, xa], K.Grid.tiles_y(K.div_ceil(k, 256), 1))
-        p = P.MatmulQuant(rows=rows, n=n, k=k, col0=0, out_stride=n, k_slice=k)
-        mul = b.add(K.Kernel.matmul_q8_0, p, [qx, wa, out, dx], K.Grid.tiles_y(K.div_ceil(n, K.matmul_quant_tile_n), K.matmul_quant_tile_t))
-        launches.append(env["Chain"]([quant, mul], rows))
-    b.finish()
-    env["flush"]()
-    steps = max(1, env["args"].steps // 4)
-    wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 4), per_step=2)
-    got = env["read"](out)[: rows * n].reshape(rows, n).astype(np.float64)
-    w = oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k)
-    xs = oracle.round_like_llama(oracle.Q8_0, x)
-    want = xs.astype(np.float64) @ w.astype(np.float64).T
     ops = 2 * rows * n * k
-    return {
-        "workload": "C4 shape through quantize_q8 + matmul_q8_0: f32 activations rounded to Q8_0 blocks, int8 MFMA, f32 scaling per 32-weight unit",
-        "ops_per_step": ops,
-        "us_per_step_wall": round(wall / steps * 1e6, 3),
-        "us_per_step_gpu": round(gpu_s / steps * 1e6, 3),
-        "TOPs_gpu": round(ops * steps / gpu_s / 1e12, 1),
-        "int8_mfma_frac": round(ops * steps / gpu_s / 1e12 / MFMA_INT8_PEAK_TOPS, 4),
-        "max_err_over_max_want": float(np.max(np.abs(got - want)) / np.max(np.abs(want))),
-    }
+
+    def one(t, raw, otype, what):
+        block = K.act_block(t)
+        src = env["upload"](raw)
+        rb = K.row_bytes(t, k)
+        qx, dx = env["output"](rows * k), env["output"](4 * rows * k // block)
+        launches = []
+        for _ in range(4):
+            wa = env["output"](n * rb)
+            if K.needs_layout(t):
+                K.Launcher(rec, kset).layout(t, src, wa, n, k)
+            else:
+                rec.copy_buffer(src.buffer, src.offset, wa.buffer, wa.offset, raw.size)
+            quant = b.add(K.Kernel.quantize_q8, P.QuantizeQ8(k=k, block=block), [xa, qx, dx, xa], K.Grid.tiles_y(K.div_ceil(k, 256), 1))
+            p = P.MatmulQuant(rows=rows, n=n, k=k, col0=0, out_stride=n, k_slice=k)
+            mul = b.add(K.weight_kernel("matmul", t), p, [qx, wa, out, dx], K.Grid.tiles_y(K.div_ceil(n, K.matmul_quant_tile_n), K.matmul_quant_tile_t))
+            launches.append(env["Chain"]([quant, mul], rows))
+        b.finish()
+        env["flush"]()
+        steps = max(1, env["args"].steps // 4)
+        wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 4), per_step=2)
+        got = env["read"](out)[: rows * n].reshape(rows, n).astype(np.float64)
+        w = oracle.dequantize(otype, raw, n * k).reshape(n, k)
+        xs = oracle.round_like_llama(otype, x)
+        want = xs.astype(np.float64) @ w.astype(np.float64).T
+        return {
+            "workload": what,
+            "ops_per_step": ops,
+            "us_per_step_wall": round(wall / steps * 1e6, 3),
+            "us_per_step_gpu": round(gpu_s / steps * 1e6, 3),
+            "TOPs_gpu": round(ops * steps / gpu_s / 1e12, 1),
+            "int8_mfma_frac": round(ops * steps / gpu_s / 1e12 / MFMA_INT8_PEAK_TOPS, 4),
+            "max_err_over_max_want": float(np.max(np.abs(got - want)) / np.max(np.abs(want))),
+        }
+
+    res = one(TensorType.q8_0, synth.q8_0_rows(g, n, k), oracle.Q8_0,
+              "C4 shape through quantize_q8 + matmul_q8_0: f32 activations rounded to Q8_0 blocks, int8 MFMA, f32 scaling per 32-weight unit")
+    res["k_formats"] = {}
+    for t, otype in ((TensorType.q4_k, oracle.Q4_K), (TensorType.q5_k, oracle.Q5_K), (TensorType.q6_k, oracle.Q6_K), (TensorType.q3_k, oracle.Q3_K)):
+        r = one(t, synth.random_blocks(g, t.name, n, k), otype, f"the same shape through quantize_q8 (Q8_K blocks) + matmul_{t.name}")
+        res["k_formats"][t.name] = {key: r[key] for key in ("us_per_step_gpu", "TOPs_gpu", "max_err_over_max_want")}
+    return res
 
 
 def bench_c5(env):
