@@ -210,6 +210,11 @@ MFMA_VARIANT = K.MatvecVariant(wg=512, lanes=64, rows=16)
     (True, 5, 96, 4096),      # four slabs
     (False, 3, 100, 2048),    # accumulate epilogue, an odd token count
     (False, 1, 530, 1024),    # one token, more than one workgroup
+    # k of 2048 or 4096 and whole tiles: the kernel with the tokens' operands in registers
+    (False, 8, 4112, 4096),   # 257 tiles: a second tile for the first workgroup
+    (True, 8, 4128, 4096),    # gate and up tiles of 258 output tiles
+    (True, 3, 64, 2048),      # one block a wave
+    (False, 2, 48, 2048),
 ])
 def test_quant_matvec_mfma_variant(ctx, pair, rows, n, k):
     """The matrix-core variant of matvec_q4_k (a wave per sixteen rows): every

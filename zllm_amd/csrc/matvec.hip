@@ -115,6 +115,8 @@ __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
 // The matrix-core variant of matvec_q4_k (matvec_mfma.hip).
 bool matvec_q4k_mfma_accepts(const MvArgs &a);
 zhip_result launch_matvec_q4k_mfma(const Dispatch &d, const MvArgs &a, uint64_t x_bytes, uint64_t w_bytes);
+bool matvec_q4k_mfma_resident_accepts(const MvArgs &a);
+zhip_result launch_matvec_q4k_mfma_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
 // The tuned multiply (matvec_quant.hip): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
 zhip_result launch_matvec_quant(const Dispatch &d, const MvArgs &a, int type);
 
@@ -191,6 +193,9 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     a.norm_w = norm ? reinterpret_cast<const float *>(d.bind[4].ptr) : nullptr;
 
     // MatvecVariant (wg 512, lanes 64, rows 16) names the matrix-core variant: a wave per sixteen rows.
+    // (k of 2048 or 4096 and whole tiles: the kernel that keeps the tokens' operands in registers.)
+    if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && v.act_div == 0u && matvec_q4k_mfma_resident_accepts(a))
+        return launch_matvec_q4k_mfma_resident(d, a, d.bind[2].size);
     if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && v.act_div == 0u && matvec_q4k_mfma_accepts(a))
         return launch_matvec_q4k_mfma(d, a, d.bind[1].size, d.bind[2].size);
     // The tuned kernel takes rows of whole 64-weight tasks.

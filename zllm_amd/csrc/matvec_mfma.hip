@@ -169,10 +169,15 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_kernel(MfArgs q) {
     // Each token's scale: the power of two that puts its largest magnitude in [2^14, 2^15).
     if (wave < a.m) {
         const float4 *xr = reinterpret_cast<const float4 *>(a.x + (size_t)wave * a.xr);
+        // Sixteen vectors a lane at a time, all loaded before any is used: one trip to memory
+        // per 4096 positions, not one per vector.
         float big = 0.f;
-        for (uint32_t i = lane; i < a.k / 4u; i += 64u) {
-            const float4 v = xr[i];
-            big = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fmaxf(fabsf(v.z), fabsf(v.w)), big));
+        for (uint32_t base = lane; base < a.k / 4u; base += 1024u) {
+            float4 v[16];
+#pragma unroll
+            for (uint32_t i = 0; i < 16; i++) v[i] = base + 64u * i < a.k / 4u ? xr[base + 64u * i] : float4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (uint32_t i = 0; i < 16; i++) big = fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)), fmaxf(fmaxf(fabsf(v[i].z), fabsf(v[i].w)), big));
         }
 #pragma unroll
         for (int off = 32; off > 0; off >>= 1) big = fmaxf(big, __shfl_xor(big, off, 64));

@@ -1,0 +1,321 @@
+// matvec_q4_k, matrix-core variant for k = 2048 or 4096: the same arithmetic as
+// matvec_mfma.hip (weights as exact f16 values 16 + q, every token as two f16
+// rows, per-token power-of-two scale; see there), laid out so that nothing
+// is recomputed and nothing but partial results crosses LDS.
+//
+// A 512-thread workgroup is eight waves that split k eight ways (one or two
+// 256-weight blocks a wave). A wave builds its k range of all tokens' f16 rows
+// once, straight into matrix-core operands that stay in registers for the
+// whole kernel (64 VGPRs at k = 4096), together with the rows' sub-block sums
+// (32 VGPRs). It then walks over sixteen-row weight tiles, persistent
+// workgroups taking tiles b, b + G, ...: its blocks of the tile's sixteen rows
+// (144 sixteen-byte chunks a block, three wave-wide direct loads into a private
+// ring of LDS slots: whole-line accesses; a lane loading its own row's bytes
+// straight into registers costs fifty cache accesses a load) arrive a tile
+// ahead, each lane reads its row's header and nibbles back, and multiplies;
+// the eight waves' partial sums (512 bytes a wave and tile) meet in LDS, where
+// 128 threads add the eight for one output each (row i % 16, token i / 16) in
+// the order of the k ranges, apply the SILU_PAIR / ACCUMULATE epilogue and store. One
+// barrier a tile; no barrier waits for the loads in flight.
+//
+// Contract as the other variants (src/kernels/matvec_quant.wgsl.hbs); a token's
+// result does not depend on how many tokens share the launch.
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "decode.cuh"
+#include "matvec_common.cuh"
+
+namespace zhip {
+
+typedef _Float16 rf16x8 __attribute__((ext_vector_type(8)));
+typedef float rf32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t ru32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t ru32x2 __attribute__((ext_vector_type(2)));
+
+namespace {
+
+constexpr uint32_t THREADS = 512, WAVES = 8;
+constexpr int DEPTH = 2;  // ring slots a wave: one tile multiplied, the others in flight
+constexpr uint32_t SLOT = 3u * 1024u;  // a block: 2304 bytes; the third load's idle lanes land behind them
+
+struct ResArgs {
+    MvArgs a;
+    uint32_t w_bytes;
+    uint32_t nibble_mask, sixteen;  // 0x03C003C0, 0x4C004C00 (see nibbles)
+    uint32_t out_tiles;             // sixteen-output tiles
+};
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, (int)bytes, 0x00020000);
+}
+
+// A barrier that waits for this wave's LDS traffic only: the weight loads of the
+// tile ahead stay in flight.
+__device__ __forceinline__ void lds_barrier() {
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
+typedef __attribute__((address_space(3))) void *lds_ptr;
+
+// One wave-wide load of 16 bytes a lane straight into LDS (lane l lands at dst + 16 l). The
+// destination reaches the load as a bare LDS address, so the compiler keeps no dependency
+// between these loads and later LDS reads; the explicit waits order them.
+__device__ __forceinline__ void load_lds_b128(__amdgpu_buffer_rsrc_t buf, uint8_t *dst, uint32_t voffset, uint32_t soffset) {
+    uint32_t address = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);
+    asm volatile("" : "+s"(address));
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)(uintptr_t)address, 16, voffset, soffset, 0, 0);
+}
+
+template <int LEFT>
+__device__ __forceinline__ void wait_loads() {
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LEFT) : "memory");
+}
+
+// A 4-byte store the compiler's wait-count bookkeeping does not see as a store: with one
+// pending it would turn every wait for a weight load into a wait for all loads in flight
+// (loads and stores complete out of order with each other). A wait that counts only the
+// loads issued after the awaited one stays sufficient while a store is outstanding.
+__device__ __forceinline__ void store_apart(float *at, float v) {
+    asm volatile("global_store_dword %0, %1, off\n\ts_nop 0" ::"v"(at), "v"(v) : "memory");
+}
+
+// Eight nibbles of two words as f16 values 16 + q in the order k0 k2 k1 k3 k4 k6 k5 k7 (the
+// inputs' operands are built in the same order). `mask` arrives in a scalar register and
+// `sixteen` in a vector one: a shift and one v_and_or_b32 a pair.
+template <bool HIGH>
+__device__ __forceinline__ rf16x8 nibbles(ru32x2 w, uint32_t mask, uint32_t sixteen) {
+    ru32x4 r;
+    if (HIGH) {
+        r.x = ((w.x << 2) & mask) | sixteen;
+        r.y = ((w.x >> 6) & mask) | sixteen;
+        r.z = ((w.y << 2) & mask) | sixteen;
+        r.w = ((w.y >> 6) & mask) | sixteen;
+    } else {
+        r.x = ((w.x << 6) & mask) | sixteen;
+        r.y = ((w.x >> 2) & mask) | sixteen;
+        r.z = ((w.y << 6) & mask) | sixteen;
+        r.w = ((w.y >> 2) & mask) | sixteen;
+    }
+    return __builtin_bit_cast(rf16x8, r);
+}
+
+// NB: 256-weight blocks of a wave's k range (k = 2048 NB).
+template <bool PAIR, int NB>
+__global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResArgs q) {
+    const MvArgs &a = q.a;
+    __shared__ float lds_scale[16];               // [8] scale, [8] its inverse
+    __shared__ float lds_part[2][WAVES][128];     // [tile parity][wave][2 lane + token of the lane's two]
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+    const __amdgpu_buffer_rsrc_t wbuf = make_buffer(a.w, q.w_bytes);
+    uint32_t sixteen = q.sixteen;
+    asm volatile("" : "+v"(sixteen));
+
+    // The workgroup's weight tiles: output tiles b, b + G, ...; with SILU_PAIR the gate tile
+    // and then the up tile of each. Tile p of the run starts at matrix row:
+    const uint32_t per = PAIR ? 2u : 1u;
+    const uint32_t mine = blockIdx.x < q.out_tiles ? (q.out_tiles - 1u - blockIdx.x) / gridDim.x + 1u : 0u;
+    const uint32_t count = per * mine;
+    auto out_tile = [&](uint32_t p) { return blockIdx.x + (p / per) * gridDim.x; };
+    auto row0 = [&](uint32_t p) { return 16u * out_tile(p) + ((PAIR && (p & 1u)) ? a.half : 0u); };
+
+    // A tile's loads: chunk c of a block's 144 (row c / 9, sixteen bytes c % 9) by lane c % 64 of
+    // load c / 64; past 144 a lane asks beyond the buffer and zeros land. The tile's part of
+    // the offset is uniform and travels in a scalar register (the buffer's range check does
+    // not see it: every row of a tile exists here). Past the run's last tile the loads still
+    // run, so that the waits count the same loads every step, but fetch the matrix's first rows.
+    __shared__ __align__(16) uint8_t lds_ring[WAVES * DEPTH * NB * SLOT];
+    uint8_t *ring = lds_ring + wave * (DEPTH * NB * SLOT);
+    uint32_t woff[3];
+#pragma unroll
+    for (uint32_t j = 0; j < 3; j++) {
+        const uint32_t c = 64u * j + lane;
+        woff[j] = c < 144u ? (c / 9u) * a.row_bytes + 16u * (c % 9u) + NB * wave * 144u : 0xfffffff0u - 144u * NB;
+    }
+    auto load_tile = [&](uint32_t p, uint32_t slot) __attribute__((always_inline)) {
+        const uint32_t base = (p < count ? row0(p) : 0u) * a.row_bytes;
+#pragma unroll
+        for (uint32_t i = 0; i < NB; i++)
+#pragma unroll
+            for (uint32_t j = 0; j < 3; j++) load_lds_b128(wbuf, ring + (slot * NB + i) * SLOT + 1024u * j, woff[j] + 144u * i, base);
+    };
+    constexpr int LOADS = 3 * NB;  // a tile's loads of one wave
+    load_tile(0, 0);
+
+    // Each token's scale: the power of two that puts its largest magnitude in [2^14, 2^15).
+    if (wave < a.m) {
+        const float4 *xr = reinterpret_cast<const float4 *>(a.x + (size_t)wave * a.xr);
+        // (all of the lane's loads first: one trip to memory, not one per vector)
+        float4 v[NB * 8];
+#pragma unroll
+        for (int i = 0; i < NB * 8; i++) v[i] = xr[lane + 64u * i];
+        float big = 0.f;
+#pragma unroll
+        for (int i = 0; i < NB * 8; i++) big = fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)), fmaxf(fmaxf(fabsf(v[i].z), fabsf(v[i].w)), big));
+#pragma unroll
+        for (int off = 32; off > 0; off >>= 1) big = fmaxf(big, __shfl_xor(big, off, 64));
+        if (lane == 0) {
+            const int e = (int)((__float_as_uint(big) >> 23) & 0xffu);  // biased exponent; 0 for zero and subnormals
+            int se = 127 + 14 - (e - 127);                               // scale = 2^(14 - (e - 127)), kept normal both ways
+            se = se < 1 ? 1 : se > 253 ? 253 : se;
+            lds_scale[wave] = (e == 0 || e == 255) ? 1.0f : __uint_as_float((uint32_t)se << 23);
+            lds_scale[8 + wave] = (e == 0 || e == 255) ? 1.0f : __uint_as_float((uint32_t)(254 - se) << 23);
+        }
+    } else if (lane == 0) {
+        lds_scale[wave] = lds_scale[8 + wave] = 1.0f;
+    }
+    lds_barrier();
+
+    // This wave's k range of the tokens as matrix-core operands: operand row l16 is token
+    // l16 / 2, the f16 rounding of its scaled inputs (even rows) or what that left, times
+    // 2^11 (odd rows); the lane's eight positions of sub-block s are 8 g .. 8 g + 7, in the
+    // order k0 k2 k1 k3 k4 k6 k5 k7. Rows of tokens the step does not have are zeros.
+    rf16x8 xf[NB * 8];
+    {
+        // (an absent token's rows read the last token's inputs under a scale of zero: no branches,
+        // so all of the lane's loads go out together)
+        const uint32_t t = l16 >> 1, tsrc = t < a.m ? t : a.m - 1u;
+        const float scale = t < a.m ? lds_scale[t] : 0.f;
+        const float *xt = a.x + (size_t)tsrc * a.xr + NB * 256u * wave + 8u * g;
+        float4 raw[NB * 8][2];
+#pragma unroll
+        for (int s = 0; s < NB * 8; s++) {
+            raw[s][0] = *reinterpret_cast<const float4 *>(xt + 32 * s);
+            raw[s][1] = *reinterpret_cast<const float4 *>(xt + 32 * s + 4);
+        }
+#pragma unroll
+        for (int s = 0; s < NB * 8; s++) {
+            const float x[8] = {raw[s][0].x, raw[s][0].y, raw[s][0].z, raw[s][0].w, raw[s][1].x, raw[s][1].y, raw[s][1].z, raw[s][1].w};
+            // Both rows' values for every lane (even lanes keep the first, odd lanes the second);
+            // the scale is a power of two, so x * scale - hi in one fused operation is exact.
+            _Float16 hi[8], lo[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                hi[e] = (_Float16)(x[e] * scale);
+                lo[e] = (_Float16)(fmaf(x[e], scale, -(float)hi[e]) * 2048.0f);
+            }
+            const rf16x8 first = {hi[0], hi[2], hi[1], hi[3], hi[4], hi[6], hi[5], hi[7]};
+            const rf16x8 second = {lo[0], lo[2], lo[1], lo[3], lo[4], lo[6], lo[5], lo[7]};
+            const ru32x4 f4 = __builtin_bit_cast(ru32x4, first), s4 = __builtin_bit_cast(ru32x4, second);
+            const bool odd = l16 & 1u;
+            const ru32x4 pick = {odd ? s4.x : f4.x, odd ? s4.y : f4.y, odd ? s4.z : f4.z, odd ? s4.w : f4.w};
+            xf[s] = __builtin_bit_cast(rf16x8, pick);
+        }
+    }
+    // The rows' sub-block sums, by the matrix cores (the rows times a column of ones): every
+    // lane gets the sums of its own two tokens (operand rows 4 g .. 4 g + 3), whatever its column.
+    float2 xsum[NB * 8];
+    {
+        const ru32x4 ones = {0x3C003C00u, 0x3C003C00u, 0x3C003C00u, 0x3C003C00u};
+#pragma unroll
+        for (int s = 0; s < NB * 8; s++) {
+            const rf32x4 d = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[s], __builtin_bit_cast(rf16x8, ones), rf32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+            xsum[s] = float2{fmaf(d[1], 1.0f / 2048.0f, d[0]), fmaf(d[3], 1.0f / 2048.0f, d[2])};
+        }
+    }
+
+    float held = 0.f;  // the gate tile's result, until the up tile's arrives
+    auto step = [&](uint32_t p, uint32_t slot) __attribute__((always_inline)) {
+        float acc[2] = {0.f, 0.f};  // tokens 2 g and 2 g + 1, matrix row row0 + l16, this wave's k range
+#pragma unroll
+        for (int i = 0; i < NB; i++) {
+            const uint8_t *block = ring + (slot * NB + i) * SLOT + l16 * 144u;
+            const ru32x4 h = *reinterpret_cast<const ru32x4 *>(block);
+            const float d = half_bits_to_float(h.x & 0xffffu), dmin = half_bits_to_float(h.x >> 16);
+            // The eight 6-bit scales and minimums as bytes of four words (src/ref/tensor.zig:94-98).
+            const uint32_t sc_lo_ = h.y & 0x3f3f3f3fu, mn_lo_ = h.z & 0x3f3f3f3fu;
+            const uint32_t sc_hi_ = (h.w & 0x0f0f0f0fu) | ((h.y >> 2) & 0x30303030u);
+            uint32_t mn_hi = ((h.w >> 4) & 0x0f0f0f0fu) | ((h.z >> 2) & 0x30303030u);
+            // (kept apart from the masks above: a clean byte converts to f32 in one instruction,
+            // a 6-bit field of the raw word needs two)
+            uint32_t sc_lo = sc_lo_, mn_lo = mn_lo_, sc_hi = sc_hi_;
+            asm volatile("" : "+v"(sc_lo), "+v"(mn_lo), "+v"(sc_hi), "+v"(mn_hi));
+#pragma unroll
+            for (uint32_t c = 0; c < 4; c++) {
+                const ru32x2 wq = *reinterpret_cast<const ru32x2 *>(block + 16u + 32u * c + 8u * g);
+#pragma unroll
+                for (uint32_t half = 0; half < 2; half++) {
+                    const uint32_t sb = 2u * c + half, shift = 8u * (sb & 3u);
+                    const float dsc = d * (float)(((sb < 4u ? sc_lo : sc_hi) >> shift) & 0xffu);
+                    const float off = fmaf(16.0f, dsc, dmin * (float)(((sb < 4u ? mn_lo : mn_hi) >> shift) & 0xffu));
+                    const rf16x8 wf = half ? nibbles<true>(wq, q.nibble_mask, sixteen) : nibbles<false>(wq, q.nibble_mask, sixteen);
+                    const rf32x4 r = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[8 * i + sb], wf, rf32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
+                    const float2 xs = xsum[8 * i + sb];
+                    acc[0] = fmaf(-off, xs.x, fmaf(dsc, fmaf(r[1], 1.0f / 2048.0f, r[0]), acc[0]));
+                    acc[1] = fmaf(-off, xs.y, fmaf(dsc, fmaf(r[3], 1.0f / 2048.0f, r[2]), acc[1]));
+                }
+            }
+        }
+        float *part = &lds_part[p & 1u][0][0];
+        *reinterpret_cast<float2 *>(part + wave * 128u + 2u * lane) = float2{acc[0], acc[1]};
+        lds_barrier();
+        // Buffer p % 2 is written again in step p + 2, after the barrier of step p + 1, which
+        // a wave passes only when it has read what it needs here.
+        // The 128 outputs of a tile are summed by one pair of waves, a different pair from one
+        // output tile to the next (the extra work does not make the same waves late every time).
+        if ((tid >> 7) == ((p / per) & 3u)) {
+            const uint32_t row = tid & 15u, t = (tid >> 4) & 7u;
+            const float *src = part + 2u * ((t >> 1) * 16u + row) + (t & 1u);
+            float sum = src[0];
+#pragma unroll
+            for (uint32_t wv = 1; wv < WAVES; wv++) sum += src[wv * 128u];
+            sum *= lds_scale[8 + t];
+            if (PAIR && !(p & 1u)) {
+                held = sum;
+            } else {
+                const float v = PAIR ? silu_f(held) * sum : sum;
+                if (t < a.m) {
+                    float *o = a.out + (size_t)t * a.out_stride + a.col0 + 16u * out_tile(p) + row;
+                    store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + v : v);
+                }
+            }
+        }
+    };
+
+    // DEPTH ring slots in rotation: DEPTH - 1 tiles in flight behind the one multiplied. Every
+    // wave of the workgroup runs the same steps (the barrier inside). Before tile p is read,
+    // all but the loads of the DEPTH - 1 tiles after it have landed.
+#pragma unroll
+    for (int s = 1; s < DEPTH - 1; s++) load_tile(s, s);
+    for (uint32_t p = 0; p < count; p += DEPTH) {
+#pragma unroll
+        for (int s = 0; s < DEPTH; s++) {
+            load_tile(p + s + (DEPTH - 1), (s + DEPTH - 1) % DEPTH);
+            wait_loads<(DEPTH - 1) * LOADS>();
+            if (p + s < count) step(p + s, s);
+        }
+    }
+    wait_loads<0>();  // nothing may still land in LDS once the workgroup is gone
+}
+
+}  // namespace
+
+// Whether this kernel can run the (already validated) arguments: whole tiles, k split into
+// one or two blocks a wave, no prologue.
+bool matvec_q4k_mfma_resident_accepts(const MvArgs &a) {
+    const bool pair = a.flags & FLAG_SILU_PAIR;
+    return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u) && !(a.flags & FLAG_NORM) && a.act_div == 0.f && a.rows % 16u == 0 &&
+           (!pair || a.half % 16u == 0);
+}
+
+zhip_result launch_matvec_q4k_mfma_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) {
+    const bool pair = a.flags & FLAG_SILU_PAIR;
+    // 32-bit byte offsets.
+    const uint64_t reach = ((uint64_t)(pair ? a.half : 0u) + a.rows + 16u) * a.row_bytes;
+    if (w_bytes >= 0xfffffff0ull || reach >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "matvec_q4_k: operands of 4 GiB or more");
+    ResArgs q{a, (uint32_t)w_bytes, 0x03C003C0u, 0x4C004C00u, a.rows / 16u};
+    const uint32_t cus = (uint32_t)d.dev->compute_units;
+    const dim3 grid(q.out_tiles < cus ? q.out_tiles : cus);
+    if (a.k == 2048u) {
+        if (pair) hipLaunchKernelGGL((matvec_q4k_mfma_resident_kernel<true, 1>), grid, dim3(THREADS), 0, d.stream, q);
+        else hipLaunchKernelGGL((matvec_q4k_mfma_resident_kernel<false, 1>), grid, dim3(THREADS), 0, d.stream, q);
+    } else {
+        if (pair) hipLaunchKernelGGL((matvec_q4k_mfma_resident_kernel<true, 2>), grid, dim3(THREADS), 0, d.stream, q);
+        else hipLaunchKernelGGL((matvec_q4k_mfma_resident_kernel<false, 2>), grid, dim3(THREADS), 0, d.stream, q);
+    }
+    return check_launch(d, "matvec_q4_k");
+}
+
+}  // namespace zhip
