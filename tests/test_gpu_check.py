@@ -513,6 +513,40 @@ def test_matmul_bf16_streamed_chunk(ctx, rows, n, k, col0, pad, accumulate, pack
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
 
 
+@pytest.mark.parametrize("rows,n,k,col0,pad,accumulate,packed", [
+    (128, 16400, 1024, 0, 0, False, True),
+    (50, 16400, 512, 4, 4, True, False),
+])
+def test_matmul_q8_0_float_streamed_chunk(ctx, rows, n, k, col0, pad, accumulate, packed):
+    """The same shape class with Q8_0 weights (matmul_q8_0_float on the bf16 rung):
+    weights bf16(q * d), against the rung's operand contract; a token's bits the
+    same in the chunk or alone."""
+    c = ctx
+    rung = K.Prefill.bf16_mfma_xbf16 if packed else K.Prefill.bf16_mfma
+    x = c.random(rows * k, 1).reshape(rows, k)
+    xs = synth.bf16_round(x).astype(np.float64)
+    raw, wq = quant_rows(c, TensorType.q8_0, n, k)
+    wa = c.gpu_weights(TensorType.q8_0, raw, k)
+    stride = n + pad
+    init = c.random(rows * stride, 0.5).reshape(rows, stride)
+    c.set.select_prefill(c.rec, rung)
+
+    def run(first, count):
+        xa = c.upload(synth.to_bf16_bits(x[first : first + count]) if packed else x[first : first + count])
+        out = c.upload(init[first : first + count])
+        c.launcher().launch(Kernel.matmul_q8_0_float, P.MatmulQuant(rows=count, n=n, k=k, col0=col0, out_stride=stride, accumulate=int(accumulate), k_slice=k),
+                            [xa, wa, out], (K.div_ceil(n, 64), K.div_ceil(count, 16), 1))
+        return c.read(out).reshape(count, stride)
+
+    got = run(0, rows)
+    want = xs @ synth.bf16_round(wq).astype(np.float64).T + (init[:, col0 : col0 + n] if accumulate else 0)
+    assert rel_err(got[:, col0 : col0 + n], want) <= 1e-5
+    assert np.array_equal(got[:, :col0], init[:, :col0]) and np.array_equal(got[:, col0 + n :], init[:, col0 + n :]), "columns outside the chunk were written"
+    for first, count in ((0, 1), (rows - 1, 1), (rows // 3, min(20, rows - rows // 3))):
+        assert run(first, count).tobytes() == got[first : first + count].tobytes(), "a token's bits depend on its chunk"
+    c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
+
+
 def launch_float_q8(c, x, weights, out, rows, accumulate, slices, chunked):
     """Two weight chunks exercise nonzero col0 and a padded output stride;
     split-k partials are dense per chunk (src/kernels/check.zig:752-770)."""

@@ -362,9 +362,9 @@ __global__ __launch_bounds__(256) void narrow_bf16_kernel(const f32x4 *src, u32x
 zhip_result validate_matmul(const Dispatch &d, const char *name, bool sliced, bool q8_0, uint32_t x_bytes, bool *empty);
 
 // The streaming kernel for few tokens over a short k (matmul_stream.hip).
-bool matmul_bf16_stream_accepts(const Dispatch &d, const float *out, uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride);
-zhip_result launch_matmul_bf16_stream(const Dispatch &d, const char *name, const uint8_t *x, const uint8_t *w, float *out,
-    uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate);
+bool matmul_stream_accepts(const Dispatch &d, bool q8_0, const float *out, uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride);
+zhip_result launch_matmul_stream(const Dispatch &d, const char *name, bool q8_0, const uint8_t *x, const uint8_t *w, float *out,
+    uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, uint32_t row_bytes);
 
 // The 256-token tiling (matmul_mfma_wide.hip).
 zhip_result launch_mfma_wide(const Dispatch &d, const char *name, bool q8_0, const uint8_t *x, const uint8_t *w, float *out,
@@ -421,10 +421,10 @@ static zhip_result launch_mfma(const Dispatch &d, const char *name, bool sliced,
         a.x = d.work->data;
     }
     const uint32_t slices = sliced ? d.grid[2] : 1u;
-    // A chunk of up to 128 tokens against a tall bf16 matrix with a short k is one pass over
-    // the weights: the kernel that streams them into registers.
-    if (std::is_same<W, WBf16>::value && slices == 1u && matmul_bf16_stream_accepts(d, a.out, a.rows, a.n, a.k, a.col0, a.out_stride))
-        return launch_matmul_bf16_stream(d, name, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate);
+    // A chunk of up to 128 tokens against a tall matrix with a short k is one pass over the
+    // weights: the kernel that streams them into registers.
+    if (slices == 1u && a.k_slice >= a.k && matmul_stream_accepts(d, q8_0, a.out, a.rows, a.n, a.k, a.col0, a.out_stride))
+        return launch_matmul_stream(d, name, q8_0, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes);
     // Long steps whose 256 x 128 tiles fill the CUs take that tiling: each
     // weight is converted once per 256 tokens and half the bytes cross from L2.
     if (slices == 1u && a.k_slice >= a.k && (uint64_t)((a.rows + 255u) / 256u) * ((a.n + 127u) / 128u) >= (uint64_t)d.dev->compute_units)

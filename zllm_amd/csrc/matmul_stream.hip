@@ -1,6 +1,8 @@
-// matmul_bf16 on the matrix cores for steps of up to 128 tokens over a short k
-// (up to 1024) and many matrix rows: the vocabulary projection of a prefill
-// chunk (src/kernels/matmul_half.wgsl's contract, the bf16 rung's operands).
+// matmul_bf16 and matmul_q8_0_float on the matrix cores for steps of up to 128
+// tokens over a short k (up to 1024) and many matrix rows: the vocabulary
+// projection of a prefill chunk (the contracts of src/kernels/matmul_half.wgsl
+// and matmul_q8_0_float.wgsl, the bf16 rung's operands: Q8_0 weights become
+// bf16(q * d)).
 // Such a step is bound by the one pass over the weights, like a decode
 // multiply, so the kernel is built like one: the weights stream from memory
 // straight into the registers of the wave that multiplies them, each byte
@@ -25,6 +27,7 @@
 #include <hip/hip_runtime.h>
 
 #include "common.h"
+#include "decode.cuh"
 
 namespace zhip {
 
@@ -43,8 +46,19 @@ struct StreamArgs {
     float *out;
     uint32_t rows, n, k, col0, out_stride, accumulate;
     uint32_t x_bytes, w_bytes;
+    uint32_t row_bytes; // bytes between weight rows
     uint32_t tiles;     // sixteen-row weight tiles
 };
+
+typedef uint32_t su32x2 __attribute__((ext_vector_type(2)));
+typedef __bf16 sbf16x2 __attribute__((ext_vector_type(2)));
+typedef float sf32x2 __attribute__((ext_vector_type(2)));
+
+// Two floats to packed bf16, round to nearest even (src/ref/matmul.zig:250-255).
+__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
+    const sf32x2 v = {lo, hi};
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, sbf16x2));
+}
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const uint8_t *base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, (int)bytes, 0x00020000);
@@ -82,14 +96,19 @@ __device__ __forceinline__ sf32x4 from_lane(sf32x4 v, uint32_t from) {
 
 // MT: token tiles of sixteen (rows <= 16 MT); KC: 32-position chunks of a wave's
 // k range (k = 256 KC).
-template <int MT, int KC>
-__global__ __launch_bounds__(THREADS) void matmul_bf16_stream_kernel(StreamArgs a) {
+template <int MT, int KC, bool Q8>
+__global__ __launch_bounds__(THREADS) void matmul_stream_kernel(StreamArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];  // [2][wave][MT * 64 lanes] partial vectors
     constexpr uint32_t PART = MT * 64u * 16u;                       // bytes a wave writes per tile
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
     const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.x, a.x_bytes), wbuf = make_buffer(a.w, a.w_bytes);
-    // The lane's eight positions of chunk c: k = 32 KC wave + 32 c + 8 g.
-    const uint32_t kbyte = 2u * (32u * KC * wave + 8u * g);
+    // The lane's eight positions of chunk c. BF16 rows: k = 32 KC wave + 32 c + 8 g (a 16-byte
+    // load a chunk). Q8_0 rows: a 16-byte load holds sixteen weights, two chunks' worth, so
+    // chunk c = 2 j + h takes k = 32 KC wave + 64 j + 16 g + 8 h: the lane's load j covers
+    // 16 g .. 16 g + 15 of the 64 and a row's four lanes 64 contiguous bytes either way.
+    static_assert(!Q8 || KC % 2 == 0, "a Q8_0 load feeds two chunks");
+    const uint32_t kw = 32u * KC * wave;
+    auto kpos = [&](int c) { return Q8 ? kw + 64u * (c >> 1) + 16u * g + 8u * (c & 1) : kw + 32u * c + 8u * g; };
 
     // This wave's part of every token (tokens past `rows` lie past the buffer: zeros).
     sbf16x8 xf[MT][KC];
@@ -97,7 +116,7 @@ __global__ __launch_bounds__(THREADS) void matmul_bf16_stream_kernel(StreamArgs 
     for (int i = 0; i < MT; i++)
 #pragma unroll
         for (int c = 0; c < KC; c++)
-            xf[i][c] = __builtin_bit_cast(sbf16x8, __builtin_amdgcn_raw_buffer_load_b128(xbuf, (16u * i + l16) * a.k * 2u + kbyte + 64u * c, 0, 0));
+            xf[i][c] = __builtin_bit_cast(sbf16x8, __builtin_amdgcn_raw_buffer_load_b128(xbuf, ((16u * i + l16) * a.k + kpos(c)) * 2u, 0, 0));
 
     // This workgroup's tiles, in pairs (a pair's outputs fill whole 128-byte lines): pairs
     // b, b + G, b + 2 G ... of the G workgroups, so that at any time the chip reads one
@@ -114,11 +133,35 @@ __global__ __launch_bounds__(THREADS) void matmul_bf16_stream_kernel(StreamArgs 
     // check does not see: n is a multiple of sixteen here, every row of a tile exists).
     // Past the workgroup's last tile the loads still run, so that every wait counts the same
     // loads on every path, but fetch the matrix's first tile again (from cache; unused).
-    const uint32_t wlane = l16 * a.k * 2u + kbyte, tile_bytes = 32u * a.k;
-    auto load_tile = [&](uint32_t p, su32x4 (&b)[KC]) __attribute__((always_inline)) {
+    struct Tile {
+        su32x4 b[Q8 ? KC / 2 : KC];  // the lane's weights as stored
+        su32x2 d;                    // Q8_0: the f16 scales of the wave's KC blocks of the lane's row
+    };
+    const uint32_t wlane = l16 * a.row_bytes + (Q8 ? kw + 16u * g : 2u * (kw + 8u * g));
+    const uint32_t dlane = l16 * a.row_bytes + a.k + 2u * KC * wave, tile_bytes = 16u * a.row_bytes;
+    auto load_tile = [&](uint32_t p, Tile &t) __attribute__((always_inline)) {
         const uint32_t base = (p < count ? tile_of(p) : 0u) * tile_bytes;
 #pragma unroll
-        for (int c = 0; c < KC; c++) b[c] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, wlane + 64u * c, base, 0);
+        for (int c = 0; c < (Q8 ? KC / 2 : KC); c++) t.b[c] = __builtin_amdgcn_raw_buffer_load_b128(wbuf, wlane + 64u * c, base, 0);
+        if (Q8) {
+            if (KC == 4) t.d = __builtin_amdgcn_raw_buffer_load_b64(wbuf, dlane, base, 0);
+            else t.d.x = __builtin_amdgcn_raw_buffer_load_b32(wbuf, dlane, base, 0);
+        }
+    };
+    // Chunk c of a tile as a matrix-core operand: BF16 as stored; Q8_0 as bf16(q * d), one
+    // rounding of the exact f32 product, d the scale of the block the lane's weights lie in.
+    auto operand = [&](const Tile &t, int c) __attribute__((always_inline)) -> sbf16x8 {
+        if (!Q8) return __builtin_bit_cast(sbf16x8, t.b[c]);
+        const uint32_t block = 2u * (c >> 1) + (g >> 1);  // of the wave's KC
+        const uint32_t word = block < 2u ? t.d.x : t.d.y;
+        const float d = half_bits_to_float((block & 1u) ? word >> 16 : word & 0xffffu);
+        const int32_t lo = (int32_t)((c & 1) ? t.b[c >> 1].z : t.b[c >> 1].x), hi = (int32_t)((c & 1) ? t.b[c >> 1].w : t.b[c >> 1].y);
+        const su32x4 v = {
+            pack_bf16((float)(int8_t)(lo) * d, (float)(int8_t)(lo >> 8) * d),
+            pack_bf16((float)(int8_t)(lo >> 16) * d, (float)(lo >> 24) * d),
+            pack_bf16((float)(int8_t)(hi) * d, (float)(int8_t)(hi >> 8) * d),
+            pack_bf16((float)(int8_t)(hi >> 16) * d, (float)(hi >> 24) * d)};
+        return __builtin_bit_cast(sbf16x8, v);
     };
     // Tile q of the run: its matrix-core instructions, with the reads of tile q - 1's eight
     // partial vectors in between (the matrix cores work while LDS answers), then the sum and
@@ -127,7 +170,10 @@ __global__ __launch_bounds__(THREADS) void matmul_bf16_stream_kernel(StreamArgs 
     // that barrier, which every wave passes only when it has read what it needs.
     static_assert(MT <= (int)WAVES, "one partial vector is read per token tile's instructions");
     sf32x4 held = {0.f, 0.f, 0.f, 0.f};
-    auto step = [&](uint32_t q, const su32x4 (&b)[KC]) __attribute__((always_inline)) {
+    auto step = [&](uint32_t q, const Tile &t) __attribute__((always_inline)) {
+        sbf16x8 wf[KC];
+#pragma unroll
+        for (int c = 0; c < KC; c++) wf[c] = operand(t, c);
         // (the four vectors of a token are stored permuted, see below)
         const uint8_t *prev = lds + ((q & 1u) ^ 1u) * (WAVES * PART) + ((tid & (MT * 64u - 1u)) ^ ((tid >> 4) & 3u)) * 16u;
         constexpr int PER = WAVES / MT;  // partial vectors read per token tile's instructions
@@ -141,7 +187,7 @@ __global__ __launch_bounds__(THREADS) void matmul_bf16_stream_kernel(StreamArgs 
         for (int i = 0; i < MT; i++) {
             acc[i & 1] = sf32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-            for (int c = 0; c < KC; c++) acc[i & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(sbf16x8, b[c]), xf[i][c], acc[i & 1], 0, 0, 0);
+            for (int c = 0; c < KC; c++) acc[i & 1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(wf[c], xf[i][c], acc[i & 1], 0, 0, 0);
             __builtin_amdgcn_sched_barrier(0);
             if (i > 0) {
                 *reinterpret_cast<sf32x4 *>(mine + (i - 1) * 1024u) = acc[(i - 1) & 1];
@@ -192,7 +238,7 @@ __global__ __launch_bounds__(THREADS) void matmul_bf16_stream_kernel(StreamArgs 
     // Every wave of the workgroup runs the same steps (the barrier inside); one step past
     // the last tile sums and stores that tile (its own instructions multiply stale registers
     // into partial sums nobody reads).
-    su32x4 b[DEPTH][KC];
+    Tile b[DEPTH];
 #pragma unroll
     for (int s = 0; s < DEPTH - 1; s++) load_tile(s, b[s]);
     const uint32_t rounds = count ? count + 1u : 0u;
@@ -205,9 +251,9 @@ __global__ __launch_bounds__(THREADS) void matmul_bf16_stream_kernel(StreamArgs 
     }
 }
 
-template <int MT, int KC>
+template <int MT, int KC, bool Q8>
 static zhip_result launch(const Dispatch &d, const char *name, const StreamArgs &a, uint32_t groups) {
-    auto kernel = matmul_bf16_stream_kernel<MT, KC>;
+    auto kernel = matmul_stream_kernel<MT, KC, Q8>;
     constexpr int bytes = 2 * WAVES * MT * 64 * 16;
     static bool configured = false;
     if (!configured) {
@@ -222,37 +268,39 @@ static zhip_result launch(const Dispatch &d, const char *name, const StreamArgs 
 }
 
 template <int MT>
-static zhip_result launch_k(const Dispatch &d, const char *name, const StreamArgs &a, uint32_t groups) {
+static zhip_result launch_k(const Dispatch &d, const char *name, const StreamArgs &a, uint32_t groups, bool q8_0) {
+    if (q8_0) return a.k == 512u ? launch<MT, 2, true>(d, name, a, groups) : launch<MT, 4, true>(d, name, a, groups);
     switch (a.k / 256u) {
-    case 1: return launch<MT, 1>(d, name, a, groups);
-    case 2: return launch<MT, 2>(d, name, a, groups);
-    case 3: return launch<MT, 3>(d, name, a, groups);
-    default: return launch<MT, 4>(d, name, a, groups);
+    case 1: return launch<MT, 1, false>(d, name, a, groups);
+    case 2: return launch<MT, 2, false>(d, name, a, groups);
+    case 3: return launch<MT, 3, false>(d, name, a, groups);
+    default: return launch<MT, 4, false>(d, name, a, groups);
     }
 }
 
 }  // namespace
 
-// Whether the streaming kernel suits a (validated) bf16 step: few tokens, a short
-// k in whole chunks, enough whole weight tiles to occupy every CU several times,
-// and outputs that can be stored 16 bytes at a time.
-bool matmul_bf16_stream_accepts(const Dispatch &d, const float *out, uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride) {
-    return rows >= 1 && rows <= 128 && k >= 256 && k <= 1024 && k % 256u == 0 && (n + 15u) / 16u >= 4u * (uint32_t)d.dev->compute_units &&
+// Whether the streaming kernel suits a (validated) step on the bf16 rung: few tokens, a
+// short k in whole chunks (Q8_0: two or four blocks a wave), enough whole weight tiles to
+// occupy every CU several times, and outputs that can be stored 16 bytes at a time.
+bool matmul_stream_accepts(const Dispatch &d, bool q8_0, const float *out, uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride) {
+    const bool k_fits = q8_0 ? (k == 512u || k == 1024u) : (k >= 256u && k <= 1024u && k % 256u == 0);
+    return rows >= 1 && rows <= 128 && k_fits && (n + 15u) / 16u >= 4u * (uint32_t)d.dev->compute_units &&
            (uintptr_t)out % 16u == 0 && out_stride % 4u == 0 && col0 % 4u == 0 && n % 16u == 0;
 }
 
-zhip_result launch_matmul_bf16_stream(const Dispatch &d, const char *name, const uint8_t *x, const uint8_t *w, float *out,
-    uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate) {
-    const uint64_t x_bytes = (uint64_t)rows * k * 2u, w_bytes = (uint64_t)n * k * 2u;
+zhip_result launch_matmul_stream(const Dispatch &d, const char *name, bool q8_0, const uint8_t *x, const uint8_t *w, float *out,
+    uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, uint32_t row_bytes) {
+    const uint64_t x_bytes = (uint64_t)rows * k * 2u, w_bytes = (uint64_t)n * row_bytes;
     // 32-bit byte offsets, up to a tile of sixteen past the last token and row.
-    if (w_bytes + 32ull * k >= 0xfffffff0ull - 256u) return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
+    if (w_bytes + 16ull * row_bytes >= 0xfffffff0ull - 256u) return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
     StreamArgs a{};
     a.x = x; a.w = w; a.out = out;
     a.rows = rows; a.n = n; a.k = k; a.col0 = col0; a.out_stride = out_stride; a.accumulate = accumulate;
-    a.x_bytes = (uint32_t)x_bytes; a.w_bytes = (uint32_t)w_bytes;
+    a.x_bytes = (uint32_t)x_bytes; a.w_bytes = (uint32_t)w_bytes; a.row_bytes = row_bytes;
     a.tiles = (n + 15u) / 16u;
     const uint32_t groups = a.tiles < (uint32_t)d.dev->compute_units ? a.tiles : (uint32_t)d.dev->compute_units;
-    return rows <= 64u ? launch_k<4>(d, name, a, groups) : launch_k<8>(d, name, a, groups);
+    return rows <= 64u ? launch_k<4>(d, name, a, groups, q8_0) : launch_k<8>(d, name, a, groups, q8_0);
 }
 
 }  // namespace zhip
