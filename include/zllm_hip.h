@@ -45,9 +45,16 @@ enum {
     ZHIP_E_INVALID_ARGUMENT = -11   /* a null or undersized argument to this API */
 };
 
+/* zhip_options.flags. A submit that is only dispatches (then reads) and repeats an
+ * earlier one exactly is replayed from a HIP graph captured the second time it is
+ * seen; this flag (or the environment variable ZHIP_NO_REPLAY) keeps every
+ * submit a sequence of plain launches. No counterpart in the reference: its
+ * hosts record command lists per submit (src/agility/host.zig:520-548). */
+#define ZHIP_OPTION_NO_REPLAY 1u
+
 typedef struct zhip_options {
     uint32_t device_index; /* HIP device ordinal */
-    uint32_t flags;        /* reserved, 0 */
+    uint32_t flags;        /* ZHIP_OPTION_* */
 } zhip_options;
 
 /* What gpu.Device.adapter/limits/memoryBudget report (src/gpu/host.zig:30-46,
@@ -125,6 +132,9 @@ zhip_result zhip_profile_read(zhip_context *context, zhip_timing *out, size_t ca
  * pair on the host's stream), in nanoseconds, and how many dispatches it ran:
  * the measurement a tuner's batched timing takes (src/tune/tune.zig:8-11). */
 zhip_result zhip_last_submit(zhip_context *context, uint64_t *out_ns, uint64_t *out_dispatches);
+/* How many submits so far ran their dispatches from a replayed graph (see
+ * ZHIP_OPTION_NO_REPLAY). No counterpart in the reference; for tests and reports. */
+zhip_result zhip_replayed_submits(zhip_context *context, uint64_t *out_count);
 
 /* Replaces Device.errorMessage (src/gpu/host.zig:128-133; agility.h:108-109):
  * copies the last error message, NUL-terminated; returns its length. */

@@ -1,0 +1,159 @@
+"""Repeated submits replayed from a HIP graph give the results of the same
+submits run launch by launch.
+
+A decode step in the reference is a fixed list of prebuilt launches recorded
+again for every token (src/kernels/kernels.zig:1031-1044): the host replays
+such a list from a graph captured the second time it sees it. Every replay
+here is checked bit for bit against a device that never replays, with other
+submits, writes and reads between the replays."""
+import numpy as np
+import pytest
+
+import oracle
+from gpucheck import Ctx, rel_err
+from zllm_amd import Device, synth
+from zllm_amd import kernels as K
+from zllm_amd.kernels import Kernel, TensorType, params as P
+
+pytestmark = pytest.mark.gpu
+
+N, KDIM, LAYERS, EPS = 512, 1024, 4, 1e-6  # feed-forward width N, hidden width k, chained layers
+
+
+class Stack:
+    """LAYERS x (RMS norm + fused gate/up + SiLU multiply, then down): 2 * LAYERS
+    prebuilt launches, each layer reading the one before, on one context."""
+
+    def __init__(self, c: Ctx, m: int, weights):
+        self.c, self.m = c, m
+        self.x = c.output(m * KDIM)
+        b = K.Builder(c.rec, c.set)
+        self.launches = []
+        cur = self.x
+        for gate_up, down, norm in weights:
+            wg = c.gpu_weights(TensorType.q4_k, gate_up, KDIM)
+            wd = c.gpu_weights(TensorType.q8_0, down, N)
+            act, nxt = c.output(m * N), c.output(m * KDIM)
+            v = K.MatvecVariant()
+            self.launches.append(b.add(
+                K.weight_kernel("matvec", TensorType.q4_k), P.MatvecBf16(n=N, k=KDIM, col0=0, out_stride=N, eps=EPS, norm=True, silu_pair=True, half=N),
+                [cur, wg, act, c.upload(norm)], K.Grid.rows_y(K.div_ceil(N, v.group_rows()))))
+            self.launches.append(b.add(
+                K.weight_kernel("matvec", TensorType.q8_0), P.MatvecBf16(n=KDIM, k=N, col0=0, out_stride=KDIM, silu_pair=False, half=0),
+                [act, wd, nxt, wd], K.Grid.rows_y(K.div_ceil(KDIM, v.group_rows()))))
+            cur = nxt
+        self.out = cur
+        self.builder = b
+        b.finish()
+        c.flush()
+
+    def uniform_of_last(self) -> tuple[int, int]:
+        """Buffer and byte offset of the last launch's parameter block."""
+        assert len(self.builder.pages) == 1
+        return self.builder.pages[0][0], (len(self.launches) - 1) * K.Builder.slot
+
+    def step(self, x: np.ndarray, rows: int | None = None) -> np.ndarray:
+        """Writes the step's input, records the launches and one read, submits."""
+        c = self.c
+        rows = self.m if rows is None else rows
+        c.rec.write_buffer(self.x.buffer, 0, np.ascontiguousarray(x, dtype=np.float32).reshape(-1).view(np.uint8))
+        for l in self.launches:
+            l.record(c.rec, K.Extent(rows=rows))
+        return c.read(self.out)[: rows * KDIM].reshape(rows, KDIM).copy()
+
+
+def make_weights():
+    g = synth.rng(0x6A9)
+    return [(synth.q4_k_rows(g, 2 * N, KDIM), synth.q8_0_rows(g, KDIM, N), synth.activations(g, 1, KDIM).reshape(-1)) for _ in range(LAYERS)]
+
+
+def unrelated_work(c: Ctx, seed: int) -> None:
+    """A short submit of another shape, a write and a read: eager work between replays."""
+    rows, width = 2, 96
+    gu = synth.activations(synth.rng(seed), rows, 2 * width)
+    act = c.output(rows * width)
+    c.launcher().launch(Kernel.silu_mul, P.SiluMul(rows * width, width), [c.upload(gu), act], K.elementwise(rows * width))
+    got = c.read(act).reshape(rows, width)
+    g64 = gu[:, :width].astype(np.float64)
+    assert np.max(np.abs(got - g64 / (1 + np.exp(-g64)) * gu[:, width:])) < 1e-5
+
+
+@pytest.fixture()
+def pair():
+    """The same stack on a replaying device and on one that never replays."""
+    weights = make_weights()
+    devs = [Device.open(0), Device.open(0, Device.NO_REPLAY)]
+    yield [Stack(Ctx(d), 2, weights) for d in devs]
+    for d in devs:
+        d.deinit()
+
+
+def test_every_replay_matches_the_eager_run(pair):
+    replaying, eager = pair
+    seen = []
+    for i in range(7):
+        x = synth.activations(synth.rng(0x700 + i), 2, KDIM)
+        got, want = replaying.step(x), eager.step(x)
+        assert np.array_equal(got, want), f"step {i}"
+        seen.append(got)
+        unrelated_work(replaying.c, 0x800 + i)
+    # First sight runs as recorded, the second captures and replays, as does every later one.
+    assert replaying.c.host.replayed_submits() == 6
+    assert eager.c.host.replayed_submits() == 0
+    assert not np.array_equal(seen[0], seen[1])  # the inputs did differ
+    # And the chain is the right arithmetic, not only the same on both devices.
+    x = synth.activations(synth.rng(0x700), 2, KDIM)
+    cur = x.astype(np.float64)
+    for gate_up, down, norm in make_weights():
+        xn = cur / np.sqrt(np.mean(cur * cur, axis=1, keepdims=True) + EPS) * norm
+        both = xn @ oracle.Matrix(oracle.Q4_K, gate_up, 2 * N, KDIM).rows().astype(np.float64).T
+        act = both[:, :N] / (1 + np.exp(-both[:, :N])) * both[:, N:]
+        cur = act @ oracle.Matrix(oracle.Q8_0, down, KDIM, N).rows().astype(np.float64).T
+    assert rel_err(seen[0], cur) <= 1e-4
+
+
+def test_steps_of_different_extents_keep_their_own_graphs(pair):
+    """Alternating one-token and two-token steps: two recorded sequences, each
+    replayed from its own graph once it has been seen."""
+    replaying, eager = pair
+    for i in range(8):
+        rows = 1 + (i & 1)
+        x = synth.activations(synth.rng(0x900 + i), 2, KDIM)
+        assert np.array_equal(replaying.step(x, rows), eager.step(x, rows)), f"step {i}"
+    assert replaying.c.host.replayed_submits() == 6
+
+
+def test_changed_parameters_are_not_replayed_from_the_old_graph(pair):
+    """A parameter block rewritten between steps changes the launches: the old
+    graph must not run for them."""
+    replaying, eager = pair
+    x = synth.activations(synth.rng(0xA00), 2, KDIM)
+    for _ in range(3):
+        assert np.array_equal(replaying.step(x), eager.step(x))
+    assert replaying.c.host.replayed_submits() == 2
+    # Turn the last launch into an accumulating one (out += W act) in its parameter block.
+    prev = replaying.step(x)
+    assert np.array_equal(prev, eager.step(x))
+    before = replaying.c.host.replayed_submits()
+    changed = np.frombuffer(P.MatvecBf16(n=KDIM, k=N, col0=0, out_stride=KDIM, accumulate=True).pack(), dtype=np.uint8)
+    for s in pair:
+        buf, offset = s.uniform_of_last()
+        s.c.rec.write_buffer(buf, offset, changed)
+    got, want = replaying.step(x), eager.step(x)
+    assert np.array_equal(got, want)
+    assert np.array_equal(got, prev + prev)  # the old graph would have given prev again
+    assert replaying.c.host.replayed_submits() == before  # first sight of the changed sequence
+
+
+def test_profiling_runs_launch_by_launch(pair):
+    replaying, eager = pair
+    x = synth.activations(synth.rng(0xB00), 2, KDIM)
+    for _ in range(3):
+        assert np.array_equal(replaying.step(x), eager.step(x))
+    replaying.c.host.start_profile()
+    assert np.array_equal(replaying.step(x), eager.step(x))
+    t = replaying.c.host.timings()
+    replaying.c.host.stop_profile()
+    assert sum(v.count for v in t.totals.values()) == 2 * LAYERS  # every launch timed on its own
+    assert np.array_equal(replaying.step(x), eager.step(x))      # and replayed again afterwards
+    assert replaying.c.host.replayed_submits() == 3

@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(HERE, "libzllm_hip.so")
 # Every entry point include/zllm_hip.h declares.
 EXPORTS = (
     "zhip_create", "zhip_destroy", "zhip_get_caps", "zhip_supports_prefill", "zhip_set_file", "zhip_execute",
-    "zhip_profile_start", "zhip_profile_stop", "zhip_profile_read", "zhip_last_submit", "zhip_last_error",
+    "zhip_profile_start", "zhip_profile_stop", "zhip_profile_read", "zhip_last_submit", "zhip_replayed_submits", "zhip_last_error",
     "zhip_force_loss", "zhip_kernel_artifact", "zhip_backend_source", "zhip_kernel_ordinal",
 )
 
@@ -63,6 +63,8 @@ def _load() -> C.CDLL:
     lib.zhip_profile_read.argtypes = [ctx, C.POINTER(CTiming), C.c_size_t, C.POINTER(C.c_size_t), C.POINTER(C.c_uint64)]
     lib.zhip_last_submit.restype = C.c_int32
     lib.zhip_last_submit.argtypes = [ctx, C.POINTER(C.c_uint64), C.POINTER(C.c_uint64)]
+    lib.zhip_replayed_submits.restype = C.c_int32
+    lib.zhip_replayed_submits.argtypes = [ctx, C.POINTER(C.c_uint64)]
     lib.zhip_last_error.restype = C.c_size_t
     lib.zhip_last_error.argtypes = [ctx, C.c_char_p, C.c_size_t]
     lib.zhip_force_loss.restype = C.c_int32

@@ -25,6 +25,7 @@
 #include <algorithm>
 #include <cstdarg>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <map>
 #include <new>
@@ -264,6 +265,19 @@ struct zhip_context {
     uint64_t untimed = 0;
     std::vector<hipEvent_t> events;
     uint64_t last_ns = 0, last_dispatches = 0;
+
+    // Replayed submits: a submit that is nothing but dispatches (then reads) and has been
+    // seen before with exactly the same launches runs as a HIP graph (see submit()).
+    struct Replay {
+        std::vector<uint8_t> key;   // every launch's function, grid, bound ranges and parameter bytes
+        hipGraphExec_t exec = nullptr;
+        bool unusable = false;      // capturing it failed once: stay eager
+        uint64_t used = 0;
+    };
+    std::vector<Replay> replays;
+    uint64_t replay_clock = 0;
+    bool use_graphs = true;
+    uint64_t replayed_submits = 0;
 };
 
 namespace {
@@ -333,20 +347,21 @@ void mark_written(Buffer &b) {
     if (b.shadowed) b.shadow_stale = true;
 }
 
-zhip_result run_dispatch(zhip_context *c, const Op &op, size_t &timed) {
-    Pipeline *pl = get(c->pipelines, op.pipeline);
+// Resolves a queued dispatch: its pipeline, the device ranges of its bindings and
+// its parameter block on the host. `err` receives the launcher's message.
+zhip_result prepare_dispatch(zhip_context *c, const Op &op, Dispatch &d, Pipeline *&pl, char *err, size_t err_cap) {
+    pl = get(c->pipelines, op.pipeline);
     // The pipeline was checked when the dispatch was recorded and destroys of
     // pipelines are not deferred, so look it up again.
     if (!pl || !pl->launch) return set_error(c, ZHIP_E_BAD_ID, "dispatch: pipeline %u was destroyed before the submit", op.pipeline);
-    Dispatch d;
     d.stream = c->stream;
     d.dev = &c->info;
     d.work = &c->work;
     d.variant = pl->variant;
     memcpy(d.grid, op.grid, sizeof d.grid);
-    char err[384] = "";
+    err[0] = 0;
     d.err = err;
-    d.err_cap = sizeof err;
+    d.err_cap = err_cap;
     for (uint32_t b = 0; b < 8; b++) {
         const Entry &e = op.group.e[b];
         if (!e.bound) continue;
@@ -362,6 +377,20 @@ zhip_result run_dispatch(zhip_context *c, const Op &op, size_t &timed) {
     if (zhip_result r = refresh_shadow(c, *ub)) return r;
     d.params = ub->shadow.data() + op.group.e[0].offset;
     d.params_size = op.group.e[0].size;
+    return ZHIP_OK;
+}
+
+void mark_outputs(zhip_context *c, const Op &op, const Pipeline &pl) {
+    for (uint32_t b = 1; b < 8; b++)
+        if (op.group.e[b].bound && (pl.info->writes >> b & 1u))
+            if (Buffer *buf = get(c->buffers, op.group.e[b].buffer)) mark_written(*buf);
+}
+
+zhip_result run_dispatch(zhip_context *c, const Op &op, size_t &timed) {
+    Dispatch d;
+    Pipeline *pl = nullptr;
+    char err[384] = "";
+    if (zhip_result r = prepare_dispatch(c, op, d, pl, err, sizeof err)) return r;
 
     const bool timed_now = c->profiling && timed < kTimingCapacity;
     if (c->profiling && !timed_now) c->untimed++;
@@ -382,9 +411,120 @@ zhip_result run_dispatch(zhip_context *c, const Op &op, size_t &timed) {
         if (zhip_result e = hip_check(c, hipEventRecord(c->events[2 * timed + 1], c->stream), "hipEventRecord")) return e;
         timed++;
     }
-    for (uint32_t b = 1; b < 8; b++)
-        if (op.group.e[b].bound && (pl->info->writes >> b & 1u))
-            if (Buffer *buf = get(c->buffers, op.group.e[b].buffer)) mark_written(*buf);
+    mark_outputs(c, op, *pl);
+    return ZHIP_OK;
+}
+
+// ---- replayed submits ------------------------------------------------------------------
+// Launching a kernel costs the CPU about 2.9 us here; a HIP graph replays its kernels
+// 1.6 us apart. A decode step is hundreds of launches of a few microseconds each, the same
+// ones token after token, so a submit whose leading dispatches (everything before its
+// reads) equal an earlier submit's exactly, function by function and byte by byte of their
+// arguments, is replayed from a graph captured the second time it is seen (the first time
+// it runs as it is, which also lets launchers do their one-time set-up outside a capture).
+// Only kernels are captured: no copies, clears or memsets.
+constexpr size_t kMinReplayDispatches = 8, kMaxReplays = 16;
+
+// The leading dispatches of the queue if what follows them is only reads, else 0.
+size_t replayable_prefix(const zhip_context *c) {
+    size_t n = 0;
+    while (n < c->ops.size() && c->ops[n].kind == Op::dispatch) n++;
+    for (size_t i = n; i < c->ops.size(); i++)
+        if (c->ops[i].kind != Op::read) return 0;
+    return n >= kMinReplayDispatches ? n : 0;
+}
+
+zhip_result replay_key(zhip_context *c, size_t count, std::vector<uint8_t> &key) {
+    key.clear();
+    auto put_bytes = [&](const void *p, size_t n) { key.insert(key.end(), (const uint8_t *)p, (const uint8_t *)p + n); };
+    char err[384];
+    // Launchers may point kernels at the workspace: a graph captured with an allocation
+    // that has since been replaced must never match again.
+    const uint64_t work[2] = {(uint64_t)(uintptr_t)c->work.data, c->work.bytes};
+    put_bytes(work, sizeof work);
+    for (size_t i = 0; i < count; i++) {
+        Dispatch d;
+        Pipeline *pl = nullptr;
+        if (zhip_result r = prepare_dispatch(c, c->ops[i], d, pl, err, sizeof err)) return r;
+        const LaunchFn fn = pl->launch;
+        put_bytes(&fn, sizeof fn);
+        put_bytes(&d.variant, sizeof d.variant);
+        put_bytes(d.grid, sizeof d.grid);
+        for (uint32_t b = 0; b < 8; b++) {
+            const uint64_t range[3] = {d.bind[b].bound ? 1ull : 0ull, (uint64_t)(uintptr_t)d.bind[b].ptr, d.bind[b].size};
+            put_bytes(range, sizeof range);
+        }
+        put_bytes(d.params, d.params_size);
+    }
+    return ZHIP_OK;
+}
+
+// Captures the queue's first `count` dispatches into an executable graph. Nothing runs.
+zhip_result capture_replay(zhip_context *c, size_t count, hipGraphExec_t *out) {
+    *out = nullptr;
+    if (hipStreamBeginCapture(c->stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+        (void)hipGetLastError();
+        return ZHIP_E_GPU;
+    }
+    zhip_result failed = ZHIP_OK;
+    char err[384];
+    for (size_t i = 0; i < count && failed == ZHIP_OK; i++) {
+        Dispatch d;
+        Pipeline *pl = nullptr;
+        failed = prepare_dispatch(c, c->ops[i], d, pl, err, sizeof err);
+        if (failed == ZHIP_OK) failed = pl->launch(d);
+    }
+    hipGraph_t graph = nullptr;
+    const hipError_t ended = hipStreamEndCapture(c->stream, &graph);
+    if (ended != hipSuccess || failed != ZHIP_OK || !graph) {
+        (void)hipGetLastError();
+        if (graph) (void)hipGraphDestroy(graph);
+        return failed != ZHIP_OK ? failed : ZHIP_E_GPU;
+    }
+    const hipError_t made = hipGraphInstantiate(out, graph, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(graph);
+    if (made != hipSuccess) {
+        (void)hipGetLastError();
+        *out = nullptr;
+        return ZHIP_E_GPU;
+    }
+    return ZHIP_OK;
+}
+
+// The graph of the queue's first `count` dispatches if this exact sequence has been seen
+// before (captured now if this is the second time), else null: the caller then runs them
+// one by one.
+zhip_result find_replay(zhip_context *c, size_t count, zhip_context::Replay **out) {
+    *out = nullptr;
+    std::vector<uint8_t> key;
+    if (zhip_result r = replay_key(c, count, key)) return r;
+    zhip_context::Replay *entry = nullptr;
+    for (auto &e : c->replays)
+        if (e.key.size() == key.size() && memcmp(e.key.data(), key.data(), key.size()) == 0) entry = &e;
+    if (!entry) {
+        // First sight: remember it (replacing the least recently used) and run as recorded.
+        if (c->replays.size() < kMaxReplays) {
+            c->replays.emplace_back();
+            entry = &c->replays.back();
+        } else {
+            entry = &c->replays[0];
+            for (auto &e : c->replays)
+                if (e.used < entry->used) entry = &e;
+            if (entry->exec) (void)hipGraphExecDestroy(entry->exec);
+            *entry = zhip_context::Replay();
+        }
+        entry->key = std::move(key);
+        entry->used = ++c->replay_clock;
+        return ZHIP_OK;
+    }
+    entry->used = ++c->replay_clock;
+    if (entry->unusable) return ZHIP_OK;
+    if (!entry->exec && capture_replay(c, count, &entry->exec) != ZHIP_OK) {
+        entry->unusable = true;
+        entry->exec = nullptr;
+        return ZHIP_OK;
+    }
+    *out = entry;
     return ZHIP_OK;
 }
 
@@ -402,8 +542,30 @@ zhip_result submit(zhip_context *c) {
     std::vector<TimingKey> keys;
     uint64_t dispatches = 0;
     size_t next_read = 0;
+    // Parameter blocks the GPU wrote are read back while resolving the launches: before the
+    // timed region and before any capture.
+    const size_t prefix = (c->use_graphs && !c->profiling) ? replayable_prefix(c) : 0;
+    zhip_context::Replay *replay = nullptr;
+    if (prefix > 0)
+        if (zhip_result r = find_replay(c, prefix, &replay)) return r;
     if (zhip_result r = hip_check(c, hipEventRecord(c->ev_begin, c->stream), "hipEventRecord")) return r;
-    for (const Op &op : c->ops) {
+    bool replayed = false;
+    if (replay) {
+        if (hipGraphLaunch(replay->exec, c->stream) == hipSuccess) {
+            for (size_t i = 0; i < prefix; i++)
+                if (Pipeline *pl = get(c->pipelines, c->ops[i].pipeline)) mark_outputs(c, c->ops[i], *pl);
+            c->replayed_submits++;
+            dispatches = prefix;
+            replayed = true;
+        } else {
+            (void)hipGetLastError();
+            (void)hipGraphExecDestroy(replay->exec);
+            replay->exec = nullptr;
+            replay->unusable = true;
+        }
+    }
+    for (size_t at = replayed ? prefix : 0; at < c->ops.size(); at++) {
+        const Op &op = c->ops[at];
         switch (op.kind) {
         case Op::dispatch: {
             const size_t before = timed;
@@ -715,6 +877,7 @@ zhip_result zhip_create(const zhip_options *options, zhip_context **out_context)
     zhip_context *c = new (std::nothrow) zhip_context();
     if (!c) return ZHIP_E_OUT_OF_MEMORY;
     c->device = index;
+    c->use_graphs = !(options && (options->flags & ZHIP_OPTION_NO_REPLAY)) && !getenv("ZHIP_NO_REPLAY");
     c->info.compute_units = prop.multiProcessorCount;
     c->info.max_lds = (int)prop.sharedMemPerBlock;
     c->caps.abi_version = ZHIP_ABI_VERSION;
@@ -744,6 +907,8 @@ zhip_result zhip_destroy(zhip_context *c) {
     if (c->stream) (void)hipStreamSynchronize(c->stream);
     for (Buffer &b : c->buffers)
         if (b.alive && b.dev) (void)hipFree(b.dev);
+    for (auto &e : c->replays)
+        if (e.exec) (void)hipGraphExecDestroy(e.exec);
     c->work.release();
     for (hipEvent_t ev : c->events) (void)hipEventDestroy(ev);
     if (c->download) (void)hipHostFree(c->download);
@@ -837,6 +1002,12 @@ zhip_result zhip_profile_read(zhip_context *c, zhip_timing *out, size_t capacity
         out[i].count = kv.second.count;
         i++;
     }
+    return ZHIP_OK;
+}
+
+zhip_result zhip_replayed_submits(zhip_context *c, uint64_t *out) {
+    if (!c || !out) return ZHIP_E_INVALID_ARGUMENT;
+    *out = c->replayed_submits;
     return ZHIP_OK;
 }
 

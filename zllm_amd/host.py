@@ -101,9 +101,11 @@ class Timings:
 class Device:
     """One MI355X (src/gpu/host.zig:48-135)."""
 
-    def __init__(self, index: int = 0) -> None:
+    NO_REPLAY = 1  # ZHIP_OPTION_NO_REPLAY: never replay a repeated submit from a HIP graph
+
+    def __init__(self, index: int = 0, flags: int = 0) -> None:
         self.ctx = C.c_void_p()
-        opts = _lib.Options(index, 0)
+        opts = _lib.Options(index, flags)
         r = _lib.lib.zhip_create(C.byref(opts), C.byref(self.ctx))
         if r < 0:
             self.ctx = C.c_void_p()
@@ -112,8 +114,8 @@ class Device:
         self.check(_lib.lib.zhip_get_caps(self.ctx, C.byref(self.caps)))
 
     @classmethod
-    def open(cls, index: int = 0) -> "Device":
-        return cls(index)
+    def open(cls, index: int = 0, flags: int = 0) -> "Device":
+        return cls(index, flags)
 
     def deinit(self) -> None:
         if self.ctx:
@@ -207,6 +209,12 @@ class Host:
         self.d.check(_lib.lib.zhip_profile_read(self.d.ctx, rows, n.value, C.byref(n), C.byref(untimed)))
         totals = {TimingKey(rows[i].pipeline, tuple(rows[i].grid)): TimingTotal(rows[i].ns, rows[i].count) for i in range(n.value)}
         return Timings(totals, untimed.value)
+
+    def replayed_submits(self) -> int:
+        """Submits so far whose dispatches ran from a replayed HIP graph."""
+        n = C.c_uint64(0)
+        self.d.check(_lib.lib.zhip_replayed_submits(self.d.ctx, C.byref(n)))
+        return n.value
 
     def last_submit(self) -> tuple[int, int]:
         """GPU nanoseconds and dispatch count of the last submit's work."""
