@@ -36,9 +36,10 @@
 // The four k quarters are added through LDS at the end, always as
 // (q0 + q2) + (q1 + q3).
 //
-// v_mfma_f32_16x16x32_bf16 takes from lane l eight k values of token l % 16 and
-// eight of matrix row l % 16: lane group g = l / 16 owns positions 8 g .. 8 g + 7
-// of the wave's 32.
+// v_mfma_f32_16x16x32_bf16 takes from lane l eight k values of matrix row l % 16
+// (its first operand) and eight of token l % 16: lane group g = l / 16 owns
+// positions 8 g .. 8 g + 7 of the wave's 32, and ends up with outputs 4 g .. 4 g + 3
+// of token l % 16, which it stores as one 16-byte piece.
 //
 // Pipeline: buffer loads straight into LDS (no registers, no LDS store
 // instructions; anything past the end of a binding reads as zero), three LDS
@@ -277,7 +278,7 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
 #pragma unroll
         for (int i = 0; i < MT; i++) {
 #pragma unroll
-            for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bf[j], acc[i][j], 0, 0, 0);
+            for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);
             af[i] = *reinterpret_cast<const bf16x8 *>(xn + 2048 * i);
         }
         convert(wf, kc + BK);
@@ -326,22 +327,31 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     __syncthreads();
     if (kq >= 2u) return;
     const float *src = xchg + (size_t)(((kq ^ 1u) * 2u + wn) * (REGS / 2)) * 64u + lane;
-    // D[token][output]: the lane holds output column lane % 16 and token rows
-    // 4 * (lane / 16) .. + 3 of each 16 x 16 tile.
+    // D[output][token] (the weights are the MFMA's first operand): the lane holds
+    // outputs 4 (lane / 16) .. + 3 of token lane % 16 in each 16 x 16 tile, sixteen
+    // contiguous bytes of the token's row.
+    const bool aligned = ((a.out_stride | a.col0 | a.slice_stride) & 3u) == 0u && (reinterpret_cast<uintptr_t>(a.out) & 15u) == 0u;
 #pragma unroll
     for (int i = 0; i < KEEP; i++) {
+        const uint32_t t = t0 + 16u * (kq ? i + KEEP : i) + lrow;
 #pragma unroll
         for (int j = 0; j < 2; j++) {
-            const uint32_t col = j0 + 32u * wn + 16u * j + lrow;
+            const uint32_t col = j0 + 32u * wn + 16u * j + 4u * g;
+            f32x4 other;
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const float other = src[((i * 2 + j) * 4 + r) * 64];
-                const float mine = kq ? acc[i + KEEP][j][r] : acc[i][j][r];
-                const float v = kq ? other + mine : mine + other;  // (q0 + q2) + (q1 + q3)
-                const uint32_t t = t0 + 16u * (kq ? i + KEEP : i) + 4u * g + r;
-                if (col >= a.n || t >= a.rows) continue;
-                const size_t o = (size_t)z * a.slice_stride + (size_t)t * a.out_stride + a.col0 + col;
-                a.out[o] = a.accumulate ? a.out[o] + v : v;
+            for (int r = 0; r < 4; r++) other[r] = src[((i * 2 + j) * 4 + r) * 64];
+            const f32x4 mine = kq ? acc[i + KEEP][j] : acc[i][j];
+            f32x4 v = kq ? other + mine : mine + other;  // (q0 + q2) + (q1 + q3)
+            if (t >= a.rows || col >= a.n) continue;
+            float *o = a.out + (size_t)z * a.slice_stride + (size_t)t * a.out_stride + a.col0 + col;
+            if (aligned && col + 3u < a.n) {
+                f32x4 *o4 = reinterpret_cast<f32x4 *>(o);
+                if (a.accumulate) v += *o4;
+                *o4 = v;
+            } else {
+#pragma unroll
+                for (int r = 0; r < 4; r++)
+                    if (col + r < a.n) o[r] = a.accumulate ? o[r] + v[r] : v[r];
             }
         }
     }

@@ -168,7 +168,7 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_wide_kernel(Args a) {
 #pragma unroll
             for (int i = 0; i < 4; i++)
 #pragma unroll
-                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
         }
         if (kc + GK < ke) commit(cur ^ 1u, kc + GK, wnext, xnext);
         __syncthreads();
@@ -196,21 +196,27 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_wide_kernel(Args a) {
         if (k0 + GK < ke) tile(k0 + GK, w1, x1, w2, x2);
     }
 
-    // D[token][output]: the lane holds output column lane % 16 and token rows
-    // 4 * (lane / 16) .. + 3 of each 16 x 16 tile.
+    // D[output][token] (the weights are the MFMA's first operand): the lane holds
+    // outputs 4 (lane / 16) .. + 3 of token lane % 16 in each 16 x 16 tile, sixteen
+    // contiguous bytes of the token's row.
+    const bool aligned = ((a.out_stride | a.col0) & 3u) == 0u && (reinterpret_cast<uintptr_t>(a.out) & 15u) == 0u;
 #pragma unroll
     for (int i = 0; i < 4; i++) {
+        const uint32_t t = t0 + wm + 16 * i + lrow;
 #pragma unroll
         for (int j = 0; j < 4; j++) {
-            const uint32_t col = j0 + wn + 16 * j + lrow;
-            if (col >= a.n) continue;
+            const uint32_t col = j0 + wn + 16 * j + 4 * (lane >> 4);
+            if (t >= a.rows || col >= a.n) continue;
+            float *o = a.out + (size_t)t * a.out_stride + a.col0 + col;
+            f32x4 v = acc[i][j];
+            if (aligned && col + 3u < a.n) {
+                f32x4 *o4 = reinterpret_cast<f32x4 *>(o);
+                if (a.accumulate) v += *o4;
+                *o4 = v;
+            } else {
 #pragma unroll
-            for (int r = 0; r < 4; r++) {
-                const uint32_t t = t0 + wm + 16 * i + 4 * (lane >> 4) + r;
-                if (t >= a.rows) continue;
-                const size_t o = (size_t)t * a.out_stride + a.col0 + col;
-                const float v = acc[i][j][r];
-                a.out[o] = a.accumulate ? a.out[o] + v : v;
+                for (int r = 0; r < 4; r++)
+                    if (col + r < a.n) o[r] = a.accumulate ? o[r] + v[r] : v[r];
             }
         }
     }
