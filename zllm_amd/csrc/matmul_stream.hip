@@ -80,8 +80,11 @@ __device__ __forceinline__ void lds_barrier() {
 // while a store is outstanding (loads complete in order among themselves; the
 // store only makes the wait stricter). The two idle cycles keep a following
 // instruction from overwriting the data registers before the store has read them.
+// The outputs are written once and not read again by this kernel: the non-temporal
+// hint keeps them from displacing the weight stream in L2 (measured 86.6 -> 84.4 us
+// on 128 x 1024 x 151936).
 __device__ __forceinline__ void store_apart(sf32x4 *at, sf32x4 v) {
-    asm volatile("global_store_dwordx4 %0, %1, off\n\ts_nop 1" ::"v"(at), "v"(v) : "memory");
+    asm volatile("global_store_dwordx4 %0, %1, off nt\n\ts_nop 1" ::"v"(at), "v"(v) : "memory");
 }
 
 // Each lane's vector of the lane whose number times four is `from`.
