@@ -157,3 +157,59 @@ def test_profiling_runs_launch_by_launch(pair):
     assert sum(v.count for v in t.totals.values()) == 2 * LAYERS  # every launch timed on its own
     assert np.array_equal(replaying.step(x), eager.step(x))      # and replayed again afterwards
     assert replaying.c.host.replayed_submits() == 3
+
+
+def test_a_regrown_workspace_retires_the_graphs_that_pointed_into_it():
+    """The bf16 rung narrows f32 activations into the context's workspace; a graph
+    captured with one allocation must not run once a larger step has replaced it."""
+    rows, n, k = 32, 128, 256
+    g = synth.rng(0xC0DE)
+    raw = synth.q8_0_rows(g, n, k)
+    big_rows = 20480  # 10 MB of narrowed activations: beyond the 8 MB the workspace starts with
+    big_x = synth.activations(synth.rng(1), big_rows, k, bf16=True)
+    devs = [Device.open(0), Device.open(0, Device.NO_REPLAY)]
+    try:
+        steps = []
+        for d in devs:
+            c = Ctx(d)
+            c.set.select_prefill(c.rec, K.Prefill.bf16_mfma)
+            wa = c.gpu_weights(TensorType.q8_0, raw, k)
+            xa, big_xa = c.output(rows * k), c.upload(big_x)
+            outs = [c.output(rows * n) for _ in range(8)]
+            big_out = c.output(big_rows * n)
+            b = K.Builder(c.rec, c.set)
+            p = P.MatmulQuant(rows=rows, n=n, k=k, col0=0, out_stride=n, k_slice=k)
+            ls = [b.add(Kernel.matmul_q8_0_float, p, [xa, wa, o], K.Grid.tiles_y(K.div_ceil(n, 64), 16)) for o in outs]
+            big = b.add(Kernel.matmul_q8_0_float, P.MatmulQuant(rows=big_rows, n=n, k=k, col0=0, out_stride=n, k_slice=k), [big_xa, wa, big_out],
+                        K.Grid.tiles_y(K.div_ceil(n, 64), 16))
+            b.finish()
+            c.flush()
+
+            def step(x, c=c, xa=xa, ls=ls, outs=outs):
+                c.rec.write_buffer(xa.buffer, 0, np.ascontiguousarray(x).reshape(-1).view(np.uint8))
+                for l in ls:
+                    l.record(c.rec, K.Extent(rows=rows))
+                return c.read(outs[-1]).copy()
+
+            def grow(c=c, big=big, big_out=big_out):
+                big.record(c.rec, K.Extent(rows=big_rows))
+                return c.read(big_out).copy()
+
+            steps.append((c, step, grow))
+        (rc, rstep, rgrow), (ec, estep, egrow) = steps
+        for i in range(3):
+            x = synth.activations(synth.rng(0xD00 + i), rows, k, bf16=True)
+            assert np.array_equal(rstep(x), estep(x)), f"step {i}"
+        # The first step allocated the workspace, so the second was the first sight of the
+        # sequence with that allocation and the third was captured and replayed.
+        assert rc.host.replayed_submits() == 1
+        assert np.array_equal(rgrow(), egrow())  # replaces the workspace
+        for i in range(3):
+            x = synth.activations(synth.rng(0xE00 + i), rows, k, bf16=True)
+            assert np.array_equal(rstep(x), estep(x)), f"step {i} after the regrowth"
+        assert rc.host.replayed_submits() == 3  # seen again with the new allocation, then replayed twice
+        want = synth.activations(synth.rng(0xE02), rows, k, bf16=True).astype(np.float64) @ oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k).astype(np.float64).T
+        assert rel_err(rstep(synth.activations(synth.rng(0xE02), rows, k, bf16=True)).reshape(rows, n), want) <= 2e-2
+    finally:
+        for d in devs:
+            d.deinit()
