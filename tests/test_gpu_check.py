@@ -153,6 +153,15 @@ def quant_matvec(c, t: TensorType, k: int, pair: bool, variants=None):
     (TensorType.q6_k, 1024, False),   # "matvec q6_k norm+="
     (TensorType.q6_k, 2304, True),    # the SiLU pair on Q6_K, nine blocks a row
     (TensorType.q5_k, 4096, True),
+    # k above 4096: the lane walks several tasks, inputs read from LDS.
+    (TensorType.q4_k, 14336, False),
+    (TensorType.q4_k, 5120, True),
+    (TensorType.q8_0, 14336, True),
+    (TensorType.q8_0, 8224, False),   # 128.5 tasks: a tail in the third wave
+    (TensorType.q6_k, 8192, False),
+    (TensorType.q3_k, 16384, True),
+    (TensorType.q5_k, 4352, True),
+    (TensorType.q4_k, 16640, False),
 ])
 def test_quant_matvec(ctx, t, k, pair):
     worst, split_exact = quant_matvec(ctx, t, k, pair)
