@@ -34,7 +34,7 @@
 // Q8_0 block), so each SIMD holds two waves to overlap LDS reads, conversions
 // and MFMAs, and no wave converts or reads a weight another one also needs.
 // The four k quarters are added through LDS at the end, always as
-// (q0 + q2) + (q1 + q3).
+// (q0 + q2) + (q1 + q3), each wave finishing a quarter of the token tiles.
 //
 // v_mfma_f32_16x16x32_bf16 takes from lane l eight k values of matrix row l % 16
 // (its first operand) and eight of token l % 16: lane group g = l / 16 owns
@@ -183,6 +183,9 @@ struct WBf16 {
 
 template <class W, int MT> constexpr int buf_bytes() { return 16 * MT * 256 + W::WBUF; }
 template <class W, int MT> constexpr int lds_bytes() { return 3 * buf_bytes<W, MT>(); }
+// The exchange of the k quarters at the end reuses the buffers: 8 waves x 3 inboxes x MT / 4
+// tiles x 2 x 1 KB.
+static_assert(lds_bytes<WQ8_0, 8>() >= 8 * 3 * 2 * 2 * 1024 && lds_bytes<WQ8_0, 4>() >= 8 * 3 * 1 * 2 * 1024, "the exchange must fit the buffers");
 
 template <class W, int MT, bool RAGGED>
 __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
@@ -289,71 +292,68 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still land in LDS below
     __syncthreads();
 
-    // Add the four k quarters through LDS, in a fixed order whatever the
-    // timing: quarters 2 and 3 hand everything to 0 and 1, then 0 and 1 swap
-    // halves (quarter 0 keeps the lower token tiles), so four waves store.
-    float *xchg = reinterpret_cast<float *>(lds);
-    constexpr int REGS = MT * 8;  // accumulator floats per lane
-    if (kq >= 2u) {
-        float *dst = xchg + (size_t)(((kq - 2u) * 2u + wn) * REGS) * 64u + lane;
+    // Add the four k quarters through LDS in one exchange: the wave of quarter q keeps token
+    // tiles OWN q .. + OWN - 1 of its 32 matrix rows and hands its sums of the other tiles to
+    // the waves that keep those; after one barrier every wave adds the four quarters of its
+    // tiles in a fixed order, (q0 + q2) + (q1 + q3), and stores them. The quarter is a
+    // constant in each copy of the code, so that the accumulators are indexed statically.
+    constexpr int OWN = MT / 4;
+    f32x4 *inbox = reinterpret_cast<f32x4 *>(lds);
+    // Where quarter `from` puts tile ii, j for the wave of quarter `owner` (from != owner).
+    auto slot = [&](uint32_t owner, uint32_t from, int ii, int j) {
+        return ((((owner * 2u + wn) * 3u + ((from + 3u - owner) & 3u)) * OWN + ii) * 2u + j) * 64u + lane;
+    };
+    auto send = [&](auto quarter) __attribute__((always_inline)) {
+        constexpr int Q = decltype(quarter)::value;
 #pragma unroll
-        for (int i = 0; i < MT; i++)
+        for (int i = 0; i < MT; i++) {
+            if (i / OWN == Q) continue;
 #pragma unroll
-            for (int j = 0; j < 2; j++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) dst[((i * 2 + j) * 4 + r) * 64] = acc[i][j][r];
-    }
-    __syncthreads();
-    if (kq < 2u) {
-        const float *src = xchg + (size_t)((kq * 2u + wn) * REGS) * 64u + lane;
-#pragma unroll
-        for (int i = 0; i < MT; i++)
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) acc[i][j][r] += src[((i * 2 + j) * 4 + r) * 64];
-    }
-    __syncthreads();
-    constexpr int KEEP = MT / 2;  // token tiles each of the two keeps
-    if (kq < 2u) {
-        float *dst = xchg + (size_t)((kq * 2u + wn) * (REGS / 2)) * 64u + lane;
-#pragma unroll
-        for (int i = 0; i < KEEP; i++)
-#pragma unroll
-            for (int j = 0; j < 2; j++)
-#pragma unroll
-                for (int r = 0; r < 4; r++) dst[((i * 2 + j) * 4 + r) * 64] = kq ? acc[i][j][r] : acc[i + KEEP][j][r];
-    }
-    __syncthreads();
-    if (kq >= 2u) return;
-    const float *src = xchg + (size_t)(((kq ^ 1u) * 2u + wn) * (REGS / 2)) * 64u + lane;
+            for (int j = 0; j < 2; j++) inbox[slot(i / OWN, Q, i % OWN, j)] = acc[i][j];
+        }
+    };
     // D[output][token] (the weights are the MFMA's first operand): the lane holds
     // outputs 4 (lane / 16) .. + 3 of token lane % 16 in each 16 x 16 tile, sixteen
     // contiguous bytes of the token's row.
     const bool aligned = ((a.out_stride | a.col0 | a.slice_stride) & 3u) == 0u && (reinterpret_cast<uintptr_t>(a.out) & 15u) == 0u;
+    auto collect = [&](auto quarter) __attribute__((always_inline)) {
+        constexpr int Q = decltype(quarter)::value;
 #pragma unroll
-    for (int i = 0; i < KEEP; i++) {
-        const uint32_t t = t0 + 16u * (kq ? i + KEEP : i) + lrow;
+        for (int ii = 0; ii < OWN; ii++) {
+            const uint32_t t = t0 + 16u * (OWN * Q + ii) + lrow;
 #pragma unroll
-        for (int j = 0; j < 2; j++) {
-            const uint32_t col = j0 + 32u * wn + 16u * j + 4u * g;
-            f32x4 other;
+            for (int j = 0; j < 2; j++) {
+                f32x4 p[4];
 #pragma unroll
-            for (int r = 0; r < 4; r++) other[r] = src[((i * 2 + j) * 4 + r) * 64];
-            const f32x4 mine = kq ? acc[i + KEEP][j] : acc[i][j];
-            f32x4 v = kq ? other + mine : mine + other;  // (q0 + q2) + (q1 + q3)
-            if (t >= a.rows || col >= a.n) continue;
-            float *o = a.out + (size_t)z * a.slice_stride + (size_t)t * a.out_stride + a.col0 + col;
-            if (aligned && col + 3u < a.n) {
-                f32x4 *o4 = reinterpret_cast<f32x4 *>(o);
-                if (a.accumulate) v += *o4;
-                *o4 = v;
-            } else {
+                for (int from = 0; from < 4; from++) p[from] = from == Q ? acc[OWN * Q + ii][j] : inbox[slot(Q, from, ii, j)];
+                f32x4 v = (p[0] + p[2]) + (p[1] + p[3]);
+                const uint32_t col = j0 + 32u * wn + 16u * j + 4u * g;
+                if (t >= a.rows || col >= a.n) continue;
+                float *o = a.out + (size_t)z * a.slice_stride + (size_t)t * a.out_stride + a.col0 + col;
+                if (aligned && col + 3u < a.n) {
+                    f32x4 *o4 = reinterpret_cast<f32x4 *>(o);
+                    if (a.accumulate) v += *o4;
+                    *o4 = v;
+                } else {
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (col + r < a.n) o[r] = a.accumulate ? o[r] + v[r] : v[r];
+                    for (int r = 0; r < 4; r++)
+                        if (col + r < a.n) o[r] = a.accumulate ? o[r] + v[r] : v[r];
+                }
             }
         }
+    };
+    switch (kq) {
+    case 0: send(std::integral_constant<int, 0>{}); break;
+    case 1: send(std::integral_constant<int, 1>{}); break;
+    case 2: send(std::integral_constant<int, 2>{}); break;
+    default: send(std::integral_constant<int, 3>{}); break;
+    }
+    __syncthreads();
+    switch (kq) {
+    case 0: collect(std::integral_constant<int, 0>{}); break;
+    case 1: collect(std::integral_constant<int, 1>{}); break;
+    case 2: collect(std::integral_constant<int, 2>{}); break;
+    default: collect(std::integral_constant<int, 3>{}); break;
     }
 }
 
