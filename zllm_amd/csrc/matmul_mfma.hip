@@ -440,7 +440,11 @@ static zhip_result launch_mfma(const Dispatch &d, const char *name, bool sliced,
     if (slices == 1u && a.k_slice >= a.k && (uint64_t)((a.rows + 255u) / 256u) * ((a.n + 127u) / 128u) >= (uint64_t)d.dev->compute_units)
         return launch_mfma_wide(d, name, q8_0, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes);
     const bool ragged = a.k % BK != 0 || a.k_slice % BK != 0;
-    if (a.rows > 64u) return ragged ? launch_kernel<W, 8, true>(d, name, a, slices) : launch_kernel<W, 8, false>(d, name, a, slices);
+    // 128-token tiles unless those leave half of the CUs idle and 64-token tiles (which
+    // convert every weight twice as often) still run in one round.
+    const uint64_t tall = (uint64_t)((a.rows + 127u) / 128u) * ((a.n + BN - 1) / BN) * slices;
+    if (a.rows > 64u && 2u * tall > (uint64_t)d.dev->compute_units)
+        return ragged ? launch_kernel<W, 8, true>(d, name, a, slices) : launch_kernel<W, 8, false>(d, name, a, slices);
     return ragged ? launch_kernel<W, 4, true>(d, name, a, slices) : launch_kernel<W, 4, false>(d, name, a, slices);
 }
 
