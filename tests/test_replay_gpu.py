@@ -26,14 +26,16 @@ class Stack:
 
     def __init__(self, c: Ctx, m: int, weights):
         self.c, self.m = c, m
+        self.skip = 0  # trailing launches a step leaves out
         self.x = c.output(m * KDIM)
         b = K.Builder(c.rec, c.set)
-        self.launches = []
+        self.launches, self.outputs = [], []
         cur = self.x
         for gate_up, down, norm in weights:
             wg = c.gpu_weights(TensorType.q4_k, gate_up, KDIM)
             wd = c.gpu_weights(TensorType.q8_0, down, N)
             act, nxt = c.output(m * N), c.output(m * KDIM)
+            self.outputs += [act, nxt]
             v = K.MatvecVariant()
             self.launches.append(b.add(
                 K.weight_kernel("matvec", TensorType.q4_k), P.MatvecBf16(n=N, k=KDIM, col0=0, out_stride=N, eps=EPS, norm=True, silu_pair=True, half=N),
@@ -57,9 +59,11 @@ class Stack:
         c = self.c
         rows = self.m if rows is None else rows
         c.rec.write_buffer(self.x.buffer, 0, np.ascontiguousarray(x, dtype=np.float32).reshape(-1).view(np.uint8))
-        for l in self.launches:
+        used = self.launches[: len(self.launches) - self.skip]
+        for l in used:
             l.record(c.rec, K.Extent(rows=rows))
-        return c.read(self.out)[: rows * KDIM].reshape(rows, KDIM).copy()
+        out = self.out if self.skip == 0 else self.outputs[len(used) - 1]
+        return c.read(out)[: rows * (N if len(used) % 2 else KDIM)].copy()
 
 
 def make_weights():
@@ -110,6 +114,36 @@ def test_every_replay_matches_the_eager_run(pair):
         act = both[:, :N] / (1 + np.exp(-both[:, :N])) * both[:, N:]
         cur = act @ oracle.Matrix(oracle.Q8_0, down, KDIM, N).rows().astype(np.float64).T
     assert rel_err(seen[0], cur) <= 1e-4
+
+
+def test_more_sequences_than_kept_graphs():
+    """Twenty different steps in rotation (sixteen graphs are kept, the least recently used
+    replaced): none is seen twice before it is forgotten, every result is still right; ten in
+    rotation are replayed from their second round on."""
+    g = synth.rng(0x6AA)
+    weights = [(synth.q4_k_rows(g, 2 * N, KDIM), synth.q8_0_rows(g, KDIM, N), synth.activations(g, 1, KDIM).reshape(-1)) for _ in range(5)]
+    devs = [Device.open(0), Device.open(0, Device.NO_REPLAY)]
+    try:
+        replaying, eager = [Stack(Ctx(d), 8, weights) for d in devs]
+        variants = [(rows, skip) for skip in (0, 1, 2) for rows in range(1, 9)][:20]  # 10, 9 or 8 launches of 1..8 rows
+
+        def run(variant, seed):
+            rows, skip = variant
+            x = synth.activations(synth.rng(seed), 8, KDIM)
+            replaying.skip = eager.skip = skip
+            return np.array_equal(replaying.step(x, rows), eager.step(x, rows))
+
+        for cycle in range(3):
+            for i, v in enumerate(variants):
+                assert run(v, 0xF00 + 32 * cycle + i), f"cycle {cycle}, variant {v}"
+        assert replaying.c.host.replayed_submits() == 0
+        for cycle in range(3):
+            for i, v in enumerate(variants[:10]):
+                assert run(v, 0xF80 + 32 * cycle + i), f"cycle {cycle}, variant {v}"
+        assert 10 <= replaying.c.host.replayed_submits() <= 30
+    finally:
+        for d in devs:
+            d.deinit()
 
 
 def test_steps_of_different_extents_keep_their_own_graphs(pair):
