@@ -425,13 +425,21 @@ zhip_result run_dispatch(zhip_context *c, const Op &op, size_t &timed) {
 // Only kernels are captured: no copies, clears or memsets.
 constexpr size_t kMinReplayDispatches = 8, kMaxReplays = 16;
 
-// The leading dispatches of the queue if what follows them is only reads, else 0.
-size_t replayable_prefix(const zhip_context *c) {
+// The leading dispatches of the queue if what follows them is only reads, else 0. Every
+// parameter block must sit in a uniform-usage buffer whose host copy is current: any other
+// would be read back from the GPU while the launches are resolved, which a capture forbids.
+size_t replayable_prefix(zhip_context *c) {
     size_t n = 0;
     while (n < c->ops.size() && c->ops[n].kind == Op::dispatch) n++;
     for (size_t i = n; i < c->ops.size(); i++)
         if (c->ops[i].kind != Op::read) return 0;
-    return n >= kMinReplayDispatches ? n : 0;
+    if (n < kMinReplayDispatches) return 0;
+    for (size_t i = 0; i < n; i++) {
+        const Entry &e = c->ops[i].group.e[0];
+        const Buffer *ub = e.bound ? get(c->buffers, e.buffer) : nullptr;
+        if (!ub || !ub->shadowed || ub->shadow_stale) return 0;
+    }
+    return n;
 }
 
 zhip_result replay_key(zhip_context *c, size_t count, std::vector<uint8_t> &key) {
