@@ -556,6 +556,55 @@ def test_matmul_q8_0_float_streamed_chunk(ctx, rows, n, k, col0, pad, accumulate
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
 
 
+@pytest.mark.parametrize("weights", ["bf16", "f16", "q8_0"])
+@pytest.mark.parametrize("rows,n,k,col0,pad,accumulate", [
+    (19, 100, 1024, 0, 0, False),    # partial tiles in both dimensions
+    (133, 150, 96, 3, 6, True),      # a step of 96 positions, accumulate, padded rows
+    (300, 4100, 128, 0, 0, False),   # 128-token tiles
+    (67, 70, 320, 0, 0, False),
+])
+def test_prefill_fp16_single_rung(ctx, weights, rows, n, k, col0, pad, accumulate):
+    """The reference's fp16_single rung: activations rounded to f16, weights rounded
+    to f16 (Q8_0: the f32 product d * q rounded once), fp32 accumulation
+    (src/agility/kernels/matmul_q8_0_float_linalg_single.hlsl:36-58,
+    src/agility/kernels/matmul_half_linalg.hlsl:34-52). Against that operand contract in
+    float64; a token's bits the same in the step or alone."""
+    c = ctx
+    x = c.random(rows * k, 2).reshape(rows, k)
+    x[0, :4] = [70000.0, -3e-6, 1.0009765625 + 2.0 ** -12, 65519.0]  # beyond the range, below the normals, a tie, the last value that rounds to a finite one
+    if weights == "q8_0":
+        raw, values = quant_rows(c, TensorType.q8_0, n, k)
+        wa, kernel = c.gpu_weights(TensorType.q8_0, raw, k), Kernel.matmul_q8_0_float
+        p = lambda count: P.MatmulQuant(rows=count, n=n, k=k, col0=col0, out_stride=n + pad, accumulate=int(accumulate), k_slice=k)
+    else:
+        bits, values = random_half(c, n * k, 1, weights)
+        wa, kernel = c.upload(bits.reshape(n, k)), Kernel["matmul_" + weights]
+        p = lambda count: P.MatmulBf16(rows=count, n=n, k=k, col0=col0, out_stride=n + pad, accumulate=int(accumulate))
+    stride = n + pad
+    init = c.random(rows * stride, 0.5).reshape(rows, stride)
+    c.set.select_prefill(c.rec, K.Prefill.fp16_single)
+
+    def run(first, count):
+        out = c.upload(init[first : first + count])
+        c.launcher().launch(kernel, p(count), [c.upload(x[first : first + count]), wa, out], (K.div_ceil(n, 64), K.div_ceil(count, 16), 1))
+        return c.read(out).reshape(count, stride)
+
+    got = run(0, rows)
+    with np.errstate(over="ignore"):
+        x16 = x.astype(np.float16).astype(np.float64)
+        w16 = values.reshape(n, k).astype(np.float32).astype(np.float16).astype(np.float64)
+    assert np.isinf(x16[0, 0]) and x16[0, 3] == 65504.0
+    with np.errstate(invalid="ignore"):
+        want = x16 @ w16.T + (init[:, col0 : col0 + n] if accumulate else 0)
+    # Token 0 holds an infinity: its outputs are infinities or NaN, as the reference's are.
+    assert not np.isfinite(got[0, col0 : col0 + n]).any()
+    assert rel_err(got[1:, col0 : col0 + n], want[1:]) <= 1e-5
+    assert np.array_equal(got[:, :col0], init[:, :col0]) and np.array_equal(got[:, col0 + n :], init[:, col0 + n :]), "columns outside the step were written"
+    for first, count in ((1, 1), (rows - 1, 1), (rows // 3, min(20, rows - rows // 3))):
+        assert run(first, count).tobytes() == got[first : first + count].tobytes(), "a token's bits depend on its step"
+    c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
+
+
 def launch_float_q8(c, x, weights, out, rows, accumulate, slices, chunked):
     """Two weight chunks exercise nonzero col0 and a padded output stride;
     split-k partials are dense per chunk (src/kernels/check.zig:752-770)."""

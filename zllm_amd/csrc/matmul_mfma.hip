@@ -57,6 +57,8 @@ namespace zhip {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 // Native vectors rather than HIP's uint4/float4 structs: their copies are plain
@@ -83,6 +85,27 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
     const f32x2 v = {lo, hi};
     return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
 }
+
+// The format both operands enter the matrix cores in. Bf16 is this backend's own rung;
+// F16 is the reference's fp16_single rung (activations and weights rounded to f16, fp32
+// accumulation: src/agility/kernels/matmul_q8_0_float_linalg_single.hlsl:36-58,
+// src/agility/kernels/matmul_half_linalg.hlsl:34-52 with SINGLE_PRODUCT).
+struct Bf16 {
+    typedef bf16x8 vec8;
+    __device__ static uint32_t pack(float lo, float hi) { return pack_bf16(lo, hi); }
+    __device__ static float widen(uint32_t bits) { return __builtin_bit_cast(float, bits << 16); }
+    __device__ static f32x4 mfma(vec8 a, vec8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0); }
+};
+struct F16 {
+    typedef f16x8 vec8;
+    // Round to nearest even; values beyond the f16 range become infinities, as (half)v does.
+    __device__ static uint32_t pack(float lo, float hi) {
+        const f32x2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+    }
+    __device__ static float widen(uint32_t bits) { return (float)__builtin_bit_cast(_Float16, (uint16_t)bits); }
+    __device__ static f32x4 mfma(vec8 a, vec8 b, f32x4 c) { return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0); }
+};
 
 // A raw buffer: loads past `bytes` return zero instead of faulting.
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const uint8_t *base, uint32_t bytes) {
@@ -147,20 +170,25 @@ struct WQ8_0 {
         f.q = *reinterpret_cast<const u32x2 *>(buf + row * 128u + 16u * ((2u * kq + (g >> 1)) ^ key) + 8u * (g & 1u));
         f.d = *reinterpret_cast<const uint16_t *>(buf + SCALES + 8u * row + 2u * kq);
     }
-    // bf16(q * d) of the lane's eight weights.
-    __device__ static bf16x8 frag(const Frag &f) {
+    // q * d of the lane's eight weights (exact in f32), rounded once to the operand format.
+    template <class H>
+    __device__ static typename H::vec8 frag(const Frag &f) {
         const float d = half_bits_to_float(f.d);
         const int32_t lo = (int32_t)f.q.x, hi = (int32_t)f.q.y;
         const u32x4 v = {
-            pack_bf16((float)(int8_t)(lo) * d, (float)(int8_t)(lo >> 8) * d),
-            pack_bf16((float)(int8_t)(lo >> 16) * d, (float)(lo >> 24) * d),
-            pack_bf16((float)(int8_t)(hi) * d, (float)(int8_t)(hi >> 8) * d),
-            pack_bf16((float)(int8_t)(hi >> 16) * d, (float)(hi >> 24) * d)};
-        return __builtin_bit_cast(bf16x8, v);
+            H::pack((float)(int8_t)(lo) * d, (float)(int8_t)(lo >> 8) * d),
+            H::pack((float)(int8_t)(lo >> 16) * d, (float)(lo >> 24) * d),
+            H::pack((float)(int8_t)(hi) * d, (float)(int8_t)(hi >> 8) * d),
+            H::pack((float)(int8_t)(hi >> 16) * d, (float)(hi >> 24) * d)};
+        return __builtin_bit_cast(typename H::vec8, v);
     }
 };
 
-struct WBf16 {
+// Weights stored as 16-bit floats of format S (Bf16 or F16): used as stored when the
+// operands have that format, else widened and rounded to the operands' (the reference rounds
+// decoded weights to f16: src/agility/kernels/matmul_half_linalg.hlsl:46-52).
+template <class S>
+struct WHalf {
     static constexpr int WBUF = 2 * BN * 128;  // two lines a row: [line][row][128]
     static constexpr int LOADS = 2;
     struct Offsets { uint32_t q[2]; };
@@ -178,8 +206,20 @@ struct WBf16 {
     __device__ static void read(const uint8_t *buf, uint32_t row, uint32_t key, uint32_t g, uint32_t kq, Frag &f) {
         f.v = *reinterpret_cast<const u32x4 *>(buf + (kq >> 1) * (BN * 128) + row * 128u + 16u * ((4u * (kq & 1u) + g) ^ key));
     }
-    __device__ static bf16x8 frag(const Frag &f) { return __builtin_bit_cast(bf16x8, f.v); }
+    template <class H>
+    __device__ static typename H::vec8 frag(const Frag &f) {
+        if constexpr (std::is_same<H, S>::value) {
+            return __builtin_bit_cast(typename H::vec8, f.v);
+        } else {
+            u32x4 v;
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[i] = H::pack(S::widen(f.v[i] & 0xffffu), S::widen(f.v[i] >> 16));
+            return __builtin_bit_cast(typename H::vec8, v);
+        }
+    }
 };
+typedef WHalf<Bf16> WBf16;
+typedef WHalf<F16> WF16;
 
 template <class W, int MT> constexpr int buf_bytes() { return 16 * MT * 256 + W::WBUF; }
 template <class W, int MT> constexpr int lds_bytes() { return 3 * buf_bytes<W, MT>(); }
@@ -187,8 +227,9 @@ template <class W, int MT> constexpr int lds_bytes() { return 3 * buf_bytes<W, M
 // tiles x 2 x 1 KB.
 static_assert(lds_bytes<WQ8_0, 8>() >= 8 * 3 * 2 * 2 * 1024 && lds_bytes<WQ8_0, 4>() >= 8 * 3 * 1 * 2 * 1024, "the exchange must fit the buffers");
 
-template <class W, int MT, bool RAGGED>
+template <class W, class H, int MT, bool RAGGED>
 __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
+    typedef typename H::vec8 vec8;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int BM = 16 * MT, XBUF = BM * 256;   // activations: [line][row][128]
     constexpr int BUF = XBUF + W::WBUF;            // one buffer: activations, then weights
@@ -233,7 +274,7 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     // of line kq / 2.
     const uint32_t key = line_key(lrow);
     const uint32_t a_at = (kq >> 1) * (BM * 128) + lrow * 128u + 16u * ((4u * (kq & 1u) + g) ^ key);
-    bf16x8 af[MT], bf[2];
+    vec8 af[MT], bf[2];
     auto read_b = [&](uint32_t buf, typename W::Frag (&wf)[2]) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < 2; j++) W::read(lds + buf * BUF + XBUF, 32u * wn + 16u * j + lrow, key, g, kq, wf[j]);
@@ -241,7 +282,7 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     auto convert = [&](const typename W::Frag (&wf)[2], uint32_t k0) __attribute__((always_inline)) {
         const bool live = !RAGGED || k0 + 32u * kq < ke;
 #pragma unroll
-        for (int j = 0; j < 2; j++) bf[j] = live ? W::frag(wf[j]) : __builtin_bit_cast(bf16x8, u32x4{0u, 0u, 0u, 0u});
+        for (int j = 0; j < 2; j++) bf[j] = live ? W::template frag<H>(wf[j]) : __builtin_bit_cast(vec8, u32x4{0u, 0u, 0u, 0u});
     };
 
     const uint32_t steps = (ke - kb + BK - 1) / BK;
@@ -253,7 +294,7 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
         typename W::Frag wf[2];
         read_b(0, wf);
 #pragma unroll
-        for (int i = 0; i < MT; i++) af[i] = *reinterpret_cast<const bf16x8 *>(lds + a_at + 2048 * i);
+        for (int i = 0; i < MT; i++) af[i] = *reinterpret_cast<const vec8 *>(lds + a_at + 2048 * i);
         convert(wf, kb);
     }
     // Every wave has its fragments of step 0 (buffer 0 may be refilled) and its
@@ -281,8 +322,8 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
 #pragma unroll
         for (int i = 0; i < MT; i++) {
 #pragma unroll
-            for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bf[j], af[i], acc[i][j], 0, 0, 0);
-            af[i] = *reinterpret_cast<const bf16x8 *>(xn + 2048 * i);
+            for (int j = 0; j < 2; j++) acc[i][j] = H::mfma(bf[j], af[i], acc[i][j]);
+            af[i] = *reinterpret_cast<const vec8 *>(xn + 2048 * i);
         }
         convert(wf, kc + BK);
         if (kq >= 2u) fetch(cur, kc + 3u * BK);
@@ -357,11 +398,12 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     }
 }
 
-// f32 activations to packed bf16, eight per thread.
-__global__ __launch_bounds__(256) void narrow_bf16_kernel(const f32x4 *src, u32x4 *dst, uint64_t groups) {
+// f32 activations to the packed operand format, eight per thread.
+template <class H>
+__global__ __launch_bounds__(256) void narrow_kernel(const f32x4 *src, u32x4 *dst, uint64_t groups) {
     for (uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x; i < groups; i += (uint64_t)gridDim.x * 256u) {
         const f32x4 lo = src[2 * i], hi = src[2 * i + 1];
-        dst[i] = u32x4{pack_bf16(lo.x, lo.y), pack_bf16(lo.z, lo.w), pack_bf16(hi.x, hi.y), pack_bf16(hi.z, hi.w)};
+        dst[i] = u32x4{H::pack(lo.x, lo.y), H::pack(lo.z, lo.w), H::pack(hi.x, hi.y), H::pack(hi.z, hi.w)};
     }
 }
 
@@ -380,9 +422,9 @@ zhip_result launch_matmul_stream(const Dispatch &d, const char *name, bool q8_0,
 zhip_result launch_mfma_wide(const Dispatch &d, const char *name, bool q8_0, const uint8_t *x, const uint8_t *w, float *out,
     uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, uint32_t row_bytes);
 
-template <class W, int MT, bool RAGGED>
+template <class W, class H, int MT, bool RAGGED>
 static zhip_result launch_kernel(const Dispatch &d, const char *name, const MfmaArgs &a, uint32_t slices) {
-    auto kernel = matmul_mfma_kernel<W, MT, RAGGED>;
+    auto kernel = matmul_mfma_kernel<W, H, MT, RAGGED>;
     constexpr int bytes = lds_bytes<W, MT>();
     static bool configured = false;
     if (!configured) {
@@ -397,8 +439,11 @@ static zhip_result launch_kernel(const Dispatch &d, const char *name, const Mfma
     return check_launch(d, name);
 }
 
-template <class W, bool XBF16>
+// XPACKED: the activations are bound already packed in the operand format (an extension of
+// the contract, bf16 only); otherwise they are bound as f32 and narrowed first.
+template <class W, bool XPACKED, class H = Bf16>
 static zhip_result launch_mfma(const Dispatch &d, const char *name, bool sliced, bool q8_0) {
+    constexpr bool XBF16 = XPACKED;
     bool empty = false;
     if (zhip_result r = validate_matmul(d, name, sliced, q8_0, XBF16 ? 2u : 4u, &empty)) return r;
     if (empty) return ZHIP_OK;
@@ -426,31 +471,36 @@ static zhip_result launch_mfma(const Dispatch &d, const char *name, bool sliced,
         if (zhip_result r = d.work->reserve(d, x_bytes)) return r;
         const uint64_t groups = x_bytes / 16u;
         const uint64_t blocks = (groups + 255u) / 256u;
-        hipLaunchKernelGGL(narrow_bf16_kernel, dim3((uint32_t)(blocks < 4096u ? blocks : 4096u)), dim3(256), 0, d.stream,
+        hipLaunchKernelGGL(narrow_kernel<H>, dim3((uint32_t)(blocks < 4096u ? blocks : 4096u)), dim3(256), 0, d.stream,
             reinterpret_cast<const f32x4 *>(a.x), reinterpret_cast<u32x4 *>(d.work->data), groups);
         a.x = d.work->data;
     }
     const uint32_t slices = sliced ? d.grid[2] : 1u;
     // A chunk of up to 128 tokens against a tall matrix with a short k is one pass over the
     // weights: the kernel that streams them into registers.
-    if (slices == 1u && a.k_slice >= a.k && matmul_stream_accepts(d, q8_0, a.out, a.rows, a.n, a.k, a.col0, a.out_stride))
+    constexpr bool kBf16Rung = std::is_same<H, Bf16>::value && (std::is_same<W, WBf16>::value || std::is_same<W, WQ8_0>::value);
+    if (kBf16Rung && slices == 1u && a.k_slice >= a.k && matmul_stream_accepts(d, q8_0, a.out, a.rows, a.n, a.k, a.col0, a.out_stride))
         return launch_matmul_stream(d, name, q8_0, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes);
     // Long steps whose 256 x 128 tiles fill the CUs take that tiling: each
     // weight is converted once per 256 tokens and half the bytes cross from L2.
-    if (slices == 1u && a.k_slice >= a.k && (uint64_t)((a.rows + 255u) / 256u) * ((a.n + 127u) / 128u) >= (uint64_t)d.dev->compute_units)
+    if (kBf16Rung && slices == 1u && a.k_slice >= a.k && (uint64_t)((a.rows + 255u) / 256u) * ((a.n + 127u) / 128u) >= (uint64_t)d.dev->compute_units)
         return launch_mfma_wide(d, name, q8_0, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes);
     const bool ragged = a.k % BK != 0 || a.k_slice % BK != 0;
     // 128-token tiles unless those leave half of the CUs idle and 64-token tiles (which
     // convert every weight twice as often) still run in one round.
     const uint64_t tall = (uint64_t)((a.rows + 127u) / 128u) * ((a.n + BN - 1) / BN) * slices;
     if (a.rows > 64u && 2u * tall > (uint64_t)d.dev->compute_units)
-        return ragged ? launch_kernel<W, 8, true>(d, name, a, slices) : launch_kernel<W, 8, false>(d, name, a, slices);
-    return ragged ? launch_kernel<W, 4, true>(d, name, a, slices) : launch_kernel<W, 4, false>(d, name, a, slices);
+        return ragged ? launch_kernel<W, H, 8, true>(d, name, a, slices) : launch_kernel<W, H, 8, false>(d, name, a, slices);
+    return ragged ? launch_kernel<W, H, 4, true>(d, name, a, slices) : launch_kernel<W, H, 4, false>(d, name, a, slices);
 }
 
 zhip_result launch_matmul_bf16_mfma(const Dispatch &d) { return launch_mfma<WBf16, false>(d, "matmul_bf16", false, false); }
 zhip_result launch_matmul_q8_0_float_mfma(const Dispatch &d) { return launch_mfma<WQ8_0, false>(d, "matmul_q8_0_float", true, true); }
 zhip_result launch_matmul_bf16_mfma_xbf16(const Dispatch &d) { return launch_mfma<WBf16, true>(d, "matmul_bf16", false, false); }
 zhip_result launch_matmul_q8_0_float_mfma_xbf16(const Dispatch &d) { return launch_mfma<WQ8_0, true>(d, "matmul_q8_0_float", true, true); }
+// The reference's fp16_single rung: f32-bound activations rounded to f16, weights rounded to f16.
+zhip_result launch_matmul_bf16_f16(const Dispatch &d) { return launch_mfma<WBf16, false, F16>(d, "matmul_bf16", false, false); }
+zhip_result launch_matmul_f16_f16(const Dispatch &d) { return launch_mfma<WF16, false, F16>(d, "matmul_f16", false, false); }
+zhip_result launch_matmul_q8_0_float_f16(const Dispatch &d) { return launch_mfma<WQ8_0, false, F16>(d, "matmul_q8_0_float", true, true); }
 
 }  // namespace zhip

@@ -210,7 +210,15 @@ class Prefill(enum.IntEnum):
 
 
 PREFILL_VARIANT = {Prefill.scalar_f32: 0, Prefill.fp16_single: 0xFFFC0000, Prefill.fp16_compensated: 0xFFFF0000, Prefill.bf16_mfma: 0xFFFB0000, Prefill.bf16_mfma_xbf16: 0xFFFA0000}
-prefill_kernels = (Kernel.matmul_q8_0_float, Kernel.matmul_bf16)
+# The identities a prefill rung switches (src/agility/kernels.zig:111-112, without gyro_matmul).
+# The bf16 rungs are this backend's own and leave matmul_f16 on the exact f32 kernel.
+prefill_kernels = (Kernel.matmul_q8_0_float, Kernel.matmul_bf16, Kernel.matmul_f16)
+
+
+def prefill_kernels_of(rung: "Prefill") -> tuple:
+    if rung in (Prefill.bf16_mfma, Prefill.bf16_mfma_xbf16):
+        return (Kernel.matmul_q8_0_float, Kernel.matmul_bf16)
+    return prefill_kernels
 
 
 class params:
@@ -379,9 +387,11 @@ class Set:
                 self.pipelines[k] = self.scalar_prefill[k]
             return
         for k in prefill_kernels:
+            self.pipelines[k] = self.scalar_prefill[k]
+        for k in prefill_kernels_of(rung):
             if (rung, k) not in self.prefill_variants:
                 self.prefill_variants[(rung, k)] = rec.create_kernel(int(k), PREFILL_VARIANT[rung], contract(k).writes, artifact(k, PREFILL_VARIANT[rung]))
-        for k in prefill_kernels:
+        for k in prefill_kernels_of(rung):
             self.pipelines[k] = self.prefill_variants[(rung, k)]
 
     def matvec(self, rec: cmd.Recorder, k: Kernel, v: MatvecVariant) -> int:
