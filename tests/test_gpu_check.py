@@ -605,6 +605,56 @@ def test_prefill_fp16_single_rung(ctx, weights, rows, n, k, col0, pad, accumulat
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
 
 
+@pytest.mark.parametrize("weights", ["bf16", "f16", "q8_0"])
+@pytest.mark.parametrize("rows,n,k,col0,pad,accumulate", [
+    (19, 100, 1024, 0, 0, False),
+    (133, 150, 96, 3, 6, True),
+    (300, 4100, 128, 0, 0, False),
+    (67, 70, 320, 0, 0, False),
+])
+def test_prefill_fp16_compensated_rung(ctx, weights, rows, n, k, col0, pad, accumulate):
+    """The reference's fp16_compensated rung: every activation as its f16 value plus
+    the f16 of the remainder; Q8_0 weights as exact integers with the block scale
+    applied to the block's sum, stored halves rounded to f16
+    (src/agility/kernels/matmul_q8_0_float_linalg.hlsl:40-101,
+    src/agility/kernels/matmul_half_linalg.hlsl:34-75). Against that operand contract
+    in float64, and, because the activations keep about 22 bits, within 1e-5 of the
+    product of the unrounded activations too (Q8_0; stored halves keep their f16 rounding)."""
+    c = ctx
+    x = c.random(rows * k, 2).reshape(rows, k)
+    if weights == "q8_0":
+        raw, values = quant_rows(c, TensorType.q8_0, n, k)
+        wa, kernel = c.gpu_weights(TensorType.q8_0, raw, k), Kernel.matmul_q8_0_float
+        p = lambda count: P.MatmulQuant(rows=count, n=n, k=k, col0=col0, out_stride=n + pad, accumulate=int(accumulate), k_slice=k)
+        w_used = values.reshape(n, k).astype(np.float64)           # exact: integers times the block's scale
+    else:
+        bits, values = random_half(c, n * k, 1, weights)
+        wa, kernel = c.upload(bits.reshape(n, k)), Kernel["matmul_" + weights]
+        p = lambda count: P.MatmulBf16(rows=count, n=n, k=k, col0=col0, out_stride=n + pad, accumulate=int(accumulate))
+        w_used = values.reshape(n, k).astype(np.float32).astype(np.float16).astype(np.float64)
+    stride = n + pad
+    init = c.random(rows * stride, 0.5).reshape(rows, stride)
+    c.set.select_prefill(c.rec, K.Prefill.fp16_compensated)
+
+    def run(first, count):
+        out = c.upload(init[first : first + count])
+        c.launcher().launch(kernel, p(count), [c.upload(x[first : first + count]), wa, out], (K.div_ceil(n, 64), K.div_ceil(count, 16), 1))
+        return c.read(out).reshape(count, stride)
+
+    got = run(0, rows)
+    hi = x.astype(np.float16)
+    lo = (x - hi.astype(np.float32)).astype(np.float16)
+    x_used = hi.astype(np.float64) + lo.astype(np.float64)
+    base = init[:, col0 : col0 + n] if accumulate else 0
+    assert rel_err(got[:, col0 : col0 + n], x_used @ w_used.T + base) <= 1e-5
+    if weights == "q8_0":
+        assert rel_err(got[:, col0 : col0 + n], x.astype(np.float64) @ w_used.T + base) <= 1e-5
+    assert np.array_equal(got[:, :col0], init[:, :col0]) and np.array_equal(got[:, col0 + n :], init[:, col0 + n :]), "columns outside the step were written"
+    for first, count in ((0, 1), (rows - 1, 1), (rows // 3, min(20, rows - rows // 3))):
+        assert run(first, count).tobytes() == got[first : first + count].tobytes(), "a token's bits depend on its step"
+    c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
+
+
 def launch_float_q8(c, x, weights, out, rows, accumulate, slices, chunked):
     """Two weight chunks exercise nonzero col0 and a padded output stride;
     split-k partials are dense per chunk (src/kernels/check.zig:752-770)."""

@@ -27,7 +27,7 @@ def test_caps_and_adapter(device):
     assert device.memory_budget() > 100 << 30
     assert device.caps.wavefront == 64 and device.caps.compute_units >= 200
     assert device.supports_prefill(K.Prefill.scalar_f32) and device.supports_prefill(K.Prefill.bf16_mfma)
-    assert device.supports_prefill(K.Prefill.fp16_single) and not device.supports_prefill(K.Prefill.fp16_compensated)
+    assert device.supports_prefill(K.Prefill.fp16_single) and device.supports_prefill(K.Prefill.fp16_compensated)
     assert device.backend().name == "hip"
 
 
@@ -215,8 +215,8 @@ def test_missing_kernels_fail_the_batch_and_drop_the_submission(ctx):
 def test_create_kernel_rejects_what_it_does_not_implement(ctx):
     c = ctx
     writes = K.contract(Kernel.matmul_bf16).writes
-    rung = K.Prefill.fp16_compensated
-    expect(c, host.UnsupportedPrefill, lambda: c.rec.create_kernel(int(Kernel.matmul_bf16), K.PREFILL_VARIANT[rung], writes, K.artifact(Kernel.matmul_bf16)))
+    # A prefill variant id that is neither the reference's nor this backend's.
+    expect(c, host.BadCommand, lambda: c.rec.create_kernel(int(Kernel.matmul_bf16), 0xFFF90000, writes, K.artifact(Kernel.matmul_bf16, 0xFFF90000)))
     # matmul_f16 has only the exact f32 rung.
     expect(c, host.UnsupportedPrefill, lambda: c.rec.create_kernel(int(Kernel.matmul_f16), K.PREFILL_VARIANT[K.Prefill.bf16_mfma], writes, K.artifact(Kernel.matmul_f16, K.PREFILL_VARIANT[K.Prefill.bf16_mfma])))
     expect(c, host.BadCommand, lambda: c.rec.create_kernel(int(Kernel.matmul_bf16), 0, writes, b"@compute fn main() {}"))           # another backend's artifact

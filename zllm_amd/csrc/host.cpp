@@ -76,6 +76,9 @@ zhip_result launch_matmul_q8_0_float_mfma_xbf16(const Dispatch &);
 zhip_result launch_matmul_bf16_f16(const Dispatch &);
 zhip_result launch_matmul_f16_f16(const Dispatch &);
 zhip_result launch_matmul_q8_0_float_f16(const Dispatch &);
+zhip_result launch_matmul_bf16_f16c(const Dispatch &);
+zhip_result launch_matmul_f16_f16c(const Dispatch &);
+zhip_result launch_matmul_q8_0_float_f16c(const Dispatch &);
 
 struct KernelInfo {
     const char *name;
@@ -86,39 +89,40 @@ struct KernelInfo {
     LaunchFn launch_bf16;  // the bf16 MFMA rung of a prefill identity
     LaunchFn launch_bf16x; // the same with packed bf16 activations
     LaunchFn launch_f16;   // the reference's fp16_single rung
+    LaunchFn launch_f16c;  // the reference's fp16_compensated rung
     int revision;          // bumped when the implementation changes (plan-cache key)
 };
 
 static const KernelInfo kImplemented[] = {
-    {"matvec_q8_0", 5, 0b01000, VariantKind::matvec, launch_matvec_q8_0, nullptr, nullptr, nullptr, 1},
-    {"matvec_q3_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q3_k, nullptr, nullptr, nullptr, 1},
-    {"matvec_q4_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q4_k, nullptr, nullptr, nullptr, 1},
-    {"matvec_q5_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q5_k, nullptr, nullptr, nullptr, 1},
-    {"matvec_q6_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q6_k, nullptr, nullptr, nullptr, 1},
-    {"matvec_bf16", 5, 0b01000, VariantKind::none, launch_matvec_bf16, nullptr, nullptr, nullptr, 1},
-    {"matvec_f16", 5, 0b01000, VariantKind::none, launch_matvec_f16, nullptr, nullptr, nullptr, 1},
-    {"matmul_f16", 4, 0b1000, VariantKind::prefill, launch_matmul_f16_f32, nullptr, nullptr, launch_matmul_f16_f16, 1},
-    {"matmul_bf16", 4, 0b1000, VariantKind::prefill, launch_matmul_bf16_f32, launch_matmul_bf16_mfma, launch_matmul_bf16_mfma_xbf16, launch_matmul_bf16_f16, 1},
-    {"matmul_q8_0_float", 4, 0b1000, VariantKind::prefill, launch_matmul_q8_0_float_f32, launch_matmul_q8_0_float_mfma, launch_matmul_q8_0_float_mfma_xbf16, launch_matmul_q8_0_float_f16, 1},
-    {"matmul_q8_0", 5, 0b01000, VariantKind::none, launch_matmul_q8_0, nullptr, nullptr, nullptr, 1},
-    {"matmul_q3_k", 5, 0b01000, VariantKind::none, launch_matmul_q3_k, nullptr, nullptr, nullptr, 1},
-    {"matmul_q4_k", 5, 0b01000, VariantKind::none, launch_matmul_q4_k, nullptr, nullptr, nullptr, 1},
-    {"matmul_q5_k", 5, 0b01000, VariantKind::none, launch_matmul_q5_k, nullptr, nullptr, nullptr, 1},
-    {"matmul_q6_k", 5, 0b01000, VariantKind::none, launch_matmul_q6_k, nullptr, nullptr, nullptr, 1},
-    {"quantize_q8", 5, 0b01100, VariantKind::none, launch_quantize_q8, nullptr, nullptr, nullptr, 1},
-    {"matmul_reduce", 3, 0b100, VariantKind::none, launch_matmul_reduce, nullptr, nullptr, nullptr, 1},
-    {"silu_mul", 3, 0b100, VariantKind::none, launch_silu_mul, nullptr, nullptr, nullptr, 1},
-    {"repack_q8_0", 3, 0b100, VariantKind::none, launch_repack_q8_0, nullptr, nullptr, nullptr, 1},
-    {"repack_q3_k", 3, 0b100, VariantKind::none, launch_repack_q3_k, nullptr, nullptr, nullptr, 1},
-    {"repad", 3, 0b100, VariantKind::none, launch_repad, nullptr, nullptr, nullptr, 1},
-    {"embed_q8_0", 4, 0b1000, VariantKind::none, launch_embed_q8_0, nullptr, nullptr, nullptr, 1},
-    {"embed_q3_k", 4, 0b1000, VariantKind::none, launch_embed_q3_k, nullptr, nullptr, nullptr, 1},
-    {"embed_q4_k", 4, 0b1000, VariantKind::none, launch_embed_q4_k, nullptr, nullptr, nullptr, 1},
-    {"embed_q5_k", 4, 0b1000, VariantKind::none, launch_embed_q5_k, nullptr, nullptr, nullptr, 1},
-    {"embed_q6_k", 4, 0b1000, VariantKind::none, launch_embed_q6_k, nullptr, nullptr, nullptr, 1},
-    {"embed_bf16", 4, 0b1000, VariantKind::none, launch_embed_bf16, nullptr, nullptr, nullptr, 1},
-    {"embed_f16", 4, 0b1000, VariantKind::none, launch_embed_f16, nullptr, nullptr, nullptr, 1},
-    {"embed_iq4_xs", 4, 0b1000, VariantKind::none, launch_embed_iq4_xs, nullptr, nullptr, nullptr, 1},
+    {"matvec_q8_0", 5, 0b01000, VariantKind::matvec, launch_matvec_q8_0, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matvec_q3_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q3_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matvec_q4_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q4_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matvec_q5_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q5_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matvec_q6_k", 5, 0b01000, VariantKind::matvec, launch_matvec_q6_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matvec_bf16", 5, 0b01000, VariantKind::none, launch_matvec_bf16, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matvec_f16", 5, 0b01000, VariantKind::none, launch_matvec_f16, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matmul_f16", 4, 0b1000, VariantKind::prefill, launch_matmul_f16_f32, nullptr, nullptr, launch_matmul_f16_f16, launch_matmul_f16_f16c, 1},
+    {"matmul_bf16", 4, 0b1000, VariantKind::prefill, launch_matmul_bf16_f32, launch_matmul_bf16_mfma, launch_matmul_bf16_mfma_xbf16, launch_matmul_bf16_f16, launch_matmul_bf16_f16c, 1},
+    {"matmul_q8_0_float", 4, 0b1000, VariantKind::prefill, launch_matmul_q8_0_float_f32, launch_matmul_q8_0_float_mfma, launch_matmul_q8_0_float_mfma_xbf16, launch_matmul_q8_0_float_f16, launch_matmul_q8_0_float_f16c, 1},
+    {"matmul_q8_0", 5, 0b01000, VariantKind::none, launch_matmul_q8_0, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matmul_q3_k", 5, 0b01000, VariantKind::none, launch_matmul_q3_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matmul_q4_k", 5, 0b01000, VariantKind::none, launch_matmul_q4_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matmul_q5_k", 5, 0b01000, VariantKind::none, launch_matmul_q5_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matmul_q6_k", 5, 0b01000, VariantKind::none, launch_matmul_q6_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"quantize_q8", 5, 0b01100, VariantKind::none, launch_quantize_q8, nullptr, nullptr, nullptr, nullptr, 1},
+    {"matmul_reduce", 3, 0b100, VariantKind::none, launch_matmul_reduce, nullptr, nullptr, nullptr, nullptr, 1},
+    {"silu_mul", 3, 0b100, VariantKind::none, launch_silu_mul, nullptr, nullptr, nullptr, nullptr, 1},
+    {"repack_q8_0", 3, 0b100, VariantKind::none, launch_repack_q8_0, nullptr, nullptr, nullptr, nullptr, 1},
+    {"repack_q3_k", 3, 0b100, VariantKind::none, launch_repack_q3_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"repad", 3, 0b100, VariantKind::none, launch_repad, nullptr, nullptr, nullptr, nullptr, 1},
+    {"embed_q8_0", 4, 0b1000, VariantKind::none, launch_embed_q8_0, nullptr, nullptr, nullptr, nullptr, 1},
+    {"embed_q3_k", 4, 0b1000, VariantKind::none, launch_embed_q3_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"embed_q4_k", 4, 0b1000, VariantKind::none, launch_embed_q4_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"embed_q5_k", 4, 0b1000, VariantKind::none, launch_embed_q5_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"embed_q6_k", 4, 0b1000, VariantKind::none, launch_embed_q6_k, nullptr, nullptr, nullptr, nullptr, 1},
+    {"embed_bf16", 4, 0b1000, VariantKind::none, launch_embed_bf16, nullptr, nullptr, nullptr, nullptr, 1},
+    {"embed_f16", 4, 0b1000, VariantKind::none, launch_embed_f16, nullptr, nullptr, nullptr, nullptr, 1},
+    {"embed_iq4_xs", 4, 0b1000, VariantKind::none, launch_embed_iq4_xs, nullptr, nullptr, nullptr, nullptr, 1},
 };
 
 static const KernelInfo *find_kernel(const char *name, size_t len) {
@@ -676,9 +680,8 @@ zhip_result create_kernel(zhip_context *c, const Command &cmd) {
             return set_error(c, ZHIP_E_BAD_COMMAND, "create_kernel: %s variant 0x%08x is not a MatvecVariant id", info->name, p.variant);
         break;
     case VariantKind::prefill:
-        if (p.variant == kVariantFp16Compensated)
-            return set_error(c, ZHIP_E_UNSUPPORTED_PREFILL, "create_kernel: %s: the compensated fp16 rung is not implemented on HIP", info->name);
         if (p.variant == kVariantFp16Single) p.launch = info->launch_f16;
+        else if (p.variant == kVariantFp16Compensated) p.launch = info->launch_f16c;
         else if (p.variant == kVariantBf16) p.launch = info->launch_bf16;
         else if (p.variant == kVariantBf16X) p.launch = info->launch_bf16x;
         else if (p.variant != 0) return set_error(c, ZHIP_E_BAD_COMMAND, "create_kernel: %s has no variant 0x%08x", info->name, p.variant);
@@ -943,9 +946,9 @@ zhip_result zhip_get_caps(zhip_context *c, zhip_caps *out) {
 
 int32_t zhip_supports_prefill(zhip_context *c, uint32_t rung) {
     if (!c || c->lost) return 0;
-    // scalar_f32 and fp16_single of the reference's ladder; the bf16 MFMA rungs are this
-    // backend's own (3: f32 activations as bound by the contract, 4: packed bf16 activations).
-    return rung == ZHIP_PREFILL_SCALAR_F32 || rung == ZHIP_PREFILL_FP16_SINGLE || rung == 3u || rung == 4u;
+    // The reference's ladder (scalar_f32, fp16_single, fp16_compensated); the bf16 MFMA rungs
+    // are this backend's own (3: f32 activations as bound by the contract, 4: packed bf16).
+    return rung <= ZHIP_PREFILL_FP16_COMPENSATED || rung == 3u || rung == 4u;
 }
 
 zhip_result zhip_set_file(zhip_context *c, const void *bytes, size_t len) {

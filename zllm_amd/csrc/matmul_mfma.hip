@@ -77,6 +77,7 @@ struct MfmaArgs {
     uint32_t rows, n, k, col0, out_stride, accumulate, k_slice, slice_stride;
     uint32_t row_bytes;
     uint32_t x_bytes, w_bytes;  // bytes the kernel may read behind x and w
+    uint32_t x_plane;           // compensated rung: bytes from the activations' f16 values to their residuals
 };
 
 // Two floats to packed bf16, round to nearest even as the reference narrows
@@ -170,6 +171,27 @@ struct WQ8_0 {
         f.q = *reinterpret_cast<const u32x2 *>(buf + row * 128u + 16u * ((2u * kq + (g >> 1)) ^ key) + 8u * (g & 1u));
         f.d = *reinterpret_cast<const uint16_t *>(buf + SCALES + 8u * row + 2u * kq);
     }
+    // The compensated rung keeps the weights as the integers they are and applies the
+    // block's scale to the block's sum (src/agility/kernels/matmul_q8_0_float_linalg.hlsl:21-25).
+    static constexpr bool BLOCK_SCALED = true;
+    struct ScaleRaw { uint32_t s[4]; };
+    // The scales of rows row0 .. row0 + 3 for k quarter kq.
+    __device__ static void read_scales(const uint8_t *buf, uint32_t row0, uint32_t kq, ScaleRaw &r) {
+#pragma unroll
+        for (int i = 0; i < 4; i++) r.s[i] = *reinterpret_cast<const uint16_t *>(buf + SCALES + 8u * (row0 + i) + 2u * kq);
+    }
+    __device__ static f32x4 scales(const ScaleRaw &r) {
+        return f32x4{half_bits_to_float(r.s[0]), half_bits_to_float(r.s[1]), half_bits_to_float(r.s[2]), half_bits_to_float(r.s[3])};
+    }
+    // The lane's eight weights as integers in the operand format (exact: |q| <= 128).
+    template <class H>
+    __device__ static typename H::vec8 frag_exact(const Frag &f) {
+        const int32_t lo = (int32_t)f.q.x, hi = (int32_t)f.q.y;
+        const u32x4 v = {
+            H::pack((float)(int8_t)(lo), (float)(int8_t)(lo >> 8)), H::pack((float)(int8_t)(lo >> 16), (float)(lo >> 24)),
+            H::pack((float)(int8_t)(hi), (float)(int8_t)(hi >> 8)), H::pack((float)(int8_t)(hi >> 16), (float)(hi >> 24))};
+        return __builtin_bit_cast(typename H::vec8, v);
+    }
     // q * d of the lane's eight weights (exact in f32), rounded once to the operand format.
     template <class H>
     __device__ static typename H::vec8 frag(const Frag &f) {
@@ -206,6 +228,12 @@ struct WHalf {
     __device__ static void read(const uint8_t *buf, uint32_t row, uint32_t key, uint32_t g, uint32_t kq, Frag &f) {
         f.v = *reinterpret_cast<const u32x4 *>(buf + (kq >> 1) * (BN * 128) + row * 128u + 16u * ((4u * (kq & 1u) + g) ^ key));
     }
+    static constexpr bool BLOCK_SCALED = false;
+    struct ScaleRaw {};
+    __device__ static void read_scales(const uint8_t *, uint32_t, uint32_t, ScaleRaw &) {}
+    __device__ static f32x4 scales(const ScaleRaw &) { return f32x4{1.f, 1.f, 1.f, 1.f}; }
+    template <class H>
+    __device__ static typename H::vec8 frag_exact(const Frag &f) { return frag<H>(f); }
     template <class H>
     __device__ static typename H::vec8 frag(const Frag &f) {
         if constexpr (std::is_same<H, S>::value) {
@@ -221,19 +249,26 @@ struct WHalf {
 typedef WHalf<Bf16> WBf16;
 typedef WHalf<F16> WF16;
 
-template <class W, int MT> constexpr int buf_bytes() { return 16 * MT * 256 + W::WBUF; }
-template <class W, int MT> constexpr int lds_bytes() { return 3 * buf_bytes<W, MT>(); }
+template <class W, int MT, bool COMP = false> constexpr int buf_bytes() { return (COMP ? 2 : 1) * 16 * MT * 256 + W::WBUF; }
+template <class W, int MT, bool COMP = false> constexpr int lds_bytes() { return 3 * buf_bytes<W, MT, COMP>(); }
 // The exchange of the k quarters at the end reuses the buffers: 8 waves x 3 inboxes x MT / 4
 // tiles x 2 x 1 KB.
 static_assert(lds_bytes<WQ8_0, 8>() >= 8 * 3 * 2 * 2 * 1024 && lds_bytes<WQ8_0, 4>() >= 8 * 3 * 1 * 2 * 1024, "the exchange must fit the buffers");
 
-template <class W, class H, int MT, bool RAGGED>
+// COMP: the reference's compensated rung. Every activation enters twice, as its f16 value
+// and as the f16 of what that rounding left (two planes of the narrowed copy, two planes in
+// LDS, two MFMAs a tile); Q8_0 weights enter as their integers and a block's scale multiplies
+// the block's sum (src/agility/kernels/matmul_q8_0_float_linalg.hlsl:79-101), stored halves
+// are rounded to f16 and both products are summed (matmul_half_linalg.hlsl:53-60).
+template <class W, class H, int MT, bool RAGGED, bool COMP = false>
 __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     typedef typename H::vec8 vec8;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    constexpr int BM = 16 * MT, XBUF = BM * 256;   // activations: [line][row][128]
-    constexpr int BUF = XBUF + W::WBUF;            // one buffer: activations, then weights
-    constexpr int XLOADS = MT / 2;                 // wave-wide activation loads a step issues per wave
+    constexpr int BM = 16 * MT, XPLANE = BM * 256;           // activations: [line][row][128]
+    constexpr int PLANES = COMP ? 2 : 1, XBUF = PLANES * XPLANE;
+    constexpr int BUF = XBUF + W::WBUF;                      // one buffer: activations, then weights
+    constexpr int XLOADS = PLANES * MT / 2;                  // wave-wide activation loads a step issues per wave
+    constexpr bool SCALED = COMP && W::BLOCK_SCALED;
     constexpr int LOADS = XLOADS + W::LOADS;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t j0 = blockIdx.x * BN, t0 = blockIdx.y * BM, z = blockIdx.z;
@@ -258,9 +293,9 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     uint32_t xoff[XLOADS], xdst[XLOADS];
 #pragma unroll
     for (int i = 0; i < XLOADS; i++) {
-        const uint32_t b = wave + 8u * i, line = b / (BM / 8), row = 8u * (b % (BM / 8)) + (lane >> 3);
-        xoff[i] = (t0 + row) * a.k * 2u + 128u * line + 16u * ((lane & 7u) ^ line_key(row));
-        xdst[i] = line * (BM * 128) + 1024u * (b % (BM / 8));
+        const uint32_t plane = i / (MT / 2), b = wave + 8u * (i % (MT / 2)), line = b / (BM / 8), row = 8u * (b % (BM / 8)) + (lane >> 3);
+        xoff[i] = plane * a.x_plane + (t0 + row) * a.k * 2u + 128u * line + 16u * ((lane & 7u) ^ line_key(row));
+        xdst[i] = plane * XPLANE + line * (BM * 128) + 1024u * (b % (BM / 8));
     }
     auto fetch = [&](uint32_t buf, uint32_t k0) __attribute__((always_inline)) {
         uint8_t *base = lds + buf * BUF;
@@ -274,15 +309,41 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     // of line kq / 2.
     const uint32_t key = line_key(lrow);
     const uint32_t a_at = (kq >> 1) * (BM * 128) + lrow * 128u + 16u * ((4u * (kq & 1u) + g) ^ key);
-    vec8 af[MT], bf[2];
-    auto read_b = [&](uint32_t buf, typename W::Frag (&wf)[2]) __attribute__((always_inline)) {
-#pragma unroll
-        for (int j = 0; j < 2; j++) W::read(lds + buf * BUF + XBUF, 32u * wn + 16u * j + lrow, key, g, kq, wf[j]);
+    vec8 af[MT], af2[COMP ? MT : 1], bf[2];
+    f32x4 sc[2];  // SCALED: the block scales of the lane's four outputs in each of its two tiles
+    struct Raw {
+        typename W::Frag wf[2];
+        typename W::ScaleRaw sr[2];
     };
-    auto convert = [&](const typename W::Frag (&wf)[2], uint32_t k0) __attribute__((always_inline)) {
+    auto read_b = [&](uint32_t buf, Raw &r) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            W::read(lds + buf * BUF + XBUF, 32u * wn + 16u * j + lrow, key, g, kq, r.wf[j]);
+            if (SCALED) W::read_scales(lds + buf * BUF + XBUF, 32u * wn + 16u * j + 4u * g, kq, r.sr[j]);
+        }
+    };
+    auto convert = [&](const Raw &r, uint32_t k0) __attribute__((always_inline)) {
         const bool live = !RAGGED || k0 + 32u * kq < ke;
 #pragma unroll
-        for (int j = 0; j < 2; j++) bf[j] = live ? W::template frag<H>(wf[j]) : __builtin_bit_cast(vec8, u32x4{0u, 0u, 0u, 0u});
+        for (int j = 0; j < 2; j++) {
+            bf[j] = live ? (SCALED ? W::template frag_exact<H>(r.wf[j]) : W::template frag<H>(r.wf[j])) : __builtin_bit_cast(vec8, u32x4{0u, 0u, 0u, 0u});
+            if (SCALED) sc[j] = live ? W::scales(r.sr[j]) : f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    // One token tile against the wave's two weight tiles.
+    auto multiply = [&](int i) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < 2; j++) {
+            if constexpr (SCALED) {
+                f32x4 part = H::mfma(bf[j], af[i], f32x4{0.f, 0.f, 0.f, 0.f});
+                part = H::mfma(bf[j], af2[i], part);
+                acc[i][j] = part * sc[j] + acc[i][j];
+            } else if constexpr (COMP) {
+                acc[i][j] = H::mfma(bf[j], af2[i], H::mfma(bf[j], af[i], acc[i][j]));
+            } else {
+                acc[i][j] = H::mfma(bf[j], af[i], acc[i][j]);
+            }
+        }
     };
 
     const uint32_t steps = (ke - kb + BK - 1) / BK;
@@ -291,11 +352,14 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     fetch(2, kb + 2 * BK);
     sync_keeping_loads<2 * LOADS>();
     {
-        typename W::Frag wf[2];
-        read_b(0, wf);
+        Raw r;
+        read_b(0, r);
 #pragma unroll
-        for (int i = 0; i < MT; i++) af[i] = *reinterpret_cast<const vec8 *>(lds + a_at + 2048 * i);
-        convert(wf, kb);
+        for (int i = 0; i < MT; i++) {
+            af[i] = *reinterpret_cast<const vec8 *>(lds + a_at + 2048 * i);
+            if (COMP) af2[i] = *reinterpret_cast<const vec8 *>(lds + a_at + XPLANE + 2048 * i);
+        }
+        convert(r, kb);
     }
     // Every wave has its fragments of step 0 (buffer 0 may be refilled) and its
     // loads of step 1, which step 0 reads, have landed.
@@ -317,15 +381,15 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
         // on 512 x 4096 x 4096).
         if (kq < 2u) fetch(cur, kc + 3u * BK);
         const uint8_t *xn = lds + nxt * BUF + a_at;
-        typename W::Frag wf[2];
-        read_b(nxt, wf);
+        Raw r;
+        read_b(nxt, r);
 #pragma unroll
         for (int i = 0; i < MT; i++) {
-#pragma unroll
-            for (int j = 0; j < 2; j++) acc[i][j] = H::mfma(bf[j], af[i], acc[i][j]);
+            multiply(i);
             af[i] = *reinterpret_cast<const vec8 *>(xn + 2048 * i);
+            if (COMP) af2[i] = *reinterpret_cast<const vec8 *>(xn + XPLANE + 2048 * i);
         }
-        convert(wf, kc + BK);
+        convert(r, kc + BK);
         if (kq >= 2u) fetch(cur, kc + 3u * BK);
         sync_keeping_loads<LOADS>();
         cur = nxt;
@@ -407,6 +471,23 @@ __global__ __launch_bounds__(256) void narrow_kernel(const f32x4 *src, u32x4 *ds
     }
 }
 
+// f32 activations to two f16 planes: the rounded values, and the f16 of what each rounding
+// left (src/agility/kernels/matmul_q8_0_float_linalg.hlsl:47-52); eight per thread.
+__global__ __launch_bounds__(256) void narrow_split_kernel(const f32x4 *src, u32x4 *hi_out, u32x4 *lo_out, uint64_t groups) {
+    for (uint64_t i = (uint64_t)blockIdx.x * 256u + threadIdx.x; i < groups; i += (uint64_t)gridDim.x * 256u) {
+        const f32x4 v[2] = {src[2 * i], src[2 * i + 1]};
+        u32x4 hi, lo;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const float a0 = v[e >> 1][2 * (e & 1)], a1 = v[e >> 1][2 * (e & 1) + 1];
+            hi[e] = F16::pack(a0, a1);
+            lo[e] = F16::pack(__fsub_rn(a0, F16::widen(hi[e] & 0xffffu)), __fsub_rn(a1, F16::widen(hi[e] >> 16)));
+        }
+        hi_out[i] = hi;
+        lo_out[i] = lo;
+    }
+}
+
 }  // namespace
 
 // Validation shared with the f32 rung (matmul_f32.hip); x_bytes = 4 for f32
@@ -422,10 +503,11 @@ zhip_result launch_matmul_stream(const Dispatch &d, const char *name, bool q8_0,
 zhip_result launch_mfma_wide(const Dispatch &d, const char *name, bool q8_0, const uint8_t *x, const uint8_t *w, float *out,
     uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, uint32_t row_bytes);
 
-template <class W, class H, int MT, bool RAGGED>
+template <class W, class H, int MT, bool RAGGED, bool COMP = false>
 static zhip_result launch_kernel(const Dispatch &d, const char *name, const MfmaArgs &a, uint32_t slices) {
-    auto kernel = matmul_mfma_kernel<W, H, MT, RAGGED>;
-    constexpr int bytes = lds_bytes<W, MT>();
+    auto kernel = matmul_mfma_kernel<W, H, MT, RAGGED, COMP>;
+    constexpr int bytes = lds_bytes<W, MT, COMP>();
+    static_assert(bytes <= 160 * 1024, "three buffers must fit the CU's LDS");
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
@@ -441,8 +523,9 @@ static zhip_result launch_kernel(const Dispatch &d, const char *name, const Mfma
 
 // XPACKED: the activations are bound already packed in the operand format (an extension of
 // the contract, bf16 only); otherwise they are bound as f32 and narrowed first.
-template <class W, bool XPACKED, class H = Bf16>
+template <class W, bool XPACKED, class H = Bf16, bool COMP = false>
 static zhip_result launch_mfma(const Dispatch &d, const char *name, bool sliced, bool q8_0) {
+    static_assert(!COMP || (!XPACKED && std::is_same<H, F16>::value), "the compensated rung narrows f32 activations to two f16 planes");
     constexpr bool XBF16 = XPACKED;
     bool empty = false;
     if (zhip_result r = validate_matmul(d, name, sliced, q8_0, XBF16 ? 2u : 4u, &empty)) return r;
@@ -468,11 +551,21 @@ static zhip_result launch_mfma(const Dispatch &d, const char *name, bool sliced,
     if (!XBF16) {
         // Narrow the step's activations once, into the workspace.
         if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", name);
-        if (zhip_result r = d.work->reserve(d, x_bytes)) return r;
+        const uint64_t plane = (x_bytes + 255u) & ~(uint64_t)255u;
+        if (COMP && plane + x_bytes >= (1ull << 32)) return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
+        if (zhip_result r = d.work->reserve(d, COMP ? plane + x_bytes : x_bytes)) return r;
         const uint64_t groups = x_bytes / 16u;
         const uint64_t blocks = (groups + 255u) / 256u;
-        hipLaunchKernelGGL(narrow_kernel<H>, dim3((uint32_t)(blocks < 4096u ? blocks : 4096u)), dim3(256), 0, d.stream,
-            reinterpret_cast<const f32x4 *>(a.x), reinterpret_cast<u32x4 *>(d.work->data), groups);
+        const dim3 ngrid((uint32_t)(blocks < 4096u ? blocks : 4096u));
+        if (COMP) {
+            hipLaunchKernelGGL(narrow_split_kernel, ngrid, dim3(256), 0, d.stream, reinterpret_cast<const f32x4 *>(a.x),
+                reinterpret_cast<u32x4 *>(d.work->data), reinterpret_cast<u32x4 *>(d.work->data + plane), groups);
+            a.x_plane = (uint32_t)plane;
+            a.x_bytes = (uint32_t)(plane + x_bytes);
+        } else {
+            hipLaunchKernelGGL(narrow_kernel<H>, ngrid, dim3(256), 0, d.stream,
+                reinterpret_cast<const f32x4 *>(a.x), reinterpret_cast<u32x4 *>(d.work->data), groups);
+        }
         a.x = d.work->data;
     }
     const uint32_t slices = sliced ? d.grid[2] : 1u;
@@ -486,6 +579,10 @@ static zhip_result launch_mfma(const Dispatch &d, const char *name, bool sliced,
     if (kBf16Rung && slices == 1u && a.k_slice >= a.k && (uint64_t)((a.rows + 255u) / 256u) * ((a.n + 127u) / 128u) >= (uint64_t)d.dev->compute_units)
         return launch_mfma_wide(d, name, q8_0, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes);
     const bool ragged = a.k % BK != 0 || a.k_slice % BK != 0;
+    if constexpr (COMP) {
+        // Two planes of activations in LDS: 64-token tiles.
+        return ragged ? launch_kernel<W, H, 4, true, true>(d, name, a, slices) : launch_kernel<W, H, 4, false, true>(d, name, a, slices);
+    }
     // 128-token tiles unless those leave half of the CUs idle and 64-token tiles (which
     // convert every weight twice as often) still run in one round.
     const uint64_t tall = (uint64_t)((a.rows + 127u) / 128u) * ((a.n + BN - 1) / BN) * slices;
@@ -502,5 +599,9 @@ zhip_result launch_matmul_q8_0_float_mfma_xbf16(const Dispatch &d) { return laun
 zhip_result launch_matmul_bf16_f16(const Dispatch &d) { return launch_mfma<WBf16, false, F16>(d, "matmul_bf16", false, false); }
 zhip_result launch_matmul_f16_f16(const Dispatch &d) { return launch_mfma<WF16, false, F16>(d, "matmul_f16", false, false); }
 zhip_result launch_matmul_q8_0_float_f16(const Dispatch &d) { return launch_mfma<WQ8_0, false, F16>(d, "matmul_q8_0_float", true, true); }
+// The reference's fp16_compensated rung.
+zhip_result launch_matmul_bf16_f16c(const Dispatch &d) { return launch_mfma<WBf16, false, F16, true>(d, "matmul_bf16", false, false); }
+zhip_result launch_matmul_f16_f16c(const Dispatch &d) { return launch_mfma<WF16, false, F16, true>(d, "matmul_f16", false, false); }
+zhip_result launch_matmul_q8_0_float_f16c(const Dispatch &d) { return launch_mfma<WQ8_0, false, F16, true>(d, "matmul_q8_0_float", true, true); }
 
 }  // namespace zhip
