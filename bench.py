@@ -368,9 +368,10 @@ def bench_c4(env):
     xa = env["upload"](synth.to_bf16_bits(x))
     rb = K.row_bytes(TensorType.q8_0, k)
     out = env["output"](4 * rows * n)
-    launches = []
+    launches, weight_copies = [], []
     for _ in range(4):
         wa = env["output"](n * rb)
+        weight_copies.append(wa)
         K.Launcher(rec, kset).layout(TensorType.q8_0, src, wa, n, k)
         p = P.MatmulQuant(rows=rows, n=n, k=k, col0=0, out_stride=n, k_slice=k)
         launches.append(env["L"](b.add(K.Kernel.matmul_q8_0_float, p, [xa, wa, out], K.Grid.tiles_y(K.div_ceil(n, 64), 16)), rows))
@@ -379,9 +380,25 @@ def bench_c4(env):
     steps = max(1, env["args"].steps // 4)
     wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 4))
     got = env["read"](out)[: rows * n].reshape(rows, n).astype(np.float64)
-    kset.select_prefill(rec, K.Prefill.scalar_f32)
     w = oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k)
     want = x.astype(np.float64) @ w.astype(np.float64).T
+    # The reference's own ladder on the same shape, activations bound as f32 as its contract
+    # says: the exact f32 rung and the two f16 matrix-core rungs.
+    xf = env["upload"](x)
+    ladder = {}
+    for rung, share in ((K.Prefill.fp16_single, 4), (K.Prefill.fp16_compensated, 4), (K.Prefill.scalar_f32, 40)):
+        kset.select_prefill(rec, rung)
+        rl = []
+        for wa in weight_copies:
+            rl.append(env["L"](b.add(K.Kernel.matmul_q8_0_float, P.MatmulQuant(rows=rows, n=n, k=k, col0=0, out_stride=n, k_slice=k), [xf, wa, out], K.Grid.tiles_y(K.div_ceil(n, 64), 16)), rows))
+        b.finish()
+        env["flush"]()
+        rsteps = max(4, env["args"].steps // share)
+        _, rgpu = env["timed"](rl, rsteps, max(1, rsteps // 10))
+        rgot = env["read"](out)[: rows * n].reshape(rows, n).astype(np.float64)
+        ladder[rung.name] = {"us_per_launch_gpu": round(rgpu / rsteps * 1e6, 3), "TFLOPs_gpu": round(2 * rows * n * k * rsteps / rgpu / 1e12, 1),
+                             "max_err_over_max_want": float(np.max(np.abs(rgot - want)) / np.max(np.abs(want)))}
+    kset.select_prefill(rec, K.Prefill.scalar_f32)
     wn = np.linalg.norm(w.astype(np.float64), axis=1)
     xn = np.linalg.norm(x.astype(np.float64), axis=1)
     bound = float(np.max(np.abs(got - want) / (xn[:, None] * wn[None, :])))
@@ -396,6 +413,7 @@ def bench_c4(env):
         "mfma_frac": round(flops * steps / gpu_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
         "max_err_over_row_x_norms": bound,
         "max_err_over_max_want": float(np.max(np.abs(got - want)) / np.max(np.abs(want))),
+        "reference_ladder_f32_activations": ladder,
     }
 
 

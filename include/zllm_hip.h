@@ -99,9 +99,13 @@ zhip_result zhip_create(const zhip_options *options, zhip_context **out_context)
 zhip_result zhip_destroy(zhip_context *context);
 /* Replaces Device.limits/adapter/memoryBudget (src/gpu/host.zig:81-126). */
 zhip_result zhip_get_caps(zhip_context *context, zhip_caps *out_caps);
-/* Replaces Device.supportsPrefill (src/gpu/host.zig:70-77): 1 or 0. The scalar
- * rung is always supported; the fp16 rungs are D3D12 LinAlg contracts this
- * backend does not implement. */
+/* Replaces Device.supportsPrefill (src/gpu/host.zig:70-77): 1 or 0. All three
+ * rungs of the reference's ladder are supported: scalar_f32 (exact f32 kernels),
+ * fp16_single and fp16_compensated (create_kernel variants 0xfffc0000 and
+ * 0xffff0000 of matmul_q8_0_float, matmul_bf16 and matmul_f16,
+ * src/agility/kernels.zig:114-131) on the f16 matrix cores; 3 and 4 name this
+ * backend's own bf16 rungs (variants 0xfffb0000 / 0xfffa0000 of
+ * matmul_q8_0_float and matmul_bf16). */
 int32_t zhip_supports_prefill(zhip_context *context, uint32_t rung);
 /* Replaces Host.setFile (src/gpu/host.zig:158-165): the model file mapping
  * write_file commands read; it must stay mapped while they may execute. */
