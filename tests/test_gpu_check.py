@@ -672,7 +672,7 @@ def launch_float_q8(c, x, weights, out, rows, accumulate, slices, chunked):
                      [partial, out], K.elementwise(rows * n))
 
 
-@pytest.mark.parametrize("rung", [K.Prefill.scalar_f32, K.Prefill.bf16_mfma, K.Prefill.bf16_mfma_xbf16])
+@pytest.mark.parametrize("rung", [K.Prefill.scalar_f32, K.Prefill.fp16_single, K.Prefill.fp16_compensated, K.Prefill.bf16_mfma, K.Prefill.bf16_mfma_xbf16])
 def test_matmul_q8_0_float(ctx, rung):
     """Unrounded float activations, k = 320, full and partial tiles, weight
     chunks, padding, accumulate and split-k; within each split-k path token
@@ -688,7 +688,12 @@ def test_matmul_q8_0_float(ctx, rung):
     xa = c.upload(xin)
     init = c.random(rows * stride, 0.25).reshape(rows, stride)
     c.set.select_prefill(c.rec, rung)
-    if rung != K.Prefill.scalar_f32:
+    if rung == K.Prefill.fp16_single:
+        xs, ws, tol = x.astype(np.float16), values.astype(np.float16), 1e-5
+    elif rung == K.Prefill.fp16_compensated:
+        hi = x.astype(np.float16)
+        xs, ws, tol = hi.astype(np.float64) + (x - hi.astype(np.float32)).astype(np.float16).astype(np.float64), values, 1e-5
+    elif rung != K.Prefill.scalar_f32:
         # The rung's operand contract: both operands rounded to bf16.
         xs, ws, tol = synth.bf16_round(x), synth.bf16_round(values), 1e-5
     else:
