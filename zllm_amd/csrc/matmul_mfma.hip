@@ -1,6 +1,11 @@
 // Prefill multiplies on the CDNA4 matrix cores: the bf16 rung of matmul_bf16
 // and matmul_q8_0_float (same parameter blocks, bindings and grids as
-// src/kernels/matmul_half.wgsl and src/kernels/matmul_q8_0_float.wgsl).
+// src/kernels/matmul_half.wgsl and src/kernels/matmul_q8_0_float.wgsl), and,
+// with f16 operands, the reference's fp16_single and fp16_compensated rungs of
+// those two and matmul_f16 (src/agility/kernels/matmul_q8_0_float_linalg.hlsl,
+// matmul_q8_0_float_linalg_single.hlsl, matmul_half_linalg.hlsl); what follows
+// describes the bf16 rung, the f16 rungs differ in the operand format only
+// (see Bf16 / F16 and the COMP parameter of the kernel).
 //
 // out[t][col0 + j] (+)= sum_i bf16(x[t][i]) * bf16(w[j][i]), fp32 accumulate.
 // Q8_0 weights become bf16(q * d), one rounding of the exact f32 product; BF16
