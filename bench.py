@@ -45,7 +45,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,c5,formats for the 'also' section; 'none' skips it")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,c5,formats,replay for the 'also' section; 'none' skips it")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run 4 plain elementwise copies (256 MiB read + 256 MiB written each) so a counter run has a kernel of known traffic to scale by")
@@ -273,7 +273,7 @@ def main() -> int:
     only = [s for s in args.only.split(",") if s]
     also = {}
     if "none" not in only:
-        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c4_int8", bench_c4_int8), ("c5", bench_c5), ("formats", bench_formats)):
+        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c4_int8", bench_c4_int8), ("c5", bench_c5), ("formats", bench_formats), ("replay", bench_replay)):
             if not only or name in only:
                 try:
                     also[name] = fn(locals())
@@ -301,6 +301,63 @@ def bench_c1(env):
     nbytes = n * k // 32 * 34 + 4 * k + 4 * n  # GGUF bytes: 3,358,720
     return env["hbm_entry"]("C1: Q8_0 decode matvec M=1 K=1024 N=3072", nbytes, wall, gpu_s, steps,
                             {"copies": len(launches), "max_err_over_row_x_norms": bound, "max_err_over_max_want": rel})
+
+
+def bench_replay(env):
+    """A decode step's worth of small dependent-looking launches (224 one-row Q8_0 multiplies,
+    K = 1024, N = 3072, the same batch submitted again and again as a decoder does per
+    token): wall time per submit when the host replays the batch from a HIP graph and when
+    it launches it kernel by kernel, each on a context of its own."""
+    import time
+
+    from zllm_amd import Device, Host, cmd
+    synth, K, TensorType, P = env["synth"], env["K"], env["TensorType"], env["P"]
+    n, k, count, submits = 3072, 1024, 224, 12
+    g = synth.rng(0xC1)
+    raw, x = synth.q8_0_rows(g, n, k), synth.activations(g, 1, k)
+    storage = cmd.Usage.storage | cmd.Usage.copy_dst | cmd.Usage.copy_src
+    out = {}
+    for name, flags in (("replayed", 0), ("launched", Device.NO_REPLAY)):
+        dev = Device.open(0, flags)
+        host, rec = Host(dev), cmd.Recorder()
+        kset = K.Set.create(rec)
+        token = [0]
+
+        def flush():
+            token[0] += 1
+            rec.submit(token[0])
+            t0 = time.perf_counter()
+            host.execute(rec.batch(), [])
+            wall = time.perf_counter() - t0
+            rec.clear()
+            return wall
+
+        def upload(arr):
+            a8 = np.ascontiguousarray(arr).reshape(-1).view(np.uint8)
+            buf = rec.create_buffer(a8.size, storage)
+            rec.write_buffer(buf, 0, a8)
+            return K.Arg(buf, a8.size)
+
+        src, xa = upload(raw), upload(x)
+        wa = K.Arg(rec.create_buffer(n * K.row_bytes(TensorType.q8_0, k), storage), n * K.row_bytes(TensorType.q8_0, k))
+        K.Launcher(rec, kset).layout(TensorType.q8_0, src, wa, n, k)
+        oa = K.Arg(rec.create_buffer(4 * n, storage), 4 * n)
+        b = K.Builder(rec, kset)
+        launch = b.add(K.weight_kernel("matvec", TensorType.q8_0), P.MatvecBf16(n=n, k=k, col0=0, out_stride=n), [xa, wa, oa, wa],
+                       K.Grid.rows_y(K.div_ceil(n, K.MatvecVariant().group_rows())))
+        b.finish()
+        flush()
+        walls, gpus = [], []
+        for _ in range(submits):
+            for _ in range(count):
+                launch.record(rec, K.Extent(rows=1))
+            walls.append(flush())
+            gpus.append(host.last_submit()[0])
+        out[name] = {"us_per_submit_wall": round(float(np.median(walls[3:])) * 1e6, 1), "us_per_submit_gpu": round(float(np.median(gpus[3:])) * 1e-3, 1),
+                     "replayed_submits": host.replayed_submits()}
+        dev.deinit()
+    out["workload"] = f"{count} x matvec_q8_0 M=1 K={k} N={n} per submit, {submits} submits, medians after the third"
+    return out
 
 
 def bench_formats(env):
