@@ -283,3 +283,33 @@ def matmul_q8(t: int, raw: np.ndarray, q: np.ndarray, d: np.ndarray, n: int) -> 
     if _lib.zref_matmul_q8(t, _ptr(raw), _ptr(q), _ptr(d), rows, n, k, _ptr(out)) != 0:
         raise ValueError("matmul_q8: unsupported type")
     return out
+
+
+def prefill_fp16_single(x: np.ndarray, w: np.ndarray) -> np.ndarray:
+    """The fp16_single prefill rung's product in float64: activations rounded to f16
+    ((half)v, src/agility/kernels/matmul_q8_0_float_linalg_single.hlsl:36-40,
+    matmul_half_linalg.hlsl:38-41), weights rounded to f16 (Q8_0: (half)(scale * q),
+    matmul_q8_0_float_linalg_single.hlsl:50-57; stored halves: matmul_half_linalg.hlsl:50-51),
+    fp32 accumulation on the matrix units, restated here without its rounding.
+    x is tokens x k (f32), w outputs x k: the dequantized weights as f32 (for Q8_0 the
+    product d * q is exact in f32). Values beyond the f16 range become infinities."""
+    with np.errstate(over="ignore", invalid="ignore"):
+        x16 = np.asarray(x, dtype=np.float32).astype(np.float16).astype(np.float64)
+        w16 = np.asarray(w, dtype=np.float32).astype(np.float16).astype(np.float64)
+        return x16 @ w16.T
+
+
+def prefill_fp16_compensated(x: np.ndarray, w: np.ndarray, exact_weights: bool) -> np.ndarray:
+    """The fp16_compensated prefill rung's product in float64: every activation as
+    hi = (half)v and lo = (half)(v - (float)hi)
+    (src/agility/kernels/matmul_q8_0_float_linalg.hlsl:47-52). Q8_0 weights
+    (exact_weights) stay exact, integers with the block's scale applied to the block's
+    sum of both products (matmul_q8_0_float_linalg.hlsl:62-69,84-100); stored halves are
+    rounded to f16 and the two products are added at the end (matmul_half_linalg.hlsl:50-51,70-73)."""
+    x = np.asarray(x, dtype=np.float32)
+    with np.errstate(over="ignore", invalid="ignore"):
+        hi = x.astype(np.float16)
+        lo = (x - hi.astype(np.float32)).astype(np.float16)
+        w = np.asarray(w, dtype=np.float32)
+        wu = w.astype(np.float64) if exact_weights else w.astype(np.float16).astype(np.float64)
+        return hi.astype(np.float64) @ wu.T + lo.astype(np.float64) @ wu.T

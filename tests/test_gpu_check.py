@@ -591,11 +591,9 @@ def test_prefill_fp16_single_rung(ctx, weights, rows, n, k, col0, pad, accumulat
 
     got = run(0, rows)
     with np.errstate(over="ignore"):
-        x16 = x.astype(np.float16).astype(np.float64)
-        w16 = values.reshape(n, k).astype(np.float32).astype(np.float16).astype(np.float64)
+        x16 = x.astype(np.float16)
     assert np.isinf(x16[0, 0]) and x16[0, 3] == 65504.0
-    with np.errstate(invalid="ignore"):
-        want = x16 @ w16.T + (init[:, col0 : col0 + n] if accumulate else 0)
+    want = oracle.prefill_fp16_single(x, values.reshape(n, k)) + (init[:, col0 : col0 + n] if accumulate else 0)
     # Token 0 holds an infinity: its outputs are infinities or NaN, as the reference's are.
     assert not np.isfinite(got[0, col0 : col0 + n]).any()
     assert rel_err(got[1:, col0 : col0 + n], want[1:]) <= 1e-5
@@ -642,11 +640,8 @@ def test_prefill_fp16_compensated_rung(ctx, weights, rows, n, k, col0, pad, accu
         return c.read(out).reshape(count, stride)
 
     got = run(0, rows)
-    hi = x.astype(np.float16)
-    lo = (x - hi.astype(np.float32)).astype(np.float16)
-    x_used = hi.astype(np.float64) + lo.astype(np.float64)
     base = init[:, col0 : col0 + n] if accumulate else 0
-    assert rel_err(got[:, col0 : col0 + n], x_used @ w_used.T + base) <= 1e-5
+    assert rel_err(got[:, col0 : col0 + n], oracle.prefill_fp16_compensated(x, values.reshape(n, k), exact_weights=weights == "q8_0") + base) <= 1e-5
     if weights == "q8_0":
         assert rel_err(got[:, col0 : col0 + n], x.astype(np.float64) @ w_used.T + base) <= 1e-5
     assert np.array_equal(got[:, :col0], init[:, :col0]) and np.array_equal(got[:, col0 + n :], init[:, col0 + n :]), "columns outside the step were written"
@@ -688,17 +683,18 @@ def test_matmul_q8_0_float(ctx, rung):
     xa = c.upload(xin)
     init = c.random(rows * stride, 0.25).reshape(rows, stride)
     c.set.select_prefill(c.rec, rung)
+    prod = None
     if rung == K.Prefill.fp16_single:
-        xs, ws, tol = x.astype(np.float16), values.astype(np.float16), 1e-5
+        prod, tol = oracle.prefill_fp16_single(x, values), 1e-5
     elif rung == K.Prefill.fp16_compensated:
-        hi = x.astype(np.float16)
-        xs, ws, tol = hi.astype(np.float64) + (x - hi.astype(np.float32)).astype(np.float16).astype(np.float64), values, 1e-5
+        prod, tol = oracle.prefill_fp16_compensated(x, values, exact_weights=True), 1e-5
     elif rung != K.Prefill.scalar_f32:
         # The rung's operand contract: both operands rounded to bf16.
         xs, ws, tol = synth.bf16_round(x), synth.bf16_round(values), 1e-5
     else:
         xs, ws, tol = x, values, 1e-5
-    prod = xs.astype(np.float64) @ ws.astype(np.float64).T
+    if prod is None:
+        prod = xs.astype(np.float64) @ ws.astype(np.float64).T
     for accumulate in (0, 1):
         want = prod + (init[:, 3 : 3 + n] if accumulate else 0)
         for slices, chunked in ((1, 0), (1, 1), (2, 0), (2, 1)):

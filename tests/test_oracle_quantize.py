@@ -175,3 +175,57 @@ def test_matmul_q8_equals_rounded_activations_times_decoded_weights(t, name):
     # differ by f32 roundings.
     tol = 1e-12 if t == oracle.Q8_0 else 2e-7
     assert np.max(np.abs(got - want)) <= tol * scale
+
+
+# ---- the f16 prefill rungs' operand contracts ------------------------------------------
+
+def _shader_q8_compensated(x, q, d):
+    """matmul_q8_0_float_linalg.hlsl:40-101 for one token and one row, in the shader's own
+    steps with f32 arithmetic: per block part_hi, part_lo over the exact integers, then
+    total += (part_hi + part_lo) * scale."""
+    total = np.float32(0)
+    for b in range(len(d)):
+        part_hi = part_lo = np.float32(0)
+        for i in range(32 * b, 32 * b + 32):
+            hi = np.float16(x[i])
+            lo = np.float16(np.float32(x[i]) - np.float32(hi))
+            part_hi = np.float32(part_hi + np.float32(hi) * np.float32(q[i]))
+            part_lo = np.float32(part_lo + np.float32(lo) * np.float32(q[i]))
+        total = np.float32(total + np.float32(part_hi + part_lo) * np.float32(d[b]))
+    return float(total)
+
+
+def test_fp16_rungs_operand_contracts():
+    g = np.random.Generator(np.random.PCG64(0xF16))
+    k, n, rows = 96, 5, 3
+    q = g.integers(-128, 128, size=(n, k)).astype(np.int8)
+    d = (g.random((n, k // 32)) * 0.01 + 0.001).astype(np.float16)
+    w = (q.astype(np.float32).reshape(n, k // 32, 32) * d.astype(np.float32)[:, :, None]).reshape(n, k)
+    x = (g.standard_normal((rows, k)) * 3).astype(np.float32)
+    # Compensated, Q8_0: the shader's own loop (f32 steps) agrees to f32 rounding, and the
+    # result is the unrounded product to about 2^-22: a dropped residual, a rounded weight or
+    # a scale applied per product instead of per block would each show at 1e-4 or more.
+    got = oracle.prefill_fp16_compensated(x, w, exact_weights=True)
+    exact = x.astype(np.float64) @ w.astype(np.float64).T
+    scale = np.max(np.abs(exact))
+    for t in range(rows):
+        for j in range(n):
+            assert abs(_shader_q8_compensated(x[t], q[j], d[j]) - got[t, j]) <= 1e-6 * scale
+    assert np.max(np.abs(got - exact)) <= 1e-6 * scale
+    # Single: exactly the product of the f16-rounded operands; its distance from the exact
+    # product is the f16 rounding (2^-11 relative per operand), far above the compensated one's.
+    single = oracle.prefill_fp16_single(x, w)
+    x16, w16 = x.astype(np.float16).astype(np.float64), w.astype(np.float16).astype(np.float64)
+    assert np.array_equal(single, x16 @ w16.T)
+    assert 1e-5 * scale < np.max(np.abs(single - exact)) < 1e-2 * scale
+    # Stored halves: weights rounded to f16, activations compensated.
+    halves = oracle.prefill_fp16_compensated(x, w, exact_weights=False)
+    assert np.max(np.abs(halves - x.astype(np.float64) @ w16.T)) <= 1e-6 * scale
+    # Special values: hi + lo is exact for values with at most 22 significant bits in range,
+    # and anything beyond the f16 range is an infinity in both rungs.
+    v = np.array([[1.0 + 2.0 ** -11 + 2.0 ** -20], [70000.0], [-65520.0], [2.0 ** -30]], dtype=np.float32)  # one value a token
+    one = np.ones((1, 1), dtype=np.float32)
+    c = oracle.prefill_fp16_compensated(v, one, exact_weights=True)[:, 0]
+    assert c[0] == float(v[0, 0]) and np.isnan(c[1]) and np.isnan(c[2])  # inf + (-inf) residual
+    s = oracle.prefill_fp16_single(v, one)[:, 0]
+    assert s[0] == 1.0 + 2.0 ** -10 and np.isinf(s[1]) and s[2] == -np.inf and s[3] == float(np.float16(2.0 ** -30))
