@@ -232,14 +232,17 @@ struct DecBF16 {
     static const char *name() { return "matvec_bf16"; }
     static uint32_t row_bytes(uint32_t k) { return 2u * k; }
     __device__ static uint32_t xoff(uint32_t task, int h) { return 8u * task + 4u * h; }
-    __device__ static void decode(const uint8_t *row, uint32_t, uint32_t task, float (&w)[E]) {
-        const uint4 q = *reinterpret_cast<const uint4 *>(row + 16u * task);
+    // A task as loaded, and its eight weights.
+    __device__ static void expand(const uint4 &q, float (&w)[E]) {
         const uint32_t words[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             w[2 * e + 0] = __uint_as_float(words[e] << 16);
             w[2 * e + 1] = __uint_as_float(words[e] & 0xffff0000u);
         }
+    }
+    __device__ static void decode(const uint8_t *row, uint32_t, uint32_t task, float (&w)[E]) {
+        expand(*reinterpret_cast<const uint4 *>(row + 16u * task), w);
     }
 };
 
@@ -253,14 +256,16 @@ struct DecF16 {
     static const char *name() { return "matvec_f16"; }
     static uint32_t row_bytes(uint32_t k) { return 2u * k; }
     __device__ static uint32_t xoff(uint32_t task, int h) { return 8u * task + 4u * h; }
-    __device__ static void decode(const uint8_t *row, uint32_t, uint32_t task, float (&w)[E]) {
-        const uint4 q = *reinterpret_cast<const uint4 *>(row + 16u * task);
+    __device__ static void expand(const uint4 &q, float (&w)[E]) {
         const uint32_t words[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
         for (int e = 0; e < 4; e++) {
             w[2 * e + 0] = half_bits_to_float(words[e] & 0xffffu);
             w[2 * e + 1] = half_bits_to_float(words[e] >> 16);
         }
+    }
+    __device__ static void decode(const uint8_t *row, uint32_t, uint32_t task, float (&w)[E]) {
+        expand(*reinterpret_cast<const uint4 *>(row + 16u * task), w);
     }
 };
 

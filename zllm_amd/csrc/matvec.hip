@@ -15,11 +15,19 @@
 // (the reference's split invariant, matvec_quant.wgsl.hbs:14-18).
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "decode.cuh"
 #include "matvec_common.cuh"
 
 namespace zhip {
+
+// The 16-bit formats' tasks are eight weights against two neighbouring input vectors. Lanes
+// reading vector 2 task (then 2 task + 1) of a token would touch every other 16 bytes of LDS,
+// two lanes to a bank; their inputs are therefore staged with the even vectors first and the
+// odd ones behind them, so that each read covers consecutive vectors.
+template <class D> constexpr bool kSplitInputs = std::is_same<D, DecBF16>::value || std::is_same<D, DecF16>::value;
 
 template <class D, int MT>
 __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
@@ -44,10 +52,103 @@ __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
                 for (uint32_t i = tid; i < k4; i += 256u) dst[i] = make_float4(0.f, 0.f, 0.f, 0.f);
                 continue;
             }
-            stage_token(a, t0 + t, dst, red);
+            if constexpr (kSplitInputs<D>) stage_token(a, t0 + t, dst, red, [k4](uint32_t i) { return (i & 1u) * (k4 / 2u) + (i >> 1); });
+            else stage_token(a, t0 + t, dst, red);
         }
         __syncthreads();
 
+        if constexpr (kSplitInputs<D>) {
+            // The 16-bit formats: a wave walks (group, 64-task slice) positions with the next
+            // position's two 16-byte loads in flight while it multiplies the current one (past
+            // its last position the loads are clamped to a valid one and their data unused).
+            const uint32_t iters = (tasks + 63u) / 64u;
+            auto rows_of = [&](uint32_t g, uint32_t &j0, uint32_t &r1, bool &has1) {
+                j0 = pair ? g : 2u * g;
+                r1 = pair ? a.half + g : j0 + 1u;
+                has1 = pair || r1 < a.rows;
+            };
+            auto load_at = [&](uint32_t g, uint32_t it, uint4 &q0, uint4 &q1) {
+                uint32_t j0, r1;
+                bool has1;
+                rows_of(g < groups ? g : groups - 1u, j0, r1, has1);
+                const uint32_t task = lane + 64u * it, tk = task < tasks ? task : 0u;
+                q0 = *reinterpret_cast<const uint4 *>(a.w + (size_t)j0 * a.row_bytes + 16u * tk);
+                q1 = *reinterpret_cast<const uint4 *>(a.w + (size_t)(has1 ? r1 : j0) * a.row_bytes + 16u * tk);
+            };
+            float acc0[MT], acc1[MT];
+#pragma unroll
+            for (int t = 0; t < MT; t++) acc0[t] = acc1[t] = 0.f;
+            uint32_t g = gwave, it = 0;
+            uint4 c0, c1;
+            load_at(g, it, c0, c1);
+            while (g < groups) {
+                uint32_t ng = g, nit = it + 1u;
+                if (nit == iters) {
+                    nit = 0;
+                    ng = g + nwaves;
+                }
+                uint4 n0, n1;
+                load_at(ng, nit, n0, n1);
+                const uint32_t task = lane + 64u * it;
+                if (task < tasks) {
+                    float w0[D::E], w1[D::E];
+                    D::expand(c0, w0);
+                    D::expand(c1, w1);
+#pragma unroll
+                    for (int t = 0; t < MT; t++) {
+                        const float *xt = xs + (size_t)t * a.k;
+                        float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                        for (int h = 0; h < 2; h++) {
+                            const float4 v = *reinterpret_cast<const float4 *>(xt + 4u * ((uint32_t)h * (k4 / 2u) + task));
+                            const int b = 4 * h;
+                            s0 = fmaf(w0[b + 0], v.x, s0); s1 = fmaf(w1[b + 0], v.x, s1);
+                            s0 = fmaf(w0[b + 1], v.y, s0); s1 = fmaf(w1[b + 1], v.y, s1);
+                            s0 = fmaf(w0[b + 2], v.z, s0); s1 = fmaf(w1[b + 2], v.z, s1);
+                            s0 = fmaf(w0[b + 3], v.w, s0); s1 = fmaf(w1[b + 3], v.w, s1);
+                        }
+                        acc0[t] += s0;
+                        acc1[t] += s1;
+                    }
+                }
+                if (it + 1u == iters) {
+                    uint32_t j0, r1;
+                    bool has1;
+                    rows_of(g, j0, r1, has1);
+#pragma unroll
+                    for (int t = 0; t < MT; t++) {
+                        acc0[t] = wave_sum(acc0[t]);
+                        acc1[t] = wave_sum(acc1[t]);
+                    }
+                    if (lane == 0) {
+                        for (uint32_t t = 0; t < mt; t++) {
+                            const size_t o = (size_t)(t0 + t) * a.out_stride + a.col0 + j0;
+                            if (pair) {
+                                float v = silu_f(acc0[t]) * acc1[t];
+                                if (a.flags & FLAG_ACCUMULATE) v += a.out[o];
+                                a.out[o] = v;
+                            } else {
+                                float v = acc0[t];
+                                if (a.flags & FLAG_ACCUMULATE) v += a.out[o];
+                                a.out[o] = v;
+                                if (has1) {
+                                    float u = acc1[t];
+                                    if (a.flags & FLAG_ACCUMULATE) u += a.out[o + 1];
+                                    a.out[o + 1] = u;
+                                }
+                            }
+                        }
+                    }
+#pragma unroll
+                    for (int t = 0; t < MT; t++) acc0[t] = acc1[t] = 0.f;
+                }
+                c0 = n0;
+                c1 = n1;
+                g = ng;
+                it = nit;
+            }
+            continue;
+        }
         for (uint32_t g = gwave; g < groups; g += nwaves) {
             // The group's two weight rows and whether each exists.
             const uint32_t j0 = pair ? g : 2u * g;
@@ -204,14 +305,15 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     // Tokens per pass over the weights: as many as fit workgroup memory.
     const uint64_t row_lds = (uint64_t)p.k * 4u;
     const uint64_t max_lds = 160u * 1024u - 64u;
-    uint32_t mt = a.m >= 3 ? 4u : a.m;
+    uint32_t mt = a.m >= 5 ? 8u : a.m >= 3 ? 4u : a.m;
     while (mt > 1 && mt * row_lds > 65536u) mt >>= 1;
     if (mt * row_lds > max_lds) return fail(d, ZHIP_E_BAD_COMMAND, "%s: k = %u does not fit workgroup memory", D::name(), p.k);
     const uint32_t lds = (uint32_t)(mt * row_lds);
     switch (mt) {
     case 1: return run<D, 1>(d, a, lds);
     case 2: return run<D, 2>(d, a, lds);
-    default: return run<D, 4>(d, a, lds);
+    case 4: return run<D, 4>(d, a, lds);
+    default: return run<D, 8>(d, a, lds);
     }
 }
 
