@@ -552,6 +552,15 @@ def bench_c5(env):
     res["m1"] = env["hbm_entry"]("C5: bf16 lm_head matvec M=1 K=1024 N=151936", nbytes, wall, gpu_s, steps,
                                  {"copies": len(launches), "max_err_over_row_x_norms": bound, "max_err_over_max_want": rel,
                                   "argmax_equal": bool(int(np.argmax(got[0])) == oracle.argmax(want[0].astype(np.float32)))})
+    # M = 4 and 8: the widths of a speculative verify step, still the decode multiply.
+    for m in (4, 8):
+        xm = synth.activations(g, m, k, bf16=True)
+        launches, out = env["matvec_workload"](TensorType.bf16, wbits, n, k, m, False, xm)
+        wall, gpu_s = env["timed"](launches, max(1, steps // 2), max(1, env["args"].warmup // 20))
+        got = env["read"](out)[: m * n].reshape(m, n)
+        wantm = oracle.matmul_f64(xm, w)
+        res[f"m{m}"] = env["hbm_entry"](f"C5: bf16 lm_head matvec M={m} K=1024 N=151936", 2 * n * k + 4 * m * k + 4 * m * n, wall, gpu_s, max(1, steps // 2),
+                                        {"copies": len(launches), "max_err_over_max_want": float(np.max(np.abs(got - wantm)) / np.max(np.abs(wantm)))})
     # M = 128: the prefill multiply on the bf16 MFMA rung.
     rows = 128
     x = synth.activations(g, rows, k, bf16=True)
