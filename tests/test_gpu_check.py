@@ -261,6 +261,46 @@ def test_quant_matvec_mfma_variant(ctx, pair, rows, n, k):
         assert got[tk].tobytes() == c.read(single)[:stride].tobytes(), "a token's sums differ between a lone launch and a multi-token launch"
 
 
+@pytest.mark.parametrize("rows,n,k,col0,pad,accumulate", [
+    (8, 200, 1024, 3, 7, True),      # partial last tile, unaligned rows
+    (5, 96, 4096, 4, 8, False),      # aligned rows: 16-byte stores
+    (3, 100, 2080, 0, 0, True),      # k = 65 blocks: a ragged last step
+    (1, 530, 1024, 0, 2, False),     # one token
+    (8, 4112, 4096, 0, 0, False),    # 65 tiles of 64 rows
+])
+def test_matvec_q8_0_mfma_variant(ctx, rows, n, k, col0, pad, accumulate):
+    """The matrix-core variant of matvec_q8_0 (the id of a wave per sixteen rows): every
+    token within 1e-5 of float64 over the decoded weights whatever its magnitude (each token
+    is scaled by its own power of two), each token bitwise equal to its lone launch, nothing
+    outside the outputs touched."""
+    c = ctx
+    x = c.random(rows * k, 3).reshape(rows, k)
+    x[0] *= np.float32(1e-6)          # tokens of very different magnitudes, beyond the f16 range both ways
+    x[rows - 1] *= np.float32(3e6)
+    raw, values = quant_rows(c, TensorType.q8_0, n, k)
+    stride = n + pad
+    init = c.random(rows * stride, 2).reshape(rows, stride)
+    xa, wa = c.upload(x), c.gpu_weights(TensorType.q8_0, raw, k)
+    want = x.astype(np.float64) @ values.astype(np.float64).T + (init[:, col0 : col0 + n] if accumulate else 0)
+    p = lambda: P.MatvecBf16(n=n, k=k, col0=col0, out_stride=stride, accumulate=accumulate)
+    pipeline = c.set.matvec(c.rec, Kernel.matvec_q8_0, MFMA_VARIANT)
+    grid_x = K.div_ceil(n, MFMA_VARIANT.group_rows())
+    out = c.upload(init)
+    c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, wa], (grid_x, rows, 1))
+    got = c.read(out).reshape(rows, stride)
+    prod = x.astype(np.float64) @ values.astype(np.float64).T
+    for tk in range(rows):
+        # Against the product's own scale (an accumulated init may dwarf a tiny token's product).
+        assert np.max(np.abs(got[tk, col0 : col0 + n] - want[tk])) <= 1e-5 * max(np.max(np.abs(prod[tk])), 1e-30) + 1e-6 * np.max(np.abs(want[tk])), tk
+    mask = np.ones(stride, dtype=bool)
+    mask[col0 : col0 + n] = False
+    assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32))
+    for tk in range(rows):
+        single = c.upload(init[tk])
+        c.launcher().launch_pipeline(pipeline, p(), [c.upload(x[tk]), wa, single, wa], (grid_x, 1, 1))
+        assert got[tk].tobytes() == c.read(single)[:stride].tobytes(), "a token's sums differ between a lone launch and a multi-token launch"
+
+
 # ---- block decoders bit for bit, through the embedding gathers: check.zig:873-905 -----
 
 @pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q3_k, TensorType.q4_k, TensorType.q5_k, TensorType.q6_k])

@@ -57,6 +57,7 @@
 
 #include "common.h"
 #include "decode.cuh"
+#include "matvec_common.cuh"
 
 namespace zhip {
 
@@ -83,6 +84,7 @@ struct MfmaArgs {
     uint32_t row_bytes;
     uint32_t x_bytes, w_bytes;  // bytes the kernel may read behind x and w
     uint32_t x_plane;           // compensated rung: bytes from the activations' f16 values to their residuals
+    const float *token_scale;   // decode variant: what each token's sums are multiplied by at the end, or null
 };
 
 // Two floats to packed bf16, round to nearest even as the reference narrows
@@ -258,7 +260,7 @@ template <class W, int MT, bool COMP = false> constexpr int buf_bytes() { return
 template <class W, int MT, bool COMP = false> constexpr int lds_bytes() { return 3 * buf_bytes<W, MT, COMP>(); }
 // The exchange of the k quarters at the end reuses the buffers: 8 waves x 3 inboxes x MT / 4
 // tiles x 2 x 1 KB.
-static_assert(lds_bytes<WQ8_0, 8>() >= 8 * 3 * 2 * 2 * 1024 && lds_bytes<WQ8_0, 4>() >= 8 * 3 * 1 * 2 * 1024, "the exchange must fit the buffers");
+static_assert(lds_bytes<WQ8_0, 8>() >= 8 * 3 * 4 * 1024 && lds_bytes<WQ8_0, 4>() >= 8 * 3 * 2 * 1024 && lds_bytes<WQ8_0, 2, true>() >= 8 * 3 * 1024, "the exchange must fit the buffers");
 
 // COMP: the reference's compensated rung. Every activation enters twice, as its f16 value
 // and as the f16 of what that rounding left (two planes of the narrowed copy, two planes in
@@ -402,24 +404,25 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still land in LDS below
     __syncthreads();
 
-    // Add the four k quarters through LDS in one exchange: the wave of quarter q keeps token
-    // tiles OWN q .. + OWN - 1 of its 32 matrix rows and hands its sums of the other tiles to
-    // the waves that keep those; after one barrier every wave adds the four quarters of its
-    // tiles in a fixed order, (q0 + q2) + (q1 + q3), and stores them. The quarter is a
-    // constant in each copy of the code, so that the accumulators are indexed statically.
-    constexpr int OWN = MT / 4;
+    // Add the four k quarters through LDS in one exchange: of the wave's 2 MT tiles (tile
+    // 2 i + j: token tile i, weight tile j of its 32 matrix rows) the wave of quarter q keeps
+    // tiles OWN q .. + OWN - 1 and hands its sums of the others to the waves that keep those;
+    // after one barrier every wave adds the four quarters of its tiles in a fixed order,
+    // (q0 + q2) + (q1 + q3), and stores them. The quarter is a constant in each copy of the
+    // code, so that the accumulators are indexed statically.
+    constexpr int OWN = 2 * MT / 4;
+    static_assert(OWN >= 1 && 2 * MT % 4 == 0, "a quarter finishes a whole number of tiles");
     f32x4 *inbox = reinterpret_cast<f32x4 *>(lds);
-    // Where quarter `from` puts tile ii, j for the wave of quarter `owner` (from != owner).
-    auto slot = [&](uint32_t owner, uint32_t from, int ii, int j) {
-        return ((((owner * 2u + wn) * 3u + ((from + 3u - owner) & 3u)) * OWN + ii) * 2u + j) * 64u + lane;
+    // Where quarter `from` puts its tile number tt of those the wave of quarter `owner` keeps (from != owner).
+    auto slot = [&](uint32_t owner, uint32_t from, int tt) {
+        return (((owner * 2u + wn) * 3u + ((from + 3u - owner) & 3u)) * OWN + tt) * 64u + lane;
     };
     auto send = [&](auto quarter) __attribute__((always_inline)) {
         constexpr int Q = decltype(quarter)::value;
 #pragma unroll
-        for (int i = 0; i < MT; i++) {
-            if (i / OWN == Q) continue;
-#pragma unroll
-            for (int j = 0; j < 2; j++) inbox[slot(i / OWN, Q, i % OWN, j)] = acc[i][j];
+        for (int tile = 0; tile < 2 * MT; tile++) {
+            if (tile / OWN == Q) continue;
+            inbox[slot(tile / OWN, Q, tile % OWN)] = acc[tile / 2][tile % 2];
         }
     };
     // D[output][token] (the weights are the MFMA's first operand): the lane holds
@@ -429,16 +432,17 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
     auto collect = [&](auto quarter) __attribute__((always_inline)) {
         constexpr int Q = decltype(quarter)::value;
 #pragma unroll
-        for (int ii = 0; ii < OWN; ii++) {
-            const uint32_t t = t0 + 16u * (OWN * Q + ii) + lrow;
-#pragma unroll
-            for (int j = 0; j < 2; j++) {
+        for (int tt = 0; tt < OWN; tt++) {
+            {
+                const int tile = OWN * Q + tt, i = tile / 2, j = tile % 2;
+                const uint32_t t = t0 + 16u * i + lrow;
                 f32x4 p[4];
 #pragma unroll
-                for (int from = 0; from < 4; from++) p[from] = from == Q ? acc[OWN * Q + ii][j] : inbox[slot(Q, from, ii, j)];
+                for (int from = 0; from < 4; from++) p[from] = from == Q ? acc[i][j] : inbox[slot(Q, from, tt)];
                 f32x4 v = (p[0] + p[2]) + (p[1] + p[3]);
                 const uint32_t col = j0 + 32u * wn + 16u * j + 4u * g;
                 if (t >= a.rows || col >= a.n) continue;
+                if (a.token_scale) v *= a.token_scale[t];
                 float *o = a.out + (size_t)z * a.slice_stride + (size_t)t * a.out_stride + a.col0 + col;
                 if (aligned && col + 3u < a.n) {
                     f32x4 *o4 = reinterpret_cast<f32x4 *>(o);
@@ -490,6 +494,38 @@ __global__ __launch_bounds__(256) void narrow_split_kernel(const f32x4 *src, u32
         }
         hi_out[i] = hi;
         lo_out[i] = lo;
+    }
+}
+
+// The decode variant's activations: one workgroup a token. The token is scaled by a power of
+// two that brings its largest magnitude to [2^13, 2^14) (exact, and no value leaves the f16
+// range whatever the token's scale), then split like the compensated rung's; the inverse power
+// goes to scale_out[token] and multiplies the token's sums at the end.
+__global__ __launch_bounds__(256) void narrow_split_scaled_kernel(const float *x, uint32_t x_stride, uint32_t k, uint16_t *hi_out, uint16_t *lo_out, float *scale_out) {
+    __shared__ float red[4];
+    const uint32_t t = blockIdx.x, tid = threadIdx.x;
+    const float *row = x + (size_t)t * x_stride;
+    float big = 0.f;
+    for (uint32_t i = tid; i < k; i += 256u) big = fmaxf(big, fabsf(row[i]));
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) big = fmaxf(big, __shfl_xor(big, o));
+    if ((tid & 63u) == 0u) red[tid >> 6] = big;
+    __syncthreads();
+    big = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    int e = 0;
+    if (big > 0.f && big < __builtin_inff()) {
+        int ex;
+        (void)frexpf(big, &ex);  // big = m 2^ex, m in [0.5, 1)
+        e = 14 - ex;
+        e = e > 100 ? 100 : e < -100 ? -100 : e;
+    }
+    const float up = ldexpf(1.0f, e);
+    if (tid == 0) scale_out[t] = ldexpf(1.0f, -e);
+    for (uint32_t i = tid; i < k; i += 256u) {
+        const float v = row[i] * up;
+        const _Float16 h = (_Float16)v;
+        hi_out[(size_t)t * k + i] = __builtin_bit_cast(uint16_t, h);
+        lo_out[(size_t)t * k + i] = __builtin_bit_cast(uint16_t, (_Float16)__fsub_rn(v, (float)h));
     }
 }
 
@@ -608,5 +644,36 @@ zhip_result launch_matmul_q8_0_float_f16(const Dispatch &d) { return launch_mfma
 zhip_result launch_matmul_bf16_f16c(const Dispatch &d) { return launch_mfma<WBf16, false, F16, true>(d, "matmul_bf16", false, false); }
 zhip_result launch_matmul_f16_f16c(const Dispatch &d) { return launch_mfma<WF16, false, F16, true>(d, "matmul_f16", false, false); }
 zhip_result launch_matmul_q8_0_float_f16c(const Dispatch &d) { return launch_mfma<WQ8_0, false, F16, true>(d, "matmul_q8_0_float", true, true); }
+
+// The matrix-core variant of matvec_q8_0 for steps of several tokens (a speculative verify
+// step): the compensated arithmetic above on tiles of 32 tokens, every token scaled by its own
+// power of two first, so that the per-weight work is done once for all tokens of the step.
+// Validated arguments; no NORM / activation prologue and no SiLU pair (matvec.hip routes those
+// to the default kernel).
+zhip_result launch_matvec_q8_0_mfma(const Dispatch &d, const MvArgs &v) {
+    const char *name = "matvec_q8_0";
+    MfmaArgs a{};
+    a.rows = v.m; a.n = v.rows; a.k = v.k; a.col0 = v.col0; a.out_stride = v.out_stride;
+    a.accumulate = (v.flags & FLAG_ACCUMULATE) ? 1u : 0u;
+    a.k_slice = v.k;
+    a.row_bytes = v.row_bytes;
+    a.w = v.w;
+    a.out = v.out;
+    const uint64_t x_bytes = (uint64_t)v.m * v.k * 2u, w_bytes = (uint64_t)v.rows * v.row_bytes;
+    const uint64_t plane = (x_bytes + 255u) & ~(uint64_t)255u;
+    if (2u * plane >= (1ull << 32) || w_bytes >= (1ull << 32)) return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
+    if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", name);
+    if (zhip_result r = d.work->reserve(d, 2u * plane + (uint64_t)v.m * 4u)) return r;
+    float *scales = reinterpret_cast<float *>(d.work->data + 2u * plane);
+    hipLaunchKernelGGL(narrow_split_scaled_kernel, dim3(v.m), dim3(256), 0, d.stream, v.x, v.xr, v.k,
+        reinterpret_cast<uint16_t *>(d.work->data), reinterpret_cast<uint16_t *>(d.work->data + plane), scales);
+    a.x = d.work->data;
+    a.x_plane = (uint32_t)plane;
+    a.x_bytes = (uint32_t)(plane + x_bytes);
+    a.w_bytes = (uint32_t)w_bytes;
+    a.token_scale = scales;
+    const bool ragged = a.k % BK != 0;
+    return ragged ? launch_kernel<WQ8_0, F16, 2, true, true>(d, name, a, 1u) : launch_kernel<WQ8_0, F16, 2, false, true>(d, name, a, 1u);
+}
 
 }  // namespace zhip

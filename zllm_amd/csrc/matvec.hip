@@ -218,6 +218,8 @@ bool matvec_q4k_mfma_accepts(const MvArgs &a);
 zhip_result launch_matvec_q4k_mfma(const Dispatch &d, const MvArgs &a, uint64_t x_bytes, uint64_t w_bytes);
 bool matvec_q4k_mfma_resident_accepts(const MvArgs &a);
 zhip_result launch_matvec_q4k_mfma_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
+// The matrix-core variant of matvec_q8_0 (matmul_mfma.hip).
+zhip_result launch_matvec_q8_0_mfma(const Dispatch &d, const MvArgs &a);
 // The tuned multiply (matvec_quant.hip): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
 zhip_result launch_matvec_quant(const Dispatch &d, const MvArgs &a, int type);
 
@@ -299,6 +301,10 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
         return launch_matvec_q4k_mfma_resident(d, a, d.bind[2].size);
     if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && v.act_div == 0u && matvec_q4k_mfma_accepts(a))
         return launch_matvec_q4k_mfma(d, a, d.bind[1].size, d.bind[2].size);
+    // The same id on matvec_q8_0, without prologue or pair (a one-token step too, so that a
+    // token's bits do not depend on the step it ran in).
+    if (D::CHUNK == 8 && v.lanes == 64u && v.rows == 16u && v.act_div == 0u && !(p.flags & (FLAG_NORM | FLAG_SILU_PAIR)) && a.m <= 32u)
+        return launch_matvec_q8_0_mfma(d, a);
     // The tuned kernel takes rows of whole 64-weight tasks.
     if (D::CHUNK != 0 && p.k % 64u == 0) return launch_matvec_quant(d, a, D::CHUNK);
 
