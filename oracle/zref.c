@@ -782,7 +782,8 @@ int zref_quantize_q8(const float *x, size_t n, unsigned block, int8_t *q, float 
 
 /* src/ref/matmul.zig:197-247: a row rounded as the multiply will see it. */
 int zref_round_like_llama(int type, float *x, size_t n) {
-    if (type == ZREF_Q8_0 || type == ZREF_Q3_K || type == ZREF_Q4_K || type == ZREF_Q5_K || type == ZREF_Q6_K) {
+    if (type == ZREF_Q8_0 || type == ZREF_Q3_K || type == ZREF_Q4_K || type == ZREF_Q5_K || type == ZREF_Q6_K ||
+        type == ZREF_IQ4_XS) {
         unsigned block = type == ZREF_Q8_0 ? 32 : 256;
         int8_t *q = malloc(n);
         float *d = malloc((n / block + 1) * sizeof(float));

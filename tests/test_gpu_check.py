@@ -793,6 +793,43 @@ def test_quantize_q8_value_for_value(ctx, t):
     assert np.array_equal(got, oracle.round_like_llama(ORACLE_TYPE[t], x))
 
 
+def _llama_kats():
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "round_like_llama_kat.json")) as f:
+        return json.load(f)["cases"]
+
+
+@pytest.mark.parametrize("case", _llama_kats(), ids=lambda c: c["name"])
+def test_quantize_q8_reference_kats(ctx, case):
+    """The reference's own known answers for its activation rounding
+    (src/ref/matmul.zig:382-419) through the quantize_q8 kernel: integer times
+    scale must be the expected value (ties to even under both block sizes,
+    127 / amax before rounding, IQ4_XS weights take 256-wide blocks)."""
+    c = ctx
+    types = {"q8_0": TensorType.q8_0, "q4_k": TensorType.q4_k, "q6_k": TensorType.q6_k, "iq4_xs": TensorType.iq4_xs}
+    x = np.array(case["input"], dtype=np.uint32).view(np.float32)
+    block = K.act_block(types[case["type"]])
+    k = (x.size + 255) // 256 * 256  # the kernel rounds 256 values a wave; blocks of zeros follow
+    xp = np.zeros(k, dtype=np.float32)
+    xp[: x.size] = x
+    qx, dx = quantize_x(c, types[case["type"]], c.upload(xp), 1, k)
+    q, d = read_q8(c, qx, dx, 1, k)
+    got = (q.astype(np.float32) * np.repeat(d[:, : k // block], block, axis=1))[0, : x.size]
+    if "expect" in case:
+        first, want = case["expect"]["first"], np.array(case["expect"]["bits"], dtype=np.uint32)
+        part = got[first : first + want.size]
+        if case["expect"]["compare"] == "bits":
+            assert np.array_equal(part.view(np.uint32), want)
+        else:
+            assert np.array_equal(part, want.view(np.float32))
+    if "same_as_type" in case:
+        assert K.act_block(types[case["same_as_type"]]) == block
+        assert not np.array_equal(got, x)
+        assert np.array_equal(got.view(np.uint32), oracle.round_like_llama(ORACLE_TYPE[types[case["same_as_type"]]], x[None])[0].view(np.uint32))
+
+
 @pytest.mark.parametrize("mode", [1, 2])
 def test_quantize_q8_fused(ctx, mode):
     """quantize_q8 computing its input first (RMSNorm, SiLU pair): every value
@@ -862,6 +899,12 @@ def test_matmul_int8_whole_and_split(ctx, t):
     launch_int8(c, t, act, wa, odd, rows, n, k, 1, (3, 352))
     for out in (whole, split, odd):
         assert rel_err(c.read(out).reshape(rows, n), want) <= 1e-5
+    # The first slice alone (one slice in the grid) stops inside a 256-weight block.
+    alone = c.upload(init)
+    c.launcher().launch(K.weight_kernel("matmul", t), P.MatmulQuant(rows=rows, n=n, k=k, col0=0, out_stride=n, accumulate=1, k_slice=352),
+                        [act[0], wa, alone, act[1]], (K.div_ceil(n, K.matmul_quant_tile_n), K.div_ceil(rows, K.matmul_quant_tile_t), 1))
+    want_alone = init + xs[:, :352].astype(np.float64) @ values[:, :352].astype(np.float64).T
+    assert rel_err(c.read(alone).reshape(rows, n), want_alone) <= 1e-5
     block = K.act_block(t)
     q, d = oracle.quantize_q8(x, block)
     formula = init + oracle.matmul_q8(ORACLE_TYPE[t], raw, q, d, n)

@@ -19,7 +19,7 @@ ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 
 def test_library_exports_every_declared_symbol():
     header = open(os.path.join(ROOT, "include", "zllm_hip.h")).read()
-    declared = set(re.findall(r"\b(zhip_[a-z_]+)\s*\(", header))
+    declared = set(re.findall(r"\b(zhip_[a-z0-9_]+)\s*\(", header))
     assert declared == set(_lib.EXPORTS)
     for name in declared:
         assert getattr(_lib.lib, name) is not None

@@ -229,3 +229,36 @@ def test_fp16_rungs_operand_contracts():
     assert c[0] == float(v[0, 0]) and np.isnan(c[1]) and np.isnan(c[2])  # inf + (-inf) residual
     s = oracle.prefill_fp16_single(v, one)[:, 0]
     assert s[0] == 1.0 + 2.0 ** -10 and np.isinf(s[1]) and s[2] == -np.inf and s[3] == float(np.float16(2.0 ** -30))
+
+
+# ---- the reference's own known answers for its activation rounding (src/ref/matmul.zig:382-419) ----
+
+def llama_kats():
+    import json
+    import os
+
+    with open(os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "round_like_llama_kat.json")) as f:
+        return json.load(f)["cases"]
+
+
+KAT_TYPES = {"q8_0": oracle.Q8_0, "q4_k": oracle.Q4_K, "q6_k": oracle.Q6_K, "iq4_xs": oracle.IQ4_XS}
+
+
+@pytest.mark.parametrize("case", llama_kats(), ids=lambda c: c["name"])
+def test_round_like_llama_reference_kats(case):
+    """Ties to even under Q8_K and the x86 Q8_0 rule, 127 / amax (not 1 / (amax / 127))
+    before rounding, and IQ4_XS taking the Q8_K rule: expected bits as the
+    reference's tests state them."""
+    x = np.array(case["input"], dtype=np.uint32).view(np.float32)
+    got = oracle.round_like_llama(KAT_TYPES[case["type"]], x[None])[0]
+    if "expect" in case:
+        first, want = case["expect"]["first"], np.array(case["expect"]["bits"], dtype=np.uint32)
+        part = got[first : first + want.size]
+        if case["expect"]["compare"] == "bits":
+            assert np.array_equal(part.view(np.uint32), want)
+        else:
+            assert np.array_equal(part, want.view(np.float32))
+    if "same_as_type" in case:
+        other = oracle.round_like_llama(KAT_TYPES[case["same_as_type"]], x[None])[0]
+        assert not np.array_equal(got, x)
+        assert np.array_equal(got.view(np.uint32), other.view(np.uint32))

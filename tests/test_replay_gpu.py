@@ -247,3 +247,49 @@ def test_a_regrown_workspace_retires_the_graphs_that_pointed_into_it():
     finally:
         for d in devs:
             d.deinit()
+
+
+def test_a_parameter_block_written_by_a_kernel_of_the_step_is_not_replayed():
+    """A step whose first launch writes the parameter block of its second: a graph
+    would hold the block as the host last wrote it, so such a step always runs
+    launch by launch and gives the launched result."""
+    from zllm_amd import cmd
+
+    width, fillers = 128, 8
+    results = []
+    devs = [Device.open(0), Device.open(0, Device.NO_REPLAY)]
+    try:
+        for d in devs:
+            c = Ctx(d)
+            gu = synth.activations(synth.rng(0xD00), 1, 2 * width)
+            src, act = c.upload(gu), c.output(width)
+            staged = c.upload(np.frombuffer(P.SiluMul(width, width).pack(), dtype=np.uint8))
+            ub = c.rec.create_buffer(16, cmd.Usage.uniform | cmd.Usage.storage | cmd.Usage.copy_dst)
+            pipeline = c.set.pipelines[Kernel.silu_mul]
+            bg = K.bind_group(c.rec, pipeline, K.Arg(ub, 16), [src, act])
+            b = K.Builder(c.rec, c.set)
+            copy = b.add(Kernel.repad, P.Repad(1, 16, 16), [staged, K.Arg(ub, 16)], K.Grid.fixed_(K.elementwise(4)))
+            others = [b.add(Kernel.silu_mul, P.SiluMul(width, width), [src, c.output(width)], K.Grid.fixed_(K.elementwise(width))) for _ in range(fillers)]
+            b.finish()
+            c.flush()
+            outs = []
+            for step in range(4):
+                c.rec.write_buffer(ub, 0, np.frombuffer(P.SiluMul(1, 1).pack(), dtype=np.uint8))  # what a graph would keep
+                c.flush()
+                copy.record(c.rec, K.Extent(rows=1))
+                c.rec.dispatch(pipeline, K.elementwise(width), [bg])
+                for l in others:
+                    l.record(c.rec, K.Extent(rows=1))
+                outs.append(c.read(act).copy())
+                c.rec.clear_buffer(act.buffer, 0, 4 * width)
+                c.flush()
+            results.append(outs)
+            assert c.host.replayed_submits() == 0
+        g64 = gu[0, :width].astype(np.float64)
+        want = g64 / (1 + np.exp(-g64)) * gu[0, width:]
+        for got, eager in zip(*results):
+            assert np.array_equal(got, eager)
+            assert np.max(np.abs(got - want)) < 1e-5
+    finally:
+        for d in devs:
+            d.deinit()

@@ -446,6 +446,16 @@ size_t replayable_prefix(zhip_context *c) {
         const Entry &e = c->ops[i].group.e[0];
         const Buffer *ub = e.bound ? get(c->buffers, e.buffer) : nullptr;
         if (!ub || !ub->shadowed || ub->shadow_stale) return 0;
+        // A kernel of the prefix that writes a parameter buffer: a later dispatch would
+        // have to see the written values, and a captured launch holds the ones from before.
+        const Pipeline *pl = get(c->pipelines, c->ops[i].pipeline);
+        if (!pl || !pl->info) return 0;
+        for (uint32_t b = 1; b < 8; b++) {
+            const Entry &w = c->ops[i].group.e[b];
+            if (!w.bound || !(pl->info->writes >> b & 1u)) continue;
+            const Buffer *wb = get(c->buffers, w.buffer);
+            if (!wb || wb->shadowed) return 0;
+        }
     }
     return n;
 }
@@ -545,7 +555,7 @@ zhip_result find_replay(zhip_context *c, size_t count, zhip_context::Replay **ou
 }
 
 // Runs everything queued since the last submit, waits for it, completes reads.
-zhip_result submit(zhip_context *c) {
+zhip_result run_queue(zhip_context *c) {
     if (c->read_bytes > c->download_size) {
         if (c->download) (void)hipHostFree(c->download);
         c->download = nullptr;
@@ -628,11 +638,34 @@ zhip_result submit(zhip_context *c) {
     }
     for (const Read &rd : c->reads)
         if (rd.size > 0) memcpy(rd.dst, c->download + rd.staging_offset, rd.size);
-    c->ops.clear();
-    for (uint32_t id : c->released)
-        if (zhip_result r = release_buffer(c, id)) return r;
-    c->released.clear();
     return ZHIP_OK;
+}
+
+// A submit. When the queue fails part-way, what it had already started is still running
+// on the stream: wait for it (whatever that wait says) so that later writes and frees,
+// which do not order against the stream, cannot overtake it. Buffers destroyed while work
+// was queued are released on both paths; an id destroyed twice is released once.
+zhip_result submit(zhip_context *c) {
+    zhip_result result = run_queue(c);
+    std::string message;
+    if (result != ZHIP_OK) {
+        message = c->message;
+        (void)hipStreamSynchronize(c->stream);
+        (void)hipGetLastError();
+    }
+    c->ops.clear();
+    std::vector<uint32_t> released;
+    released.swap(c->released);
+    for (uint32_t id : released) {
+        if (!get(c->buffers, id)) continue;
+        const zhip_result r = release_buffer(c, id);
+        if (result == ZHIP_OK && r != ZHIP_OK) {
+            result = r;
+            message = c->message;
+        }
+    }
+    if (result != ZHIP_OK) c->message = message;
+    return result;
 }
 
 struct Command {

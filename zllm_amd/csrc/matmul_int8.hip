@@ -525,7 +525,7 @@ static zhip_result launch_int8(const Dispatch &d, const char *name, int type) {
     a.accumulate = p.accumulate; a.k_slice = p.k_slice; a.slice_stride = p.slice_stride; a.row_bytes = (uint32_t)row_bytes;
     a.qx_bytes = (uint32_t)x_need; a.w_bytes = (uint32_t)w_need; a.dx_bytes = (uint32_t)d_need;
     const dim3 grid((uint32_t)tiles_n, (uint32_t)tiles_t, (uint32_t)slices);
-    const bool ragged = p.k % STEP != 0 || (slices > 1 && p.k_slice % STEP != 0);
+    const bool ragged = p.k % STEP != 0 || (p.k_slice < p.k && p.k_slice % STEP != 0);
     if (type == 3) {
         hipLaunchKernelGGL(matmul_kquant_i8_kernel<I8Q3>, grid, dim3(256), 0, d.stream, a);
     } else if (type == 4) {
