@@ -140,6 +140,29 @@ zhip_result zhip_last_submit(zhip_context *context, uint64_t *out_ns, uint64_t *
  * ZHIP_OPTION_NO_REPLAY). No counterpart in the reference; for tests and reports. */
 zhip_result zhip_replayed_submits(zhip_context *context, uint64_t *out_count);
 
+/* No counterpart in the reference. For callers that cannot allocate device
+ * memory (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc): the multiply of a matmul_q8_0_float dispatch in this
+ * backend's bf16 rung (create_kernel variant 0xfffb0000: f32-bound activations,
+ * Q8_0 weights in split rows, bf16 matrix cores, fp32 accumulation), given as
+ * device pointers instead of a command stream, with the kernels' one scratch
+ * buffer (the bf16 copy of the step's activations, which zhip_execute keeps
+ * in a workspace it grows with hipMalloc) in a fixed array inside the library.
+ *   out[t * out_stride + col0 + j] (+)= sum_i x[t * k + i] * w[j][i],
+ *   t < rows, j < n; `accumulate` != 0 adds to what `out` holds.
+ * Asynchronous on `stream` (a hipStream_t; null = the null stream), which must
+ * belong to the context's device; the call allocates and frees nothing and
+ * does not synchronize. Results equal the dispatch's bit for bit. Limit:
+ * rows * k * 2 <= zhip_no_alloc_capacity() (8 MiB: 1024 tokens of 4096 inputs);
+ * more fails with ZHIP_E_BAD_COMMAND and a message. Every call on a GPU shares
+ * that GPU's one array: calls that overlap on one GPU (different streams or
+ * threads, or different contexts of one device) race. */
+zhip_result zhip_matmul_q8_0_float_no_alloc(zhip_context *context, void *stream, const float *x,
+    const void *weights, float *out, uint32_t rows, uint32_t n, uint32_t k, uint32_t col0,
+    uint32_t out_stride, uint32_t accumulate);
+/* Bytes of the fixed scratch array the call above narrows activations into. */
+uint64_t zhip_no_alloc_capacity(void);
+
 /* Replaces Device.errorMessage (src/gpu/host.zig:128-133; agility.h:108-109):
  * copies the last error message, NUL-terminated; returns its length. */
 size_t zhip_last_error(zhip_context *context, char *out, size_t capacity);

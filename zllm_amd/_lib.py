@@ -15,6 +15,7 @@ EXPORTS = (
     "zhip_create", "zhip_destroy", "zhip_get_caps", "zhip_supports_prefill", "zhip_set_file", "zhip_execute",
     "zhip_profile_start", "zhip_profile_stop", "zhip_profile_read", "zhip_last_submit", "zhip_replayed_submits", "zhip_last_error",
     "zhip_force_loss", "zhip_kernel_artifact", "zhip_backend_source", "zhip_kernel_ordinal",
+    "zhip_matmul_q8_0_float_no_alloc", "zhip_no_alloc_capacity",
 )
 
 
@@ -75,6 +76,10 @@ def _load() -> C.CDLL:
     lib.zhip_backend_source.argtypes = [C.c_char_p, C.c_char_p, C.c_size_t]
     lib.zhip_kernel_ordinal.restype = C.c_int32
     lib.zhip_kernel_ordinal.argtypes = [C.c_char_p]
+    lib.zhip_matmul_q8_0_float_no_alloc.restype = C.c_int32
+    lib.zhip_matmul_q8_0_float_no_alloc.argtypes = [ctx, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p] + [C.c_uint32] * 6
+    lib.zhip_no_alloc_capacity.restype = C.c_uint64
+    lib.zhip_no_alloc_capacity.argtypes = []
     return lib
 
 

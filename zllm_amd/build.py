@@ -11,7 +11,7 @@ CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libzllm_hip.so")
 
 SOURCES = ["host.cpp", "matvec.hip", "matvec_quant.hip", "matvec_mfma.hip", "matvec_mfma_resident.hip", "matmul_f32.hip", "matmul_mfma.hip", "matmul_mfma_wide.hip", "matmul_stream.hip", "matmul_int8.hip",
-           "quantize_q8.hip", "elementwise.hip"]
+           "quantize_q8.hip", "elementwise.hip", "no_alloc.hip"]
 HEADERS = ["common.h", "decode.cuh", "matvec_common.cuh", os.path.join("..", "..", "include", "zllm_hip.h")]
 
 # -packed-fp32-ops off: some packed-FP32 forms have given wrong results on the

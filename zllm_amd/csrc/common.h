@@ -71,7 +71,8 @@ struct Dispatch;
 struct Workspace {
     uint8_t *data = nullptr;
     uint64_t bytes = 0;
-    // Makes at least `want` bytes available.
+    bool fixed = false;  // memory the workspace does not own: never grown, never freed
+    // Makes at least `want` bytes available (fails on a fixed workspace that is too small).
     zhip_result reserve(const Dispatch &d, uint64_t want);
     void release();
 };
@@ -126,6 +127,13 @@ zhip_result launch_embed_iq4_xs(const Dispatch &);
 // Host-side helpers shared by the launchers.
 zhip_result fail(const Dispatch &d, zhip_result code, const char *fmt, ...);
 zhip_result check_launch(const Dispatch &d, const char *kernel);
+
+// The entry point that allocates nothing (no_alloc.hip): its fixed scratch array's address is
+// looked up once per device, with that device current.
+zhip_result no_alloc_setup(int device, const DeviceInfo &info);
+uint64_t no_alloc_capacity();
+zhip_result no_alloc_matmul_q8_0_float(int device, hipStream_t stream, const float *x, const void *w, float *out, uint32_t rows, uint32_t n,
+    uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, char *err, size_t err_cap);
 
 // Fills `words` 32-bit words at dst with `value` on the stream (clear_buffer;
 // also used instead of memset nodes so a captured stream stays replayable).

@@ -224,6 +224,7 @@ using namespace zhip;
 // running with the old one are waited for first.
 zhip_result Workspace::reserve(const Dispatch &d, uint64_t want) {
     if (want <= bytes) return ZHIP_OK;
+    if (fixed) return fail(d, ZHIP_E_BAD_COMMAND, "workspace: %llu bytes wanted, the fixed scratch holds %llu", (unsigned long long)want, (unsigned long long)bytes);
     const uint64_t size = (want + (8u << 20) - 1) & ~(uint64_t)((8u << 20) - 1);
     if (hipStreamSynchronize(d.stream) != hipSuccess) return fail(d, ZHIP_E_GPU, "workspace: stream synchronisation failed");
     if (data) (void)hipFree(data);
@@ -240,7 +241,7 @@ zhip_result Workspace::reserve(const Dispatch &d, uint64_t want) {
 }
 
 void Workspace::release() {
-    if (data) (void)hipFree(data);
+    if (data && !fixed) (void)hipFree(data);
     data = nullptr;
     bytes = 0;
 }
@@ -946,9 +947,30 @@ zhip_result zhip_create(const zhip_options *options, zhip_context **out_context)
         delete c;
         return ZHIP_E_GPU;
     }
+    // The device is current: the one place the fixed scratch array's address is looked up.
+    if (no_alloc_setup(index, c->info) != ZHIP_OK) {
+        (void)hipEventDestroy(c->ev_begin);
+        (void)hipEventDestroy(c->ev_end);
+        (void)hipStreamDestroy(c->stream);
+        delete c;
+        return ZHIP_E_GPU;
+    }
     *out_context = c;
     return ZHIP_OK;
 }
+
+zhip_result zhip_matmul_q8_0_float_no_alloc(zhip_context *c, void *stream, const float *x, const void *weights, float *out, uint32_t rows,
+    uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate) {
+    if (!c) return ZHIP_E_INVALID_ARGUMENT;
+    if (c->lost) return set_error(c, ZHIP_E_DEVICE_LOST, "device lost");
+    char err[384] = "";
+    const zhip_result r = no_alloc_matmul_q8_0_float(c->device, static_cast<hipStream_t>(stream), x, weights, out, rows, n, k, col0, out_stride,
+        accumulate, err, sizeof err);
+    if (r != ZHIP_OK) c->message = err[0] ? err : "matmul_q8_0_float (no allocation) failed";
+    return r;
+}
+
+uint64_t zhip_no_alloc_capacity(void) { return no_alloc_capacity(); }
 
 zhip_result zhip_destroy(zhip_context *c) {
     if (!c) return ZHIP_E_INVALID_ARGUMENT;
