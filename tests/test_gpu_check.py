@@ -524,6 +524,36 @@ def test_matmul_bf16_mfma_tilings(ctx, rows, n, k):
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
 
 
+def test_matmul_q8_0_float_bf16_whole_steps_keep_token_bits(ctx):
+    """Q8_0 weights on the bf16 rung with k a multiple of 128 take the kernel with
+    producer waves and 32 x 32 x 16 MFMAs in 128- or 64-token tiles: a token's sums
+    are the same bits whichever tile height its step runs in and whichever tokens
+    share the step; ragged rows and outputs, a column offset and a padded stride."""
+    c = ctx
+    rows, n, k, col0, stride = 300, 2830, 384, 3, 2840
+    x = c.random(rows * k, 1).reshape(rows, k)
+    raw, wq = quant_rows(c, TensorType.q8_0, n, k)
+    wa = c.gpu_weights(TensorType.q8_0, raw, k)
+    c.set.select_prefill(c.rec, K.Prefill.bf16_mfma)
+    init = c.random(rows * stride, 0.5).reshape(rows, stride)
+
+    def run(first, count):
+        out = c.upload(init[first : first + count])
+        c.launcher().launch(Kernel.matmul_q8_0_float, P.MatmulQuant(rows=count, n=n, k=k, col0=col0, out_stride=stride, accumulate=1, k_slice=k),
+                            [c.upload(x[first : first + count]), wa, out], (K.div_ceil(n, 64), K.div_ceil(count, 16), 1))
+        return c.read(out).reshape(count, stride)
+
+    got = run(0, rows)  # three 128-token tiles on 45 column tiles: the tall tiling
+    want = init[:, col0 : col0 + n] + synth.bf16_round(x).astype(np.float64) @ synth.bf16_round(wq).astype(np.float64).T
+    assert rel_err(got[:, col0 : col0 + n], want) <= 1e-5
+    mask = np.ones(stride, dtype=bool)
+    mask[col0 : col0 + n] = False
+    assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32)), "columns outside the chunk were written"
+    for first, count in ((0, 1), (1, 40), (41, 64), (105, 130), (235, 65)):  # 64-token tiles, and two tall tiles
+        assert got[first : first + count].tobytes() == run(first, count).tobytes(), "token chunking changed bits"
+    c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
+
+
 @pytest.mark.parametrize("rows,n,k,col0,pad,accumulate,packed", [
     (128, 16400, 1024, 0, 0, False, True),    # whole token tiles, vector stores
     (70, 16389, 768, 5, 9, True, False),      # ragged last weight tile, unaligned output: scalar stores
