@@ -520,6 +520,19 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     // are fetched. kDepth positions stay in flight ahead of the one multiplied
     // (deeper queues cost registers, hence occupancy, and measured no faster).
     constexpr int kDepth = 1;
+    // One-token steps load the token's inputs first (up to four vectors a thread: k <= 4096):
+    // loads complete in order within a wave, so behind the weights they would wait for them.
+    float4 xv[4], gv[4];
+    if (XREG) {
+        const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)q.t0 * a.xr);
+        const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t i = tid + 256u * j;
+            xv[j] = i < a.k / 4u ? xrow[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (a.flags & FLAG_NORM) gv[j] = i < a.k / 4u ? nw[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
     typename P::Raw buf[kDepth + 1][kRows];
     Cursor cc{gwave < units ? gwave : 0u, 0u, 0u, 0u, 0u};
     place(cc);
@@ -534,6 +547,39 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     float xsum[NSUM];
     // Stage the pass's tokens in task order, padded per task (coalesced loads;
     // a lane's own 64 inputs are 256 bytes apart from its neighbour's).
+    if (XREG) {
+        // The arithmetic of stage_token on the vectors already loaded, in the same order.
+        const uint32_t k4 = a.k / 4u;
+        float scale = 1.0f;
+        if (a.flags & FLAG_NORM) {
+            float ss = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (tid + 256u * j < k4) ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w;
+            ss = wave_sum(ss);
+            __syncthreads();
+            if (lane == 0) red[wave] = ss;
+            __syncthreads();
+            ss = (red[0] + red[1]) + (red[2] + red[3]);
+            scale = 1.0f / sqrtf(ss / (float)a.k + a.eps);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t i = tid + 256u * j;
+            if (i >= k4) continue;
+            float4 v = xv[j];
+            if (a.flags & FLAG_NORM) {
+                v.x = v.x * scale * gv[j].x; v.y = v.y * scale * gv[j].y;
+                v.z = v.z * scale * gv[j].z; v.w = v.w * scale * gv[j].w;
+            }
+            if (a.act_div > 0.f) {
+                v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
+                v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+            }
+            const uint32_t p = P::stage_index(i);
+            lds4[p + (p >> 4)] = v;
+        }
+    } else
     for (uint32_t t = 0; t < (uint32_t)MT; t++) {
         float4 *dst = lds4 + (size_t)t * tok_stride4;
         if (t < q.mt) {
