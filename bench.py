@@ -45,7 +45,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,c5,formats,replay for the 'also' section; 'none' skips it")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,c5,formats,replay,floor for the 'also' section; 'none' skips it")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run 4 plain elementwise copies (256 MiB read + 256 MiB written each) so a counter run has a kernel of known traffic to scale by")
@@ -64,6 +64,9 @@ def main() -> int:
             torch.add(a, 1.0, out=o)  # one elementwise kernel: reads 256 MiB, writes 256 MiB
         torch.cuda.synchronize()
         del a, o
+
+    only_early = [w for w in args.only.split(",") if w]
+    vendor_c4 = vendor_c4_context() if ("none" not in only_early and (not only_early or "c4" in only_early)) else None
 
     from zllm_amd import Device, Host, cmd, synth
     from zllm_amd import kernels as K
@@ -125,6 +128,32 @@ def main() -> int:
             ns, count = host.last_submit()
             assert count == n * per_step
         return wall, ns * 1e-9
+
+    def protocol(launches, per_step: int = 1):
+        """The tuner's timing protocol (src/tune/tune.zig:8-11,24-27) whatever --steps says:
+        batches of at least 200 back-to-back steps in one blocking submit (a whole number of
+        rotations over `launches`), 3 warm-up batches, then 7 timed ones; returns the median
+        batch as (wall seconds, GPU seconds from the host's stream events, steps in a batch).
+        Identical batches are replayed from a HIP graph from their second submit on, as the
+        host does for any repeated submit."""
+        n = -(-200 // len(launches)) * len(launches)
+        walls, gpus = [], []
+        for rep in range(3 + 7):
+            for i in range(n):
+                launches[i % len(launches)].record(rec, K.Extent(rows=launches[i % len(launches)].rows))
+            token[0] += 1
+            rec.submit(token[0])
+            words = rec.batch()
+            t0 = time.perf_counter()
+            host.execute(words, [])
+            wall = time.perf_counter() - t0
+            rec.clear()
+            ns, count = host.last_submit()
+            assert count == n * per_step
+            if rep >= 3:
+                walls.append(wall)
+                gpus.append(ns * 1e-9)
+        return float(np.median(walls)), float(np.median(gpus)), n
 
     class L:
         """A prebuilt launch and the token rows its grid resolves with."""
@@ -208,7 +237,8 @@ def main() -> int:
     x = synth.activations(g, 1, k)
     launches, out = matvec_workload(TensorType.q4_k, raw, n, k, 1, False, x)
     c2_bytes = n * K.row_bytes(TensorType.q4_k, k) + 4 * k + 4 * n  # 33,103,872
-    wall, gpu_s = timed(launches, args.steps, args.warmup)
+    wall, _ = timed(launches, args.steps, args.warmup)
+    _, p_gpu, p_steps = protocol(launches)
     got = read(out)[:n].reshape(1, n)
 
     import oracle  # the checker and the CPU baseline; never the measured path
@@ -259,12 +289,14 @@ def main() -> int:
         },
         "roofline": {
             "bound": "hbm",
-            "achieved": round(c2_bytes * args.steps / gpu_s / 1e9, 1),
+            "achieved": round(c2_bytes * p_steps / p_gpu / 1e9, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
-            "frac": round(c2_bytes * args.steps / gpu_s / 1e9 / HBM_PEAK_GBPS, 4),
+            "frac": round(c2_bytes * p_steps / p_gpu / 1e9 / HBM_PEAK_GBPS, 4),
             "traffic": C2_TRAFFIC_BYTES,
-            "us_per_launch": round(gpu_s / args.steps * 1e6, 3),
+            "traffic_source": "rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs of this command, profiles/matvec_quant_kernel_q4k_c2.txt",
+            "us_per_launch": round(p_gpu / p_steps * 1e6, 3),
+            "protocol": f"median of 7 batches of {p_steps} back-to-back launches after 3 warm-up batches, HIP events on the host's stream",
         },
         "cpu_baseline": cpu,
         "parity": {"max_err_over_row_x_norms": bound, "max_err_over_max_want": rel, "bound": 1e-3},
@@ -273,7 +305,7 @@ def main() -> int:
     only = [s for s in args.only.split(",") if s]
     also = {}
     if "none" not in only:
-        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c4_int8", bench_c4_int8), ("c5", bench_c5), ("formats", bench_formats), ("replay", bench_replay)):
+        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c4_int8", bench_c4_int8), ("c5", bench_c5), ("formats", bench_formats), ("replay", bench_replay), ("floor", bench_floor)):
             if not only or name in only:
                 try:
                     also[name] = fn(locals())
@@ -285,6 +317,35 @@ def main() -> int:
     return 0
 
 
+def vendor_c4_context():
+    """Context only: the vendor library's bf16 multiply of C4's shape over weights dequantised
+    beforehand (bf16 in, bf16 out; not this path's contract), same protocol. Runs before this
+    library opens the device (torch brings its own copy of the HIP runtime)."""
+    rows, k, n = 512, 4096, 4096
+    try:
+        import torch
+
+        tx = torch.randn(rows, k, device="cuda:0", dtype=torch.bfloat16)
+        tws = [torch.randn(n, k, device="cuda:0", dtype=torch.bfloat16) * 0.02 for _ in range(4)]
+        ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        ts = []
+        for rep in range(3 + 7):
+            ev0.record()
+            for i in range(200):
+                torch.matmul(tx, tws[i % 4].t())
+            ev1.record()
+            torch.cuda.synchronize()
+            if rep >= 3:
+                ts.append(ev0.elapsed_time(ev1) * 1e-3 / 200)
+        tt = float(np.median(ts))
+        del tx, tws
+        torch.cuda.empty_cache()
+        return {"what": "torch.matmul (hipBLASLt), bf16 x bf16 -> bf16, weights dequantised beforehand", "us_per_launch_gpu": round(tt * 1e6, 3),
+                "TFLOPs_gpu": round(2 * rows * n * k / tt / 1e12, 1), "mfma_frac": round(2 * rows * n * k / tt / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4)}
+    except Exception as e:  # context only
+        return {"error": f"{type(e).__name__}: {e}"}
+
+
 def bench_c1(env):
     """Q8_0 decode multiply M = 1, K = 1024, N = 3072."""
     synth, oracle, K, TensorType = env["synth"], env["oracle"], env["K"], env["TensorType"]
@@ -293,14 +354,54 @@ def bench_c1(env):
     raw = synth.q8_0_rows(g, n, k)
     x = synth.activations(g, 1, k)
     launches, out = env["matvec_workload"](TensorType.q8_0, raw, n, k, 1, False, x)
-    steps = env["args"].steps
-    wall, gpu_s = env["timed"](launches, steps, env["args"].warmup)
+    wall, gpu_s, steps = env["protocol"](launches)
     got = env["read"](out)[:n].reshape(1, n)
     w = oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k)
     bound, rel = env["check_matvec"](got, oracle.matmul_f64(x, w), w, x)
     nbytes = n * k // 32 * 34 + 4 * k + 4 * n  # GGUF bytes: 3,358,720
-    return env["hbm_entry"]("C1: Q8_0 decode matvec M=1 K=1024 N=3072", nbytes, wall, gpu_s, steps,
-                            {"copies": len(launches), "max_err_over_row_x_norms": bound, "max_err_over_max_want": rel})
+    e = env["hbm_entry"]("C1: Q8_0 decode matvec M=1 K=1024 N=3072, rotating over weight copies", nbytes, wall, gpu_s, steps,
+                         {"copies": len(launches), "max_err_over_row_x_norms": bound, "max_err_over_max_want": rel})
+    # The same launch over one copy: the weights stay in L2 (3.3 MB), what a benchmark that
+    # reuses its buffers sees.
+    hwall, hgpu, hsteps = env["protocol"](launches[:1])
+    e["hot"] = {"us_per_step_wall": round(hwall / hsteps * 1e6, 3), "us_per_launch_gpu": round(hgpu / hsteps * 1e6, 3),
+                "GBps_gpu": round(nbytes * hsteps / hgpu / 1e9, 1), "copies": 1}
+    return e
+
+
+def bench_floor(env):
+    """What the machine gives a plain copy through the same command stream: copy_buffer of
+    33 MB (the headline's weight bytes) and 311 MB (the lm_head's), rotating over distinct
+    sources beyond the Infinity Cache, batches of back-to-back copies in one blocking submit,
+    median of 7 batches after 3 warm-ups. A copy reads and writes its size."""
+    rec, host, token, cmd = env["rec"], env["host"], env["token"], env["cmd"]
+
+    res = {}
+    for name, size in (("33MB", 14336 * 2304), ("311MB", 151936 * 1024 * 2)):
+        copies = env["rotation"](size)
+        srcs = [env["output"](size) for _ in range(copies)]
+        dst = env["output"](size)
+        for sbuf in srcs:
+            rec.clear_buffer(sbuf.buffer, 0, size)
+        env["flush"]()
+        n = -(-200 // copies) * copies if size < (100 << 20) else 10 * copies
+        gpus = []
+        for rep in range(3 + 7):
+            for i in range(n):
+                rec.copy_buffer(srcs[i % copies].buffer, 0, dst.buffer, 0, size)
+            token[0] += 1
+            rec.submit(token[0])
+            host.execute(rec.batch(), [])
+            rec.clear()
+            if rep >= 3:
+                gpus.append(host.last_submit()[0] * 1e-9)
+        t = float(np.median(gpus)) / n
+        res[name] = {"bytes_copied": size, "us_per_copy": round(t * 1e6, 3), "GBps_read_plus_write": round(2 * size / t / 1e9, 1),
+                     "GBps_read": round(size / t / 1e9, 1), "sources": copies, "copies_per_batch": n}
+        for sbuf in srcs + [dst]:
+            rec.destroy(cmd.Kind.buffer, sbuf.buffer)
+        env["flush"]()
+    return res
 
 
 def bench_replay(env):
@@ -366,13 +467,12 @@ def bench_formats(env):
     synth, oracle, K, TensorType = env["synth"], env["oracle"], env["K"], env["TensorType"]
     n, k = 14336, 4096
     x = synth.activations(synth.rng(0xF0), 1, k)
-    steps = max(1, env["args"].steps // 2)
     res = {}
     for name, ot in (("q8_0", oracle.Q8_0), ("q6_k", oracle.Q6_K), ("q5_k", oracle.Q5_K), ("q3_k", oracle.Q3_K)):
         t = TensorType[name]
         raw = synth.random_blocks(synth.rng(0xF1), name, n, k)
         launches, out = env["matvec_workload"](t, raw, n, k, 1, False, x)
-        wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 2))
+        wall, gpu_s, steps = env["protocol"](launches)
         got = env["read"](out)[:n].reshape(1, n)
         w = oracle.dequantize(ot, raw, n * k).reshape(n, k)
         bound, rel = env["check_matvec"](got, oracle.matmul_f64(x, w), w, x)
@@ -391,7 +491,6 @@ def bench_c3(env):
     up = synth.q4_k_rows(synth.rng(0xC3B), n, k)
     raw = np.concatenate([gate, up])
     w = oracle.dequantize(oracle.Q4_K, raw, 2 * n * k).reshape(2 * n, k)
-    steps = max(1, env["args"].steps // 2)
     res = {}
     # The default variant, and for the multi-token steps the matrix-core variant
     # (MatvecVariant wg 512, lanes 64, rows 16) a tuner would pick for them.
@@ -400,7 +499,7 @@ def bench_c3(env):
                             (8, K.MatvecVariant(wg=512, lanes=64, rows=16), "m8_matrix_cores")):
         x = synth.activations(synth.rng(0xC30 + m), m, k)
         launches, out = env["matvec_workload"](TensorType.q4_k, raw, n, k, m, True, x, variant)
-        wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 2))
+        wall, gpu_s, steps = env["protocol"](launches)
         got = env["read"](out)[: m * n].reshape(m, n).astype(np.float64)
         both = oracle.matmul_f64(x, w)
         gt, u = both[:, :n], both[:, n:]
@@ -434,8 +533,7 @@ def bench_c4(env):
         launches.append(env["L"](b.add(K.Kernel.matmul_q8_0_float, p, [xa, wa, out], K.Grid.tiles_y(K.div_ceil(n, 64), 16)), rows))
     b.finish()
     env["flush"]()
-    steps = max(1, env["args"].steps // 4)
-    wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 4))
+    wall, gpu_s, steps = env["protocol"](launches)
     got = env["read"](out)[: rows * n].reshape(rows, n).astype(np.float64)
     w = oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k)
     want = x.astype(np.float64) @ w.astype(np.float64).T
@@ -450,18 +548,19 @@ def bench_c4(env):
             rl.append(env["L"](b.add(K.Kernel.matmul_q8_0_float, P.MatmulQuant(rows=rows, n=n, k=k, col0=0, out_stride=n, k_slice=k), [xf, wa, out], K.Grid.tiles_y(K.div_ceil(n, 64), 16)), rows))
         b.finish()
         env["flush"]()
-        rsteps = max(4, env["args"].steps // share)
-        _, rgpu = env["timed"](rl, rsteps, max(1, rsteps // 10))
+        _, rgpu, rsteps = env["protocol"](rl)
         rgot = env["read"](out)[: rows * n].reshape(rows, n).astype(np.float64)
         ladder[rung.name] = {"us_per_launch_gpu": round(rgpu / rsteps * 1e6, 3), "TFLOPs_gpu": round(2 * rows * n * k * rsteps / rgpu / 1e12, 1),
                              "max_err_over_max_want": float(np.max(np.abs(rgot - want)) / np.max(np.abs(want)))}
     kset.select_prefill(rec, K.Prefill.scalar_f32)
+    vendor = env.get("vendor_c4")
     wn = np.linalg.norm(w.astype(np.float64), axis=1)
     xn = np.linalg.norm(x.astype(np.float64), axis=1)
     bound = float(np.max(np.abs(got - want) / (xn[:, None] * wn[None, :])))
     flops = 2 * rows * n * k
     return {
-        "workload": "C4: Q8_0 prefill matmul M=512 K=4096 N=4096, bf16 activations (bound as packed bf16), bf16 MFMA, fp32 accumulate",
+        "workload": "C4: Q8_0 prefill matmul M=512 K=4096 N=4096, bf16 activations (bound as packed bf16), bf16 MFMA, fp32 accumulate; "
+                    "rotating over 4 weight copies (71 MB: within the 256 MB Infinity Cache, the kernel is bound by the path into the CUs, not by HBM)",
         "flops_per_step": flops,
         "us_per_step_wall": round(wall / steps * 1e6, 3),
         "us_per_launch_gpu": round(gpu_s / steps * 1e6, 3),
@@ -471,6 +570,7 @@ def bench_c4(env):
         "max_err_over_row_x_norms": bound,
         "max_err_over_max_want": float(np.max(np.abs(got - want)) / np.max(np.abs(want))),
         "reference_ladder_f32_activations": ladder,
+        "vendor_library_context": vendor,
     }
 
 
@@ -506,8 +606,7 @@ def bench_c4_int8(env):
             launches.append(env["Chain"]([quant, mul], rows))
         b.finish()
         env["flush"]()
-        steps = max(1, env["args"].steps // 4)
-        wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 4), per_step=2)
+        wall, gpu_s, steps = env["protocol"](launches, per_step=2)
         got = env["read"](out)[: rows * n].reshape(rows, n).astype(np.float64)
         w = oracle.dequantize(otype, raw, n * k).reshape(n, k)
         xs = oracle.round_like_llama(otype, x)
@@ -540,11 +639,10 @@ def bench_c5(env):
     wbits = synth.bf16_matrix(g, n, k, 0.02)
     w = synth.bf16_bits_to_f32(wbits)
     res = {}
-    steps = max(1, env["args"].steps // 10)
     # M = 1: the decode multiply.
     x = synth.activations(g, 1, k, bf16=True)
     launches, out = env["matvec_workload"](TensorType.bf16, wbits, n, k, 1, False, x)
-    wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 10))
+    wall, gpu_s, steps = env["protocol"](launches)
     got = env["read"](out)[:n].reshape(1, n)
     want = oracle.matmul_f64(x, w)
     bound, rel = env["check_matvec"](got, want, w, x)
@@ -556,30 +654,33 @@ def bench_c5(env):
     for m in (4, 8):
         xm = synth.activations(g, m, k, bf16=True)
         launches, out = env["matvec_workload"](TensorType.bf16, wbits, n, k, m, False, xm)
-        wall, gpu_s = env["timed"](launches, max(1, steps // 2), max(1, env["args"].warmup // 20))
+        wall, gpu_s, steps = env["protocol"](launches)
         got = env["read"](out)[: m * n].reshape(m, n)
         wantm = oracle.matmul_f64(xm, w)
-        res[f"m{m}"] = env["hbm_entry"](f"C5: bf16 lm_head matvec M={m} K=1024 N=151936", 2 * n * k + 4 * m * k + 4 * m * n, wall, gpu_s, max(1, steps // 2),
+        res[f"m{m}"] = env["hbm_entry"](f"C5: bf16 lm_head matvec M={m} K=1024 N=151936", 2 * n * k + 4 * m * k + 4 * m * n, wall, gpu_s, steps,
                                         {"copies": len(launches), "max_err_over_max_want": float(np.max(np.abs(got - wantm)) / np.max(np.abs(wantm)))})
     # M = 128: the prefill multiply on the bf16 MFMA rung.
     rows = 128
     x = synth.activations(g, rows, k, bf16=True)
     kset.select_prefill(rec, K.Prefill.bf16_mfma_xbf16)
     xa = env["upload"](synth.to_bf16_bits(x))
-    wa = env["upload"](wbits)
     out = env["output"](4 * rows * n)
     p = P.MatmulBf16(rows=rows, n=n, k=k, col0=0, out_stride=n)
-    launches = [env["L"](b.add(K.Kernel.matmul_bf16, p, [xa, wa, out], K.Grid.tiles_y(K.div_ceil(n, 64), 16)), rows)]
+    copies = env["rotation"](2 * n * k)  # three copies: 934 MB, beyond the Infinity Cache
+    launches = []
+    for _ in range(copies):
+        wa = env["upload"](wbits)
+        launches.append(env["L"](b.add(K.Kernel.matmul_bf16, p, [xa, wa, out], K.Grid.tiles_y(K.div_ceil(n, 64), 16)), rows))
     b.finish()
     env["flush"]()
-    wall, gpu_s = env["timed"](launches, steps, max(1, env["args"].warmup // 10))
+    wall, gpu_s, steps = env["protocol"](launches)
     got = env["read"](out)[: rows * n].reshape(rows, n)
     kset.select_prefill(rec, K.Prefill.scalar_f32)
     want = oracle.matmul_f64(x, w)
     rel = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
     nbytes = 2 * n * k + 2 * rows * k + 4 * rows * n
     res["m128"] = env["hbm_entry"]("C5: bf16 lm_head matmul M=128 K=1024 N=151936 (bf16 MFMA)", nbytes, wall, gpu_s, steps,
-                                   {"copies": 1, "max_err_over_max_want": rel,
+                                   {"copies": copies, "max_err_over_max_want": rel,
                                     "argmax_rows_equal": int(np.count_nonzero(np.argmax(got, axis=1) == np.argmax(want, axis=1))), "rows": rows})
     return res
 
