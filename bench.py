@@ -179,7 +179,7 @@ def main() -> int:
     def rotation(w_bytes: int) -> int:
         return max(2, -(-ROTATE_BYTES // w_bytes))
 
-    def matvec_workload(t: TensorType, raw_rows: np.ndarray, n_out: int, k: int, m: int, pair: bool, x: np.ndarray, variant=None):
+    def matvec_workload(t: TensorType, raw_rows: np.ndarray, n_out: int, k: int, m: int, pair: bool, x: np.ndarray, variant=None, norm_w=None, eps=1e-6):
         """Uploads a rotation of weight copies and builds one launch per copy."""
         kernel = K.weight_kernel("matvec", t)
         rb = K.row_bytes(t, k)
@@ -200,11 +200,12 @@ def main() -> int:
                 wa = K.Arg(buf, src.size)
             first = first or wa
             v = variant or K.MatvecVariant()
-            p = P.MatvecBf16(n=n_out, k=k, col0=0, out_stride=n_out, silu_pair=pair, half=n_out if pair else 0)
+            p = P.MatvecBf16(n=n_out, k=k, col0=0, out_stride=n_out, eps=eps if norm_w is not None else 0.0, norm=norm_w is not None, silu_pair=pair, half=n_out if pair else 0)
+            na = upload(norm_w) if norm_w is not None else wa
             if K.is_half(t):
-                launches.append(L(b.add(kernel, p, [xa, wa, out, wa], K.Grid.rows_y(K.div_ceil(n_out, K.matvec_rows))), m))
+                launches.append(L(b.add(kernel, p, [xa, wa, out, na], K.Grid.rows_y(K.div_ceil(n_out, K.matvec_rows))), m))
             else:
-                launches.append(L(b.add_matvec(kernel, v, p, [xa, wa, out, wa], K.Grid.rows_y(K.div_ceil(n_out, v.group_rows()))), m))
+                launches.append(L(b.add_matvec(kernel, v, p, [xa, wa, out, na], K.Grid.rows_y(K.div_ceil(n_out, v.group_rows()))), m))
         b.finish()
         flush()
         return launches, out
@@ -494,19 +495,24 @@ def bench_c3(env):
     res = {}
     # The default variant, and for the multi-token steps the matrix-core variant
     # (MatvecVariant wg 512, lanes 64, rows 16) a tuner would pick for them.
-    for m, variant, tag in ((1, None, "m1"), (4, None, "m4"), (8, None, "m8"),
-                            (4, K.MatvecVariant(wg=512, lanes=64, rows=16), "m4_matrix_cores"),
-                            (8, K.MatvecVariant(wg=512, lanes=64, rows=16), "m8_matrix_cores")):
+    mc = K.MatvecVariant(wg=512, lanes=64, rows=16)
+    nw = synth.activations(synth.rng(0xC3F), 1, k).reshape(-1)
+    for m, variant, tag, norm in ((1, None, "m1", False), (4, None, "m4", False), (8, None, "m8", False),
+                                  (4, mc, "m4_matrix_cores", False), (8, mc, "m8_matrix_cores", False),
+                                  (1, None, "m1_norm", True), (4, mc, "m4_matrix_cores_norm", True), (8, mc, "m8_matrix_cores_norm", True)):
         x = synth.activations(synth.rng(0xC30 + m), m, k)
-        launches, out = env["matvec_workload"](TensorType.q4_k, raw, n, k, m, True, x, variant)
+        launches, out = env["matvec_workload"](TensorType.q4_k, raw, n, k, m, True, x, variant, nw if norm else None)
         wall, gpu_s, steps = env["protocol"](launches)
         got = env["read"](out)[: m * n].reshape(m, n).astype(np.float64)
-        both = oracle.matmul_f64(x, w)
+        xin = x.astype(np.float64)
+        if norm:
+            xin = xin / np.sqrt(np.mean(xin * xin, axis=1, keepdims=True) + 1e-6) * nw.astype(np.float64)
+        both = xin @ w.astype(np.float64).T
         gt, u = both[:, :n], both[:, n:]
         want = gt / (1 + np.exp(-gt)) * u
         rel = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
         nbytes = 2 * n * K.row_bytes(TensorType.q4_k, k) + m * 4 * k + m * 4 * n
-        name = f"C3: fused gate+up Q4_K + SiLU*mul, M={m}, K=4096, N=2x14336" + (", matrix-core variant" if variant else "")
+        name = f"C3: fused gate+up Q4_K + SiLU*mul, M={m}, K=4096, N=2x14336" + (", matrix-core variant" if variant else "") + (", RMSNorm prologue as the planner's FFN launch has" if norm else "")
         res[tag] = env["hbm_entry"](name, nbytes, wall, gpu_s, steps, {"copies": len(launches), "max_err_over_max_want": rel})
     return res
 

@@ -21,19 +21,20 @@ from zllm_amd.kernels import Kernel, TensorType, params as P
 pytestmark = pytest.mark.gpu
 
 
-def decode_matvec(c, t, raw, n, k, x, pair=False, m=None, variant=None):
+def decode_matvec(c, t, raw, n, k, x, pair=False, m=None, variant=None, norm_w=None, eps=0.0):
     m = x.shape[0] if m is None else m
     wa = c.gpu_weights(t, raw, k)
     out = c.output(m * n)
     kernel = K.weight_kernel("matvec", t)
     v = variant or K.MatvecVariant()
     rows_per_group = K.matvec_rows if K.is_half(t) else v.group_rows()
-    p = P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, silu_pair=pair, half=n if pair else 0)
+    p = P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, eps=eps, norm=norm_w is not None, silu_pair=pair, half=n if pair else 0)
     grid = (K.div_ceil(n, rows_per_group), m, 1)
+    na = c.upload(norm_w) if norm_w is not None else wa
     if variant is None:
-        c.launcher().launch(kernel, p, [c.upload(x), wa, out, wa], grid)
+        c.launcher().launch(kernel, p, [c.upload(x), wa, out, na], grid)
     else:
-        c.launcher().launch_pipeline(c.set.matvec(c.rec, kernel, variant), p, [c.upload(x), wa, out, wa], grid)
+        c.launcher().launch_pipeline(c.set.matvec(c.rec, kernel, variant), p, [c.upload(x), wa, out, na], grid)
     return c.read(out)[: m * n].reshape(m, n)
 
 
@@ -88,24 +89,30 @@ def test_c3_fused_gate_up_silu(ctx, m):
             assert got[t].tobytes() == decode_matvec(ctx, TensorType.q4_k, raw, n, k, x[t : t + 1], pair=True)[0].tobytes()
 
 
+@pytest.mark.parametrize("norm", [False, True])
 @pytest.mark.parametrize("m", [4, 8])
-def test_c3_fused_gate_up_silu_matrix_core_variant(ctx, m):
+def test_c3_fused_gate_up_silu_matrix_core_variant(ctx, m, norm):
     """The same step on the matrix-core variant (MatvecVariant wg 512, lanes 64,
     rows 16): within 1e-5 of float64 row by row, every row bitwise equal to its
-    own one-token launch on the same variant."""
-    n, k = 14336, 4096
+    own one-token launch on the same variant; with and without the RMSNorm
+    prologue the planner's FFN launch carries (src/plan/qwen35.zig:1048)."""
+    n, k, eps = 14336, 4096, 1e-6
     variant = K.MatvecVariant(wg=512, lanes=64, rows=16)
     raw = np.concatenate([synth.q4_k_rows(synth.rng(0xC3A), n, k), synth.q4_k_rows(synth.rng(0xC3B), n, k)])
     x = synth.activations(synth.rng(0xC30 + m), m, k)
-    got = decode_matvec(ctx, TensorType.q4_k, raw, n, k, x, pair=True, variant=variant)
-    both = oracle.matmul_f64(x, oracle.Matrix(oracle.Q4_K, raw, 2 * n, k).rows())
+    nw = synth.activations(synth.rng(0xC3F), 1, k).reshape(-1) if norm else None
+    got = decode_matvec(ctx, TensorType.q4_k, raw, n, k, x, pair=True, variant=variant, norm_w=nw, eps=eps)
+    xin = x.astype(np.float64)
+    if norm:
+        xin = xin / np.sqrt(np.mean(xin * xin, axis=1, keepdims=True) + eps) * nw.astype(np.float64)
+    both = xin @ oracle.Matrix(oracle.Q4_K, raw, 2 * n, k).rows().astype(np.float64).T
     gate, up = both[:, :n], both[:, n:]
     with np.errstate(over="ignore"):
         want = gate / (1 + np.exp(-gate)) * up
     for t in range(m):
         assert rel_err(got[t], want[t]) <= 1e-5, t
     for t in (0, m - 1):
-        assert got[t].tobytes() == decode_matvec(ctx, TensorType.q4_k, raw, n, k, x[t : t + 1], pair=True, variant=variant)[0].tobytes()
+        assert got[t].tobytes() == decode_matvec(ctx, TensorType.q4_k, raw, n, k, x[t : t + 1], pair=True, variant=variant, norm_w=nw, eps=eps)[0].tobytes()
 
 
 @pytest.mark.parametrize("rung", [K.Prefill.bf16_mfma, K.Prefill.bf16_mfma_xbf16, K.Prefill.scalar_f32])

@@ -225,29 +225,39 @@ MFMA_VARIANT = K.MatvecVariant(wg=512, lanes=64, rows=16)
     (True, 3, 64, 2048),      # one block a wave
     (False, 2, 48, 2048),
 ])
-def test_quant_matvec_mfma_variant(ctx, pair, rows, n, k):
+@pytest.mark.parametrize("prologue", ["plain", "norm", "norm_act"])
+def test_quant_matvec_mfma_variant(ctx, pair, rows, n, k, prologue):
     """The matrix-core variant of matvec_q4_k (a wave per sixteen rows): every
     row within 1e-5 of float64 over the decoded weights, each token bitwise
-    equal to its lone launch, and nothing outside the outputs touched."""
+    equal to its lone launch, and nothing outside the outputs touched; also
+    with the prologues the planner's launches carry (RMSNorm times its weights
+    on every projection, src/plan/qwen35.zig:1006,1048, and silu(x / act_div))."""
     c = ctx
+    norm, div, eps = prologue != "plain", 4 if prologue == "norm_act" else 0, 1e-6
     x = c.random(rows * k, 3).reshape(rows, k)
     x[0] *= np.float32(1e-4)          # tokens of very different magnitudes
     x[rows - 1] *= np.float32(300.0)
+    nw = c.random(k, 1.5)
     raw, values = quant_rows(c, TensorType.q4_k, 2 * n if pair else n, k)
     stride = n + 7
     init = c.random(rows * stride, 2).reshape(rows, stride)
     xa, wa = c.upload(x), c.gpu_weights(TensorType.q4_k, raw, k)
-    v64, x64 = values.astype(np.float64), x.astype(np.float64)
+    na = c.upload(nw) if norm else wa
+    v64 = values.astype(np.float64)
+    x64 = np.stack([norm_row(r, nw if norm else None, eps) for r in x])
+    if div:
+        x64 = (x64 / div) * sigmoid64(x64 / div)
     if pair:
         g, u = x64 @ v64[:n].T, x64 @ v64[n:].T
         want = g * sigmoid64(g) * u
     else:
         want = init[:, 3 : 3 + n] + x64 @ v64.T
-    p = lambda: P.MatvecBf16(n=n, k=k, col0=3, out_stride=stride, accumulate=not pair, silu_pair=pair, half=n if pair else 0)
-    pipeline = c.set.matvec(c.rec, Kernel.matvec_q4_k, MFMA_VARIANT)
-    grid_x = K.div_ceil(n, MFMA_VARIANT.group_rows())
+    p = lambda: P.MatvecBf16(n=n, k=k, col0=3, out_stride=stride, eps=eps, norm=norm, accumulate=not pair, silu_pair=pair, half=n if pair else 0)
+    variant = K.MatvecVariant(MFMA_VARIANT.wg, MFMA_VARIANT.lanes, MFMA_VARIANT.rows, div)
+    pipeline = c.set.matvec(c.rec, Kernel.matvec_q4_k, variant)
+    grid_x = K.div_ceil(n, variant.group_rows())
     out = c.upload(init)
-    c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, wa], (grid_x, rows, 1))
+    c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, na], (grid_x, rows, 1))
     got = c.read(out).reshape(rows, stride)
     # Row by row: each token against its own output scale.
     for tk in range(rows):
@@ -257,7 +267,7 @@ def test_quant_matvec_mfma_variant(ctx, pair, rows, n, k):
     assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32))
     for tk in range(rows):
         single = c.upload(init[tk])
-        c.launcher().launch_pipeline(pipeline, p(), [c.upload(x[tk]), wa, single, wa], (grid_x, 1, 1))
+        c.launcher().launch_pipeline(pipeline, p(), [c.upload(x[tk]), wa, single, na], (grid_x, 1, 1))
         assert got[tk].tobytes() == c.read(single)[:stride].tobytes(), "a token's sums differ between a lone launch and a multi-token launch"
 
 

@@ -223,6 +223,13 @@ zhip_result launch_matvec_q8_0_mfma(const Dispatch &d, const MvArgs &a);
 // The tuned multiply (matvec_quant.hip): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
 zhip_result launch_matvec_quant(const Dispatch &d, const MvArgs &a, int type);
 
+// Token blockIdx.x as the multiplies will see it (RMSNorm times the norm weights and / or
+// silu(x / act_div)), written to dst + token * k / 4.
+__global__ __launch_bounds__(256) void matvec_prologue_kernel(MvArgs a, float4 *dst) {
+    __shared__ float red[4];
+    stage_token(a, blockIdx.x, dst + (size_t)blockIdx.x * (a.k / 4u), red);
+}
+
 template <class D, int MT>
 static zhip_result run(const Dispatch &d, const MvArgs &a, uint32_t lds_bytes) {
     static int configured_device = -1;  // dynamic LDS above 64 KiB needs opting in once
@@ -295,15 +302,39 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     a.out = reinterpret_cast<float *>(d.bind[3].ptr);
     a.norm_w = norm ? reinterpret_cast<const float *>(d.bind[4].ptr) : nullptr;
 
+    // The matrix-core variants take their inputs as they are: a step with a prologue (RMSNorm,
+    // silu(x / act_div): src/kernels/matvec_quant.wgsl.hbs:73-89) first writes the transformed
+    // tokens to the workspace, one workgroup a token with the staging arithmetic of the default
+    // variant, and the multiply reads those.
+    const bool matrix_cores = quant && v.lanes == 64u && v.rows == 16u && D::CHUNK == 4;
+    uint64_t x_bound = d.bind[1].size;
+    // (Computing the prologue inside the multiply was tried on the kernel for k of 2048 or 4096:
+    // every workgroup repeats the row sums and takes its norm weights in dependent trips to
+    // memory, 36 us against 28 us with this pass in front, 22.5 us without a prologue.)
+    if (matrix_cores && (norm || a.act_div > 0.f) && a.m <= 8u && p.k % 1024u == 0) {
+        if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", D::name());
+        const uint64_t bytes = (uint64_t)a.m * p.k * 4u;
+        if (zhip_result r = d.work->reserve(d, bytes)) return r;
+        hipLaunchKernelGGL(matvec_prologue_kernel, dim3(a.m), dim3(256), 0, d.stream, a, reinterpret_cast<float4 *>(d.work->data));
+        if (zhip_result r = check_launch(d, D::name())) return r;
+        a.x = reinterpret_cast<const float *>(d.work->data);
+        a.xr = p.k;
+        a.flags &= ~FLAG_NORM;
+        a.act_div = 0.f;
+        a.norm_w = nullptr;
+        x_bound = bytes;
+        v.act_div = 0u;
+    }
+    const bool plain = !(a.flags & FLAG_NORM) && a.act_div == 0.f;
     // MatvecVariant (wg 512, lanes 64, rows 16) names the matrix-core variant: a wave per sixteen rows.
     // (k of 2048 or 4096 and whole tiles: the kernel that keeps the tokens' operands in registers.)
-    if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && v.act_div == 0u && matvec_q4k_mfma_resident_accepts(a))
+    if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && plain && matvec_q4k_mfma_resident_accepts(a))
         return launch_matvec_q4k_mfma_resident(d, a, d.bind[2].size);
-    if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && v.act_div == 0u && matvec_q4k_mfma_accepts(a))
-        return launch_matvec_q4k_mfma(d, a, d.bind[1].size, d.bind[2].size);
+    if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && plain && matvec_q4k_mfma_accepts(a))
+        return launch_matvec_q4k_mfma(d, a, x_bound, d.bind[2].size);
     // The same id on matvec_q8_0, without prologue or pair (a one-token step too, so that a
     // token's bits do not depend on the step it ran in).
-    if (D::CHUNK == 8 && v.lanes == 64u && v.rows == 16u && v.act_div == 0u && !(p.flags & (FLAG_NORM | FLAG_SILU_PAIR)) && a.m <= 32u)
+    if (D::CHUNK == 8 && v.lanes == 64u && v.rows == 16u && plain && !pair && a.m <= 32u)
         return launch_matvec_q8_0_mfma(d, a);
     // The tuned kernel takes rows of whole 64-weight tasks.
     if (D::CHUNK != 0 && p.k % 64u == 0) return launch_matvec_quant(d, a, D::CHUNK);
