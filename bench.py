@@ -47,6 +47,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,c5,formats,replay,floor for the 'also' section; 'none' skips it")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
+    ap.add_argument("--no-replay", action="store_true",
+                    help="launch every dispatch of a repeated submit instead of replaying it from a HIP graph (for runs under a kernel tracer, "
+                         "which has crashed on replayed graphs of several hundred kernel nodes)")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run 4 plain elementwise copies (256 MiB read + 256 MiB written each) so a counter run has a kernel of known traffic to scale by")
     args = ap.parse_args()
@@ -72,7 +75,7 @@ def main() -> int:
     from zllm_amd import kernels as K
     from zllm_amd.kernels import Kernel, TensorType, params as P
 
-    dev = Device.open(0)
+    dev = Device.open(0, Device.NO_REPLAY if args.no_replay else 0)
     host = Host(dev)
     rec = cmd.Recorder()
     kset = K.Set.create(rec)

@@ -986,6 +986,39 @@ def test_matmul_int8_shapes(ctx, t, rows, n, k):
     assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32))
 
 
+def test_matmul_q8_0_int8_whole_steps_keep_token_bits(ctx):
+    """matmul_q8_0 with k a multiple of 128, unsliced, takes the kernel whose scale products
+    run on the matrix cores, in 128- or 64-token tiles: a token's sums are the same bits
+    whichever tile height its step runs in and whichever tokens share the step; ragged
+    rows and outputs, a column offset and a padded stride; against float64 over the
+    rounded activations, 1e-5 (src/kernels/check.zig:839-871), and the unit formula."""
+    c = ctx
+    t = TensorType.q8_0
+    rows, n, k, col0, stride = 300, 2830, 640, 3, 2840
+    x = c.random(rows * k, 1).reshape(rows, k)
+    xs = oracle.round_like_llama(ORACLE_TYPE[t], x)
+    raw, values = quant_rows(c, t, n, k)
+    wa = c.gpu_weights(t, raw, k)
+    init = c.random(rows * stride, 0.5).reshape(rows, stride)
+
+    def run(first, count):
+        out = c.upload(init[first : first + count])
+        launch_int8(c, t, quantize_x(c, t, c.upload(x[first : first + count]), count, k), wa, out, count, n, k, 1, None, col0=col0, stride=stride)
+        return c.read(out).reshape(count, stride)
+
+    got = run(0, rows)  # three 128-token tiles on 45 column tiles: the tall tiling
+    want = init[:, col0 : col0 + n] + xs.astype(np.float64) @ values.astype(np.float64).T
+    assert rel_err(got[:, col0 : col0 + n], want) <= 1e-5
+    q, d = oracle.quantize_q8(x, 32)
+    formula = init[:, col0 : col0 + n] + oracle.matmul_q8(ORACLE_TYPE[t], raw, q, d, n)
+    assert rel_err(got[:, col0 : col0 + n], formula) <= 2e-6
+    mask = np.ones(stride, dtype=bool)
+    mask[col0 : col0 + n] = False
+    assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32)), "columns outside the chunk were written"
+    for first, count in ((0, 1), (1, 40), (41, 64), (105, 130), (235, 65)):  # 64-token tiles, and two tall tiles
+        assert got[first : first + count].tobytes() == run(first, count).tobytes(), "token chunking changed bits"
+
+
 def test_silu_mul(ctx):
     c = ctx
     rows, width = 7, 10_001

@@ -485,6 +485,12 @@ __global__ __launch_bounds__(256, 2) void matmul_kquant_i8_kernel(I8Args a) {
 
 }  // namespace
 
+// matmul_q8_i8.hip
+bool matmul_q8_i8_accepts(uint32_t k, uint32_t k_slice, uint32_t slices);
+zhip_result launch_matmul_q8_i8(const Dispatch &d, const char *name, const uint8_t *qx, const uint8_t *w, const uint8_t *dx, float *out, uint32_t rows,
+    uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, uint32_t row_bytes, uint32_t qx_bytes, uint32_t w_bytes,
+    uint32_t dx_bytes);
+
 // matmul_quant.wgsl's workgroup is 128 outputs x 32 tokens: the grid says how
 // much of the product a dispatch covers, whatever tiling computes it.
 static zhip_result launch_int8(const Dispatch &d, const char *name, int type) {
@@ -524,6 +530,9 @@ static zhip_result launch_int8(const Dispatch &d, const char *name, int type) {
     a.rows = (uint32_t)rows; a.n = (uint32_t)n; a.k = p.k; a.col0 = p.col0; a.out_stride = p.out_stride;
     a.accumulate = p.accumulate; a.k_slice = p.k_slice; a.slice_stride = p.slice_stride; a.row_bytes = (uint32_t)row_bytes;
     a.qx_bytes = (uint32_t)x_need; a.w_bytes = (uint32_t)w_need; a.dx_bytes = (uint32_t)d_need;
+    if (type == 8 && matmul_q8_i8_accepts(p.k, p.k_slice, (uint32_t)slices))
+        return launch_matmul_q8_i8(d, name, a.qx, a.w, a.dx, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes, a.qx_bytes,
+            a.w_bytes, a.dx_bytes);
     const dim3 grid((uint32_t)tiles_n, (uint32_t)tiles_t, (uint32_t)slices);
     const bool ragged = p.k % STEP != 0 || (p.k_slice < p.k && p.k_slice % STEP != 0);
     if (type == 3) {
