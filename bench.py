@@ -484,6 +484,22 @@ def bench_formats(env):
         nbytes = n * (k // e) * bb + 4 * k + 4 * n
         res[name] = env["hbm_entry"](f"{name} decode matvec M=1 K={k} N={n}", nbytes, wall, gpu_s, steps,
                                      {"copies": len(launches), "max_err_over_row_x_norms": bound, "max_err_over_max_want": rel})
+    # Steps of several tokens on Q8_0 (a speculative verify step): the default variant, and the
+    # matrix-core variant (MatvecVariant wg 512, lanes 64, rows 16) a tuner would pick for them.
+    mc = K.MatvecVariant(wg=512, lanes=64, rows=16)
+    raw = synth.random_blocks(synth.rng(0xF1), "q8_0", n, k)
+    w = oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k)
+    e, bb = K.LAYOUT[TensorType.q8_0]
+    for m, variant, tag in ((4, None, "q8_0_m4"), (2, mc, "q8_0_m2_matrix_cores"), (4, mc, "q8_0_m4_matrix_cores"), (8, mc, "q8_0_m8_matrix_cores")):
+        xm = synth.activations(synth.rng(0xF8 + m), m, k)
+        launches, out = env["matvec_workload"](TensorType.q8_0, raw, n, k, m, False, xm, variant)
+        wall, gpu_s, steps = env["protocol"](launches)
+        got = env["read"](out)[: m * n].reshape(m, n).astype(np.float64)
+        want = xm.astype(np.float64) @ w.astype(np.float64).T
+        rel = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+        nbytes = n * (k // e) * bb + m * 4 * k + m * 4 * n
+        res[tag] = env["hbm_entry"](f"q8_0 decode matvec M={m} K={k} N={n}" + (", matrix-core variant" if variant else ""), nbytes, wall, gpu_s, steps,
+                                    {"copies": len(launches), "max_err_over_max_want": rel})
     return res
 
 

@@ -276,7 +276,9 @@ def test_quant_matvec_mfma_variant(ctx, pair, rows, n, k, prologue):
     (5, 96, 4096, 4, 8, False),      # aligned rows: 16-byte stores
     (3, 100, 2080, 0, 0, True),      # k = 65 blocks: a ragged last step
     (1, 530, 1024, 0, 2, False),     # one token
-    (8, 4112, 4096, 0, 0, False),    # 65 tiles of 64 rows
+    (8, 4112, 4096, 0, 0, False),    # 257 sixteen-row tiles: the kernel that streams whole tiles, two tiles on one workgroup
+    (7, 4112, 2048, 5, 7, True),     # the same with eight blocks a wave, unaligned outputs, accumulating
+    (2, 1536, 4096, 0, 0, True),
 ])
 def test_matvec_q8_0_mfma_variant(ctx, rows, n, k, col0, pad, accumulate):
     """The matrix-core variant of matvec_q8_0 (the id of a wave per sixteen rows): every
@@ -309,6 +311,40 @@ def test_matvec_q8_0_mfma_variant(ctx, rows, n, k, col0, pad, accumulate):
         single = c.upload(init[tk])
         c.launcher().launch_pipeline(pipeline, p(), [c.upload(x[tk]), wa, single, wa], (grid_x, 1, 1))
         assert got[tk].tobytes() == c.read(single)[:stride].tobytes(), "a token's sums differ between a lone launch and a multi-token launch"
+
+
+@pytest.mark.parametrize("prologue", ["norm", "norm_act"])
+@pytest.mark.parametrize("rows,n,k", [(6, 4112, 4096), (3, 96, 2048), (2, 200, 1024)])
+def test_matvec_q8_0_mfma_variant_prologues(ctx, rows, n, k, prologue):
+    """The matrix-core variant of matvec_q8_0 on steps with the RMSNorm and silu(x / act_div)
+    prologues (src/kernels/matvec_quant.wgsl.hbs:73-89): the transformed tokens reach the
+    multiply through the workspace; 1e-5 against float64, each token bitwise equal to its
+    lone launch."""
+    c = ctx
+    div, eps = 4 if prologue == "norm_act" else 0, 1e-6
+    x = c.random(rows * k, 3).reshape(rows, k)
+    x[0] *= np.float32(1e-4)
+    nw = c.random(k, 1.5)
+    raw, values = quant_rows(c, TensorType.q8_0, n, k)
+    init = c.random(rows * n, 2).reshape(rows, n)
+    xa, wa, na = c.upload(x), c.gpu_weights(TensorType.q8_0, raw, k), c.upload(nw)
+    x64 = np.stack([norm_row(r, nw, eps) for r in x])
+    if div:
+        x64 = (x64 / div) * sigmoid64(x64 / div)
+    want = init + x64 @ values.astype(np.float64).T
+    p = lambda: P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, eps=eps, norm=True, accumulate=True)
+    variant = K.MatvecVariant(MFMA_VARIANT.wg, MFMA_VARIANT.lanes, MFMA_VARIANT.rows, div)
+    pipeline = c.set.matvec(c.rec, Kernel.matvec_q8_0, variant)
+    grid_x = K.div_ceil(n, variant.group_rows())
+    out = c.upload(init)
+    c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, na], (grid_x, rows, 1))
+    got = c.read(out).reshape(rows, n)
+    for tk in range(rows):
+        assert rel_err(got[tk], want[tk]) <= 1e-5, tk
+    for tk in range(rows):
+        single = c.upload(init[tk])
+        c.launcher().launch_pipeline(pipeline, p(), [c.upload(x[tk]), wa, single, na], (grid_x, 1, 1))
+        assert got[tk].tobytes() == c.read(single)[:n].tobytes(), "a token's sums differ between a lone launch and a multi-token launch"
 
 
 # ---- block decoders bit for bit, through the embedding gathers: check.zig:873-905 -----

@@ -218,6 +218,9 @@ bool matvec_q4k_mfma_accepts(const MvArgs &a);
 zhip_result launch_matvec_q4k_mfma(const Dispatch &d, const MvArgs &a, uint64_t x_bytes, uint64_t w_bytes);
 bool matvec_q4k_mfma_resident_accepts(const MvArgs &a);
 zhip_result launch_matvec_q4k_mfma_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
+// The matrix-core variant of matvec_q8_0 for k of 2048 or 4096 (matvec_q8_mfma_stream.hip).
+bool matvec_q8_mfma_stream_accepts(const MvArgs &a);
+zhip_result launch_matvec_q8_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
 // The matrix-core variant of matvec_q8_0 (matmul_mfma.hip).
 zhip_result launch_matvec_q8_0_mfma(const Dispatch &d, const MvArgs &a);
 // The tuned multiply (matvec_quant.hip): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
@@ -306,12 +309,15 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     // silu(x / act_div): src/kernels/matvec_quant.wgsl.hbs:73-89) first writes the transformed
     // tokens to the workspace, one workgroup a token with the staging arithmetic of the default
     // variant, and the multiply reads those.
-    const bool matrix_cores = quant && v.lanes == 64u && v.rows == 16u && D::CHUNK == 4;
+    const bool matrix_cores = quant && v.lanes == 64u && v.rows == 16u && (D::CHUNK == 4 || D::CHUNK == 8);
     uint64_t x_bound = d.bind[1].size;
     // (Computing the prologue inside the multiply was tried on the kernel for k of 2048 or 4096:
     // every workgroup repeats the row sums and takes its norm weights in dependent trips to
     // memory, 36 us against 28 us with this pass in front, 22.5 us without a prologue.)
-    if (matrix_cores && (norm || a.act_div > 0.f) && a.m <= 8u && p.k % 1024u == 0) {
+    // (On matvec_q8_0 only where the kernel that streams whole tiles takes the step: the other
+    // matrix-core kernel of that operation narrows its inputs into the same workspace.)
+    const bool prepass = D::CHUNK == 4 ? p.k % 1024u == 0 : ((p.k == 2048u || p.k == 4096u) && a.rows % 16u == 0 && !pair);
+    if (matrix_cores && (norm || a.act_div > 0.f) && a.m <= 8u && prepass) {
         if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", D::name());
         const uint64_t bytes = (uint64_t)a.m * p.k * 4u;
         if (zhip_result r = d.work->reserve(d, bytes)) return r;
@@ -334,6 +340,8 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
         return launch_matvec_q4k_mfma(d, a, x_bound, d.bind[2].size);
     // The same id on matvec_q8_0, without prologue or pair (a one-token step too, so that a
     // token's bits do not depend on the step it ran in).
+    if (D::CHUNK == 8 && v.lanes == 64u && v.rows == 16u && plain && !pair && matvec_q8_mfma_stream_accepts(a))
+        return launch_matvec_q8_mfma_stream(d, a, d.bind[2].size);
     if (D::CHUNK == 8 && v.lanes == 64u && v.rows == 16u && plain && !pair && a.m <= 32u)
         return launch_matvec_q8_0_mfma(d, a);
     // The tuned kernel takes rows of whole 64-weight tasks.
