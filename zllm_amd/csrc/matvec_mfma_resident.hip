@@ -109,7 +109,7 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
     __shared__ float lds_scale[16];               // [8] scale, [8] its inverse
     __shared__ float lds_part[2][WAVES][128];     // [tile parity][wave][2 lane + token of the lane's two]
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
-    const __amdgpu_buffer_rsrc_t wbuf = make_buffer(a.w, q.w_bytes);
+    const __amdgpu_buffer_rsrc_t wbuf = make_buffer(a.w, q.w_bytes), nobuf = make_buffer(a.w, 0);
     uint32_t sixteen = q.sixteen;
     asm volatile("" : "+v"(sixteen));
 
@@ -125,7 +125,8 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
     // load c / 64; past 144 a lane asks beyond the buffer and zeros land. The tile's part of
     // the offset is uniform and travels in a scalar register (the buffer's range check does
     // not see it: every row of a tile exists here). Past the run's last tile the loads still
-    // run, so that the waits count the same loads every step, but fetch the matrix's first rows.
+    // run, so that the waits count the same loads every step, but against an empty buffer:
+    // zeros land and nothing is fetched.
     __shared__ __align__(16) uint8_t lds_ring[WAVES * DEPTH * NB * SLOT];
     uint8_t *ring = lds_ring + wave * (DEPTH * NB * SLOT);
     uint32_t woff[3];
@@ -135,11 +136,13 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
         woff[j] = c < 144u ? (c / 9u) * a.row_bytes + 16u * (c % 9u) + NB * wave * 144u : 0xfffffff0u - 144u * NB;
     }
     auto load_tile = [&](uint32_t p, uint32_t slot) __attribute__((always_inline)) {
-        const uint32_t base = (p < count ? row0(p) : 0u) * a.row_bytes;
+        const bool real = p < count;
+        const __amdgpu_buffer_rsrc_t buf = real ? wbuf : nobuf;
+        const uint32_t base = (real ? row0(p) : 0u) * a.row_bytes;
 #pragma unroll
         for (uint32_t i = 0; i < NB; i++)
 #pragma unroll
-            for (uint32_t j = 0; j < 3; j++) load_lds_b128(wbuf, ring + (slot * NB + i) * SLOT + 1024u * j, woff[j] + 144u * i, base);
+            for (uint32_t j = 0; j < 3; j++) load_lds_b128(buf, ring + (slot * NB + i) * SLOT + 1024u * j, woff[j] + 144u * i, base);
     };
     constexpr int LOADS = 3 * NB;  // a tile's loads of one wave
     load_tile(0, 0);
