@@ -12,7 +12,7 @@
 #include <hip/hip_runtime.h>
 
 #include "common.h"
-#include "decode.cuh"
+#include "decode.h"
 
 namespace zhip {
 

@@ -56,8 +56,8 @@
 #include <type_traits>
 
 #include "common.h"
-#include "decode.cuh"
-#include "matvec_common.cuh"
+#include "decode.h"
+#include "matvec_common.h"
 
 namespace zhip {
 

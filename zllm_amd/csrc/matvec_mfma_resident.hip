@@ -23,8 +23,8 @@
 #include <hip/hip_runtime.h>
 
 #include "common.h"
-#include "decode.cuh"
-#include "matvec_common.cuh"
+#include "decode.h"
+#include "matvec_common.h"
 
 namespace zhip {
 

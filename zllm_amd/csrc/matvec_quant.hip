@@ -33,12 +33,15 @@
 // from a bank-conflict-free padded LDS copy kept in task order, once per task
 // for both rows of a pass (two outputs, or the gate and up rows of one output
 // with SILU_PAIR). In both, the next task's vectors are loaded before the
-// current one is multiplied.
+// current one is multiplied. An XREG workgroup asks for the token's inputs (and
+// norm weights) before its first weights: loads complete in order within a
+// wave, so inputs requested behind a weight row would wait for that row's trip
+// to memory before the staging could start.
 #include <hip/hip_runtime.h>
 
 #include "common.h"
-#include "decode.cuh"
-#include "matvec_common.cuh"
+#include "decode.h"
+#include "matvec_common.h"
 
 namespace zhip {
 
