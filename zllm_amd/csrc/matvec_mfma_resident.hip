@@ -29,6 +29,7 @@
 namespace zhip {
 
 typedef _Float16 rf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 rf16x4 __attribute__((ext_vector_type(4)));
 typedef float rf32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t ru32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t ru32x2 __attribute__((ext_vector_type(2)));
@@ -106,7 +107,8 @@ __device__ __forceinline__ rf16x8 nibbles(ru32x2 w, uint32_t mask, uint32_t sixt
 template <bool PAIR, int NB>
 __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResArgs q) {
     const MvArgs &a = q.a;
-    __shared__ float lds_scale[16];               // [8] scale, [8] its inverse
+    __shared__ float lds_scale[16];               // [8 ..]: one over each token's scale
+    __shared__ float lds_max[WAVES * 8];          // [wave][token]: the largest magnitude in the wave's range
     __shared__ float lds_part[2][WAVES][128];     // [tile parity][wave][2 lane + token of the lane's two]
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
     const __amdgpu_buffer_rsrc_t wbuf = make_buffer(a.w, q.w_bytes), nobuf = make_buffer(a.w, 0);
@@ -145,65 +147,69 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
             for (uint32_t j = 0; j < 3; j++) load_lds_b128(buf, ring + (slot * NB + i) * SLOT + 1024u * j, woff[j] + 144u * i, base);
     };
     constexpr int LOADS = 3 * NB;  // a tile's loads of one wave
+
+    // The tokens' inputs first: loads complete in order within a wave, and behind the weight
+    // loads below the first use of an input would wait for a round trip of the weight stream.
+    // Operand row l16 of the matrix instruction is token l16 / 2: the f16 rounding of its scaled
+    // inputs (even rows) or what that left, times 2^11 (odd rows); the lane's eight positions of
+    // sub-block s are 8 g .. 8 g + 7 in the order k0 k2 k1 k3 k4 k6 k5 k7. The two lanes of a
+    // token and group share the work: the even one loads and splits positions 0 .. 3, the odd
+    // one 4 .. 7, and they swap what the other needs. An absent token's rows read the last
+    // token's inputs under a scale of zero: no branches, so all of the lane's loads go out together.
+    const uint32_t tok = l16 >> 1, sub = l16 & 1u, tsrc = tok < a.m ? tok : a.m - 1u;
+    float4 raw[NB * 8];
+    {
+        const float *xt = a.x + (size_t)tsrc * a.xr + NB * 256u * wave + 8u * g + 4u * sub;
+#pragma unroll
+        for (int s = 0; s < NB * 8; s++) raw[s] = *reinterpret_cast<const float4 *>(xt + 32 * s);
+    }
     load_tile(0, 0);
 
-    // Each token's scale: the power of two that puts its largest magnitude in [2^14, 2^15).
-    if (wave < a.m) {
-        const float4 *xr = reinterpret_cast<const float4 *>(a.x + (size_t)wave * a.xr);
-        // (all of the lane's loads first: one trip to memory, not one per vector)
-        float4 v[NB * 8];
-#pragma unroll
-        for (int i = 0; i < NB * 8; i++) v[i] = xr[lane + 64u * i];
+    // Each token's scale: the power of two that puts its largest magnitude in [2^14, 2^15). The
+    // eight lanes of a token (two rows, four groups) hold this wave's range of it; the eight
+    // waves' maxima meet in LDS.
+    {
         float big = 0.f;
 #pragma unroll
-        for (int i = 0; i < NB * 8; i++) big = fmaxf(fmaxf(fabsf(v[i].x), fabsf(v[i].y)), fmaxf(fmaxf(fabsf(v[i].z), fabsf(v[i].w)), big));
-#pragma unroll
-        for (int off = 32; off > 0; off >>= 1) big = fmaxf(big, __shfl_xor(big, off, 64));
-        if (lane == 0) {
-            const int e = (int)((__float_as_uint(big) >> 23) & 0xffu);  // biased exponent; 0 for zero and subnormals
-            int se = 127 + 14 - (e - 127);                               // scale = 2^(14 - (e - 127)), kept normal both ways
-            se = se < 1 ? 1 : se > 253 ? 253 : se;
-            lds_scale[wave] = (e == 0 || e == 255) ? 1.0f : __uint_as_float((uint32_t)se << 23);
-            lds_scale[8 + wave] = (e == 0 || e == 255) ? 1.0f : __uint_as_float((uint32_t)(254 - se) << 23);
-        }
-    } else if (lane == 0) {
-        lds_scale[wave] = lds_scale[8 + wave] = 1.0f;
+        for (int s = 0; s < NB * 8; s++) big = fmaxf(fmaxf(fabsf(raw[s].x), fabsf(raw[s].y)), fmaxf(fmaxf(fabsf(raw[s].z), fabsf(raw[s].w)), big));
+        big = fmaxf(big, __shfl_xor(big, 1, 64));
+        big = fmaxf(big, __shfl_xor(big, 16, 64));
+        big = fmaxf(big, __shfl_xor(big, 32, 64));
+        if (g == 0u && sub == 0u) lds_max[8u * wave + tok] = big;
     }
     lds_barrier();
-
-    // This wave's k range of the tokens as matrix-core operands: operand row l16 is token
-    // l16 / 2, the f16 rounding of its scaled inputs (even rows) or what that left, times
-    // 2^11 (odd rows); the lane's eight positions of sub-block s are 8 g .. 8 g + 7, in the
-    // order k0 k2 k1 k3 k4 k6 k5 k7. Rows of tokens the step does not have are zeros.
+    auto scale_of = [&](uint32_t t, bool inverse) {
+        float big = lds_max[t];
+#pragma unroll
+        for (uint32_t wv = 1; wv < WAVES; wv++) big = fmaxf(big, lds_max[8u * wv + t]);
+        const int e = (int)((__float_as_uint(big) >> 23) & 0xffu);  // biased exponent; 0 for zero and subnormals
+        int se = 127 + 14 - (e - 127);                               // scale = 2^(14 - (e - 127)), kept normal both ways
+        se = se < 1 ? 1 : se > 253 ? 253 : se;
+        if (e == 0 || e == 255) return 1.0f;
+        return __uint_as_float((uint32_t)(inverse ? 254 - se : se) << 23);
+    };
+    if (tid < 8u) lds_scale[8 + tid] = tid < a.m ? scale_of(tid, true) : 1.0f;  // read after a later barrier
     rf16x8 xf[NB * 8];
     {
-        // (an absent token's rows read the last token's inputs under a scale of zero: no branches,
-        // so all of the lane's loads go out together)
-        const uint32_t t = l16 >> 1, tsrc = t < a.m ? t : a.m - 1u;
-        const float scale = t < a.m ? lds_scale[t] : 0.f;
-        const float *xt = a.x + (size_t)tsrc * a.xr + NB * 256u * wave + 8u * g;
-        float4 raw[NB * 8][2];
+        const float scale = tok < a.m ? scale_of(tok, false) : 0.f;
 #pragma unroll
         for (int s = 0; s < NB * 8; s++) {
-            raw[s][0] = *reinterpret_cast<const float4 *>(xt + 32 * s);
-            raw[s][1] = *reinterpret_cast<const float4 *>(xt + 32 * s + 4);
-        }
+            const float x[4] = {raw[s].x, raw[s].y, raw[s].z, raw[s].w};
+            // The scale is a power of two, so x * scale - hi in one fused operation is exact.
+            _Float16 hi[4], lo[4];
 #pragma unroll
-        for (int s = 0; s < NB * 8; s++) {
-            const float x[8] = {raw[s][0].x, raw[s][0].y, raw[s][0].z, raw[s][0].w, raw[s][1].x, raw[s][1].y, raw[s][1].z, raw[s][1].w};
-            // Both rows' values for every lane (even lanes keep the first, odd lanes the second);
-            // the scale is a power of two, so x * scale - hi in one fused operation is exact.
-            _Float16 hi[8], lo[8];
-#pragma unroll
-            for (int e = 0; e < 8; e++) {
+            for (int e = 0; e < 4; e++) {
                 hi[e] = (_Float16)(x[e] * scale);
                 lo[e] = (_Float16)(fmaf(x[e], scale, -(float)hi[e]) * 2048.0f);
             }
-            const rf16x8 first = {hi[0], hi[2], hi[1], hi[3], hi[4], hi[6], hi[5], hi[7]};
-            const rf16x8 second = {lo[0], lo[2], lo[1], lo[3], lo[4], lo[6], lo[5], lo[7]};
-            const ru32x4 f4 = __builtin_bit_cast(ru32x4, first), s4 = __builtin_bit_cast(ru32x4, second);
-            const bool odd = l16 & 1u;
-            const ru32x4 pick = {odd ? s4.x : f4.x, odd ? s4.y : f4.y, odd ? s4.z : f4.z, odd ? s4.w : f4.w};
+            const ru32x2 h2 = __builtin_bit_cast(ru32x2, rf16x4{hi[0], hi[2], hi[1], hi[3]}), l2 = __builtin_bit_cast(ru32x2, rf16x4{lo[0], lo[2], lo[1], lo[3]});
+            // The even lane keeps its first roundings and needs the odd lane's; the odd lane keeps
+            // its remainders and needs the even lane's.
+            const ru32x2 give = sub ? h2 : l2;
+            ru32x2 got;
+            got.x = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)give.x, 0xB1, 0xf, 0xf, false);  // quad_perm [1, 0, 3, 2]: the neighbour's
+            got.y = (uint32_t)__builtin_amdgcn_update_dpp(0, (int)give.y, 0xB1, 0xf, 0xf, false);
+            const ru32x4 pick = {sub ? got.x : h2.x, sub ? got.y : h2.y, sub ? l2.x : got.x, sub ? l2.y : got.y};
             xf[s] = __builtin_bit_cast(rf16x8, pick);
         }
     }
