@@ -37,14 +37,16 @@ typedef uint32_t ru32x2 __attribute__((ext_vector_type(2)));
 namespace {
 
 constexpr uint32_t THREADS = 512, WAVES = 8;
-constexpr int DEPTH = 2;  // ring slots a wave: one tile multiplied, the others in flight
+constexpr int DEPTH = 3;  // ring slots a wave: one tile multiplied, the others in flight
 constexpr uint32_t SLOT = 3u * 1024u;  // a block: 2304 bytes; the third load's idle lanes land behind them
 
 struct ResArgs {
     MvArgs a;
     uint32_t w_bytes;
     uint32_t nibble_mask, sixteen;  // 0x03C003C0, 0x4C004C00 (see nibbles)
-    uint32_t out_tiles;             // sixteen-output tiles
+    uint32_t rounds;                // sixteen-output tiles every workgroup takes: tiles b, b + G, ...
+    uint32_t left;                  // output tiles after those, fewer than G: one for each of the first workgroups,
+    uint32_t split;                 // or (split) eight outputs of one for each of the first 2 * left
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void *base, uint32_t bytes) {
@@ -118,10 +120,16 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
     // The workgroup's weight tiles: output tiles b, b + G, ...; with SILU_PAIR the gate tile
     // and then the up tile of each. Tile p of the run starts at matrix row:
     const uint32_t per = PAIR ? 2u : 1u;
-    const uint32_t mine = blockIdx.x < q.out_tiles ? (q.out_tiles - 1u - blockIdx.x) / gridDim.x + 1u : 0u;
+    // When the output tiles left over after whole rounds are at most half as many as the
+    // workgroups, two workgroups share each, eight rows apiece: a whole tile more on half of
+    // the CUs would be the launch's tail.
+    const bool extra = blockIdx.x < (q.split ? 2u * q.left : q.left);
+    const uint32_t mine = q.rounds + (extra ? 1u : 0u);
     const uint32_t count = per * mine;
-    auto out_tile = [&](uint32_t p) { return blockIdx.x + (p / per) * gridDim.x; };
-    auto row0 = [&](uint32_t p) { return 16u * out_tile(p) + ((PAIR && (p & 1u)) ? a.half : 0u); };
+    const uint32_t last_out = 16u * (q.rounds * gridDim.x + (q.split ? blockIdx.x >> 1 : blockIdx.x)) + (q.split ? 8u * (blockIdx.x & 1u) : 0u);
+    auto out0 = [&](uint32_t p) { return p / per < q.rounds ? 16u * (blockIdx.x + (p / per) * gridDim.x) : last_out; };  // first output of tile p
+    auto rows_of = [&](uint32_t p) { return (q.split && p / per >= q.rounds) ? 8u : 16u; };
+    auto row0 = [&](uint32_t p) { return out0(p) + ((PAIR && (p & 1u)) ? a.half : 0u); };
 
     // A tile's loads: chunk c of a block's 144 (row c / 9, sixteen bytes c % 9) by lane c % 64 of
     // load c / 64; past 144 a lane asks beyond the buffer and zeros land. The tile's part of
@@ -131,20 +139,22 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
     // zeros land and nothing is fetched.
     __shared__ __align__(16) uint8_t lds_ring[WAVES * DEPTH * NB * SLOT];
     uint8_t *ring = lds_ring + wave * (DEPTH * NB * SLOT);
-    uint32_t woff[3];
+    uint32_t woff[3], woff8[3];  // (woff8: the same for an eight-row share, whose other rows are not fetched)
 #pragma unroll
     for (uint32_t j = 0; j < 3; j++) {
         const uint32_t c = 64u * j + lane;
         woff[j] = c < 144u ? (c / 9u) * a.row_bytes + 16u * (c % 9u) + NB * wave * 144u : 0xfffffff0u - 144u * NB;
+        woff8[j] = c < 72u ? woff[j] : 0xfffffff0u - 144u * NB;
     }
     auto load_tile = [&](uint32_t p, uint32_t slot) __attribute__((always_inline)) {
         const bool real = p < count;
         const __amdgpu_buffer_rsrc_t buf = real ? wbuf : nobuf;
         const uint32_t base = (real ? row0(p) : 0u) * a.row_bytes;
+        const bool whole = rows_of(p) == 16u;
 #pragma unroll
         for (uint32_t i = 0; i < NB; i++)
 #pragma unroll
-            for (uint32_t j = 0; j < 3; j++) load_lds_b128(buf, ring + (slot * NB + i) * SLOT + 1024u * j, woff[j] + 144u * i, base);
+            for (uint32_t j = 0; j < 3; j++) load_lds_b128(buf, ring + (slot * NB + i) * SLOT + 1024u * j, (whole ? woff[j] : woff8[j]) + 144u * i, base);
     };
     constexpr int LOADS = 3 * NB;  // a tile's loads of one wave
 
@@ -275,8 +285,8 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
                 held = sum;
             } else {
                 const float v = PAIR ? silu_f(held) * sum : sum;
-                if (t < a.m) {
-                    float *o = a.out + (size_t)t * a.out_stride + a.col0 + 16u * out_tile(p) + row;
+                if (t < a.m && row < rows_of(p)) {
+                    float *o = a.out + (size_t)t * a.out_stride + a.col0 + out0(p) + row;
                     store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + v : v);
                 }
             }
@@ -314,9 +324,12 @@ zhip_result launch_matvec_q4k_mfma_resident(const Dispatch &d, const MvArgs &a, 
     // 32-bit byte offsets.
     const uint64_t reach = ((uint64_t)(pair ? a.half : 0u) + a.rows + 16u) * a.row_bytes;
     if (w_bytes >= 0xfffffff0ull || reach >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "matvec_q4_k: operands of 4 GiB or more");
-    ResArgs q{a, (uint32_t)w_bytes, 0x03C003C0u, 0x4C004C00u, a.rows / 16u};
-    const uint32_t cus = (uint32_t)d.dev->compute_units;
-    const dim3 grid(q.out_tiles < cus ? q.out_tiles : cus);
+    const uint32_t cus = (uint32_t)d.dev->compute_units, tiles = a.rows / 16u;
+    const uint32_t groups = tiles < cus ? (2u * tiles <= cus ? 2u * tiles : tiles) : cus;
+    const bool halves = tiles < groups;  // every workgroup takes eight outputs of one tile
+    const uint32_t left = halves ? tiles : tiles % groups;
+    ResArgs q{a, (uint32_t)w_bytes, 0x03C003C0u, 0x4C004C00u, halves ? 0u : tiles / groups, left, (halves || 2u * left <= groups) ? 1u : 0u};
+    const dim3 grid(groups);
     if (a.k == 2048u) {
         if (pair) hipLaunchKernelGGL((matvec_q4k_mfma_resident_kernel<true, 1>), grid, dim3(THREADS), 0, d.stream, q);
         else hipLaunchKernelGGL((matvec_q4k_mfma_resident_kernel<false, 1>), grid, dim3(THREADS), 0, d.stream, q);
