@@ -66,6 +66,13 @@ __device__ __forceinline__ void load_lds_b128(__amdgpu_buffer_rsrc_t buf, uint8_
     asm volatile("" : "+s"(address));
     __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)(uintptr_t)address, 16, offset, 0, 0, 0);
 }
+// The same with a uniform part of the offset in a scalar register (the buffer's range check
+// sees the lane's part only).
+__device__ __forceinline__ void load_lds_b128(__amdgpu_buffer_rsrc_t buf, uint8_t *dst, uint32_t offset, uint32_t uniform_offset) {
+    uint32_t address = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);
+    asm volatile("" : "+s"(address));
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)(uintptr_t)address, 16, offset, uniform_offset, 0, 0);
+}
 
 // Every load of this wave has landed, every wave's LDS traffic is done: the
 // buffer just filled may be read, the one just read may be filled.
@@ -240,7 +247,10 @@ __device__ __forceinline__ void store_tile(const I8Args &a, const if32x4 (&acc)[
 }
 
 // ---- K formats (256-weight blocks), Q8_K activations ---------------------------------
-// A format gives the bytes a lane loads for one block of its row (Raw, load) and
+// A format gives the bytes a lane reads of one block of its row (Raw, load: from the wave's
+// LDS slot, where the sixteen rows' blocks arrive by whole-line direct loads; a lane loading
+// its own row's 8- and 16-byte pieces from memory makes the vector memory unit look up a
+// cache line per lane, and that rate bounded the kernel) and
 // unit u's operand: the eight signed integers at positions 8 g .. 8 g + 7 of the
 // unit with the scales of the unit's two halves of sixteen and its minimum
 // (src/kernels/quant/q3_k.wgsl, q4_k.wgsl, q5_k.wgsl, q6_k.wgsl: head, scales, quad_i8).
@@ -256,10 +266,10 @@ struct I8Q4 {
         iu32x4 h;       // d, dmin and the twelve scale bytes
         iu32x2 q[4];    // 8 bytes of each 64-weight chunk: low nibbles unit 2c, high 2c + 1
     };
-    static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t w, uint32_t blk, uint32_t g, Raw &r) {
-        r.h = __builtin_amdgcn_raw_buffer_load_b128(w, blk, 0, 0);
+    static __device__ __forceinline__ void load(const uint8_t *blk, uint32_t g, Raw &r) {
+        r.h = *reinterpret_cast<const iu32x4 *>(blk);
 #pragma unroll
-        for (uint32_t c = 0; c < 4; c++) r.q[c] = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 16u + 32u * c + 8u * g, 0, 0);
+        for (uint32_t c = 0; c < 4; c++) r.q[c] = *reinterpret_cast<const iu32x2 *>(blk + 16u + 32u * c + 8u * g);
     }
     static __device__ __forceinline__ void block(const Raw &r, float &d, float &dmin) {
         d = half_bits_to_float(r.h.x & 0xffffu);
@@ -283,11 +293,11 @@ struct I8Q5 {
         iu32x2 qh;      // the fifth bits of positions 8 g .. 8 g + 7, bit u for unit u
         iu32x2 q[4];
     };
-    static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t w, uint32_t blk, uint32_t g, Raw &r) {
-        r.h = __builtin_amdgcn_raw_buffer_load_b128(w, blk, 0, 0);
-        r.qh = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 16u + 8u * g, 0, 0);
+    static __device__ __forceinline__ void load(const uint8_t *blk, uint32_t g, Raw &r) {
+        r.h = *reinterpret_cast<const iu32x4 *>(blk);
+        r.qh = *reinterpret_cast<const iu32x2 *>(blk + 16u + 8u * g);
 #pragma unroll
-        for (uint32_t c = 0; c < 4; c++) r.q[c] = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 48u + 32u * c + 8u * g, 0, 0);
+        for (uint32_t c = 0; c < 4; c++) r.q[c] = *reinterpret_cast<const iu32x2 *>(blk + 48u + 32u * c + 8u * g);
     }
     static __device__ __forceinline__ void block(const Raw &r, float &d, float &dmin) {
         d = half_bits_to_float(r.h.x & 0xffffu);
@@ -312,13 +322,13 @@ struct I8Q6 {
         iu32x4 sc;      // sixteen signed scales
         uint32_t d;
     };
-    static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t w, uint32_t blk, uint32_t g, Raw &r) {
+    static __device__ __forceinline__ void load(const uint8_t *blk, uint32_t g, Raw &r) {
 #pragma unroll
-        for (uint32_t i = 0; i < 4; i++) r.ql[i] = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 32u * i + 8u * g, 0, 0);
+        for (uint32_t i = 0; i < 4; i++) r.ql[i] = *reinterpret_cast<const iu32x2 *>(blk + 32u * i + 8u * g);
 #pragma unroll
-        for (uint32_t n = 0; n < 2; n++) r.qh[n] = __builtin_amdgcn_raw_buffer_load_b64(w, blk + 128u + 32u * n + 8u * g, 0, 0);
-        r.sc = __builtin_amdgcn_raw_buffer_load_b128(w, blk + 192u, 0, 0);
-        r.d = __builtin_amdgcn_raw_buffer_load_b32(w, blk + 208u, 0, 0);
+        for (uint32_t n = 0; n < 2; n++) r.qh[n] = *reinterpret_cast<const iu32x2 *>(blk + 128u + 32u * n + 8u * g);
+        r.sc = *reinterpret_cast<const iu32x4 *>(blk + 192u);
+        r.d = *reinterpret_cast<const uint32_t *>(blk + 208u);
     }
     static __device__ __forceinline__ void block(const Raw &r, float &d, float &dmin) {
         d = half_bits_to_float(r.d & 0xffffu);
@@ -341,9 +351,9 @@ struct I8Q3 {
     struct Raw {
         iu32x4 u[8];  // two words of 2-bit values, the high bits, scales - 32 and d
     };
-    static __device__ __forceinline__ void load(__amdgpu_buffer_rsrc_t w, uint32_t blk, uint32_t, Raw &r) {
+    static __device__ __forceinline__ void load(const uint8_t *blk, uint32_t, Raw &r) {
 #pragma unroll
-        for (uint32_t i = 0; i < 8; i++) r.u[i] = __builtin_amdgcn_raw_buffer_load_b128(w, blk + 16u * i, 0, 0);
+        for (uint32_t i = 0; i < 8; i++) r.u[i] = *reinterpret_cast<const iu32x4 *>(blk + 16u * i);
     }
     static __device__ __forceinline__ void block(const Raw &r, float &d, float &dmin) {
         d = half_bits_to_float(r.u[0].w >> 16);  // every unit of a block carries the block's d
@@ -365,7 +375,13 @@ template <class P>
 __global__ __launch_bounds__(256, 2) void matmul_kquant_i8_kernel(I8Args a) {
     __shared__ __align__(16) uint8_t lds_q[2][TT * LINE];
     __shared__ __align__(16) float lds_d[2][TT];      // the tokens' block scales
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
+    // The weights: per wave and buffer its sixteen rows' blocks, [row][BLOCK bytes], as WLOADS
+    // wave-wide loads of 16 bytes a lane (chunk c = 64 load + lane: row c / CPR, piece c % CPR;
+    // lanes past the sixteenth row ask past the buffer and zeros land behind the blocks).
+    constexpr uint32_t CPR = P::BLOCK / 16u, WLOADS = (16u * CPR + 63u) / 64u, WSLOT = WLOADS * 1024u;
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_w[];  // [2][4 waves][WSLOT]
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t n0 = blockIdx.x * TN, t0 = blockIdx.y * TT;
     const uint32_t kb = blockIdx.z * a.k_slice, ke = min(a.k, kb + a.k_slice);
     const uint32_t k_first = kb & ~(STEP - 1u);
@@ -377,16 +393,25 @@ __global__ __launch_bounds__(256, 2) void matmul_kquant_i8_kernel(I8Args a) {
     const uint32_t aoff = (t0 + atok) * a.k + 64u * aq;
     const uint32_t doff = (t0 + atok) * (a.k / 256u) * 4u;
     const uint32_t j = n0 + 16u * wave + l16;
-    const uint32_t wrow = j * a.row_bytes;
+    uint32_t woff[WLOADS];
+#pragma unroll
+    for (uint32_t i = 0; i < WLOADS; i++) {
+        const uint32_t c = 64u * i + lane;
+        woff[i] = c < 16u * CPR ? (n0 + 16u * wave + c / CPR) * a.row_bytes + 16u * (c % CPR) : 0xfffffff0u - a.row_bytes;
+    }
 
     iu32x4 ra[4];
     uint32_t rd;
-    typename P::Raw cur, next;
-    auto fetch = [&](uint32_t k0, typename P::Raw &r) __attribute__((always_inline)) {
+    typename P::Raw cur;
+    // Step k0's operands: the tokens' bytes and scales into registers (stashed in LDS after the
+    // multiply), the weights straight into LDS buffer `buf`.
+    auto fetch = [&](uint32_t k0, uint32_t buf) __attribute__((always_inline)) {
 #pragma unroll
         for (uint32_t i = 0; i < 4; i++) ra[i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, aoff + k0 + 16u * i, 0, 0);
         rd = __builtin_amdgcn_raw_buffer_load_b32(dbuf, doff + k0 / 64u, 0, 0);
-        P::load(wbuf, wrow + k0 / 256u * P::BLOCK, g, r);
+        uint8_t *dst = lds_w + (buf * 4u + wave) * WSLOT;
+#pragma unroll
+        for (uint32_t i = 0; i < WLOADS; i++) load_lds_b128(wbuf, dst + 1024u * i, woff[i], k0 / 256u * P::BLOCK);
     };
     auto stash = [&](uint32_t buf) __attribute__((always_inline)) {
         uint8_t *line = &lds_q[buf][atok * LINE + 64u * aq];
@@ -402,17 +427,21 @@ __global__ __launch_bounds__(256, 2) void matmul_kquant_i8_kernel(I8Args a) {
 #pragma unroll
     for (int mt = 0; mt < 4; mt++) acc[mt] = if32x4{0.f, 0.f, 0.f, 0.f};
 
-    fetch(k_first, cur);
+    fetch(k_first, 0);
     stash(0);
-    __syncthreads();
+    sync_after_loads();
     for (uint32_t s = 0; s < steps; s++) {
         const uint32_t k0 = k_first + s * STEP, buf = s & 1u;
         const bool more = s + 1u < steps;
-        if (more) fetch(k0 + STEP, next);
+        P::load(lds_w + (buf * 4u + wave) * WSLOT + l16 * P::BLOCK, g, cur);
+        if (more) fetch(k0 + STEP, buf ^ 1u);
         // A block's units are summed in integers: a unit's exact sum times its 6- or 8-bit
         // scale (one 24-bit multiply-add a result), the minimums as one more matrix
         // instruction a unit whose second operand is the unit's minimum in all 32 positions,
-        // accumulated by the matrix cores. The block's two f32 scales are applied once.
+        // accumulated by the matrix cores. The block's two f32 scales are applied once. (The
+        // minimums' term as two matrix instructions a block, the tokens' unit sums against the
+        // rows' eight minimums, was tried: taking the sums while staging costs more than the six
+        // instructions it saves, 48.1 against 46.3 us for Q4_K.)
         i32x4 isum[4], msum[4];
 #pragma unroll
         for (int mt = 0; mt < 4; mt++) isum[mt] = msum[mt] = i32x4{0, 0, 0, 0};
@@ -474,13 +503,28 @@ __global__ __launch_bounds__(256, 2) void matmul_kquant_i8_kernel(I8Args a) {
                 acc[mt][i] = fmaf(dxv[i], part, acc[mt][i]);
             }
         }
-        if (more) {
-            stash(buf ^ 1u);
-            cur = next;
-        }
-        __syncthreads();
+        if (more) stash(buf ^ 1u);
+        sync_after_loads();
     }
     store_tile(a, acc, t0, j, g);
+}
+
+// The K-format kernel's weight buffers are dynamic LDS (with the static token buffers a
+// workgroup takes 57 - 66 KB, two workgroups a CU).
+template <class P>
+zhip_result launch_kquant(const Dispatch &d, const char *name, dim3 grid, const I8Args &a) {
+    constexpr uint32_t bytes = 2u * 4u * ((16u * (P::BLOCK / 16u) + 63u) / 64u) * 1024u;
+    auto kernel = matmul_kquant_i8_kernel<P>;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", name, bytes);
+        }
+        configured = true;
+    }
+    hipLaunchKernelGGL(kernel, grid, dim3(256), bytes, d.stream, a);
+    return check_launch(d, name);
 }
 
 }  // namespace
@@ -536,13 +580,13 @@ static zhip_result launch_int8(const Dispatch &d, const char *name, int type) {
     const dim3 grid((uint32_t)tiles_n, (uint32_t)tiles_t, (uint32_t)slices);
     const bool ragged = p.k % STEP != 0 || (p.k_slice < p.k && p.k_slice % STEP != 0);
     if (type == 3) {
-        hipLaunchKernelGGL(matmul_kquant_i8_kernel<I8Q3>, grid, dim3(256), 0, d.stream, a);
+        return launch_kquant<I8Q3>(d, name, grid, a);
     } else if (type == 4) {
-        hipLaunchKernelGGL(matmul_kquant_i8_kernel<I8Q4>, grid, dim3(256), 0, d.stream, a);
+        return launch_kquant<I8Q4>(d, name, grid, a);
     } else if (type == 5) {
-        hipLaunchKernelGGL(matmul_kquant_i8_kernel<I8Q5>, grid, dim3(256), 0, d.stream, a);
+        return launch_kquant<I8Q5>(d, name, grid, a);
     } else if (type == 6) {
-        hipLaunchKernelGGL(matmul_kquant_i8_kernel<I8Q6>, grid, dim3(256), 0, d.stream, a);
+        return launch_kquant<I8Q6>(d, name, grid, a);
     } else {
         if (ragged) hipLaunchKernelGGL(matmul_q8_0_i8_kernel<true>, grid, dim3(256), 0, d.stream, a);
         else hipLaunchKernelGGL(matmul_q8_0_i8_kernel<false>, grid, dim3(256), 0, d.stream, a);
