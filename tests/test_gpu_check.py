@@ -570,18 +570,20 @@ def test_matmul_bf16_mfma_tilings(ctx, rows, n, k):
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
 
 
-def test_matmul_q8_0_float_bf16_whole_steps_keep_token_bits(ctx):
-    """Q8_0 weights on the bf16 rung with k a multiple of 128 take the kernel with
-    producer waves and 32 x 32 x 16 MFMAs in 128- or 64-token tiles: a token's sums
-    are the same bits whichever tile height its step runs in and whichever tokens
-    share the step; ragged rows and outputs, a column offset and a padded stride."""
+@pytest.mark.parametrize("rung", ["bf16_mfma", "fp16_single"])
+def test_matmul_q8_0_float_bf16_whole_steps_keep_token_bits(ctx, rung):
+    """Q8_0 weights on the bf16 rung and on the reference's fp16_single rung with k a multiple
+    of 128 take the kernel with producer waves and 32 x 32 x 16 MFMAs in 128- or 64-token
+    tiles: a token's sums are the same bits whichever tile height its step runs in and
+    whichever tokens share the step; ragged rows and outputs, a column offset and a padded stride."""
     c = ctx
     rows, n, k, col0, stride = 300, 2830, 384, 3, 2840
     x = c.random(rows * k, 1).reshape(rows, k)
     raw, wq = quant_rows(c, TensorType.q8_0, n, k)
     wa = c.gpu_weights(TensorType.q8_0, raw, k)
-    c.set.select_prefill(c.rec, K.Prefill.bf16_mfma)
+    c.set.select_prefill(c.rec, K.Prefill[rung])
     init = c.random(rows * stride, 0.5).reshape(rows, stride)
+    narrow = synth.bf16_round if rung == "bf16_mfma" else (lambda v: v.astype(np.float16).astype(np.float32))
 
     def run(first, count):
         out = c.upload(init[first : first + count])
@@ -590,7 +592,7 @@ def test_matmul_q8_0_float_bf16_whole_steps_keep_token_bits(ctx):
         return c.read(out).reshape(count, stride)
 
     got = run(0, rows)  # three 128-token tiles on 45 column tiles: the tall tiling
-    want = init[:, col0 : col0 + n] + synth.bf16_round(x).astype(np.float64) @ synth.bf16_round(wq).astype(np.float64).T
+    want = init[:, col0 : col0 + n] + narrow(x).astype(np.float64) @ narrow(wq).astype(np.float64).T
     assert rel_err(got[:, col0 : col0 + n], want) <= 1e-5
     mask = np.ones(stride, dtype=bool)
     mask[col0 : col0 + n] = False

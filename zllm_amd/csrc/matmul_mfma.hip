@@ -546,7 +546,7 @@ zhip_result launch_mfma_wide(const Dispatch &d, const char *name, bool q8_0, con
 
 // Q8_0 weights on the bf16 rung over whole 128-deep steps (matmul_q8_bf16.hip).
 bool matmul_q8_bf16_accepts(uint32_t k, uint32_t k_slice, uint32_t slices);
-zhip_result launch_matmul_q8_bf16(const Dispatch &d, const char *name, const uint8_t *x, const uint8_t *w, float *out, uint32_t rows, uint32_t n,
+zhip_result launch_matmul_q8_bf16(const Dispatch &d, const char *name, bool f16, const uint8_t *x, const uint8_t *w, float *out, uint32_t rows, uint32_t n,
     uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, uint32_t row_bytes, uint32_t x_bytes, uint32_t w_bytes);
 
 template <class W, class H, int MT, bool RAGGED, bool COMP = false>
@@ -624,9 +624,10 @@ static zhip_result launch_mfma(const Dispatch &d, const char *name, bool sliced,
     // weight is converted once per 256 tokens and half the bytes cross from L2.
     if (kBf16Rung && slices == 1u && a.k_slice >= a.k && (uint64_t)((a.rows + 255u) / 256u) * ((a.n + 127u) / 128u) >= (uint64_t)d.dev->compute_units)
         return launch_mfma_wide(d, name, q8_0, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes);
-    if constexpr (std::is_same<W, WQ8_0>::value && std::is_same<H, Bf16>::value && !COMP) {
+    if constexpr (std::is_same<W, WQ8_0>::value && !COMP) {
         if (matmul_q8_bf16_accepts(a.k, a.k_slice, slices))
-            return launch_matmul_q8_bf16(d, name, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes, a.x_bytes, a.w_bytes);
+            return launch_matmul_q8_bf16(d, name, std::is_same<H, F16>::value, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes,
+                a.x_bytes, a.w_bytes);
     }
     const bool ragged = a.k % BK != 0 || a.k_slice % BK != 0;
     if constexpr (COMP) {

@@ -1,7 +1,8 @@
-// matmul_q8_0_float on the bf16 matrix cores for whole 128-deep k steps: the kernel the bf16
-// rung takes when k is a multiple of 128 and not sliced (same contract as matmul_mfma.hip:
-// out[t][col0 + j] (+)= sum_i bf16(x[t][i]) * bf16(q[j][i] * d[j][i / 32]), fp32 accumulate;
-// src/kernels/matmul_q8_0_float.wgsl:1-105 for the bindings and the parameter block).
+// matmul_q8_0_float on the matrix cores for whole 128-deep k steps: the kernel the bf16 rungs
+// and the fp16_single rung take when k is a multiple of 128 and not sliced (same contract as
+// matmul_mfma.hip: out[t][col0 + j] (+)= sum_i h(x[t][i]) * h(q[j][i] * d[j][i / 32]) with h the
+// rounding to bf16 or f16, fp32 accumulate; src/kernels/matmul_q8_0_float.wgsl:1-105 for the
+// bindings and the parameter block).
 //
 // What shapes it, measured on MI355X at 512 x 4096 x 4096:
 //  * A CU's tile is 128 tokens x 64 matrix rows (8192 outputs: the step's outputs over 256 CUs;
@@ -40,6 +41,8 @@ namespace {
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
@@ -66,10 +69,23 @@ struct Q8Args {
     uint32_t x_bytes, w_bytes;  // bytes the kernel may read behind x and w
 };
 
-__device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
-    const f32x2 v = {lo, hi};
-    return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-}
+// The operand type of a rung: two floats rounded into one word, and the matrix instruction.
+struct AsBf16 {
+    typedef bf16x8 vec;
+    static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+        const f32x2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
+    }
+    static __device__ __forceinline__ f32x16 mfma(vec a, vec b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
+};
+struct AsF16 {
+    typedef f16x8 vec;
+    static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
+        const f32x2 v = {lo, hi};
+        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
+    }
+    static __device__ __forceinline__ f32x16 mfma(vec a, vec b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
+};
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const uint8_t *base, uint32_t bytes) {
     return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, (int)bytes, 0x00020000);
 }
@@ -101,26 +117,28 @@ __device__ __forceinline__ uint32_t line_key(uint32_t row) { return (row & 7u) ^
 
 struct WRaw { u32x4 q; uint32_t d; };
 
-// Sixteen int8 weights times their block's scale (exact in f32), rounded once to bf16: the
-// first operands of the lane's two MFMAs.
-__device__ __forceinline__ void convert(const WRaw &r, bf16x8 &w0, bf16x8 &w1) {
+// Sixteen int8 weights times their block's scale (exact in f32), rounded once to the operand
+// type: the first operands of the lane's two MFMAs.
+template <class H>
+__device__ __forceinline__ void convert(const WRaw &r, typename H::vec &w0, typename H::vec &w1) {
     const float d = (float)__builtin_bit_cast(_Float16, (uint16_t)r.d);
     u32x4 lo, hi;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
         const int32_t v = (int32_t)r.q[i];
-        lo[2 * i] = pack_bf16((float)(int8_t)(v) * d, (float)(int8_t)(v >> 8) * d);
-        lo[2 * i + 1] = pack_bf16((float)(int8_t)(v >> 16) * d, (float)(v >> 24) * d);
+        lo[2 * i] = H::pack((float)(int8_t)(v) * d, (float)(int8_t)(v >> 8) * d);
+        lo[2 * i + 1] = H::pack((float)(int8_t)(v >> 16) * d, (float)(v >> 24) * d);
         const int32_t u = (int32_t)r.q[2 + i];
-        hi[2 * i] = pack_bf16((float)(int8_t)(u) * d, (float)(int8_t)(u >> 8) * d);
-        hi[2 * i + 1] = pack_bf16((float)(int8_t)(u >> 16) * d, (float)(u >> 24) * d);
+        hi[2 * i] = H::pack((float)(int8_t)(u) * d, (float)(int8_t)(u >> 8) * d);
+        hi[2 * i + 1] = H::pack((float)(int8_t)(u >> 16) * d, (float)(u >> 24) * d);
     }
-    w0 = __builtin_bit_cast(bf16x8, lo);
-    w1 = __builtin_bit_cast(bf16x8, hi);
+    w0 = __builtin_bit_cast(typename H::vec, lo);
+    w1 = __builtin_bit_cast(typename H::vec, hi);
 }
 
-template <int TT>
+template <int TT, class H>
 __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
+    typedef typename H::vec opvec;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int BM = 32 * TT, ABUF = abuf_bytes<TT>(), BUF = buf_bytes<TT>();
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -195,7 +213,7 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
     const uint32_t a_at0 = (kq >> 1) * (BM * 128) + lrow * 128u + 16u * ((4u * (kq & 1u) + 2u * h) ^ key);
     const uint32_t a_at1 = (kq >> 1) * (BM * 128) + lrow * 128u + 16u * ((4u * (kq & 1u) + 2u * h + 1u) ^ key);
 
-    bf16x8 tok[2][TT][2], wop[2][2];
+    opvec tok[2][TT][2], wop[2][2];
     auto read_frags = [&](uint32_t buf, auto set, WRaw &raw) __attribute__((always_inline)) {
         constexpr int S = decltype(set)::value;
         const uint8_t *base = lds + buf * BUF;
@@ -203,8 +221,8 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
         raw.d = *reinterpret_cast<const uint16_t *>(base + s_at);
 #pragma unroll
         for (int tt = 0; tt < TT; tt++) {
-            tok[S][tt][0] = *reinterpret_cast<const bf16x8 *>(base + a_at0 + 4096 * tt);
-            tok[S][tt][1] = *reinterpret_cast<const bf16x8 *>(base + a_at1 + 4096 * tt);
+            tok[S][tt][0] = *reinterpret_cast<const opvec *>(base + a_at0 + 4096 * tt);
+            tok[S][tt][1] = *reinterpret_cast<const opvec *>(base + a_at1 + 4096 * tt);
         }
     };
     auto multiply = [&](auto set) __attribute__((always_inline)) {
@@ -212,14 +230,14 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
 #pragma unroll
         for (int j = 0; j < 2; j++)
 #pragma unroll
-            for (int tt = 0; tt < TT; tt++) acc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wop[S][j], tok[S][tt][j], acc[tt], 0, 0, 0);
+            for (int tt = 0; tt < TT; tt++) acc[tt] = H::mfma(wop[S][j], tok[S][tt][j], acc[tt]);
     };
 
     sync_after_reads();  // step 0 has landed
     {
         WRaw raw;
         read_frags(0, std::integral_constant<int, 0>{}, raw);
-        convert(raw, wop[0][0], wop[0][1]);
+        convert<H>(raw, wop[0][0], wop[0][1]);
     }
     sync_after_reads();  // step 1 has landed, buffer 0 is free
 
@@ -232,7 +250,7 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
         WRaw raw;
         read_frags(NB, std::integral_constant<int, 1 - S>{}, raw);
         multiply(cur_set);
-        convert(raw, wop[1 - S][0], wop[1 - S][1]);
+        convert<H>(raw, wop[1 - S][0], wop[1 - S][1]);
         __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
 #pragma unroll
         for (int i = 0; i < 2 * TT; i++) {
@@ -329,9 +347,9 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
     }
 }
 
-template <int TT>
+template <int TT, class H>
 zhip_result launch_tile(const Dispatch &d, const char *name, const Q8Args &a) {
-    auto kernel = matmul_q8_bf16_kernel<TT>;
+    auto kernel = matmul_q8_bf16_kernel<TT, H>;
     constexpr int bytes = lds_bytes<TT>();
     static bool configured = false;
     if (!configured) {
@@ -352,7 +370,8 @@ zhip_result launch_tile(const Dispatch &d, const char *name, const Q8Args &a) {
 // validated the bindings).
 bool matmul_q8_bf16_accepts(uint32_t k, uint32_t k_slice, uint32_t slices) { return slices == 1u && k_slice >= k && k >= BK && k % BK == 0u; }
 
-zhip_result launch_matmul_q8_bf16(const Dispatch &d, const char *name, const uint8_t *x, const uint8_t *w, float *out, uint32_t rows, uint32_t n,
+// x: the activations packed two bytes a value, bf16 or (f16 = true) f16.
+zhip_result launch_matmul_q8_bf16(const Dispatch &d, const char *name, bool f16, const uint8_t *x, const uint8_t *w, float *out, uint32_t rows, uint32_t n,
     uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, uint32_t row_bytes, uint32_t x_bytes, uint32_t w_bytes) {
     Q8Args a{};
     a.x = x; a.w = w; a.out = out;
@@ -361,8 +380,9 @@ zhip_result launch_matmul_q8_bf16(const Dispatch &d, const char *name, const uin
     // 128-token tiles unless those leave half of the CUs idle: then 64-token tiles, which
     // convert every weight twice as often but run in one round on twice the CUs.
     const uint64_t tall = (uint64_t)((rows + 127u) / 128u) * ((n + BN - 1) / BN);
-    if (rows > 64u && 2u * tall > (uint64_t)d.dev->compute_units) return launch_tile<4>(d, name, a);
-    return launch_tile<2>(d, name, a);
+    const bool high = rows > 64u && 2u * tall > (uint64_t)d.dev->compute_units;
+    if (f16) return high ? launch_tile<4, AsF16>(d, name, a) : launch_tile<2, AsF16>(d, name, a);
+    return high ? launch_tile<4, AsBf16>(d, name, a) : launch_tile<2, AsBf16>(d, name, a);
 }
 
 }  // namespace zhip
