@@ -33,7 +33,7 @@ namespace {
 constexpr uint32_t TT = 64;     // tokens per workgroup
 constexpr uint32_t TN = 64;     // rows per workgroup
 constexpr uint32_t STEP = 256;  // positions per step
-constexpr uint32_t LINE = STEP + 8;  // bytes between register-staged token lines in LDS
+constexpr uint32_t LINE = STEP + 16;  // bytes between register-staged token lines in LDS: sixteen tokens' 8-byte reads of two lane groups cover all banks
 constexpr uint32_t UNITS = 1;  // units the K-format kernel schedules together (2 and 4 measured no faster)
 
 struct I8Args {
@@ -509,6 +509,170 @@ __global__ __launch_bounds__(256, 2) void matmul_kquant_i8_kernel(I8Args a) {
     store_tile(a, acc, t0, j, g);
 }
 
+// ---- Q4_K and Q5_K, whole unsliced k: 32 x 32 x 32 matrix instructions ---------------------
+// The same arithmetic on tiles of 32 tokens x 64 rows, two waves a workgroup (32 rows each, four
+// workgroups a CU): v_mfma_i32_32x32x32_i8 does a unit of 32 x 32 outputs in half the time four
+// 16 x 16 x 32 take, and matrix and vector instructions of a SIMD do not overlap here, so the
+// matrix instructions' own time counts. Lane l holds row l % 32 of its wave and positions
+// 16 (l / 32) .. + 15 of a unit. Tokens and weights both arrive in LDS by whole-line direct
+// loads, a step ahead: token lines unpadded with their 16-byte chunks XOR-permuted (chunk c of
+// token t at position c ^ (t % 16): the fragment reads of sixteen tokens fall in sixteen bank
+// groups), a wave's 32 rows' blocks as stored.
+typedef int i32x16 __attribute__((ext_vector_type(16)));
+
+struct W16Q4 {
+    static constexpr uint32_t BLOCK = 144;
+    struct Raw {
+        iu32x4 h;      // d, dmin and the twelve scale bytes
+        iu32x4 q[4];   // the lane's 16 bytes of each 64-weight chunk: low nibbles unit 2c, high 2c + 1
+    };
+    static __device__ __forceinline__ void load(const uint8_t *blk, uint32_t h, Raw &r) {
+        r.h = *reinterpret_cast<const iu32x4 *>(blk);
+#pragma unroll
+        for (uint32_t c = 0; c < 4; c++) r.q[c] = *reinterpret_cast<const iu32x4 *>(blk + 16u + 32u * c + 16u * h);
+    }
+    static __device__ __forceinline__ iu32x4 unit(const Raw &r, uint32_t u) {
+        iu32x4 b = r.q[u >> 1];
+        if (u & 1u) b = b >> 4;
+        return b & 0x0f0f0f0fu;
+    }
+};
+
+struct W16Q5 {
+    static constexpr uint32_t BLOCK = 176;
+    struct Raw {
+        iu32x4 h;
+        iu32x4 qh;     // the fifth bits of positions 16 h .. + 15, bit u for unit u
+        iu32x4 q[4];
+    };
+    static __device__ __forceinline__ void load(const uint8_t *blk, uint32_t h, Raw &r) {
+        r.h = *reinterpret_cast<const iu32x4 *>(blk);
+        r.qh = *reinterpret_cast<const iu32x4 *>(blk + 16u + 16u * h);
+#pragma unroll
+        for (uint32_t c = 0; c < 4; c++) r.q[c] = *reinterpret_cast<const iu32x4 *>(blk + 48u + 32u * c + 16u * h);
+    }
+    static __device__ __forceinline__ iu32x4 unit(const Raw &r, uint32_t u) {
+        iu32x4 b = r.q[u >> 1];
+        if (u & 1u) b = b >> 4;
+        return (b & 0x0f0f0f0fu) | (((r.qh >> u) & 0x01010101u) << 4);
+    }
+};
+
+constexpr uint32_t WT = 32, WN = 64;  // tokens and rows of a workgroup of the wide kernel
+template <class P> constexpr uint32_t wide_wslot() { return ((32u * (P::BLOCK / 16u) + 63u) / 64u) * 1024u; }
+template <class P> constexpr uint32_t wide_buffer() { return WT * 256u + 2u * wide_wslot<P>(); }
+
+template <class P>
+__global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_wide[];  // two buffers: token lines, two waves' blocks (token scales behind the first's)
+    constexpr uint32_t CPR = P::BLOCK / 16u, WLOADS = (32u * CPR + 63u) / 64u, WSLOT = wide_wslot<P>(), BUF = wide_buffer<P>();
+    // The token scales land behind wave 0's rows, where the idle lanes of its last weight load put
+    // zeros: the same wave asks for them after that load, and loads land in the order asked.
+    constexpr uint32_t W_AT = WT * 256u, DX_AT = W_AT + 32u * P::BLOCK;
+    static_assert(WSLOT >= 32u * P::BLOCK + 256u, "the token scales need 256 bytes behind the first wave's blocks");
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, lrow = lane & 31u, h = lane >> 5;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t n0 = blockIdx.x * WN, t0 = blockIdx.y * WT;
+    const uint32_t steps = a.k / 256u;
+    const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.qx, a.qx_bytes), wbuf = make_buffer(a.w, a.w_bytes), dbuf = make_buffer(a.dx, a.dx_bytes);
+
+    // Loads of a step. Tokens: load i of this wave brings tokens 4 (4 wave + i) .. + 3, lane l
+    // token l / 16 of them and the chunk that belongs at position l % 16. Token scales: wave 0,
+    // lanes below 32 a token each (the others ask past the buffer). Weights: the wave's 32 rows.
+    uint32_t xoff[4], woff[WLOADS];
+#pragma unroll
+    for (uint32_t i = 0; i < 4; i++) {
+        const uint32_t t = 4u * (4u * wave + i) + (lane >> 4);
+        xoff[i] = (t0 + t) * a.k + 16u * ((lane & 15u) ^ (t & 15u));
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < WLOADS; i++) {
+        const uint32_t c = 64u * i + lane;
+        woff[i] = c < 32u * CPR ? (n0 + 32u * wave + c / CPR) * a.row_bytes + 16u * (c % CPR) : 0xfffffff0u - a.row_bytes;
+    }
+    const uint32_t doff = lane < 32u ? (t0 + lane) * (a.k / 256u) * 4u : 0xfffffff0u - a.k;
+    auto fetch = [&](uint32_t s, uint32_t buf) __attribute__((always_inline)) {
+        uint8_t *base = lds_wide + buf * BUF;
+#pragma unroll
+        for (uint32_t i = 0; i < 4; i++) load_lds_b128(xbuf, base + 1024u * (4u * wave + i), xoff[i], 256u * s);
+#pragma unroll
+        for (uint32_t i = 0; i < WLOADS; i++) load_lds_b128(wbuf, base + W_AT + wave * WSLOT + 1024u * i, woff[i], s * P::BLOCK);
+        if (wave == 0u) load_lds_b32(dbuf, base + DX_AT, doff + 4u * s);
+    };
+
+    float acc[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.f;
+    const uint32_t a_line = lrow * 256u, a_key = lrow & 15u;
+
+    fetch(0, 0);
+    sync_after_loads();
+    for (uint32_t s = 0; s < steps; s++) {
+        const uint32_t buf = s & 1u;
+        const uint8_t *base = lds_wide + buf * BUF;
+        typename P::Raw cur;
+        P::load(base + W_AT + wave * WSLOT + lrow * P::BLOCK, h, cur);
+        if (s + 1u < steps) fetch(s + 1u, buf ^ 1u);
+        // A block's units are summed in integers (a unit's exact sum times its 6-bit scale, one
+        // 24-bit multiply-add a result; the minimums by one more matrix instruction a unit whose
+        // second operand is the unit's minimum in all 32 positions, accumulated by the matrix
+        // cores), and the block's two f32 scales are applied once.
+        i32x16 isum = {}, msum = {};
+#pragma unroll
+        for (uint32_t u = 0; u < 8; u++) {
+            const uint2 sm = scale_min_k4(cur.h.y, cur.h.z, cur.h.w, u);
+            const iu32x4 w16 = P::unit(cur, u);
+            const uint32_t m4 = sm.y * 0x01010101u;
+            const i32x4 af = *reinterpret_cast<const i32x4 *>(base + a_line + 16u * ((2u * u + h) ^ a_key));
+            const i32x16 zero = {};
+            const i32x16 is = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, w16), zero, 0, 0, 0);
+            msum = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, iu32x4{m4, m4, m4, m4}), msum, 0, 0, 0);
+#pragma unroll
+            for (int e = 0; e < 16; e++) isum[e] = __mul24((int)sm.x, is[e]) + isum[e];
+        }
+        const float d = half_bits_to_float(cur.h.x & 0xffffu), dmin = half_bits_to_float(cur.h.x >> 16);
+        // The lane's sixteen results are tokens 8 j + 4 h + i, j < 4, i < 4, of its row.
+#pragma unroll
+        for (uint32_t jj = 0; jj < 4; jj++) {
+            const if32x4 dxv = *reinterpret_cast<const if32x4 *>(base + DX_AT + 4u * (8u * jj + 4u * h));
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const int e = 4 * jj + i;
+                const float part = fmaf(-dmin, (float)msum[e], d * (float)isum[e]);
+                acc[e] = fmaf(dxv[i], part, acc[e]);
+            }
+        }
+        sync_after_loads();
+    }
+    const uint32_t j = n0 + 32u * wave + lrow;
+    if (j >= a.n) return;
+    float *out = a.out + a.col0 + j;
+#pragma unroll
+    for (uint32_t e = 0; e < 16; e++) {
+        const uint32_t t = t0 + 8u * (e >> 2) + 4u * h + (e & 3u);
+        if (t >= a.rows) continue;
+        float *o = out + (size_t)t * a.out_stride;
+        *o = a.accumulate ? *o + acc[e] : acc[e];
+    }
+}
+
+template <class P>
+zhip_result launch_kquant_wide(const Dispatch &d, const char *name, const I8Args &a) {
+    constexpr uint32_t bytes = 2u * wide_buffer<P>();
+    auto kernel = matmul_kquant_i8_wide_kernel<P>;
+    static bool configured = false;
+    if (!configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", name, bytes);
+        }
+        configured = true;
+    }
+    const dim3 grid((a.n + WN - 1u) / WN, (a.rows + WT - 1u) / WT);
+    hipLaunchKernelGGL(kernel, grid, dim3(128), bytes, d.stream, a);
+    return check_launch(d, name);
+}
+
 // The K-format kernel's weight buffers are dynamic LDS (with the static token buffers a
 // workgroup takes 57 - 66 KB, two workgroups a CU).
 template <class P>
@@ -579,6 +743,9 @@ static zhip_result launch_int8(const Dispatch &d, const char *name, int type) {
             a.w_bytes, a.dx_bytes);
     const dim3 grid((uint32_t)tiles_n, (uint32_t)tiles_t, (uint32_t)slices);
     const bool ragged = p.k % STEP != 0 || (p.k_slice < p.k && p.k_slice % STEP != 0);
+    const bool whole = slices == 1u && p.k_slice >= p.k;
+    if (whole && type == 4) return launch_kquant_wide<W16Q4>(d, name, a);
+    if (whole && type == 5) return launch_kquant_wide<W16Q5>(d, name, a);
     if (type == 3) {
         return launch_kquant<I8Q3>(d, name, grid, a);
     } else if (type == 4) {
