@@ -514,7 +514,7 @@ __global__ __launch_bounds__(256, 2) void matmul_kquant_i8_kernel(I8Args a) {
 // workgroups a CU): v_mfma_i32_32x32x32_i8 does a unit of 32 x 32 outputs in half the time four
 // 16 x 16 x 32 take, and matrix and vector instructions of a SIMD do not overlap here, so the
 // matrix instructions' own time counts. Lane l holds row l % 32 of its wave and positions
-// 16 (l / 32) .. + 15 of a unit. Tokens and weights both arrive in LDS by whole-line direct
+// 16 (l / 32) .. + 15 of a unit (Q4_K, Q5_K). Tokens and weights both arrive in LDS by whole-line direct
 // loads, a step ahead: token lines unpadded with their 16-byte chunks XOR-permuted (chunk c of
 // token t at position c ^ (t % 16): the fragment reads of sixteen tokens fall in sixteen bank
 // groups), a wave's 32 rows' blocks as stored.
@@ -558,23 +558,58 @@ struct W16Q5 {
     }
 };
 
-constexpr uint32_t WT = 32, WN = 64;  // tokens and rows of a workgroup of the wide kernel
-template <class P> constexpr uint32_t wide_wslot() { return ((32u * (P::BLOCK / 16u) + 63u) / 64u) * 1024u; }
-template <class P> constexpr uint32_t wide_buffer() { return WT * 256u + 2u * wide_wslot<P>(); }
+// Q6_K and Q3_K have a scale per sixteen weights: a unit is two v_mfma_i32_32x32x16_i8, lane l
+// holding positions 8 (l / 32) .. + 7 of each half. The formats' readers above serve: their
+// lane group g of four becomes h (first half) and 2 + h (second half).
+struct W8Q6 {
+    static constexpr uint32_t BLOCK = I8Q6::BLOCK;
+    struct Raw { I8Q6::Raw half[2]; };
+    static __device__ __forceinline__ void load(const uint8_t *blk, uint32_t h, Raw &r) {
+        I8Q6::load(blk, h, r.half[0]);
+        I8Q6::load(blk, 2u + h, r.half[1]);
+    }
+    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t h, iu32x2 (&b)[2], int (&sc)[2]) {
+        int s0, s1, mn;
+        I8Q6::unit(r.half[0], u, h, b[0], s0, s1, mn);
+        sc[0] = s0;
+        I8Q6::unit(r.half[1], u, 2u + h, b[1], s0, s1, mn);
+        sc[1] = s1;
+    }
+    static __device__ __forceinline__ float scale(const Raw &r) { return half_bits_to_float(r.half[0].d & 0xffffu); }
+};
+struct W8Q3 {
+    static constexpr uint32_t BLOCK = I8Q3::BLOCK;
+    struct Raw { I8Q3::Raw all; };
+    static __device__ __forceinline__ void load(const uint8_t *blk, uint32_t h, Raw &r) { I8Q3::load(blk, h, r.all); }
+    static __device__ __forceinline__ void unit(const Raw &r, uint32_t u, uint32_t h, iu32x2 (&b)[2], int (&sc)[2]) {
+        int s0, s1, mn;
+        I8Q3::unit(r.all, u, h, b[0], s0, s1, mn);
+        sc[0] = s0;
+        I8Q3::unit(r.all, u, 2u + h, b[1], s0, s1, mn);
+        sc[1] = s1;
+    }
+    static __device__ __forceinline__ float scale(const Raw &r) { return half_bits_to_float(r.all.u[0].w >> 16); }
+};
 
-template <class P>
+constexpr uint32_t WT = 32, WN = 64;  // tokens and rows of a workgroup of the wide kernel
+// LDS of a workgroup: two token buffers (32 lines of 256 bytes and 256 bytes of token scales)
+// and one slot of blocks per wave: a wave reads its rows' blocks into registers at the start of a
+// step and then asks for the next step's into the same slot, which nobody else reads.
+template <class P> constexpr uint32_t wide_wslot() { return ((32u * (P::BLOCK / 16u) + 63u) / 64u) * 1024u; }
+constexpr uint32_t WIDE_TOKENS = WT * 256u + 256u;
+template <class P> constexpr uint32_t wide_lds() { return 2u * WIDE_TOKENS + 2u * wide_wslot<P>(); }
+
+template <class P, bool HALVES>
 __global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
-    extern __shared__ __attribute__((aligned(16))) uint8_t lds_wide[];  // two buffers: token lines, two waves' blocks (token scales behind the first's)
-    constexpr uint32_t CPR = P::BLOCK / 16u, WLOADS = (32u * CPR + 63u) / 64u, WSLOT = wide_wslot<P>(), BUF = wide_buffer<P>();
-    // The token scales land behind wave 0's rows, where the idle lanes of its last weight load put
-    // zeros: the same wave asks for them after that load, and loads land in the order asked.
-    constexpr uint32_t W_AT = WT * 256u, DX_AT = W_AT + 32u * P::BLOCK;
-    static_assert(WSLOT >= 32u * P::BLOCK + 256u, "the token scales need 256 bytes behind the first wave's blocks");
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_wide[];
+    constexpr uint32_t CPR = P::BLOCK / 16u, WLOADS = (32u * CPR + 63u) / 64u, WSLOT = wide_wslot<P>();
+    constexpr uint32_t DX_AT = WT * 256u, W_AT = 2u * WIDE_TOKENS;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, lrow = lane & 31u, h = lane >> 5;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t n0 = blockIdx.x * WN, t0 = blockIdx.y * WT;
     const uint32_t steps = a.k / 256u;
     const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.qx, a.qx_bytes), wbuf = make_buffer(a.w, a.w_bytes), dbuf = make_buffer(a.dx, a.dx_bytes);
+    uint8_t *slot = lds_wide + W_AT + wave * WSLOT;
 
     // Loads of a step. Tokens: load i of this wave brings tokens 4 (4 wave + i) .. + 3, lane l
     // token l / 16 of them and the chunk that belongs at position l % 16. Token scales: wave 0,
@@ -591,13 +626,15 @@ __global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
         woff[i] = c < 32u * CPR ? (n0 + 32u * wave + c / CPR) * a.row_bytes + 16u * (c % CPR) : 0xfffffff0u - a.row_bytes;
     }
     const uint32_t doff = lane < 32u ? (t0 + lane) * (a.k / 256u) * 4u : 0xfffffff0u - a.k;
-    auto fetch = [&](uint32_t s, uint32_t buf) __attribute__((always_inline)) {
-        uint8_t *base = lds_wide + buf * BUF;
+    auto fetch_tokens = [&](uint32_t s, uint32_t buf) __attribute__((always_inline)) {
+        uint8_t *base = lds_wide + buf * WIDE_TOKENS;
 #pragma unroll
         for (uint32_t i = 0; i < 4; i++) load_lds_b128(xbuf, base + 1024u * (4u * wave + i), xoff[i], 256u * s);
-#pragma unroll
-        for (uint32_t i = 0; i < WLOADS; i++) load_lds_b128(wbuf, base + W_AT + wave * WSLOT + 1024u * i, woff[i], s * P::BLOCK);
         if (wave == 0u) load_lds_b32(dbuf, base + DX_AT, doff + 4u * s);
+    };
+    auto fetch_weights = [&](uint32_t s) __attribute__((always_inline)) {
+#pragma unroll
+        for (uint32_t i = 0; i < WLOADS; i++) load_lds_b128(wbuf, slot + 1024u * i, woff[i], s * P::BLOCK);
     };
 
     float acc[16];
@@ -605,32 +642,58 @@ __global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
     for (int e = 0; e < 16; e++) acc[e] = 0.f;
     const uint32_t a_line = lrow * 256u, a_key = lrow & 15u;
 
-    fetch(0, 0);
+    fetch_tokens(0, 0);
+    fetch_weights(0);
     sync_after_loads();
     for (uint32_t s = 0; s < steps; s++) {
         const uint32_t buf = s & 1u;
-        const uint8_t *base = lds_wide + buf * BUF;
+        const uint8_t *base = lds_wide + buf * WIDE_TOKENS;
         typename P::Raw cur;
-        P::load(base + W_AT + wave * WSLOT + lrow * P::BLOCK, h, cur);
-        if (s + 1u < steps) fetch(s + 1u, buf ^ 1u);
-        // A block's units are summed in integers (a unit's exact sum times its 6-bit scale, one
-        // 24-bit multiply-add a result; the minimums by one more matrix instruction a unit whose
+        P::load(slot + lrow * P::BLOCK, h, cur);
+        if (s + 1u < steps) {
+            fetch_tokens(s + 1u, buf ^ 1u);
+            // The slot is refilled once this wave's reads of it have returned; the compiler, which
+            // sees no dependency between the two, must not move the loads up.
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            fetch_weights(s + 1u);
+        }
+        // A block's units are summed in integers (a unit's exact sum times its scale, one 24-bit
+        // multiply-add a result; Q4_K / Q5_K minimums by one more matrix instruction a unit whose
         // second operand is the unit's minimum in all 32 positions, accumulated by the matrix
-        // cores), and the block's two f32 scales are applied once.
+        // cores), and the block's f32 scales are applied once.
         i32x16 isum = {}, msum = {};
+        const i32x16 zero = {};
 #pragma unroll
         for (uint32_t u = 0; u < 8; u++) {
-            const uint2 sm = scale_min_k4(cur.h.y, cur.h.z, cur.h.w, u);
-            const iu32x4 w16 = P::unit(cur, u);
-            const uint32_t m4 = sm.y * 0x01010101u;
-            const i32x4 af = *reinterpret_cast<const i32x4 *>(base + a_line + 16u * ((2u * u + h) ^ a_key));
-            const i32x16 zero = {};
-            const i32x16 is = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, w16), zero, 0, 0, 0);
-            msum = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, iu32x4{m4, m4, m4, m4}), msum, 0, 0, 0);
+            if constexpr (HALVES) {
+                iu32x2 w8[2];
+                int sc[2];
+                P::unit(cur, u, h, w8, sc);
 #pragma unroll
-            for (int e = 0; e < 16; e++) isum[e] = __mul24((int)sm.x, is[e]) + isum[e];
+                for (uint32_t half = 0; half < 2; half++) {
+                    const long af = *reinterpret_cast<const long *>(base + a_line + 16u * ((2u * u + half) ^ a_key) + 8u * h);
+                    const i32x16 is = __builtin_amdgcn_mfma_i32_32x32x16_i8(af, as_operand(w8[half]), zero, 0, 0, 0);
+#pragma unroll
+                    for (int e = 0; e < 16; e++) isum[e] = __mul24(sc[half], is[e]) + isum[e];
+                }
+            } else {
+                const uint2 sm = scale_min_k4(cur.h.y, cur.h.z, cur.h.w, u);
+                const iu32x4 w16 = P::unit(cur, u);
+                const uint32_t m4 = sm.y * 0x01010101u;
+                const i32x4 af = *reinterpret_cast<const i32x4 *>(base + a_line + 16u * ((2u * u + h) ^ a_key));
+                const i32x16 is = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, w16), zero, 0, 0, 0);
+                msum = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, iu32x4{m4, m4, m4, m4}), msum, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 16; e++) isum[e] = __mul24((int)sm.x, is[e]) + isum[e];
+            }
         }
-        const float d = half_bits_to_float(cur.h.x & 0xffffu), dmin = half_bits_to_float(cur.h.x >> 16);
+        float d, dmin = 0.f;
+        if constexpr (HALVES) {
+            d = P::scale(cur);
+        } else {
+            d = half_bits_to_float(cur.h.x & 0xffffu);
+            dmin = half_bits_to_float(cur.h.x >> 16);
+        }
         // The lane's sixteen results are tokens 8 j + 4 h + i, j < 4, i < 4, of its row.
 #pragma unroll
         for (uint32_t jj = 0; jj < 4; jj++) {
@@ -638,7 +701,8 @@ __global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
 #pragma unroll
             for (int i = 0; i < 4; i++) {
                 const int e = 4 * jj + i;
-                const float part = fmaf(-dmin, (float)msum[e], d * (float)isum[e]);
+                float part = d * (float)isum[e];
+                if (!HALVES) part = fmaf(-dmin, (float)msum[e], part);
                 acc[e] = fmaf(dxv[i], part, acc[e]);
             }
         }
@@ -656,10 +720,10 @@ __global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
     }
 }
 
-template <class P>
+template <class P, bool HALVES>
 zhip_result launch_kquant_wide(const Dispatch &d, const char *name, const I8Args &a) {
-    constexpr uint32_t bytes = 2u * wide_buffer<P>();
-    auto kernel = matmul_kquant_i8_wide_kernel<P>;
+    constexpr uint32_t bytes = wide_lds<P>();
+    auto kernel = matmul_kquant_i8_wide_kernel<P, HALVES>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
@@ -744,8 +808,10 @@ static zhip_result launch_int8(const Dispatch &d, const char *name, int type) {
     const dim3 grid((uint32_t)tiles_n, (uint32_t)tiles_t, (uint32_t)slices);
     const bool ragged = p.k % STEP != 0 || (p.k_slice < p.k && p.k_slice % STEP != 0);
     const bool whole = slices == 1u && p.k_slice >= p.k;
-    if (whole && type == 4) return launch_kquant_wide<W16Q4>(d, name, a);
-    if (whole && type == 5) return launch_kquant_wide<W16Q5>(d, name, a);
+    if (whole && type == 4) return launch_kquant_wide<W16Q4, false>(d, name, a);
+    if (whole && type == 5) return launch_kquant_wide<W16Q5, false>(d, name, a);
+    if (whole && type == 6) return launch_kquant_wide<W8Q6, true>(d, name, a);
+    if (whole && type == 3) return launch_kquant_wide<W8Q3, true>(d, name, a);
     if (type == 3) {
         return launch_kquant<I8Q3>(d, name, grid, a);
     } else if (type == 4) {
