@@ -663,6 +663,15 @@ __global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
         // cores), and the block's f32 scales are applied once.
         i32x16 isum = {}, msum = {};
         const i32x16 zero = {};
+        // The eight 6-bit scales and minimums of a Q4_K / Q5_K block as bytes of four words
+        // (src/ref/tensor.zig:94-98), unpacked four at a time.
+        uint32_t sc4[2] = {0u, 0u}, mn4[2] = {0u, 0u};
+        if constexpr (!HALVES) {
+            sc4[0] = cur.h.y & 0x3f3f3f3fu;
+            mn4[0] = cur.h.z & 0x3f3f3f3fu;
+            sc4[1] = (cur.h.w & 0x0f0f0f0fu) | ((cur.h.y >> 2) & 0x30303030u);
+            mn4[1] = ((cur.h.w >> 4) & 0x0f0f0f0fu) | ((cur.h.z >> 2) & 0x30303030u);
+        }
 #pragma unroll
         for (uint32_t u = 0; u < 8; u++) {
             if constexpr (HALVES) {
@@ -677,14 +686,14 @@ __global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
                     for (int e = 0; e < 16; e++) isum[e] = __mul24(sc[half], is[e]) + isum[e];
                 }
             } else {
-                const uint2 sm = scale_min_k4(cur.h.y, cur.h.z, cur.h.w, u);
+                const int scale = (int)((sc4[u >> 2] >> (8u * (u & 3u))) & 0xffu);
                 const iu32x4 w16 = P::unit(cur, u);
-                const uint32_t m4 = sm.y * 0x01010101u;
+                const uint32_t m4 = __builtin_amdgcn_perm(0u, mn4[u >> 2], 0x01010101u * (u & 3u));  // the unit's minimum in every byte
                 const i32x4 af = *reinterpret_cast<const i32x4 *>(base + a_line + 16u * ((2u * u + h) ^ a_key));
                 const i32x16 is = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, w16), zero, 0, 0, 0);
                 msum = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, iu32x4{m4, m4, m4, m4}), msum, 0, 0, 0);
 #pragma unroll
-                for (int e = 0; e < 16; e++) isum[e] = __mul24((int)sm.x, is[e]) + isum[e];
+                for (int e = 0; e < 16; e++) isum[e] = __mul24(scale, is[e]) + isum[e];
             }
         }
         float d, dmin = 0.f;
