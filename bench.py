@@ -405,6 +405,22 @@ def bench_floor(env):
         for sbuf in srcs + [dst]:
             rec.destroy(cmd.Kind.buffer, sbuf.buffer)
         env["flush"]()
+    # A read-only stream of the headline's size through the lightest decode multiply the path
+    # has: matvec_bf16 over a 33 MB bf16 matrix (two bytes and one FMA a weight, rows as long as
+    # C2's), one launch a step like C2. What this takes is what a single launch reading 33 MB
+    # takes here, whatever the format.
+    synth, oracle, TensorType = env["synth"], env["oracle"], env["TensorType"]
+    n, k = 4040, 4096
+    g = synth.rng(0xF100)
+    wbits = synth.bf16_matrix(g, n, k, 0.02)
+    x = synth.activations(g, 1, k, bf16=True)
+    launches, out = env["matvec_workload"](TensorType.bf16, wbits, n, k, 1, False, x)
+    wall, gpu_s, steps = env["protocol"](launches)
+    got = env["read"](out)[:n].reshape(1, n)
+    w = synth.bf16_bits_to_f32(wbits)
+    rel = float(np.max(np.abs(got - oracle.matmul_f64(x, w))) / np.max(np.abs(oracle.matmul_f64(x, w))))
+    res["read_33MB_bf16_matvec"] = env["hbm_entry"](f"matvec_bf16 M=1 K={k} N={n}: a read of 33 MB in one launch", 2 * n * k + 4 * k + 4 * n, wall, gpu_s, steps,
+                                                    {"copies": len(launches), "max_err_over_max_want": rel})
     return res
 
 
