@@ -156,6 +156,29 @@ def test_c5_lm_head_decode(ctx):
     assert int(np.argmax(got[0])) == oracle.argmax(ref[0])
 
 
+@pytest.mark.parametrize("norm", [False, True])
+def test_c5_lm_head_verify_width(ctx, norm):
+    """bf16 lm_head, K=1024, N=151936, M=8 (a speculative verify step through the decode multiply,
+    plain and with the final RMSNorm fused in): logits and every row's argmax."""
+    n, k, m, eps = 151936, 1024, 8, 1e-6
+    g = synth.rng(0xC5)
+    wbits = synth.bf16_matrix(g, n, k, 0.02)
+    x = synth.activations(g, m, k, bf16=not norm)
+    nw = (1.0 + 0.1 * g.standard_normal(k)).astype(np.float32) if norm else None
+    got = decode_matvec(ctx, TensorType.bf16, wbits, n, k, x, norm_w=nw, eps=eps)
+    w = synth.bf16_bits_to_f32(wbits)
+    xin = x
+    if norm:
+        x64 = x.astype(np.float64)
+        xin = (x64 / np.sqrt(np.mean(x64 * x64, axis=1, keepdims=True) + eps) * nw.astype(np.float64)).astype(np.float32)
+    want = oracle.matmul_f64(xin, w) if not norm else xin.astype(np.float64) @ w.astype(np.float64).T
+    assert bound_err(got, want, w, xin) <= 1e-3
+    assert rel_err(got, want) <= 1e-5
+    if not norm:
+        ref = oracle.matmul(x, oracle.Matrix(oracle.BF16, wbits, n, k, oracle.default_threads()), oracle.default_threads())
+        assert np.array_equal(np.argmax(got, axis=1), np.array([oracle.argmax(r) for r in ref]))
+
+
 @pytest.mark.parametrize("rung", [K.Prefill.bf16_mfma_xbf16, K.Prefill.scalar_f32])
 def test_c5_lm_head_prefill(ctx, rung):
     """bf16 lm_head, K=1024, N=151936, M=128: argmax of every row."""

@@ -85,6 +85,112 @@ def test_matvec_bf16_norm_accumulate(ctx, half):
     assert matvec_case(ctx, 1000, 37, True, half) <= 1e-5
 
 
+def bf16_tokens_case(c, m, n, k, col0=0, pad=0, accumulate=False, norm=False, x=None):
+    """A matvec_bf16 step of m tokens over n x k weights, writing columns col0 .. col0 + n of
+    rows n + col0 + pad wide; returns (got, want in float64, the launch's inputs)."""
+    eps, stride = 1e-6, col0 + n + pad
+    x = c.random(m * k, 3).reshape(m, k) if x is None else x
+    nw = c.random(k, 1)
+    bits, values = random_half(c, n * k, 1)
+    init = c.random(m * stride, 4).reshape(m, stride)
+    out = c.upload(init)
+    c.launcher().launch(Kernel.matvec_bf16, P.MatvecBf16(n=n, k=k, col0=col0, out_stride=stride, eps=eps, norm=norm, accumulate=accumulate),
+                        [c.upload(x), c.upload(bits), out, c.upload(nw)], (K.div_ceil(n, K.matvec_rows), m, 1))
+    got = c.read(out).reshape(m, stride)
+    want = init.astype(np.float64).copy()
+    prod = np.stack([norm_row(x[t], nw if norm else None, eps) @ values.reshape(n, k).astype(np.float64).T for t in range(m)])
+    want[:, col0 : col0 + n] = prod + (want[:, col0 : col0 + n] if accumulate else 0.0)
+    return got, want, (x, bits)
+
+
+# Steps of several tokens over k = 1024 ... 4096 in steps of 512 run on the matrix cores, the
+# weights read once for all tokens; every other shape keeps the one-token kernel's path.
+@pytest.mark.parametrize("m,n,k,col0,pad,accumulate,norm", [
+    (2, 64, 1024, 0, 0, False, False),
+    (8, 100, 1024, 0, 0, False, False),        # a ragged last unit of rows
+    (3, 37, 1536, 5, 3, True, False),          # unaligned columns, accumulate
+    (4, 8200, 2048, 0, 0, False, False),       # whole rounds of tiles and a tail on every workgroup
+    (5, 9000, 2560, 0, 0, False, True),        # the RMSNorm prologue
+    (7, 333, 3072, 32, 0, True, True),
+    (8, 520, 3584, 0, 0, False, False),
+    (6, 4040, 4096, 0, 0, False, False),
+    (11, 300, 1024, 0, 7, False, False),       # more than eight tokens: two launches
+    (19, 72, 4096, 8, 0, True, False),
+])
+def test_matvec_bf16_several_tokens(ctx, m, n, k, col0, pad, accumulate, norm):
+    got, want, _ = bf16_tokens_case(ctx, m, n, k, col0, pad, accumulate, norm)
+    assert rel_err(got, want) <= 1e-5
+    # Columns outside the launch's keep their contents bit for bit.
+    keep = np.ones(got.shape[1], dtype=bool)
+    keep[col0 : col0 + n] = False
+    assert np.array_equal(got[:, keep].astype(np.float32), want[:, keep].astype(np.float32))
+
+
+def test_matvec_bf16_several_tokens_many_rows(ctx):
+    """More than forty 32-row tiles on every workgroup: the outputs kept back in workgroup
+    memory are stored in the middle of the run, not only at its end."""
+    c = ctx
+    m, n, k = 2, 41 * 32 * c.device.caps.compute_units + 50, 1024
+    x = c.random(m * k, 3).reshape(m, k)
+    bits = synth.to_bf16_bits(c.rand.standard_normal(n * k, dtype=np.float32))
+    out = c.output(m * n)
+    c.launcher().launch(Kernel.matvec_bf16, P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, eps=1e-6),
+                        [c.upload(x), c.upload(bits), out, c.upload(np.ones(k, dtype=np.float32))], (K.div_ceil(n, K.matvec_rows), m, 1))
+    got = c.read(out).reshape(m, n)
+    want = x.astype(np.float64) @ synth.bf16_bits_to_f32(bits).reshape(n, k).astype(np.float64).T
+    assert rel_err(got, want) <= 1e-5
+
+
+def test_matvec_bf16_several_tokens_keep_token_bits(ctx):
+    """A token's outputs do not depend on how many tokens share the step (from two tokens
+    up), nor on where the step's columns start."""
+    c = ctx
+    m, n, k = 13, 1000, 2048
+    x = c.random(m * k, 3).reshape(m, k)
+    bits, _ = random_half(c, n * k, 1)
+    wa = c.upload(bits)
+
+    def run(tokens, rows0, rows):
+        out = c.output(len(tokens) * rows)
+        wpart = c.upload(bits.reshape(n, k)[rows0 : rows0 + rows])
+        c.launcher().launch(Kernel.matvec_bf16, P.MatvecBf16(n=rows, k=k, col0=0, out_stride=rows, eps=1e-6),
+                            [c.upload(x[tokens]), wpart, out, c.upload(np.ones(k, dtype=np.float32))], (K.div_ceil(rows, K.matvec_rows), len(tokens), 1))
+        return c.read(out).reshape(len(tokens), rows)
+
+    whole = run(list(range(m)), 0, n)
+    assert np.array_equal(run([4, 9], 0, n), whole[[4, 9]])
+    assert np.array_equal(run([12, 0, 5, 7, 3], 0, n), whole[[12, 0, 5, 7, 3]])
+    assert np.array_equal(run(list(range(8)), 424, 576), whole[:8, 424:])
+    del wa
+
+
+def test_matvec_bf16_several_tokens_special_values(ctx):
+    """Inputs the three-way split must carry exactly: full 24-bit mantissas (integer inputs
+    against weights of +-1, where every partial sum is an integer f32 holds, so the result is
+    exact whatever the order of the additions), the largest finite value, infinities and NaNs."""
+    c = ctx
+    m, n, k = 4, 64, 1024
+    x = np.zeros((m, k), dtype=np.float32)
+    r = c.rand.integers(0, 2000, size=k)
+    x[0] = (2 ** 24 - 2048 + r).astype(np.float32)                 # 24 significant bits each
+    x[1, :8] = [3.4028235e38, -3.4028235e38, 1.1754944e-38, 16777215.0, -0.0, 1e-30, 5e37, -1.0000001]
+    x[2, 3] = np.inf
+    x[3, 5] = np.nan
+    w = np.empty((n, k), dtype=np.float32)
+    w[:32] = np.where(np.arange(k) % 2 == 0, 1.0, -1.0)
+    w[32:] = 0.5
+    w[32:, 1] = -0.25
+    out = c.output(m * n)
+    c.launcher().launch(Kernel.matvec_bf16, P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, eps=1e-6),
+                        [c.upload(x), c.upload(synth.to_bf16_bits(w.reshape(-1))), out, c.upload(np.ones(k, dtype=np.float32))], (K.div_ceil(n, K.matvec_rows), m, 1))
+    got = c.read(out).reshape(m, n)
+    assert np.array_equal(got[0, :32], np.full(32, float(np.sum(r[0::2]) - np.sum(r[1::2])), dtype=np.float32))
+    want1 = x[1].astype(np.float64) @ w[32:].astype(np.float64).T  # 0.5 * max - 0.25 * (-max) stays finite in f32
+    assert np.all(np.isfinite(got[1, 32:])) and np.max(np.abs(got[1, 32:] - want1)) <= 1e-6 * np.max(np.abs(want1))
+    assert np.all(np.isposinf(got[2, 32:]))
+    assert np.all(np.isnan(got[3]))
+
+
 @pytest.mark.parametrize("half", HALVES)
 def test_matvec_bf16_silu_pair(ctx, half):
     c = ctx

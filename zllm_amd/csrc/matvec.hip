@@ -221,6 +221,9 @@ zhip_result launch_matvec_q4k_mfma_resident(const Dispatch &d, const MvArgs &a, 
 // The matrix-core variant of matvec_q8_0 for k of 2048 or 4096 (matvec_q8_mfma_stream.hip).
 bool matvec_q8_mfma_stream_accepts(const MvArgs &a);
 zhip_result launch_matvec_q8_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
+// matvec_bf16 on the matrix cores, the weights read once for all tokens (matvec_bf16_mfma_stream.hip).
+bool matvec_bf16_mfma_stream_accepts(const MvArgs &a);
+zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
 // The matrix-core variant of matvec_q8_0 (matmul_mfma.hip).
 zhip_result launch_matvec_q8_0_mfma(const Dispatch &d, const MvArgs &a);
 // The tuned multiply (matvec_quant.hip): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
@@ -317,7 +320,12 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     // (On matvec_q8_0 only where the kernel that streams whole tiles takes the step: the other
     // matrix-core kernel of that operation narrows its inputs into the same workspace.)
     const bool prepass = D::CHUNK == 4 ? p.k % 1024u == 0 : ((p.k == 2048u || p.k == 4096u) && a.rows % 16u == 0 && !pair);
-    if (matrix_cores && (norm || a.act_div > 0.f) && a.m <= 8u && prepass) {
+    // matvec_bf16 steps of several tokens go to the kernel that reads the weights once for all
+    // of them; it too takes its inputs as they are.
+    MvArgs bare = a;
+    bare.flags &= ~FLAG_NORM;
+    const bool bf16_stream = std::is_same<D, DecBF16>::value && a.m >= 2u && matvec_bf16_mfma_stream_accepts(bare);
+    if ((matrix_cores && (norm || a.act_div > 0.f) && a.m <= 8u && prepass) || (bf16_stream && norm)) {
         if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", D::name());
         const uint64_t bytes = (uint64_t)a.m * p.k * 4u;
         if (zhip_result r = d.work->reserve(d, bytes)) return r;
@@ -332,6 +340,7 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
         v.act_div = 0u;
     }
     const bool plain = !(a.flags & FLAG_NORM) && a.act_div == 0.f;
+    if (bf16_stream) return launch_matvec_bf16_mfma_stream(d, a, d.bind[2].size);
     // MatvecVariant (wg 512, lanes 64, rows 16) names the matrix-core variant: a wave per sixteen rows.
     // (k of 2048 or 4096 and whole tiles: the kernel that keeps the tokens' operands in registers.)
     if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && plain && matvec_q4k_mfma_resident_accepts(a))
