@@ -103,19 +103,22 @@ def bf16_tokens_case(c, m, n, k, col0=0, pad=0, accumulate=False, norm=False, x=
     return got, want, (x, bits)
 
 
-# Steps of several tokens over k = 1024 ... 4096 in steps of 512 run on the matrix cores, the
-# weights read once for all tokens; every other shape keeps the one-token kernel's path.
+# Steps of several tokens over k = 1024 ... 4096 in steps of 512 and 16 MB or more of weights run
+# on the matrix cores, the weights read once for all tokens; every other shape keeps the
+# one-token kernel's path.
 @pytest.mark.parametrize("m,n,k,col0,pad,accumulate,norm", [
-    (2, 64, 1024, 0, 0, False, False),
-    (8, 100, 1024, 0, 0, False, False),        # a ragged last unit of rows
-    (3, 37, 1536, 5, 3, True, False),          # unaligned columns, accumulate
-    (4, 8200, 2048, 0, 0, False, False),       # whole rounds of tiles and a tail on every workgroup
+    (2, 8192, 1024, 0, 0, False, False),
+    (8, 8300, 1024, 0, 0, False, False),       # a ragged last unit of rows
+    (3, 5501, 1536, 5, 3, True, False),        # unaligned columns, accumulate
+    (4, 8200, 2048, 0, 0, False, False),       # a tail on every workgroup
     (5, 9000, 2560, 0, 0, False, True),        # the RMSNorm prologue
-    (7, 333, 3072, 32, 0, True, True),
-    (8, 520, 3584, 0, 0, False, False),
+    (7, 2741, 3072, 32, 0, True, True),
+    (8, 2400, 3584, 0, 0, False, False),
     (6, 4040, 4096, 0, 0, False, False),
-    (11, 300, 1024, 0, 7, False, False),       # more than eight tokens: two launches
-    (19, 72, 4096, 8, 0, True, False),
+    (11, 8195, 1024, 0, 7, False, False),      # more than eight tokens: two launches
+    (4, 8192, 1024, 0, 0, False, True),        # k = 1024 with the prologue: the tokens split beforehand
+    (19, 2052, 4096, 8, 0, True, False),
+    (3, 100, 1024, 0, 0, False, False),        # a small matrix: the general kernel
 ])
 def test_matvec_bf16_several_tokens(ctx, m, n, k, col0, pad, accumulate, norm):
     got, want, _ = bf16_tokens_case(ctx, m, n, k, col0, pad, accumulate, norm)
@@ -145,7 +148,7 @@ def test_matvec_bf16_several_tokens_keep_token_bits(ctx):
     """A token's outputs do not depend on how many tokens share the step (from two tokens
     up), nor on where the step's columns start."""
     c = ctx
-    m, n, k = 13, 1000, 2048
+    m, n, k = 13, 4500, 2048
     x = c.random(m * k, 3).reshape(m, k)
     bits, _ = random_half(c, n * k, 1)
     wa = c.upload(bits)
@@ -160,7 +163,7 @@ def test_matvec_bf16_several_tokens_keep_token_bits(ctx):
     whole = run(list(range(m)), 0, n)
     assert np.array_equal(run([4, 9], 0, n), whole[[4, 9]])
     assert np.array_equal(run([12, 0, 5, 7, 3], 0, n), whole[[12, 0, 5, 7, 3]])
-    assert np.array_equal(run(list(range(8)), 424, 576), whole[:8, 424:])
+    assert np.array_equal(run(list(range(8)), 404, 4096), whole[:8, 404:])
     del wa
 
 
@@ -169,7 +172,7 @@ def test_matvec_bf16_several_tokens_special_values(ctx):
     against weights of +-1, where every partial sum is an integer f32 holds, so the result is
     exact whatever the order of the additions), the largest finite value, infinities and NaNs."""
     c = ctx
-    m, n, k = 4, 64, 1024
+    m, n, k = 4, 8192, 1024
     x = np.zeros((m, k), dtype=np.float32)
     r = c.rand.integers(0, 2000, size=k)
     x[0] = (2 ** 24 - 2048 + r).astype(np.float32)                 # 24 significant bits each
@@ -177,17 +180,18 @@ def test_matvec_bf16_several_tokens_special_values(ctx):
     x[2, 3] = np.inf
     x[3, 5] = np.nan
     w = np.empty((n, k), dtype=np.float32)
-    w[:32] = np.where(np.arange(k) % 2 == 0, 1.0, -1.0)
-    w[32:] = 0.5
-    w[32:, 1] = -0.25
+    h = n // 2
+    w[:h] = np.where(np.arange(k) % 2 == 0, 1.0, -1.0)
+    w[h:] = 0.5
+    w[h:, 1] = -0.25
     out = c.output(m * n)
     c.launcher().launch(Kernel.matvec_bf16, P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, eps=1e-6),
                         [c.upload(x), c.upload(synth.to_bf16_bits(w.reshape(-1))), out, c.upload(np.ones(k, dtype=np.float32))], (K.div_ceil(n, K.matvec_rows), m, 1))
     got = c.read(out).reshape(m, n)
-    assert np.array_equal(got[0, :32], np.full(32, float(np.sum(r[0::2]) - np.sum(r[1::2])), dtype=np.float32))
-    want1 = x[1].astype(np.float64) @ w[32:].astype(np.float64).T  # 0.5 * max - 0.25 * (-max) stays finite in f32
-    assert np.all(np.isfinite(got[1, 32:])) and np.max(np.abs(got[1, 32:] - want1)) <= 1e-6 * np.max(np.abs(want1))
-    assert np.all(np.isposinf(got[2, 32:]))
+    assert np.array_equal(got[0, :h], np.full(h, float(np.sum(r[0::2]) - np.sum(r[1::2])), dtype=np.float32))
+    want1 = x[1].astype(np.float64) @ w[h:].astype(np.float64).T  # 0.5 * max - 0.25 * (-max) stays finite in f32
+    assert np.all(np.isfinite(got[1, h:])) and np.max(np.abs(got[1, h:] - want1)) <= 1e-6 * np.max(np.abs(want1))
+    assert np.all(np.isposinf(got[2, h:]))
     assert np.all(np.isnan(got[3]))
 
 

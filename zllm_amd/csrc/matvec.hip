@@ -224,6 +224,10 @@ zhip_result launch_matvec_q8_mfma_stream(const Dispatch &d, const MvArgs &a, uin
 // matvec_bf16 on the matrix cores, the weights read once for all tokens (matvec_bf16_mfma_stream.hip).
 bool matvec_bf16_mfma_stream_accepts(const MvArgs &a);
 zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
+// Matrices from this size on take it: below, its fixed costs (the split of the tokens, a
+// workgroup's first tile) outweigh the general kernel's per-token work at two to four tokens
+// (8 MB, k = 1024: 6.4 / 6.8 / 7.8 us at 2 / 4 / 8 tokens against 4.7 / 6.2 / 9.3).
+constexpr uint64_t kBf16StreamBytes = 16ull << 20;
 // The matrix-core variant of matvec_q8_0 (matmul_mfma.hip).
 zhip_result launch_matvec_q8_0_mfma(const Dispatch &d, const MvArgs &a);
 // The tuned multiply (matvec_quant.hip): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
@@ -320,12 +324,12 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     // (On matvec_q8_0 only where the kernel that streams whole tiles takes the step: the other
     // matrix-core kernel of that operation narrows its inputs into the same workspace.)
     const bool prepass = D::CHUNK == 4 ? p.k % 1024u == 0 : ((p.k == 2048u || p.k == 4096u) && a.rows % 16u == 0 && !pair);
-    // matvec_bf16 steps of several tokens go to the kernel that reads the weights once for all
-    // of them; it too takes its inputs as they are.
-    MvArgs bare = a;
-    bare.flags &= ~FLAG_NORM;
-    const bool bf16_stream = std::is_same<D, DecBF16>::value && a.m >= 2u && matvec_bf16_mfma_stream_accepts(bare);
-    if ((matrix_cores && (norm || a.act_div > 0.f) && a.m <= 8u && prepass) || (bf16_stream && norm)) {
+    // matvec_bf16 steps of several tokens over a matrix of some size go to the kernel that reads
+    // the weights once for all of them (by the matrix, not by the step's width: a token's bits
+    // are then the same at every width from two tokens up).
+    if (std::is_same<D, DecBF16>::value && a.m >= 2u && (uint64_t)a.rows * a.row_bytes >= kBf16StreamBytes && matvec_bf16_mfma_stream_accepts(a))
+        return launch_matvec_bf16_mfma_stream(d, a, d.bind[2].size);
+    if (matrix_cores && (norm || a.act_div > 0.f) && a.m <= 8u && prepass) {
         if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", D::name());
         const uint64_t bytes = (uint64_t)a.m * p.k * 4u;
         if (zhip_result r = d.work->reserve(d, bytes)) return r;
@@ -340,7 +344,6 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
         v.act_div = 0u;
     }
     const bool plain = !(a.flags & FLAG_NORM) && a.act_div == 0.f;
-    if (bf16_stream) return launch_matvec_bf16_mfma_stream(d, a, d.bind[2].size);
     // MatvecVariant (wg 512, lanes 64, rows 16) names the matrix-core variant: a wave per sixteen rows.
     // (k of 2048 or 4096 and whole tiles: the kernel that keeps the tokens' operands in registers.)
     if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && plain && matvec_q4k_mfma_resident_accepts(a))

@@ -63,6 +63,10 @@ struct StreamArgs {
     uint32_t tail_base;  // units of eight rows after those: tail_base for every workgroup
     uint32_t tail_rem;   // and one more for each of the first tail_rem
     uint32_t by_die;     // workgroups renumbered die by die (the grid is a multiple of eight)
+    // Inputs split beforehand (SPLIT kernels): three planes [piece][token][k] of bf16.
+    const uint8_t *planes;
+    uint32_t plane_tokens;  // tokens a plane holds
+    uint32_t t0;            // the launch's first token in the planes
 };
 
 // A barrier that waits for this wave's LDS traffic only: the weight loads of the pieces ahead
@@ -114,8 +118,12 @@ __device__ __forceinline__ uint32_t piece_bits(float x, uint32_t m0, uint32_t m1
 // The upper halves of two words as a pair of bf16 values, `lo` first.
 __device__ __forceinline__ uint32_t upper_halves(uint32_t lo, uint32_t hi) { return __builtin_amdgcn_perm(hi, lo, 0x07060302u); }
 
-// NP: pieces of a wave's k range (k = 512 NP).
-template <int NP>
+// NP: pieces of a wave's k range (k = 512 NP). SPLIT: the tokens' three pieces come ready from
+// matvec_bf16_split_kernel's planes. A workgroup that splits its tokens itself spends 12 vector
+// operations a value on it, four lanes on the same value (the lanes of the three pieces and of
+// the zero rows): 1.5 us of a launch at k = 1024, less than another launch costs, but 12 us at
+// k = 4096.
+template <int NP, bool SPLIT>
 __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(StreamArgs q) {
     const MvArgs &a = q.a;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -176,6 +184,15 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
     asm volatile("" : "+v"(m0), "+v"(m1), "+v"(m2));
     const float *xt = a.x + (size_t)(tok < a.m ? tok : a.m - 1u) * a.xr + 64u * NP * wave + 8u * kap;
     hbf16x8 xf[4 * NP];
+    if constexpr (SPLIT) {
+        // Every step's operand is sixteen bytes of a plane; the lanes of absent tokens and of
+        // the zero rows ask past the buffer's end and get zeros.
+        const __amdgpu_buffer_rsrc_t pbuf = make_buffer(q.planes, 3u * q.plane_tokens * a.k * 2u);
+        const uint32_t at = live ? ((piece * q.plane_tokens + q.t0 + tok) * a.k + 64u * NP * wave + 8u * kap) * 2u : 0xfffffff0u;
+#pragma unroll
+        for (int s = 0; s < 4 * NP; s++) xf[s] = __builtin_bit_cast(hbf16x8, __builtin_amdgcn_raw_buffer_load_b128(pbuf, live ? at + 32u * s : at, 0, 0));
+        issue();
+    } else
 #pragma unroll
     for (int s0 = 0; s0 < 4 * NP; s0 += 8) {
         float4 raw[16];
@@ -279,9 +296,30 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
     wait_loads<0>();  // nothing may still land in LDS once the workgroup is gone
 }
 
-template <int NP>
+// Token blockIdx.x as the multiply sees it (normalised if the step asks for it:
+// src/kernels/matvec_half.wgsl:58-80), split into the three planes.
+__global__ __launch_bounds__(256) void matvec_bf16_split_kernel(MvArgs a, uint2 *planes) {
+    __shared__ float red[4];
+    __shared__ float4 staged[1024];
+    stage_token(a, blockIdx.x, staged, red);
+    __syncthreads();
+    const uint32_t k4 = a.k / 4u;
+    for (uint32_t i = threadIdx.x; i < k4; i += 256u) {
+        const float4 v = staged[i];
+#pragma unroll
+        for (uint32_t piece = 0; piece < 3u; piece++) {
+            const uint32_t m0 = piece == 0u ? ~0u : 0u, m1 = piece == 1u ? ~0u : 0u, m2 = piece == 2u ? ~0u : 0u;
+            uint2 w;
+            w.x = upper_halves(piece_bits(v.x, m0, m1, m2), piece_bits(v.y, m0, m1, m2));
+            w.y = upper_halves(piece_bits(v.z, m0, m1, m2), piece_bits(v.w, m0, m1, m2));
+            planes[(size_t)(piece * gridDim.x + blockIdx.x) * k4 + i] = w;
+        }
+    }
+}
+
+template <int NP, bool SPLIT>
 zhip_result launch_blocks(const Dispatch &d, const StreamArgs &q, dim3 grid) {
-    auto kernel = matvec_bf16_mfma_stream_kernel<NP>;
+    auto kernel = matvec_bf16_mfma_stream_kernel<NP, SPLIT>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess) {
@@ -297,10 +335,23 @@ zhip_result launch_blocks(const Dispatch &d, const StreamArgs &q, dim3 grid) {
 }  // namespace
 
 // Whether this kernel can run the (already validated) arguments: k split into whole lines a
-// wave, no prologue, no pair.
+// wave, no pair.
 bool matvec_bf16_mfma_stream_accepts(const MvArgs &a) {
-    return a.m >= 1 && a.k >= 1024u && a.k <= 4096u && a.k % 512u == 0 && !(a.flags & (FLAG_NORM | FLAG_SILU_PAIR)) && a.act_div == 0.f && a.rows >= 1 &&
+    return a.m >= 1 && a.k >= 1024u && a.k <= 4096u && a.k % 512u == 0 && !(a.flags & FLAG_SILU_PAIR) && a.act_div == 0.f && a.rows >= 1 &&
            a.xr % 4u == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == 2u * a.k;
+}
+
+template <bool SPLIT>
+static zhip_result launch_for_k(const Dispatch &d, const StreamArgs &q, dim3 grid) {
+    switch (q.a.k / 512u) {
+    case 2: return launch_blocks<2, SPLIT>(d, q, grid);
+    case 3: return launch_blocks<3, SPLIT>(d, q, grid);
+    case 4: return launch_blocks<4, SPLIT>(d, q, grid);
+    case 5: return launch_blocks<5, SPLIT>(d, q, grid);
+    case 6: return launch_blocks<6, SPLIT>(d, q, grid);
+    case 7: return launch_blocks<7, SPLIT>(d, q, grid);
+    default: return launch_blocks<8, SPLIT>(d, q, grid);
+    }
 }
 
 zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) {
@@ -312,23 +363,29 @@ zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, u
     const uint32_t groups = units < cus ? units : cus;
     const uint32_t rounds = (a.rows / 32u) / groups;
     const uint32_t tail = (a.rows - 32u * rounds * groups + 7u) / 8u;
-    StreamArgs q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u};
+    StreamArgs q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, nullptr, 0u, 0u};
+    // The tokens are split (and normalised) by a launch of their own where that is cheaper than
+    // every workgroup splitting them again, and wherever the step carries the RMSNorm prologue.
+    const bool split = (a.flags & FLAG_NORM) || a.k >= 2048u;
+    if (split) {
+        const uint64_t bytes = 6ull * a.m * a.k;
+        if (!d.work) return fail(d, ZHIP_E_GPU, "matvec_bf16: no workspace");
+        if (bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "matvec_bf16: a step of %u tokens", a.m);
+        if (zhip_result r = d.work->reserve(d, bytes)) return r;
+        hipLaunchKernelGGL(matvec_bf16_split_kernel, dim3(a.m), dim3(256), 0, d.stream, a, reinterpret_cast<uint2 *>(d.work->data));
+        if (zhip_result r = check_launch(d, "matvec_bf16")) return r;
+        q.planes = d.work->data;
+        q.plane_tokens = a.m;
+        q.a.flags &= ~FLAG_NORM;
+        q.a.norm_w = nullptr;
+    }
     const dim3 grid(groups);
     for (uint32_t t0 = 0; t0 < a.m; t0 += 8u) {
         q.a.x = a.x + (size_t)t0 * a.xr;
         q.a.out = a.out + (size_t)t0 * a.out_stride;
         q.a.m = a.m - t0 < 8u ? a.m - t0 : 8u;
-        zhip_result r;
-        switch (a.k / 512u) {
-        case 2: r = launch_blocks<2>(d, q, grid); break;
-        case 3: r = launch_blocks<3>(d, q, grid); break;
-        case 4: r = launch_blocks<4>(d, q, grid); break;
-        case 5: r = launch_blocks<5>(d, q, grid); break;
-        case 6: r = launch_blocks<6>(d, q, grid); break;
-        case 7: r = launch_blocks<7>(d, q, grid); break;
-        default: r = launch_blocks<8>(d, q, grid); break;
-        }
-        if (r != ZHIP_OK) return r;
+        q.t0 = t0;
+        if (zhip_result r = split ? launch_for_k<true>(d, q, grid) : launch_for_k<false>(d, q, grid)) return r;
     }
     return ZHIP_OK;
 }

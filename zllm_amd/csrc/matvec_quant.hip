@@ -105,6 +105,7 @@ __device__ __forceinline__ float dot_bytes(uint32_t word, const float4 &x, float
 // no minimum, so the input sums go unused.
 struct KQ8 {
     static constexpr int NSUM = 2;
+    static constexpr bool DEFER = false;
     static const char *name() { return "matvec_q8_0"; }
     struct Raw {
         uint4 q[4];
@@ -160,6 +161,7 @@ struct KQ8 {
 struct KQ3 {
     static constexpr uint32_t BLOCK_BYTES = 128;
     static constexpr int NSUM = 4;
+    static constexpr bool DEFER = true;
     static const char *name() { return "matvec_q3_k"; }
     struct Raw {
         uint4 u[2];
@@ -231,6 +233,7 @@ struct KQ3 {
 struct KQ4 {
     static constexpr uint32_t BLOCK_BYTES = 144;
     static constexpr int NSUM = 2;
+    static constexpr bool DEFER = true;
     static const char *name() { return "matvec_q4_k"; }
     struct Raw {
         uint4 h, q0, q1;
@@ -293,6 +296,7 @@ struct KQ4 {
 struct KQ5 {
     static constexpr uint32_t BLOCK_BYTES = 176;
     static constexpr int NSUM = 2;
+    static constexpr bool DEFER = true;
     static const char *name() { return "matvec_q5_k"; }
     struct Raw {
         uint4 h, b0, b1, q0, q1;
@@ -361,6 +365,7 @@ struct KQ5 {
 struct KQ6 {
     static constexpr uint32_t BLOCK_BYTES = 224;
     static constexpr int NSUM = 4;
+    static constexpr bool DEFER = false;
     static const char *name() { return "matvec_q6_k"; }
     struct Raw {
         uint4 l0, l1, hv;
@@ -461,6 +466,7 @@ struct KArgs {
     uint32_t seg_log2;  // lanes per row: 4, 5 or 6
     uint32_t tasks;     // k / 64
     Masks nm;
+    uint32_t defer;     // finished rows' outputs wait in registers for one store at the end of the wave's walk
 };
 
 template <class P, int MT, bool PAIR, bool XREG>
@@ -628,6 +634,22 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
 #pragma unroll
         for (int t = 0; t < MT; t++) acc[j][t] = 0.f;
 
+    // One-token steps over rows of 4096 weights keep a finished row's output in the lane of
+    // its number and store them together when the wave's walk ends (a format's DEFER: stores
+    // between the loads of the stream cost 0.1 - 0.3 us of the 14336 x 4096 launch for Q4_K,
+    // Q5_K and Q3_K; Q6_K, whose multiply needs the most registers, lost 0.4 us and Q8_0 gained
+    // nothing, so they store row by row).
+    float kept = 0.f;
+    uint32_t nkept = 0, kept_first = gwave;
+    auto flush_kept = [&]() {
+        const uint32_t j = kept_first + lane * nwaves;
+        if (lane < nkept && j < a.rows) {
+            const size_t o = (size_t)q.t0 * a.out_stride + a.col0 + j;
+            a.out[o] = (a.flags & FLAG_ACCUMULATE) ? kept + a.out[o] : kept;
+        }
+        kept_first += nkept * nwaves;
+        nkept = 0;
+    };
     // Multiplies the position `c` from `cur`; at a unit's last slice reduces
     // and stores its outputs.
     auto compute = [&](const Cursor &c, const typename P::Raw (&cur)[kRows]) {
@@ -657,6 +679,13 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
                 const float s0 = segment_sum(acc[0][t], q.seg_log2);
                 const float s1 = kRows == 2 ? segment_sum(acc[kRows - 1][t], q.seg_log2) : 0.f;
                 acc[0][t] = acc[kRows - 1][t] = 0.f;
+                if (P::DEFER && XREG && q.defer) {
+                    const float r = PAIR ? silu_f(s0) * s1 : s0;
+                    const float total = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), 63));
+                    kept = lane == nkept ? total : kept;
+                    nkept++;
+                    if (nkept == 64u) flush_kept();
+                } else
                 if (writer && (uint32_t)t < q.mt && c.j0 < a.rows) {
                     const size_t o = (size_t)(q.t0 + t) * a.out_stride + a.col0 + c.j0;
                     if (PAIR) {
@@ -691,6 +720,7 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
             done = cc.u >= units;
         }
     }
+    if (P::DEFER && XREG && q.defer) flush_kept();
 }
 
 template <class P, int MT, bool PAIR, bool XREG>
@@ -737,6 +767,7 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
         // more of them repeat the input staging, fewer leave too few loads in flight.
         const uint32_t cap = (uint32_t)d.dev->compute_units * (xreg ? 3u : 2u);
         const uint32_t blocks = want < cap ? want : cap;
+        q.defer = (P::DEFER && xreg && q.seg_log2 == 6u) ? 1u : 0u;
         zhip_result r;
         if (xreg) r = pair ? run_quant<P, 1, true, true>(d, q, lds, blocks) : run_quant<P, 1, false, true>(d, q, lds, blocks);
         else if (mt == 1u) r = pair ? run_quant<P, 1, true, false>(d, q, lds, blocks) : run_quant<P, 1, false, false>(d, q, lds, blocks);
