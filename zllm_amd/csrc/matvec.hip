@@ -323,7 +323,7 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     // memory, 36 us against 28 us with this pass in front, 22.5 us without a prologue.)
     // (On matvec_q8_0 only where the kernel that streams whole tiles takes the step: the other
     // matrix-core kernel of that operation narrows its inputs into the same workspace.)
-    const bool prepass = D::CHUNK == 4 ? p.k % 1024u == 0 : ((p.k == 2048u || p.k == 4096u) && a.rows % 16u == 0 && !pair);
+    const bool prepass = D::CHUNK == 4 ? p.k % 1024u == 0 : ((p.k == 1024u || p.k == 2048u || p.k == 4096u) && a.rows % 16u == 0 && !pair);
     // matvec_bf16 steps of several tokens over a matrix of some size go to the kernel that reads
     // the weights once for all of them (by the matrix, not by the step's width: a token's bits
     // are then the same at every width from two tokens up).

@@ -1,4 +1,4 @@
-// matvec_q8_0, matrix-core variant for steps of up to eight tokens and k = 2048 or 4096: the
+// matvec_q8_0, matrix-core variant for steps of up to eight tokens and k = 1024, 2048 or 4096: the
 // weight stream is read once for all tokens of the step and nothing but partial sums crosses
 // LDS. Contract as the other variants (src/kernels/matvec_quant.wgsl.hbs with the decoder of
 // src/kernels/quant/q8_0_dot.wgsl:5-14): out[t][col0 + j] (+)= sum over 32-weight blocks of
@@ -27,6 +27,10 @@
 // different banks. The eight waves' partial sums meet in LDS, where 128 threads add the eight
 // for one output each in the order of the k ranges and store. One barrier a tile; no barrier
 // waits for the loads in flight.
+// (k = 1024: a row and its scales are 1088 bytes, so every other row starts in the middle of a
+// cache line and a wave's 128 bytes of it lie across two: 151936 x 1024 runs at 42 us for one
+// to eight tokens, 3.9 TB/s against 6.6 TB/s at k = 4096 - still ahead of the default variant
+// from five tokens up: 29 / 42 / 78 us there at 1 / 4 / 8 tokens.)
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -111,10 +115,11 @@ __device__ __forceinline__ void load_lds_b32(__amdgpu_buffer_rsrc_t buf, uint32_
 }
 
 // NS: 32-weight blocks of a wave's k range (k = 256 NS). The ring moves half tiles: the first or
-// second NS / 2 blocks of the wave's range of a tile's sixteen rows. A slot: sixteen lines of
-// 16 NS bytes, then 256 bytes for the scales' load (NS bytes a row; zeros from idle lanes behind).
+// second NS / 2 blocks of the wave's range of a tile's sixteen rows (at k = 1024 the whole range:
+// it is one 128-byte line a row). A slot: sixteen lines, then 256 bytes for the scales' load
+// (two bytes a block and row; zeros from idle lanes behind).
 constexpr int DEPTH = 4;  // ring slots a wave: three half tiles in flight behind the one multiplied
-template <int NS> constexpr uint32_t slot_bytes() { return 16u * 16u * NS + 256u; }
+template <int NS> constexpr uint32_t slot_bytes() { return 16u * 32u * (NS >= 8 ? NS / 2 : NS) + 256u; }
 constexpr uint32_t PART_BYTES = 2u * WAVES * 128u * 4u, SCALE_BYTES = 320u;  // [8 waves][8 tokens] maxima, [8] inverse scales, pad
 template <int NS> constexpr uint32_t lds_bytes() { return PART_BYTES + SCALE_BYTES + WAVES * DEPTH * slot_bytes<NS>(); }
 static_assert(lds_bytes<16>() <= 160u * 1024u, "the rings must fit the CU's LDS");
@@ -126,7 +131,8 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
     float *lds_part = reinterpret_cast<float *>(lds);                  // [tile parity][wave][2 lane + token of the lane's two]
     float *lds_max = reinterpret_cast<float *>(lds + PART_BYTES);      // [wave][token]: the largest magnitude in the wave's range
     float *lds_inverse = lds_max + 64;                                 // [token]: one over the token's scale
-    constexpr int HB = NS / 2;  // blocks of a half tile
+    constexpr int PARTS = NS >= 8 ? 2 : 1;  // ring slots a wave's range of a tile takes (k = 1024: one 128-byte line a row already)
+    constexpr int HB = NS / PARTS;           // blocks of a half tile
     constexpr uint32_t SLOT = slot_bytes<NS>(), LINE = 32u * HB, CHUNKS = 2u * HB;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -157,15 +163,14 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
 #pragma unroll
     for (int i = 0; i < WLOADS; i++) {
         const uint32_t row = ROWS_PER_LOAD * i + lrow;
-        woff[i] = row * a.row_bytes + 2u * LINE * wave + 16u * (lpos ^ line_key(row));
+        woff[i] = row * a.row_bytes + PARTS * LINE * wave + 16u * (lpos ^ line_key(row));
     }
     constexpr uint32_t SWORDS = HB / 2;  // words of scales a row and half
-    const uint32_t soff = lane < 16u * SWORDS ? (lane / SWORDS) * a.row_bytes + a.k + 2u * NS * wave + 4u * (lane % SWORDS) : 0xfffffff0u;
-    const uint32_t soff8 = lane < 8u * SWORDS ? soff : 0xfffffff0u;  // the same for an eight-row share
+    const uint32_t soff = (lane / SWORDS) * a.row_bytes + a.k + 2u * NS * wave + 4u * (lane % SWORDS);
     auto load_half = [&](uint32_t u, uint32_t slot) __attribute__((always_inline)) {
         // (past the run's last tile the loads still run, so that the waits count the same loads
         // every step, but against an empty buffer: zeros land and nothing is fetched)
-        const uint32_t p = u >> 1, half = u & 1u;
+        const uint32_t p = u / PARTS, half = u % PARTS;
         const __amdgpu_buffer_rsrc_t buf = p < count ? wbuf : nobuf;
         const uint32_t base = first_row(p) * a.row_bytes, rows = rows_of(p);
         const uint32_t dst = ring0 + slot * SLOT;
@@ -173,7 +178,7 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
         // instructions make of their slots' old contents is never stored)
 #pragma unroll
         for (int i = 0; i < WLOADS; i++) load_lds_b128((uint32_t)(ROWS_PER_LOAD * i) < rows ? buf : nobuf, dst + 1024u * i, woff[i], base + LINE * half);
-        load_lds_b32(buf, dst + 16u * LINE, rows == 16u ? soff : soff8, base + 2u * HB * half);
+        load_lds_b32(buf, dst + 16u * LINE, lane < rows * SWORDS ? soff : 0xfffffff0u, base + 2u * HB * half);
     };
     // The tokens' inputs first: loads complete in order within a wave, and behind the weight
     // loads below the first use of an input would wait for a round trip of the weight stream.
@@ -256,6 +261,7 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
             const su32x4 v = *reinterpret_cast<const su32x4 *>(t + 16u * LINE + l16 * 16u);
             d[0] = v.x; d[1] = v.y; d[2] = v.z; d[3] = v.w;
         } else {
+            static_assert(SWORDS == 2, "two or four words of scales a row");
             const su32x2 v = *reinterpret_cast<const su32x2 *>(t + 16u * LINE + l16 * 8u);
             d[0] = v.x; d[1] = v.y;
         }
@@ -296,7 +302,7 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
     // against 20.7 us with the lanes' own loads). Every wave of the workgroup runs the same
     // steps (the barrier inside). Before half tile u is read, all but the loads of the
     // DEPTH - 1 half tiles after it have landed.
-    for (uint32_t u = 0; u < 2u * count; u += DEPTH) {
+    for (uint32_t u = 0; u < PARTS * count; u += DEPTH) {
 #pragma unroll
         for (int s = 0; s < DEPTH; s++) {
             // The slot refilled now was read by the multiply before: its reads must have returned
@@ -305,8 +311,11 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
             load_half(u + s + (DEPTH - 1), (s + DEPTH - 1) % DEPTH);
             wait_loads<(DEPTH - 1) * LOADS>();
-            if (u + s < 2u * count) {
-                if (s & 1) {
+            if (u + s < PARTS * count) {
+                if constexpr (PARTS == 1) {
+                    multiply(std::integral_constant<int, 0>{}, s);
+                    finish(u + s);
+                } else if (s & 1) {
                     multiply(std::integral_constant<int, 1>{}, s);
                     finish((u + s) >> 1);
                 } else {
@@ -323,7 +332,7 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
 // Whether this kernel can run the (already validated) arguments: whole tiles, k split into 8 or
 // 16 blocks a wave, no prologue, no pair.
 bool matvec_q8_mfma_stream_accepts(const MvArgs &a) {
-    return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u) && !(a.flags & (FLAG_NORM | FLAG_SILU_PAIR)) && a.act_div == 0.f && a.rows % 16u == 0 &&
+    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && !(a.flags & (FLAG_NORM | FLAG_SILU_PAIR)) && a.act_div == 0.f && a.rows % 16u == 0 &&
            a.xr % 4u == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0;
 }
 
@@ -351,7 +360,7 @@ zhip_result launch_matvec_q8_mfma_stream(const Dispatch &d, const MvArgs &a, uin
     StreamArgs q{a, (uint32_t)w_bytes, tiles / groups, left, (tiles < groups || 2u * left <= groups) ? 1u : 0u, 0x64646464u};
     if (tiles < groups) { q.rounds = 0; q.left = tiles; }
     const dim3 grid(groups);
-    return a.k == 2048u ? launch_blocks<8>(d, q, grid) : launch_blocks<16>(d, q, grid);
+    return a.k == 1024u ? launch_blocks<4>(d, q, grid) : a.k == 2048u ? launch_blocks<8>(d, q, grid) : launch_blocks<16>(d, q, grid);
 }
 
 }  // namespace zhip
