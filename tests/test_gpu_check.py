@@ -426,12 +426,12 @@ def test_matvec_q8_0_mfma_variant(ctx, rows, n, k, col0, pad, accumulate):
 
 
 @pytest.mark.parametrize("prologue", ["norm", "norm_act"])
-@pytest.mark.parametrize("rows,n,k", [(6, 4112, 4096), (3, 96, 2048), (2, 200, 1024)])
+@pytest.mark.parametrize("rows,n,k", [(6, 4112, 4096), (3, 96, 2048), (2, 200, 1024), (4, 4128, 1024)])
 def test_matvec_q8_0_mfma_variant_prologues(ctx, rows, n, k, prologue):
     """The matrix-core variant of matvec_q8_0 on steps with the RMSNorm and silu(x / act_div)
-    prologues (src/kernels/matvec_quant.wgsl.hbs:73-89): the transformed tokens reach the
-    multiply through the workspace; 1e-5 against float64, each token bitwise equal to its
-    lone launch."""
+    prologues (src/kernels/matvec_quant.wgsl.hbs:73-89), which the streaming kernel computes
+    as it builds the tokens' operands (200 rows: not whole tiles, the default variant's
+    kernel); 1e-5 against float64, each token bitwise equal to its lone launch."""
     c = ctx
     div, eps = 4 if prologue == "norm_act" else 0, 1e-6
     x = c.random(rows * k, 3).reshape(rows, k)

@@ -312,24 +312,26 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     a.out = reinterpret_cast<float *>(d.bind[3].ptr);
     a.norm_w = norm ? reinterpret_cast<const float *>(d.bind[4].ptr) : nullptr;
 
-    // The matrix-core variants take their inputs as they are: a step with a prologue (RMSNorm,
-    // silu(x / act_div): src/kernels/matvec_quant.wgsl.hbs:73-89) first writes the transformed
-    // tokens to the workspace, one workgroup a token with the staging arithmetic of the default
-    // variant, and the multiply reads those.
-    const bool matrix_cores = quant && v.lanes == 64u && v.rows == 16u && (D::CHUNK == 4 || D::CHUNK == 8);
-    uint64_t x_bound = d.bind[1].size;
-    // (Computing the prologue inside the multiply was tried on the kernel for k of 2048 or 4096:
-    // every workgroup repeats the row sums and takes its norm weights in dependent trips to
-    // memory, 36 us against 28 us with this pass in front, 22.5 us without a prologue.)
-    // (On matvec_q8_0 only where the kernel that streams whole tiles takes the step: the other
-    // matrix-core kernel of that operation narrows its inputs into the same workspace.)
-    const bool prepass = D::CHUNK == 4 ? p.k % 1024u == 0 : ((p.k == 1024u || p.k == 2048u || p.k == 4096u) && a.rows % 16u == 0 && !pair);
     // matvec_bf16 steps of several tokens over a matrix of some size go to the kernel that reads
     // the weights once for all of them (by the matrix, not by the step's width: a token's bits
     // are then the same at every width from two tokens up).
     if (std::is_same<D, DecBF16>::value && a.m >= 2u && (uint64_t)a.rows * a.row_bytes >= kBf16StreamBytes && matvec_bf16_mfma_stream_accepts(a))
         return launch_matvec_bf16_mfma_stream(d, a, d.bind[2].size);
-    if (matrix_cores && (norm || a.act_div > 0.f) && a.m <= 8u && prepass) {
+
+    // MatvecVariant (wg 512, lanes 64, rows 16) names the matrix-core variants: a wave per sixteen rows.
+    const bool matrix_cores = quant && v.lanes == 64u && v.rows == 16u && (D::CHUNK == 4 || D::CHUNK == 8);
+    // The kernels that keep the tokens' operands in registers (k of 2048 or 4096, for Q8_0 also
+    // 1024, and whole tiles) compute a step's prologue (RMSNorm, silu(x / act_div):
+    // src/kernels/matvec_quant.wgsl.hbs:73-89) themselves: their operands are built from one
+    // round of loads, which the norm weights join (C3 at four tokens with the FFN launch's
+    // RMSNorm: 22.6 us, 26.1 us with a pass of its own in front, 20.7 us without a prologue).
+    const bool resident = D::CHUNK == 4 && matrix_cores && matvec_q4k_mfma_resident_accepts(a);
+    const bool q8_stream = D::CHUNK == 8 && matrix_cores && !pair && matvec_q8_mfma_stream_accepts(a);
+    // The Q4_K kernel for the other multiples of 1024 takes its inputs as they are: a step with
+    // a prologue first writes the transformed tokens to the workspace, one workgroup a token
+    // with the staging arithmetic of the default variant, and the multiply reads those.
+    uint64_t x_bound = d.bind[1].size;
+    if (D::CHUNK == 4 && matrix_cores && !resident && (norm || a.act_div > 0.f) && a.m <= 8u && p.k % 1024u == 0) {
         if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", D::name());
         const uint64_t bytes = (uint64_t)a.m * p.k * 4u;
         if (zhip_result r = d.work->reserve(d, bytes)) return r;
@@ -344,16 +346,12 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
         v.act_div = 0u;
     }
     const bool plain = !(a.flags & FLAG_NORM) && a.act_div == 0.f;
-    // MatvecVariant (wg 512, lanes 64, rows 16) names the matrix-core variant: a wave per sixteen rows.
-    // (k of 2048 or 4096 and whole tiles: the kernel that keeps the tokens' operands in registers.)
-    if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && plain && matvec_q4k_mfma_resident_accepts(a))
-        return launch_matvec_q4k_mfma_resident(d, a, d.bind[2].size);
+    if (resident) return launch_matvec_q4k_mfma_resident(d, a, d.bind[2].size);
     if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && plain && matvec_q4k_mfma_accepts(a))
         return launch_matvec_q4k_mfma(d, a, x_bound, d.bind[2].size);
-    // The same id on matvec_q8_0, without prologue or pair (a one-token step too, so that a
-    // token's bits do not depend on the step it ran in).
-    if (D::CHUNK == 8 && v.lanes == 64u && v.rows == 16u && plain && !pair && matvec_q8_mfma_stream_accepts(a))
-        return launch_matvec_q8_mfma_stream(d, a, d.bind[2].size);
+    // The same id on matvec_q8_0, without pair (a one-token step too, so that a token's bits do
+    // not depend on the step it ran in); other shapes without a prologue: the prefill tiling.
+    if (q8_stream) return launch_matvec_q8_mfma_stream(d, a, d.bind[2].size);
     if (D::CHUNK == 8 && v.lanes == 64u && v.rows == 16u && plain && !pair && a.m <= 32u)
         return launch_matvec_q8_0_mfma(d, a);
     // The tuned kernel takes rows of whole 64-weight tasks.

@@ -365,7 +365,9 @@ zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, u
     const uint32_t tail = (a.rows - 32u * rounds * groups + 7u) / 8u;
     StreamArgs q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, nullptr, 0u, 0u};
     // The tokens are split (and normalised) by a launch of their own where that is cheaper than
-    // every workgroup splitting them again, and wherever the step carries the RMSNorm prologue.
+    // every workgroup splitting them again, and wherever the step carries the RMSNorm prologue
+    // (the workgroups computing the norm themselves at k = 1024 measured the same: 151936 x 1024
+    // at 2 / 4 / 8 tokens 53.3 / 54.1 / 56.3 us against 54.2 / 54.2 / 55.5 us this way).
     const bool split = (a.flags & FLAG_NORM) || a.k >= 2048u;
     if (split) {
         const uint64_t bytes = 6ull * a.m * a.k;

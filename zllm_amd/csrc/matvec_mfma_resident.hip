@@ -111,6 +111,7 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
     const MvArgs &a = q.a;
     __shared__ float lds_scale[16];               // [8 ..]: one over each token's scale
     __shared__ float lds_max[WAVES * 8];          // [wave][token]: the largest magnitude in the wave's range
+    __shared__ float lds_ss[WAVES * 8];           // [wave][token]: the range's sum of squares (RMSNorm prologue)
     __shared__ float lds_part[2][WAVES][128];     // [tile parity][wave][2 lane + token of the lane's two]
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, l16 = lane & 15u, g = lane >> 4;
     const __amdgpu_buffer_rsrc_t wbuf = make_buffer(a.w, q.w_bytes), nobuf = make_buffer(a.w, 0);
@@ -173,7 +174,43 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
 #pragma unroll
         for (int s = 0; s < NB * 8; s++) raw[s] = *reinterpret_cast<const float4 *>(xt + 32 * s);
     }
+    // A step's prologue (src/kernels/matvec_quant.wgsl.hbs:73-89) on the same registers, in the
+    // default variant's arithmetic: RMSNorm times the norm weights (the wave ranges' sums of
+    // squares meet in LDS, added in the order of the ranges) and / or silu(x / act_div).
+    const bool norm = (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
+    float4 gw[NB * 8];
+    if (norm) {
+        const float *gt = a.norm_w + NB * 256u * wave + 8u * g + 4u * sub;
+#pragma unroll
+        for (int s = 0; s < NB * 8; s++) gw[s] = *reinterpret_cast<const float4 *>(gt + 32 * s);
+    }
     load_tile(0, 0);
+    if (norm) {
+        float ss = 0.f;
+#pragma unroll
+        for (int s = 0; s < NB * 8; s++) ss += raw[s].x * raw[s].x + raw[s].y * raw[s].y + raw[s].z * raw[s].z + raw[s].w * raw[s].w;
+        ss += __shfl_xor(ss, 1, 64);
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        if (g == 0u && sub == 0u) lds_ss[8u * wave + tok] = ss;
+        lds_barrier();
+        float total = lds_ss[tok];
+#pragma unroll
+        for (uint32_t wv = 1; wv < WAVES; wv++) total += lds_ss[8u * wv + tok];
+        const float rs = 1.0f / sqrtf(total / (float)a.k + a.eps);
+#pragma unroll
+        for (int s = 0; s < NB * 8; s++) {
+            raw[s].x = raw[s].x * rs * gw[s].x; raw[s].y = raw[s].y * rs * gw[s].y;
+            raw[s].z = raw[s].z * rs * gw[s].z; raw[s].w = raw[s].w * rs * gw[s].w;
+        }
+    }
+    if (act) {
+#pragma unroll
+        for (int s = 0; s < NB * 8; s++) {
+            raw[s].x = silu_f(raw[s].x / a.act_div); raw[s].y = silu_f(raw[s].y / a.act_div);
+            raw[s].z = silu_f(raw[s].z / a.act_div); raw[s].w = silu_f(raw[s].w / a.act_div);
+        }
+    }
 
     // Each token's scale: the power of two that puts its largest magnitude in [2^14, 2^15). The
     // eight lanes of a token (two rows, four groups) hold this wave's range of it; the eight
@@ -312,11 +349,10 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
 }  // namespace
 
 // Whether this kernel can run the (already validated) arguments: whole tiles, k split into
-// one or two blocks a wave, no prologue.
+// one or two blocks a wave.
 bool matvec_q4k_mfma_resident_accepts(const MvArgs &a) {
     const bool pair = a.flags & FLAG_SILU_PAIR;
-    return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u) && !(a.flags & FLAG_NORM) && a.act_div == 0.f && a.rows % 16u == 0 &&
-           (!pair || a.half % 16u == 0);
+    return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u) && a.rows % 16u == 0 && (!pair || a.half % 16u == 0);
 }
 
 zhip_result launch_matvec_q4k_mfma_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) {

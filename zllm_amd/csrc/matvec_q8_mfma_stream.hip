@@ -120,7 +120,7 @@ __device__ __forceinline__ void load_lds_b32(__amdgpu_buffer_rsrc_t buf, uint32_
 // (two bytes a block and row; zeros from idle lanes behind).
 constexpr int DEPTH = 4;  // ring slots a wave: three half tiles in flight behind the one multiplied
 template <int NS> constexpr uint32_t slot_bytes() { return 16u * 32u * (NS >= 8 ? NS / 2 : NS) + 256u; }
-constexpr uint32_t PART_BYTES = 2u * WAVES * 128u * 4u, SCALE_BYTES = 320u;  // [8 waves][8 tokens] maxima, [8] inverse scales, pad
+constexpr uint32_t PART_BYTES = 2u * WAVES * 128u * 4u, SCALE_BYTES = 576u;  // [8 waves][8 tokens] maxima, [8] inverse scales, [8 waves][8 tokens] sums of squares
 template <int NS> constexpr uint32_t lds_bytes() { return PART_BYTES + SCALE_BYTES + WAVES * DEPTH * slot_bytes<NS>(); }
 static_assert(lds_bytes<16>() <= 160u * 1024u, "the rings must fit the CU's LDS");
 
@@ -195,10 +195,47 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
 #pragma unroll
         for (int s = 0; s < NS; s++) raw[s] = *reinterpret_cast<const float4 *>(xt + 32 * s);
     }
+    // A step's prologue (src/kernels/matvec_quant.wgsl.hbs:73-89) on the same registers, in the
+    // default variant's arithmetic: RMSNorm times the norm weights (the wave ranges' sums of
+    // squares meet in LDS, added in the order of the ranges) and / or silu(x / act_div).
+    const bool norm = (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
+    float4 gw[NS];
+    if (norm) {
+        const float *gt = a.norm_w + NS * 32u * wave + 8u * g + 4u * sub;
+#pragma unroll
+        for (int s = 0; s < NS; s++) gw[s] = *reinterpret_cast<const float4 *>(gt + 32 * s);
+    }
     // (One half tile of weights behind them for now: with more, the requests of the workgroups
     // that start first fill the memory system's queues and the inputs of the others arrive
     // after them, 4.5 us into the kernel instead of 1.7.)
     load_half(0, 0);
+    if (norm) {
+        float ss = 0.f;
+#pragma unroll
+        for (int s = 0; s < NS; s++) ss += raw[s].x * raw[s].x + raw[s].y * raw[s].y + raw[s].z * raw[s].z + raw[s].w * raw[s].w;
+        ss += __shfl_xor(ss, 1, 64);
+        ss += __shfl_xor(ss, 16, 64);
+        ss += __shfl_xor(ss, 32, 64);
+        float *lds_ss = lds_inverse + 8;  // [wave][token]: the range's sum of squares
+        if (g == 0u && sub == 0u) lds_ss[8u * wave + tok] = ss;
+        lds_barrier();
+        float total = lds_ss[tok];
+#pragma unroll
+        for (uint32_t wv = 1; wv < WAVES; wv++) total += lds_ss[8u * wv + tok];
+        const float rs = 1.0f / sqrtf(total / (float)a.k + a.eps);
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            raw[s].x = raw[s].x * rs * gw[s].x; raw[s].y = raw[s].y * rs * gw[s].y;
+            raw[s].z = raw[s].z * rs * gw[s].z; raw[s].w = raw[s].w * rs * gw[s].w;
+        }
+    }
+    if (act) {
+#pragma unroll
+        for (int s = 0; s < NS; s++) {
+            raw[s].x = silu_f(raw[s].x / a.act_div); raw[s].y = silu_f(raw[s].y / a.act_div);
+            raw[s].z = silu_f(raw[s].z / a.act_div); raw[s].w = silu_f(raw[s].w / a.act_div);
+        }
+    }
 
     // Each token's scale: the power of two that puts its largest magnitude in [2^14, 2^15). The
     // eight lanes of a token (two rows, four groups) hold this wave's range of it; the eight
@@ -329,10 +366,10 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
 
 }  // namespace
 
-// Whether this kernel can run the (already validated) arguments: whole tiles, k split into 8 or
-// 16 blocks a wave, no prologue, no pair.
+// Whether this kernel can run the (already validated) arguments: whole tiles, k split into 4, 8
+// or 16 blocks a wave, no pair.
 bool matvec_q8_mfma_stream_accepts(const MvArgs &a) {
-    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && !(a.flags & (FLAG_NORM | FLAG_SILU_PAIR)) && a.act_div == 0.f && a.rows % 16u == 0 &&
+    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && !(a.flags & FLAG_SILU_PAIR) && a.rows % 16u == 0 &&
            a.xr % 4u == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0;
 }
 
