@@ -459,6 +459,54 @@ def test_matvec_q8_0_mfma_variant_prologues(ctx, rows, n, k, prologue):
         assert got[tk].tobytes() == c.read(single)[:n].tobytes(), "a token's sums differ between a lone launch and a multi-token launch"
 
 
+@pytest.mark.parametrize("rows,n,k,col0,pad,accumulate,prologue", [
+    (8, 8224, 4096, 0, 0, False, None),        # whole rounds of 32-row tiles and a tail on every workgroup
+    (5, 9000, 4096, 0, 0, True, None),         # a ragged last unit of rows
+    (3, 100, 2048, 3, 7, True, None),          # fewer rows than workgroups, unaligned columns
+    (1, 530, 2048, 0, 2, False, None),         # one token
+    (6, 4100, 2048, 0, 0, False, "norm"),
+    (4, 300, 4096, 5, 0, True, "norm_act"),
+    (2, 64, 1024, 0, 0, False, None),          # k the kernel does not take: the default variant's
+])
+def test_matvec_q6_k_mfma_variant(ctx, rows, n, k, col0, pad, accumulate, prologue):
+    """matvec_q6_k on the matrix-core variant id (a wave per sixteen rows): the weights are read
+    once for all tokens of the step, the tokens split beforehand (with the RMSNorm and
+    silu(x / act_div) prologues of src/kernels/matvec_quant.wgsl.hbs:73-89 where the step has
+    them). 1e-5 against float64; columns outside the launch untouched; each token bitwise equal
+    to its lone launch."""
+    c = ctx
+    stride = col0 + n + pad
+    div, eps = 4 if prologue == "norm_act" else 0, 1e-6
+    x = c.random(rows * k, 3).reshape(rows, k)
+    x[0] *= np.float32(1e-4)
+    nw = c.random(k, 1.5)
+    raw, values = quant_rows(c, TensorType.q6_k, n, k)
+    init = c.random(rows * stride, 2).reshape(rows, stride)
+    xa, wa, na = c.upload(x), c.gpu_weights(TensorType.q6_k, raw, k), c.upload(nw)
+    x64 = np.stack([norm_row(r, nw if prologue else None, eps) for r in x])
+    if div:
+        x64 = (x64 / div) * sigmoid64(x64 / div)
+    prod = x64 @ values.astype(np.float64).T
+    want = prod + (init[:, col0 : col0 + n] if accumulate else 0)
+    p = lambda: P.MatvecBf16(n=n, k=k, col0=col0, out_stride=stride, eps=eps, norm=prologue is not None, accumulate=accumulate)
+    variant = K.MatvecVariant(MFMA_VARIANT.wg, MFMA_VARIANT.lanes, MFMA_VARIANT.rows, div)
+    pipeline = c.set.matvec(c.rec, Kernel.matvec_q6_k, variant)
+    grid_x = K.div_ceil(n, variant.group_rows())
+    out = c.upload(init)
+    c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, na], (grid_x, rows, 1))
+    got = c.read(out).reshape(rows, stride)
+    for tk in range(rows):
+        # Against the product's own scale (an accumulated init may dwarf a tiny token's product).
+        assert np.max(np.abs(got[tk, col0 : col0 + n] - want[tk])) <= 1e-5 * max(np.max(np.abs(prod[tk])), 1e-30) + 1e-6 * np.max(np.abs(want[tk])), tk
+    mask = np.ones(stride, dtype=bool)
+    mask[col0 : col0 + n] = False
+    assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32))
+    for tk in (0, rows - 1):
+        single = c.upload(init[tk])
+        c.launcher().launch_pipeline(pipeline, p(), [c.upload(x[tk]), wa, single, na], (grid_x, 1, 1))
+        assert got[tk].tobytes() == c.read(single)[:stride].tobytes(), "a token's sums differ between a lone launch and a multi-token launch"
+
+
 # ---- block decoders bit for bit, through the embedding gathers: check.zig:873-905 -----
 
 @pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q3_k, TensorType.q4_k, TensorType.q5_k, TensorType.q6_k])

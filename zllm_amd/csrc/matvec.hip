@@ -224,6 +224,9 @@ zhip_result launch_matvec_q8_mfma_stream(const Dispatch &d, const MvArgs &a, uin
 // matvec_bf16 on the matrix cores, the weights read once for all tokens (matvec_bf16_mfma_stream.hip).
 bool matvec_bf16_mfma_stream_accepts(const MvArgs &a);
 zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
+// matvec_q6_k on the matrix cores for k of 2048 or 4096 (matvec_q6k_mfma_stream.hip).
+bool matvec_q6k_mfma_stream_accepts(const MvArgs &a);
+zhip_result launch_matvec_q6k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
 // Matrices from this size on take it: below, its fixed costs (the split of the tokens, a
 // workgroup's first tile) outweigh the general kernel's per-token work at two to four tokens
 // (8 MB, k = 1024: 6.4 / 6.8 / 7.8 us at 2 / 4 / 8 tokens against 4.7 / 6.2 / 9.3).
@@ -319,7 +322,9 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
         return launch_matvec_bf16_mfma_stream(d, a, d.bind[2].size);
 
     // MatvecVariant (wg 512, lanes 64, rows 16) names the matrix-core variants: a wave per sixteen rows.
-    const bool matrix_cores = quant && v.lanes == 64u && v.rows == 16u && (D::CHUNK == 4 || D::CHUNK == 8);
+    const bool matrix_cores = quant && v.lanes == 64u && v.rows == 16u && (D::CHUNK == 4 || D::CHUNK == 8 || D::CHUNK == 6);
+    // (matvec_q6_k: a launch of its own splits the tokens, prologue included, for the multiply)
+    if (D::CHUNK == 6 && matrix_cores && matvec_q6k_mfma_stream_accepts(a)) return launch_matvec_q6k_mfma_stream(d, a, d.bind[2].size);
     // The kernels that keep the tokens' operands in registers (k of 2048 or 4096, for Q8_0 also
     // 1024, and whole tiles) compute a step's prologue (RMSNorm, silu(x / act_div):
     // src/kernels/matvec_quant.wgsl.hbs:73-89) themselves: their operands are built from one
