@@ -466,7 +466,9 @@ def test_matvec_q8_0_mfma_variant_prologues(ctx, rows, n, k, prologue):
     (1, 530, 2048, 0, 2, False, None),         # one token
     (6, 4100, 2048, 0, 0, False, "norm"),
     (4, 300, 4096, 5, 0, True, "norm_act"),
-    (2, 64, 1024, 0, 0, False, None),          # k the kernel does not take: the default variant's
+    (2, 64, 1024, 0, 0, False, None),          # one unit a tile
+    (7, 8232, 1024, 0, 0, True, "norm"),
+    (3, 96, 3072, 0, 0, False, None),          # k the kernel does not take: the default variant's
 ])
 def test_matvec_q6_k_mfma_variant(ctx, rows, n, k, col0, pad, accumulate, prologue):
     """matvec_q6_k on the matrix-core variant id (a wave per sixteen rows): the weights are read

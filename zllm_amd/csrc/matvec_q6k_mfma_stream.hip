@@ -1,5 +1,5 @@
 // matvec_q6_k, matrix-core variant (MatvecVariant wg 512, lanes 64, rows 16) for steps of up to
-// eight tokens and k = 2048 or 4096: the weight stream is read once for all tokens of the step
+// eight tokens and k = 1024, 2048 or 4096: the weight stream is read once for all tokens of the step
 // and the per-weight work is done once. Contract as the default variant's
 // (src/kernels/matvec_quant.wgsl.hbs with the decoder of src/kernels/quant/q6_k_dot.wgsl; block
 // formula src/ref/tensor.zig:118-140): out[t][col0 + j] (+)= sum over 16-weight sub-blocks of
@@ -17,13 +17,16 @@
 // Layout of the work. A launch of its own (matvec_q6k_split_kernel, one workgroup a token, the
 // default variant's staging arithmetic for the RMSNorm and silu(x / act_div) prologues) writes
 // the tokens' two f16 planes and inverse scales to the workspace once. In the multiply a
-// 512-thread workgroup is eight waves; its tiles are 32 matrix rows, taken as units of eight
-// 256-weight blocks a row (1792 bytes = fourteen whole lines of each row: the whole k at 2048,
-// half of it at 4096), wave w multiplying block w of the unit. A unit travels as a flat copy
-// through a ring of two LDS slots: all waves load it by wave-wide direct loads of whole lines
-// (seven a wave), each wave waits for its own and one barrier a unit tells everyone that all of
-// it has landed; the next unit's loads go out behind that barrier, so one unit is in flight
-// while the other is multiplied. Chunk c (16 bytes) of a line of row r sits at position
+// 512-thread workgroup is eight waves; its tiles are 32 matrix rows, taken as units of four
+// 256-weight blocks a row (896 bytes = seven whole lines of each row), wave w multiplying half
+// w % 2 of block w / 2 of the unit. A unit travels as a flat copy through a ring of four LDS
+// slots: the waves load it by wave-wide direct loads of whole lines (four each for seven of
+// them), each wave waits for its own and one barrier a unit tells everyone that all of it has
+// landed; the loads of the unit three ahead go out behind that barrier, so three units are in
+// flight while one is multiplied (two slots of twice the size, one unit in flight, measured the
+// same 94 us on 128256 x 4096: per 16-weight sub-block and wave the kernel issues 24 vector
+// instructions and a matrix instruction that do not overlap, 0.85 us a unit and SIMD against
+// the 1.1 us the unit's bytes need at full rate, and the two overlap only in part). Chunk c (16 bytes) of a line of row r sits at position
 // c ^ (r % 8), which keeps the 32 rows' reads of one piece of a block to four lanes a bank. The
 // waves' partial sums meet in LDS behind the same barrier, are added in the order of the blocks
 // and wait there for one burst of stores when the workgroup's run ends. Workgroups are numbered
@@ -47,12 +50,13 @@ typedef uint32_t qu32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t qu32x4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t THREADS = 512, WAVES = 8;
-constexpr uint32_t ROW_UNIT = 8u * 224u;        // a unit's bytes of one row: fourteen lines
+constexpr uint32_t ROW_UNIT = 4u * 224u;        // a unit's bytes of one row: seven lines
 constexpr uint32_t UNIT = 32u * ROW_UNIT;       // a unit in LDS
-constexpr int LOADS = 7;                        // wave-wide loads of a unit a wave issues (56 KB / 8 / 1 KB)
+constexpr int SLOTS = 4;                        // ring slots: three units in flight behind the one multiplied
+constexpr int LOADS = 4;                        // wave-wide loads of a unit a wave issues (28 of 1 KB: seven waves' worth; the eighth asks for nothing)
 constexpr uint32_t PART_BYTES = 2u * WAVES * 256u * 4u;  // [tile parity][wave][token of the lane's four][lane]
 constexpr uint32_t KEPT = 16;                   // tiles whose outputs wait in LDS for one burst of stores
-constexpr uint32_t LDS_BYTES = PART_BYTES + 2u * UNIT + KEPT * 1024u + 64u;
+constexpr uint32_t LDS_BYTES = PART_BYTES + SLOTS * UNIT + KEPT * 1024u + 64u + 1024u;  // (the last KB: where the eighth wave's loads of nothing land)
 static_assert(LDS_BYTES <= 160u * 1024u - 64u, "the ring must fit the CU's LDS");
 
 struct Q6Args {
@@ -148,14 +152,14 @@ __global__ __launch_bounds__(256) void matvec_q6k_split_kernel(MvArgs a, uint2 *
     }
 }
 
-// NU: units of a tile (k = 2048 NU).
+// NU: units of a tile (k = 1024 NU).
 template <int NU>
 __global__ __launch_bounds__(THREADS) void matvec_q6k_mfma_stream_kernel(Q6Args q) {
     const MvArgs &a = q.a;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     float *lds_part = reinterpret_cast<float *>(lds);
     uint8_t *ring = lds + PART_BYTES;
-    float *lds_kept = reinterpret_cast<float *>(lds + PART_BYTES + 2u * UNIT);  // [tile % KEPT][token][row]
+    float *lds_kept = reinterpret_cast<float *>(lds + PART_BYTES + SLOTS * UNIT);  // [tile % KEPT][token][row]
     float *lds_inverse = lds_kept + KEPT * 256u;                                 // [token]
     const uint32_t ring0 = (uint32_t)(uintptr_t)ring;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
@@ -173,28 +177,32 @@ __global__ __launch_bounds__(THREADS) void matvec_q6k_mfma_stream_kernel(Q6Args 
     auto first_row = [&](uint32_t p) { return p < q.rounds ? 32u * (b + p * G) : tail_row; };
     auto rows_of = [&](uint32_t p) { return p < q.rounds ? 32u : 8u * tail_units; };
 
-    // A unit's loads. The unit is 448 lines, row after row; load g = 7 wave + j brings lines
-    // 8 g .. 8 g + 7, lane l line 8 g + l / 8 and the chunk that belongs at position l % 8 of it.
-    // The whole address is the lane's offset, which is what the buffer's range check sees: rows
-    // past the matrix's end land as zeros.
+    // A unit's loads. The unit is 224 lines, row after row; load g = 4 wave + j brings lines
+    // 8 g .. 8 g + 7 (the eighth wave's four would be past the unit's end: they go against an
+    // empty buffer, so that every wave's waits count the same loads), lane l line 8 g + l / 8
+    // and the chunk that belongs at position l % 8 of it. The whole address is the lane's
+    // offset, which is what the buffer's range check sees: rows past the matrix's end land as zeros.
     uint32_t woff[LOADS];
 #pragma unroll
     for (int j = 0; j < LOADS; j++) {
-        const uint32_t line = 8u * (LOADS * wave + j) + (lane >> 3), row = line / 14u, in_row = line % 14u;
+        const uint32_t line = 8u * (LOADS * wave + j) + (lane >> 3), row = line / 7u, in_row = line % 7u;
         woff[j] = row * a.row_bytes + 128u * in_row + 16u * ((lane & 7u) ^ (row & 7u));
     }
-    // Unit v of the run: unit v % NU of tile v / NU. Past the run's end nothing is asked for.
+    // Unit v of the run: unit v % NU of tile v / NU. Past the run's end the loads still run, so
+    // that the waits count the same loads every step, but against an empty buffer: zeros land
+    // and nothing is fetched.
     auto issue = [&](uint32_t v, uint32_t slot) __attribute__((always_inline)) {
         const uint32_t p = v / NU, u = v % NU;
-        if (p >= count) return;
-        const uint32_t base = first_row(p) * a.row_bytes + ROW_UNIT * u, rows = rows_of(p);
-        const uint32_t dst = ring0 + slot * UNIT + 1024u * (LOADS * wave);
+        const bool real = p < count && wave < 7u;
+        const uint32_t base = (real ? first_row(p) : 0u) * a.row_bytes + ROW_UNIT * u, rows = rows_of(p);
+        // (a load against the empty buffer still lands zeros: the eighth wave's in a spare KB)
+        const uint32_t dst = wave < 7u ? ring0 + slot * UNIT + 1024u * (LOADS * wave) : ring0 + SLOTS * UNIT + KEPT * 1024u + 64u;
 #pragma unroll
         for (int j = 0; j < LOADS; j++) {
-            // (lines 8 g .. of rows the workgroup's share of the last rows does not have are not
-            // fetched: what the matrix instructions make of the slot's old contents is never stored)
-            const uint32_t first_line_row = (8u * (LOADS * wave + j)) / 14u;
-            load_lds_b128(first_line_row < rows ? wbuf : nobuf, dst + 1024u * j, woff[j] + base);
+            // (lines of rows the workgroup's share of the last rows does not have are not fetched;
+            // what the matrix instructions make of the zeros there is never stored)
+            const uint32_t first_line_row = (8u * (LOADS * wave + j)) / 7u;
+            load_lds_b128(real && first_line_row < rows ? wbuf : nobuf, wave < 7u ? dst + 1024u * j : dst, woff[j] + base);
         }
     };
 
@@ -206,69 +214,71 @@ __global__ __launch_bounds__(THREADS) void matvec_q6k_mfma_stream_kernel(Q6Args 
     const uint32_t rho = lane & 31u, kap = lane >> 5;
     const uint32_t tok = 4u * ((rho >> 2) & 1u) + (rho & 3u), piece = rho >> 3;
     const bool live = tok < a.m && piece < 2u;
-    qf16x8 xf[16 * NU];
+    // Wave w multiplies half w % 2 (sub-blocks 8 (w % 2) .. + 7, 128 positions) of block w / 2 of
+    // every unit.
+    const uint32_t blk = wave >> 1, half = wave & 1u;
+    qf16x8 xf[8 * NU];
     {
         const __amdgpu_buffer_rsrc_t pbuf = make_buffer(q.planes, 2u * a.m * a.k * 2u);
-        const uint32_t at = live ? ((piece * a.m + tok) * a.k + 256u * wave + 8u * kap) * 2u : 0xfffffff0u;
+        const uint32_t at = live ? ((piece * a.m + tok) * a.k + 256u * blk + 128u * half + 8u * kap) * 2u : 0xfffffff0u;
 #pragma unroll
         for (int u = 0; u < NU; u++)
 #pragma unroll
-            for (int s = 0; s < 16; s++)
-                xf[16 * u + s] = __builtin_bit_cast(qf16x8, __builtin_amdgcn_raw_buffer_load_b128(pbuf, live ? at + 2u * (2048u * u + 16u * s) : at, 0, 0));
+            for (int s = 0; s < 8; s++)
+                xf[8 * u + s] = __builtin_bit_cast(qf16x8, __builtin_amdgcn_raw_buffer_load_b128(pbuf, live ? at + 2u * (1024u * u + 16u * s) : at, 0, 0));
     }
     if (tid < 8u) lds_inverse[tid] = tid < a.m ? q.inverse[tid] : 1.0f;  // read behind later barriers
-    issue(0, 0);
+#pragma unroll
+    for (int v = 0; v < SLOTS - 1; v++) issue(v, v);
 
-    // The lane's reads of its wave's block of a unit: row rho of the flat copy, the block's
-    // bytes at 224 wave. Byte o of a row's unit sits at 1792 rho + 128 (o / 128) +
+    // The lane's reads of its wave's half block of a unit: row rho of the flat copy, the block's
+    // bytes at 224 (wave / 2). Byte o of a row's unit sits at 896 rho + 128 (o / 128) +
     // 16 ((o / 16 % 8) ^ (rho % 8)) + o % 16.
     auto at_byte = [&](uint32_t o) { return ROW_UNIT * rho + (o & ~127u) + 16u * (((o >> 4) & 7u) ^ (rho & 7u)) + (o & 15u); };
-    uint32_t at_ql[8], at_qh[4];  // ql: [half n][which 32 of the half's 64][which 16]; qh: [half n][which 16]
+    uint32_t at_ql[4], at_qh[2];  // ql: [which 32 of the half's 64][which 16]; qh: [which 16]
 #pragma unroll
-    for (uint32_t i = 0; i < 8; i++) at_ql[i] = at_byte(224u * wave + 64u * (i >> 2) + 32u * ((i >> 1) & 1u) + 16u * (i & 1u) + 8u * kap);
+    for (uint32_t i = 0; i < 4; i++) at_ql[i] = at_byte(224u * blk + 64u * half + 32u * (i >> 1) + 16u * (i & 1u) + 8u * kap);
 #pragma unroll
-    for (uint32_t i = 0; i < 4; i++) at_qh[i] = at_byte(224u * wave + 128u + 32u * (i >> 1) + 16u * (i & 1u) + 8u * kap);
-    const uint32_t at_sc = at_byte(224u * wave + 192u), at_d = at_byte(224u * wave + 208u);
+    for (uint32_t i = 0; i < 2; i++) at_qh[i] = at_byte(224u * blk + 128u + 32u * half + 16u * i + 8u * kap);
+    const uint32_t at_sc = at_byte(224u * blk + 192u + 8u * half), at_d = at_byte(224u * blk + 208u);
 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};  // tokens 4 (lane / 32) + i, matrix row rho of the tile, this wave's blocks
     auto multiply = [&](auto unit, uint32_t slot) __attribute__((always_inline)) {
         constexpr int U = decltype(unit)::value;
         const uint8_t *t = ring + slot * UNIT;
-        const qu32x4 sc = *reinterpret_cast<const qu32x4 *>(t + at_sc);
+        const qu32x2 sc = *reinterpret_cast<const qu32x2 *>(t + at_sc);
         const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(t + at_d));
 #pragma unroll
-        for (uint32_t n = 0; n < 2; n++)
+        for (uint32_t h16 = 0; h16 < 2; h16++) {
+            const qu32x2 qh = *reinterpret_cast<const qu32x2 *>(t + at_qh[h16]);
 #pragma unroll
-            for (uint32_t h16 = 0; h16 < 2; h16++) {
-                const qu32x2 qh = *reinterpret_cast<const qu32x2 *>(t + at_qh[2u * n + h16]);
+            for (uint32_t qp = 0; qp < 2; qp++) {
+                const qu32x2 ql = *reinterpret_cast<const qu32x2 *>(t + at_ql[2u * qp + h16]);
 #pragma unroll
-                for (uint32_t qp = 0; qp < 2; qp++) {
-                    const qu32x2 ql = *reinterpret_cast<const qu32x2 *>(t + at_ql[4u * n + 2u * qp + h16]);
+                for (uint32_t up = 0; up < 2; up++) {
+                    // Quadrant qd of the half: weights 32 qd + 16 h16 + 8 kap ... of its 128, sub-block 2 qd + h16 of its eight.
+                    const uint32_t qd = qp + 2u * up, s = 2u * qd + h16;
+                    qu32x2 v;
 #pragma unroll
-                    for (uint32_t up = 0; up < 2; up++) {
-                        // Quadrant qd of the half: weights 128 n + 32 qd + 16 h16 + 8 kap ..., sub-block 8 n + 2 qd + h16.
-                        const uint32_t qd = qp + 2u * up, s = 8u * n + 2u * qd + h16;
-                        qu32x2 v;
-#pragma unroll
-                        for (int w = 0; w < 2; w++) {
-                            const uint32_t nib = up ? (ql[w] >> 4) & 0x0f0f0f0fu : ql[w] & 0x0f0f0f0fu;
-                            const uint32_t two = (qd ? qh[w] >> (2u * qd) : qh[w]) & 0x03030303u;
-                            v[w] = nib | (two << 4);
-                        }
-                        const uint32_t word = s < 4u ? sc.x : s < 8u ? sc.y : s < 12u ? sc.z : sc.w;
-                        const float dsc = d * (float)(int8_t)((word >> (8u * (s & 3u))) & 0xffu);
-                        qf32x16 zero;
-#pragma unroll
-                        for (int e = 0; e < 16; e++) zero[e] = 0.f;
-                        const qf32x16 r = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[16 * U + s], weights_f16(v, bias), zero, 0, 0, 0);
-#pragma unroll
-                        for (int i = 0; i < 4; i++) acc[i] = fmaf(dsc, fmaf(r[4 + i], 1.0f / 2048.0f, r[i]), acc[i]);
-                        // (a sub-block's results are used up before the next sub-block's matrix
-                        // instruction: sixteen of them in flight would not fit the registers)
-                        asm volatile("" : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]));
+                    for (int w = 0; w < 2; w++) {
+                        const uint32_t nib = up ? (ql[w] >> 4) & 0x0f0f0f0fu : ql[w] & 0x0f0f0f0fu;
+                        const uint32_t two = (qd ? qh[w] >> (2u * qd) : qh[w]) & 0x03030303u;
+                        v[w] = nib | (two << 4);
                     }
+                    const uint32_t word = s < 4u ? sc.x : sc.y;
+                    const float dsc = d * (float)(int8_t)((word >> (8u * (s & 3u))) & 0xffu);
+                    qf32x16 zero;
+#pragma unroll
+                    for (int e = 0; e < 16; e++) zero[e] = 0.f;
+                    const qf32x16 r = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[8 * U + s], weights_f16(v, bias), zero, 0, 0, 0);
+#pragma unroll
+                    for (int i = 0; i < 4; i++) acc[i] = fmaf(dsc, fmaf(r[4 + i], 1.0f / 2048.0f, r[i]), acc[i]);
+                    // (a sub-block's results are used up before the next sub-block's matrix
+                    // instruction: eight of them in flight would not fit the registers)
+                    asm volatile("" : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]));
                 }
             }
+        }
     };
     // A finished tile's partial sums into LDS; they are added behind the next barrier.
     auto hand_over = [&](uint32_t p) __attribute__((always_inline)) {
@@ -306,25 +316,32 @@ __global__ __launch_bounds__(THREADS) void matvec_q6k_mfma_stream_kernel(Q6Args 
     };
 
     // One barrier a unit: behind it all of unit v has landed (every wave has waited for its own
-    // loads), nobody still reads the other slot, and the tile before's partial sums are in LDS.
+    // loads of it; those of the two units after it stay in flight), nobody still reads the slot
+    // that is refilled next, and the tile before's partial sums are in LDS.
+    auto step = [&](uint32_t p, auto unit) __attribute__((always_inline)) {
+        constexpr int U = decltype(unit)::value;
+        const uint32_t v = NU * p + U;
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SLOTS - 2) * LOADS) : "memory");
+        lds_barrier();
+        issue(v + (SLOTS - 1), (v + (SLOTS - 1)) % SLOTS);
+        if (U == 0 && p > 0u) {
+            sum_up(p - 1u);
+            // (the next tile's sums are kept only behind a later barrier, which no thread passes
+            // before it has stored what it stores here)
+            if (p % KEPT == 0u) store_kept(p - KEPT, KEPT);
+        }
+        multiply(unit, v % SLOTS);
+    };
     for (uint32_t p = 0; p < count; p++) {
-#pragma unroll
-        for (int u = 0; u < NU; u++) {
-            const uint32_t v = NU * p + u;
-            asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-            lds_barrier();
-            issue(v + 1u, (v + 1u) & 1u);
-            if (u == 0 && p > 0u) {
-                sum_up(p - 1u);
-                // (the tile's sums are kept only behind this barrier's successor, which no thread
-                // passes before it has stored what it stores here)
-                if (p % KEPT == 0u) store_kept(p - KEPT, KEPT);
-            }
-            if (u == 0) multiply(std::integral_constant<int, 0>{}, v & 1u);
-            else multiply(std::integral_constant<int, NU - 1>{}, v & 1u);
+        step(p, std::integral_constant<int, 0>{});
+        if constexpr (NU >= 2) step(p, std::integral_constant<int, 1>{});
+        if constexpr (NU >= 4) {
+            step(p, std::integral_constant<int, 2>{});
+            step(p, std::integral_constant<int, 3>{});
         }
         hand_over(p);
     }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still land in LDS once the workgroup is gone
     if (count > 0u) {
         lds_barrier();
         sum_up(count - 1u);
@@ -351,7 +368,7 @@ zhip_result launch_blocks(const Dispatch &d, const Q6Args &q, dim3 grid) {
 
 // Whether this kernel can run the (already validated) arguments: k of whole units, no pair.
 bool matvec_q6k_mfma_stream_accepts(const MvArgs &a) {
-    return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u) && !(a.flags & FLAG_SILU_PAIR) && a.rows >= 1 && a.xr % 4u == 0 &&
+    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && !(a.flags & FLAG_SILU_PAIR) && a.rows >= 1 && a.xr % 4u == 0 &&
            (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == a.k / 256u * 224u;
 }
 
@@ -376,7 +393,7 @@ zhip_result launch_matvec_q6k_mfma_stream(const Dispatch &d, const MvArgs &a, ui
     q.a.norm_w = nullptr;
     q.a.act_div = 0.f;
     const dim3 grid(groups);
-    return a.k == 2048u ? launch_blocks<1>(d, q, grid) : launch_blocks<2>(d, q, grid);
+    return a.k == 1024u ? launch_blocks<1>(d, q, grid) : a.k == 2048u ? launch_blocks<2>(d, q, grid) : launch_blocks<4>(d, q, grid);
 }
 
 }  // namespace zhip
