@@ -8,15 +8,20 @@
 // once, straight into matrix-core operands that stay in registers for the
 // whole kernel (64 VGPRs at k = 4096), together with the rows' sub-block sums
 // (32 VGPRs). It then walks over sixteen-row weight tiles, persistent
-// workgroups taking tiles b, b + G, ...: its blocks of the tile's sixteen rows
-// (144 sixteen-byte chunks a block, three wave-wide direct loads into a private
-// ring of LDS slots: whole-line accesses; a lane loading its own row's bytes
-// straight into registers costs fifty cache accesses a load) arrive a tile
-// ahead, each lane reads its row's header and nibbles back, and multiplies;
-// the eight waves' partial sums (512 bytes a wave and tile) meet in LDS, where
-// 128 threads add the eight for one output each (row i % 16, token i / 16) in
-// the order of the k ranges, apply the SILU_PAIR / ACCUMULATE epilogue and store. One
-// barrier a tile; no barrier waits for the loads in flight.
+// workgroups taking tiles b, b + G, ...: a tile's sixteen rows are one contiguous
+// stretch of the matrix and travel as a flat copy through a ring of three LDS
+// slots that the workgroup shares, every wave loading a share of it by wave-wide
+// direct loads of whole lines, two tiles ahead (a wave fetching only its own
+// blocks, 144-byte pieces that lie across line boundaries, made every line a
+// request of two or three waves: 20.7 against 19.7 us on the 2 x 14336 x 4096
+// pair at four tokens; a lane loading its own row's bytes straight into
+// registers costs fifty cache accesses a load). Each wave waits for its own
+// loads and one barrier a tile tells everyone that all of the tile has landed;
+// behind the same barrier the tile before's partial sums (512 bytes a wave) are
+// in LDS, where 128 threads add the eight for one output each (row i % 16,
+// token i / 16) in the order of the k ranges, apply the SILU_PAIR / ACCUMULATE
+// epilogue and store. Each lane reads its row's header and nibbles back from
+// the copy (chunks XOR-permuted by row against bank conflicts) and multiplies.
 //
 // Contract as the other variants (src/kernels/matvec_quant.wgsl.hbs); a token's
 // result does not depend on how many tokens share the launch.
@@ -37,8 +42,12 @@ typedef uint32_t ru32x2 __attribute__((ext_vector_type(2)));
 namespace {
 
 constexpr uint32_t THREADS = 512, WAVES = 8;
-constexpr int DEPTH = 3;  // ring slots a wave: one tile multiplied, the others in flight
-constexpr uint32_t SLOT = 3u * 1024u;  // a block: 2304 bytes; the third load's idle lanes land behind them
+constexpr int DEPTH = 3;  // ring slots: one tile multiplied, the others in flight (two slots: +0.3 us on the 2 x 14336 x 4096 pair, four: +0.8 us)
+// A tile in LDS: the flat copy of its sixteen rows (NB = 256-weight blocks of a wave's k range:
+// a row is 1152 NB bytes, nine lines a block column of the eight waves).
+template <int NB> constexpr uint32_t tile_bytes() { return 16u * 1152u * NB; }
+// Wave-wide loads of a tile a wave issues: 18 NB of 1 KB in all; the slots past them ask for nothing.
+template <int NB> constexpr int tile_loads() { return NB == 2 ? 5 : 3; }
 
 struct ResArgs {
     MvArgs a;
@@ -66,10 +75,9 @@ typedef __attribute__((address_space(3))) void *lds_ptr;
 // One wave-wide load of 16 bytes a lane straight into LDS (lane l lands at dst + 16 l). The
 // destination reaches the load as a bare LDS address, so the compiler keeps no dependency
 // between these loads and later LDS reads; the explicit waits order them.
-__device__ __forceinline__ void load_lds_b128(__amdgpu_buffer_rsrc_t buf, uint8_t *dst, uint32_t voffset, uint32_t soffset) {
-    uint32_t address = __builtin_amdgcn_readfirstlane((uint32_t)(uintptr_t)dst);
-    asm volatile("" : "+s"(address));
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)(uintptr_t)address, 16, voffset, soffset, 0, 0);
+__device__ __forceinline__ void load_lds_b128(__amdgpu_buffer_rsrc_t buf, uint32_t dst, uint32_t voffset) {
+    asm volatile("" : "+s"(dst));
+    __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)(uintptr_t)dst, 16, voffset, 0, 0, 0);
 }
 
 template <int LEFT>
@@ -132,32 +140,36 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
     auto rows_of = [&](uint32_t p) { return (q.split && p / per >= q.rounds) ? 8u : 16u; };
     auto row0 = [&](uint32_t p) { return out0(p) + ((PAIR && (p & 1u)) ? a.half : 0u); };
 
-    // A tile's loads: chunk c of a block's 144 (row c / 9, sixteen bytes c % 9) by lane c % 64 of
-    // load c / 64; past 144 a lane asks beyond the buffer and zeros land. The tile's part of
-    // the offset is uniform and travels in a scalar register (the buffer's range check does
-    // not see it: every row of a tile exists here). Past the run's last tile the loads still
-    // run, so that the waits count the same loads every step, but against an empty buffer:
-    // zeros land and nothing is fetched.
-    __shared__ __align__(16) uint8_t lds_ring[WAVES * DEPTH * NB * SLOT];
-    uint8_t *ring = lds_ring + wave * (DEPTH * NB * SLOT);
-    uint32_t woff[3], woff8[3];  // (woff8: the same for an eight-row share, whose other rows are not fetched)
+    // A tile's loads. The tile's sixteen rows are one contiguous stretch of the matrix, 18 NB
+    // KB of whole lines, and travel as a flat copy into one of the ring's slots, which the whole
+    // workgroup shares: load g = LOADS wave + j brings lines 8 g .. 8 g + 7 (the slots past the
+    // tile's last line go against an empty buffer and land their zeros in a spare KB, so that
+    // every wave's waits count the same loads), lane l line 8 g + l / 8 and the chunk that
+    // belongs at position l % 8 of it: chunk c of a line of row r sits at position c ^ (r % 8).
+    // The whole address is the lane's offset. Past the run's last tile the loads still run, but
+    // against the empty buffer: zeros land and nothing is fetched.
+    constexpr int LOADS = tile_loads<NB>();
+    constexpr uint32_t TILE = tile_bytes<NB>(), ROW_LINES = 9u * NB, TILE_LOADS = 18u * NB;
+    __shared__ __align__(16) uint8_t lds_ring[DEPTH * TILE + 1024u];
+    const uint32_t ring0 = (uint32_t)(uintptr_t)lds_ring;
+    const uint32_t uwave = __builtin_amdgcn_readfirstlane(wave);
+    uint32_t woff[LOADS];
 #pragma unroll
-    for (uint32_t j = 0; j < 3; j++) {
-        const uint32_t c = 64u * j + lane;
-        woff[j] = c < 144u ? (c / 9u) * a.row_bytes + 16u * (c % 9u) + NB * wave * 144u : 0xfffffff0u - 144u * NB;
-        woff8[j] = c < 72u ? woff[j] : 0xfffffff0u - 144u * NB;
+    for (int j = 0; j < LOADS; j++) {
+        const uint32_t line = 8u * (LOADS * wave + j) + (lane >> 3), row = line / ROW_LINES;
+        woff[j] = 128u * line + 16u * ((lane & 7u) ^ (row & 7u));
     }
     auto load_tile = [&](uint32_t p, uint32_t slot) __attribute__((always_inline)) {
         const bool real = p < count;
-        const __amdgpu_buffer_rsrc_t buf = real ? wbuf : nobuf;
-        const uint32_t base = (real ? row0(p) : 0u) * a.row_bytes;
-        const bool whole = rows_of(p) == 16u;
+        const uint32_t base = (real ? row0(p) : 0u) * a.row_bytes, rows = rows_of(p);
 #pragma unroll
-        for (uint32_t i = 0; i < NB; i++)
-#pragma unroll
-            for (uint32_t j = 0; j < 3; j++) load_lds_b128(buf, ring + (slot * NB + i) * SLOT + 1024u * j, (whole ? woff[j] : woff8[j]) + 144u * i, base);
+        for (int j = 0; j < LOADS; j++) {
+            const uint32_t g = LOADS * uwave + j;
+            // (the lines of the rows an eight-row share does not have are not fetched)
+            const bool wanted = real && g < TILE_LOADS && (8u * g) / ROW_LINES < rows;
+            load_lds_b128(wanted ? wbuf : nobuf, g < TILE_LOADS ? ring0 + slot * TILE + 1024u * g : ring0 + DEPTH * TILE, woff[j] + base);
+        }
     };
-    constexpr int LOADS = 3 * NB;  // a tile's loads of one wave
 
     // The tokens' inputs first: loads complete in order within a wave, and behind the weight
     // loads below the first use of an input would wait for a round trip of the weight stream.
@@ -272,13 +284,26 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
         }
     }
 
+    // The lane's reads of its wave's blocks of a tile: row l16 of the flat copy, blocks
+    // NB wave + i. Byte f of the copy sits at 128 (f / 128) + 16 ((f / 16 % 8) ^ (l16 % 8)) + f % 16.
+    auto at_byte = [&](uint32_t f) { return (f & ~127u) + 16u * (((f >> 4) & 7u) ^ (l16 & 7u)) + (f & 15u); };
+    uint32_t at_header[NB], at_nibbles[NB][4];
+#pragma unroll
+    for (uint32_t i = 0; i < NB; i++) {
+        const uint32_t block = 1152u * NB * l16 + 144u * (NB * wave + i);
+        at_header[i] = at_byte(block);
+#pragma unroll
+        for (uint32_t c = 0; c < 4; c++) at_nibbles[i][c] = at_byte(block + 16u + 32u * c + 8u * g);
+    }
+
     float held = 0.f;  // the gate tile's result, until the up tile's arrives
-    auto step = [&](uint32_t p, uint32_t slot) __attribute__((always_inline)) {
+    // Multiplies tile p from its slot and leaves the wave's partial sums in LDS.
+    auto multiply = [&](uint32_t p, uint32_t slot) __attribute__((always_inline)) {
         float acc[2] = {0.f, 0.f};  // tokens 2 g and 2 g + 1, matrix row row0 + l16, this wave's k range
+        const uint8_t *tile = lds_ring + slot * TILE;
 #pragma unroll
         for (int i = 0; i < NB; i++) {
-            const uint8_t *block = ring + (slot * NB + i) * SLOT + l16 * 144u;
-            const ru32x4 h = *reinterpret_cast<const ru32x4 *>(block);
+            const ru32x4 h = *reinterpret_cast<const ru32x4 *>(tile + at_header[i]);
             const float d = half_bits_to_float(h.x & 0xffffu), dmin = half_bits_to_float(h.x >> 16);
             // The eight 6-bit scales and minimums as bytes of four words (src/ref/tensor.zig:94-98).
             const uint32_t sc_lo_ = h.y & 0x3f3f3f3fu, mn_lo_ = h.z & 0x3f3f3f3fu;
@@ -290,7 +315,7 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
             asm volatile("" : "+v"(sc_lo), "+v"(mn_lo), "+v"(sc_hi), "+v"(mn_hi));
 #pragma unroll
             for (uint32_t c = 0; c < 4; c++) {
-                const ru32x2 wq = *reinterpret_cast<const ru32x2 *>(block + 16u + 32u * c + 8u * g);
+                const ru32x2 wq = *reinterpret_cast<const ru32x2 *>(tile + at_nibbles[i][c]);
 #pragma unroll
                 for (uint32_t half = 0; half < 2; half++) {
                     const uint32_t sb = 2u * c + half, shift = 8u * (sb & 3u);
@@ -306,42 +331,53 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
         }
         float *part = &lds_part[p & 1u][0][0];
         *reinterpret_cast<float2 *>(part + wave * 128u + 2u * lane) = float2{acc[0], acc[1]};
-        lds_barrier();
-        // Buffer p % 2 is written again in step p + 2, after the barrier of step p + 1, which
-        // a wave passes only when it has read what it needs here.
-        // The 128 outputs of a tile are summed by one pair of waves, a different pair from one
-        // output tile to the next (the extra work does not make the same waves late every time).
-        if ((tid >> 7) == ((p / per) & 3u)) {
-            const uint32_t row = tid & 15u, t = (tid >> 4) & 7u;
-            const float *src = part + 2u * ((t >> 1) * 16u + row) + (t & 1u);
-            float sum = src[0];
+    };
+    // Adds the eight waves' partial sums of tile p, behind the barrier that follows its
+    // multiply. Buffer p % 2 is written again by the multiply of tile p + 2, behind the next
+    // barrier, which a wave passes only when it has read what it needs here. The 128 outputs of
+    // a tile are summed by one pair of waves, a different pair from one output tile to the next
+    // (the extra work does not make the same waves late every time).
+    auto sum_up = [&](uint32_t p) __attribute__((always_inline)) {
+        if ((tid >> 7) != ((p / per) & 3u)) return;
+        const float *part = &lds_part[p & 1u][0][0];
+        const uint32_t row = tid & 15u, t = (tid >> 4) & 7u;
+        const float *src = part + 2u * ((t >> 1) * 16u + row) + (t & 1u);
+        float sum = src[0];
 #pragma unroll
-            for (uint32_t wv = 1; wv < WAVES; wv++) sum += src[wv * 128u];
-            sum *= lds_scale[8 + t];
-            if (PAIR && !(p & 1u)) {
-                held = sum;
-            } else {
-                const float v = PAIR ? silu_f(held) * sum : sum;
-                if (t < a.m && row < rows_of(p)) {
-                    float *o = a.out + (size_t)t * a.out_stride + a.col0 + out0(p) + row;
-                    store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + v : v);
-                }
+        for (uint32_t wv = 1; wv < WAVES; wv++) sum += src[wv * 128u];
+        sum *= lds_scale[8 + t];
+        if (PAIR && !(p & 1u)) {
+            held = sum;
+        } else {
+            const float v = PAIR ? silu_f(held) * sum : sum;
+            if (t < a.m && row < rows_of(p)) {
+                float *o = a.out + (size_t)t * a.out_stride + a.col0 + out0(p) + row;
+                store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + v : v);
             }
         }
     };
 
-    // DEPTH ring slots in rotation: DEPTH - 1 tiles in flight behind the one multiplied. Every
-    // wave of the workgroup runs the same steps (the barrier inside). Before tile p is read,
-    // all but the loads of the DEPTH - 1 tiles after it have landed.
+    // DEPTH ring slots in rotation: DEPTH - 1 tiles in flight behind the one multiplied. One
+    // barrier a tile: behind it all of tile p has landed (every wave has waited for its own
+    // loads of it), nobody still reads the slot that is refilled next, and the partial sums of
+    // the tile before are in LDS.
 #pragma unroll
     for (int s = 1; s < DEPTH - 1; s++) load_tile(s, s);
     for (uint32_t p = 0; p < count; p += DEPTH) {
 #pragma unroll
         for (int s = 0; s < DEPTH; s++) {
-            load_tile(p + s + (DEPTH - 1), (s + DEPTH - 1) % DEPTH);
-            wait_loads<(DEPTH - 1) * LOADS>();
-            if (p + s < count) step(p + s, s);
+            if (p + s < count) {
+                wait_loads<(DEPTH - 2) * LOADS>();
+                lds_barrier();
+                load_tile(p + s + (DEPTH - 1), (s + DEPTH - 1) % DEPTH);
+                if (p + s > 0u) sum_up(p + s - 1u);
+                multiply(p + s, s);
+            }
         }
+    }
+    if (count > 0u) {
+        lds_barrier();
+        sum_up(count - 1u);
     }
     wait_loads<0>();  // nothing may still land in LDS once the workgroup is gone
 }
