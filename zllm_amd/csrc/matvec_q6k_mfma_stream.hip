@@ -26,7 +26,8 @@
 // flight while one is multiplied (two slots of twice the size, one unit in flight, measured the
 // same 94 us on 128256 x 4096: per 16-weight sub-block and wave the kernel issues 24 vector
 // instructions and a matrix instruction that do not overlap, 0.85 us a unit and SIMD against
-// the 1.1 us the unit's bytes need at full rate, and the two overlap only in part). Chunk c (16 bytes) of a line of row r sits at position
+// the 1.1 us the unit's bytes need at full rate, and the two overlap only in part: with the
+// multiplies switched off the same launch takes 80 us, 6.1 TB/s). Chunk c (16 bytes) of a line of row r sits at position
 // c ^ (r % 8), which keeps the 32 rows' reads of one piece of a block to four lanes a bank. The
 // waves' partial sums meet in LDS behind the same barrier, are added in the order of the blocks
 // and wait there for one burst of stores when the workgroup's run ends. Workgroups are numbered
