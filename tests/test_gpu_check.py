@@ -336,8 +336,10 @@ MFMA_VARIANT = K.MatvecVariant(wg=512, lanes=64, rows=16)
     (False, 2, 48, 2048),
 ])
 @pytest.mark.parametrize("prologue", ["plain", "norm", "norm_act"])
-def test_quant_matvec_mfma_variant(ctx, pair, rows, n, k, prologue):
-    """The matrix-core variant of matvec_q4_k (a wave per sixteen rows): every
+@pytest.mark.parametrize("t", [TensorType.q4_k, TensorType.q5_k])
+def test_quant_matvec_mfma_variant(ctx, t, pair, rows, n, k, prologue):
+    """The matrix-core variant of matvec_q4_k and matvec_q5_k (a wave per sixteen rows; Q5_K has
+    it for k of 2048 or 4096 and whole tiles, its other cases run the default variant): every
     row within 1e-5 of float64 over the decoded weights, each token bitwise
     equal to its lone launch, and nothing outside the outputs touched; also
     with the prologues the planner's launches carry (RMSNorm times its weights
@@ -348,10 +350,10 @@ def test_quant_matvec_mfma_variant(ctx, pair, rows, n, k, prologue):
     x[0] *= np.float32(1e-4)          # tokens of very different magnitudes
     x[rows - 1] *= np.float32(300.0)
     nw = c.random(k, 1.5)
-    raw, values = quant_rows(c, TensorType.q4_k, 2 * n if pair else n, k)
+    raw, values = quant_rows(c, t, 2 * n if pair else n, k)
     stride = n + 7
     init = c.random(rows * stride, 2).reshape(rows, stride)
-    xa, wa = c.upload(x), c.gpu_weights(TensorType.q4_k, raw, k)
+    xa, wa = c.upload(x), c.gpu_weights(t, raw, k)
     na = c.upload(nw) if norm else wa
     v64 = values.astype(np.float64)
     x64 = np.stack([norm_row(r, nw if norm else None, eps) for r in x])
@@ -364,7 +366,7 @@ def test_quant_matvec_mfma_variant(ctx, pair, rows, n, k, prologue):
         want = init[:, 3 : 3 + n] + x64 @ v64.T
     p = lambda: P.MatvecBf16(n=n, k=k, col0=3, out_stride=stride, eps=eps, norm=norm, accumulate=not pair, silu_pair=pair, half=n if pair else 0)
     variant = K.MatvecVariant(MFMA_VARIANT.wg, MFMA_VARIANT.lanes, MFMA_VARIANT.rows, div)
-    pipeline = c.set.matvec(c.rec, Kernel.matvec_q4_k, variant)
+    pipeline = c.set.matvec(c.rec, K.weight_kernel("matvec", t), variant)
     grid_x = K.div_ceil(n, variant.group_rows())
     out = c.upload(init)
     c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, na], (grid_x, rows, 1))

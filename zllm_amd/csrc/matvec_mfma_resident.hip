@@ -1,4 +1,4 @@
-// matvec_q4_k, matrix-core variant for k = 2048 or 4096: the same arithmetic as
+// matvec_q4_k and matvec_q5_k, matrix-core variant for k = 2048 or 4096: the same arithmetic as
 // matvec_mfma.hip (weights as exact f16 values 16 + q, every token as two f16
 // rows, per-token power-of-two scale; see there), laid out so that nothing
 // is recomputed and nothing but partial results crosses LDS.
@@ -43,16 +43,33 @@ namespace {
 
 constexpr uint32_t THREADS = 512, WAVES = 8;
 constexpr int DEPTH = 3;  // ring slots: one tile multiplied, the others in flight (two slots: +0.3 us on the 2 x 14336 x 4096 pair, four: +0.8 us)
+// The formats: a 256-weight block is a 16-byte header (d, dmin, twelve bytes of 6-bit scales and
+// minimums) and 128 bytes of nibbles; Q5_K keeps a fifth bit of every weight in 32 bytes between
+// the two (src/ref/tensor.zig:100-117). A weight enters the matrix cores as the exact f16 value
+// BIAS + q: the quant dropped into the mantissa of BIAS (16.0 for four bits, 32.0 for five).
+struct ResQ4 {
+    static constexpr uint32_t BLOCK = 144, NIBBLES_AT = 16, SHIFT = 6;
+    static constexpr bool FIFTH = false;
+    static constexpr float BIAS = 16.0f;
+    static const char *name() { return "matvec_q4_k"; }
+};
+struct ResQ5 {
+    static constexpr uint32_t BLOCK = 176, NIBBLES_AT = 48, SHIFT = 5;
+    static constexpr bool FIFTH = true;
+    static constexpr float BIAS = 32.0f;
+    static const char *name() { return "matvec_q5_k"; }
+};
 // A tile in LDS: the flat copy of its sixteen rows (NB = 256-weight blocks of a wave's k range:
-// a row is 1152 NB bytes, nine lines a block column of the eight waves).
-template <int NB> constexpr uint32_t tile_bytes() { return 16u * 1152u * NB; }
-// Wave-wide loads of a tile a wave issues: 18 NB of 1 KB in all; the slots past them ask for nothing.
-template <int NB> constexpr int tile_loads() { return NB == 2 ? 5 : 3; }
+// a row is 8 NB blocks, nine or eleven lines a block column of the eight waves).
+template <class F, int NB> constexpr uint32_t tile_bytes() { return 16u * 8u * F::BLOCK * NB; }
+// Wave-wide loads of 1 KB a tile takes, and how many a wave issues (the slots past the tile's end ask for nothing).
+template <class F, int NB> constexpr uint32_t tile_kb() { return tile_bytes<F, NB>() / 1024u; }
+template <class F, int NB> constexpr int tile_loads() { return (int)((tile_kb<F, NB>() + 7u) / 8u); }
 
 struct ResArgs {
     MvArgs a;
     uint32_t w_bytes;
-    uint32_t nibble_mask, sixteen;  // 0x03C003C0, 0x4C004C00 (see nibbles)
+    uint32_t nibble_mask, sixteen;  // Q4_K: 0x03C003C0, 0x4C004C00; Q5_K: 0x01E001E0, 0x50005000 (see nibbles)
     uint32_t rounds;                // sixteen-output tiles every workgroup takes: tiles b, b + G, ...
     uint32_t left;                  // output tiles after those, fewer than G: one for each of the first workgroups,
     uint32_t split;                 // or (split) eight outputs of one for each of the first 2 * left
@@ -93,29 +110,38 @@ __device__ __forceinline__ void store_apart(float *at, float v) {
     asm volatile("global_store_dword %0, %1, off\n\ts_nop 0" ::"v"(at), "v"(v) : "memory");
 }
 
-// Eight nibbles of two words as f16 values 16 + q in the order k0 k2 k1 k3 k4 k6 k5 k7 (the
+// Eight nibbles of two words as f16 values BIAS + q in the order k0 k2 k1 k3 k4 k6 k5 k7 (the
 // inputs' operands are built in the same order). `mask` arrives in a scalar register and
-// `sixteen` in a vector one: a shift and one v_and_or_b32 a pair.
-template <bool HIGH>
-__device__ __forceinline__ rf16x8 nibbles(ru32x2 w, uint32_t mask, uint32_t sixteen) {
+// `sixteen` (the bits of BIAS, twice) in a vector one: a shift and one v_and_or_b32 a pair.
+// Q5_K: `fifth` holds the weights' fifth bits in bit 0 of its bytes.
+template <class F, bool HIGH>
+__device__ __forceinline__ rf16x8 nibbles(ru32x2 w, ru32x2 fifth, uint32_t mask, uint32_t sixteen) {
+    constexpr uint32_t S = F::SHIFT;  // the quant's lowest bit in the f16 mantissa
     ru32x4 r;
     if (HIGH) {
-        r.x = ((w.x << 2) & mask) | sixteen;
-        r.y = ((w.x >> 6) & mask) | sixteen;
-        r.z = ((w.y << 2) & mask) | sixteen;
-        r.w = ((w.y >> 6) & mask) | sixteen;
+        r.x = ((w.x << (S - 4u)) & mask) | sixteen;
+        r.y = ((w.x >> (12u - S)) & mask) | sixteen;
+        r.z = ((w.y << (S - 4u)) & mask) | sixteen;
+        r.w = ((w.y >> (12u - S)) & mask) | sixteen;
     } else {
-        r.x = ((w.x << 6) & mask) | sixteen;
-        r.y = ((w.x >> 2) & mask) | sixteen;
-        r.z = ((w.y << 6) & mask) | sixteen;
-        r.w = ((w.y >> 2) & mask) | sixteen;
+        r.x = ((w.x << S) & mask) | sixteen;
+        r.y = ((w.x >> (8u - S)) & mask) | sixteen;
+        r.z = ((w.y << S) & mask) | sixteen;
+        r.w = ((w.y >> (8u - S)) & mask) | sixteen;
+    }
+    if (F::FIFTH) {
+        // bit 0 of bytes 0 and 2 to bits 9 and 25 (k0, k2), of bytes 1 and 3 likewise (k1, k3)
+        r.x |= (fifth.x << 9) & 0x02000200u;
+        r.y |= (fifth.x << 1) & 0x02000200u;
+        r.z |= (fifth.y << 9) & 0x02000200u;
+        r.w |= (fifth.y << 1) & 0x02000200u;
     }
     return __builtin_bit_cast(rf16x8, r);
 }
 
 // NB: 256-weight blocks of a wave's k range (k = 2048 NB).
-template <bool PAIR, int NB>
-__global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResArgs q) {
+template <class F, bool PAIR, int NB>
+__global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_resident_kernel(ResArgs q) {
     const MvArgs &a = q.a;
     __shared__ float lds_scale[16];               // [8 ..]: one over each token's scale
     __shared__ float lds_max[WAVES * 8];          // [wave][token]: the largest magnitude in the wave's range
@@ -148,8 +174,8 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
     // belongs at position l % 8 of it: chunk c of a line of row r sits at position c ^ (r % 8).
     // The whole address is the lane's offset. Past the run's last tile the loads still run, but
     // against the empty buffer: zeros land and nothing is fetched.
-    constexpr int LOADS = tile_loads<NB>();
-    constexpr uint32_t TILE = tile_bytes<NB>(), ROW_LINES = 9u * NB, TILE_LOADS = 18u * NB;
+    constexpr int LOADS = tile_loads<F, NB>();
+    constexpr uint32_t TILE = tile_bytes<F, NB>(), ROW_LINES = 8u * F::BLOCK * NB / 128u, TILE_LOADS = tile_kb<F, NB>();
     __shared__ __align__(16) uint8_t lds_ring[DEPTH * TILE + 1024u];
     const uint32_t ring0 = (uint32_t)(uintptr_t)lds_ring;
     const uint32_t uwave = __builtin_amdgcn_readfirstlane(wave);
@@ -287,13 +313,14 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
     // The lane's reads of its wave's blocks of a tile: row l16 of the flat copy, blocks
     // NB wave + i. Byte f of the copy sits at 128 (f / 128) + 16 ((f / 16 % 8) ^ (l16 % 8)) + f % 16.
     auto at_byte = [&](uint32_t f) { return (f & ~127u) + 16u * (((f >> 4) & 7u) ^ (l16 & 7u)) + (f & 15u); };
-    uint32_t at_header[NB], at_nibbles[NB][4];
+    uint32_t at_header[NB], at_fifth[NB], at_nibbles[NB][4];
 #pragma unroll
     for (uint32_t i = 0; i < NB; i++) {
-        const uint32_t block = 1152u * NB * l16 + 144u * (NB * wave + i);
+        const uint32_t block = 8u * F::BLOCK * NB * l16 + F::BLOCK * (NB * wave + i);
         at_header[i] = at_byte(block);
+        at_fifth[i] = at_byte(block + 16u + 8u * g);
 #pragma unroll
-        for (uint32_t c = 0; c < 4; c++) at_nibbles[i][c] = at_byte(block + 16u + 32u * c + 8u * g);
+        for (uint32_t c = 0; c < 4; c++) at_nibbles[i][c] = at_byte(block + F::NIBBLES_AT + 32u * c + 8u * g);
     }
 
     float held = 0.f;  // the gate tile's result, until the up tile's arrives
@@ -313,6 +340,8 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
             // a 6-bit field of the raw word needs two)
             uint32_t sc_lo = sc_lo_, mn_lo = mn_lo_, sc_hi = sc_hi_;
             asm volatile("" : "+v"(sc_lo), "+v"(mn_lo), "+v"(sc_hi), "+v"(mn_hi));
+            ru32x2 bits = {0u, 0u};  // Q5_K: bit sb of a byte is the fifth bit of the position's weight in sub-block sb
+            if (F::FIFTH) bits = *reinterpret_cast<const ru32x2 *>(tile + at_fifth[i]);
 #pragma unroll
             for (uint32_t c = 0; c < 4; c++) {
                 const ru32x2 wq = *reinterpret_cast<const ru32x2 *>(tile + at_nibbles[i][c]);
@@ -320,8 +349,9 @@ __global__ __launch_bounds__(THREADS) void matvec_q4k_mfma_resident_kernel(ResAr
                 for (uint32_t half = 0; half < 2; half++) {
                     const uint32_t sb = 2u * c + half, shift = 8u * (sb & 3u);
                     const float dsc = d * (float)(((sb < 4u ? sc_lo : sc_hi) >> shift) & 0xffu);
-                    const float off = fmaf(16.0f, dsc, dmin * (float)(((sb < 4u ? mn_lo : mn_hi) >> shift) & 0xffu));
-                    const rf16x8 wf = half ? nibbles<true>(wq, q.nibble_mask, sixteen) : nibbles<false>(wq, q.nibble_mask, sixteen);
+                    const float off = fmaf(F::BIAS, dsc, dmin * (float)(((sb < 4u ? mn_lo : mn_hi) >> shift) & 0xffu));
+                    const ru32x2 fifth = {sb ? bits.x >> sb : bits.x, sb ? bits.y >> sb : bits.y};
+                    const rf16x8 wf = half ? nibbles<F, true>(wq, fifth, q.nibble_mask, sixteen) : nibbles<F, false>(wq, fifth, q.nibble_mask, sixteen);
                     const rf32x4 r = __builtin_amdgcn_mfma_f32_16x16x32_f16(xf[8 * i + sb], wf, rf32x4{0.f, 0.f, 0.f, 0.f}, 0, 0, 0);
                     const float2 xs = xsum[8 * i + sb];
                     acc[0] = fmaf(-off, xs.x, fmaf(dsc, fmaf(r[1], 1.0f / 2048.0f, r[0]), acc[0]));
@@ -391,25 +421,36 @@ bool matvec_q4k_mfma_resident_accepts(const MvArgs &a) {
     return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u) && a.rows % 16u == 0 && (!pair || a.half % 16u == 0);
 }
 
-zhip_result launch_matvec_q4k_mfma_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) {
+template <class F>
+static zhip_result launch_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes, uint32_t mask, uint32_t bias_bits) {
     const bool pair = a.flags & FLAG_SILU_PAIR;
     // 32-bit byte offsets.
     const uint64_t reach = ((uint64_t)(pair ? a.half : 0u) + a.rows + 16u) * a.row_bytes;
-    if (w_bytes >= 0xfffffff0ull || reach >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "matvec_q4_k: operands of 4 GiB or more");
+    if (w_bytes >= 0xfffffff0ull || reach >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", F::name());
     const uint32_t cus = (uint32_t)d.dev->compute_units, tiles = a.rows / 16u;
     const uint32_t groups = tiles < cus ? (2u * tiles <= cus ? 2u * tiles : tiles) : cus;
     const bool halves = tiles < groups;  // every workgroup takes eight outputs of one tile
     const uint32_t left = halves ? tiles : tiles % groups;
-    ResArgs q{a, (uint32_t)w_bytes, 0x03C003C0u, 0x4C004C00u, halves ? 0u : tiles / groups, left, (halves || 2u * left <= groups) ? 1u : 0u};
+    ResArgs q{a, (uint32_t)w_bytes, mask, bias_bits, halves ? 0u : tiles / groups, left, (halves || 2u * left <= groups) ? 1u : 0u};
     const dim3 grid(groups);
     if (a.k == 2048u) {
-        if (pair) hipLaunchKernelGGL((matvec_q4k_mfma_resident_kernel<true, 1>), grid, dim3(THREADS), 0, d.stream, q);
-        else hipLaunchKernelGGL((matvec_q4k_mfma_resident_kernel<false, 1>), grid, dim3(THREADS), 0, d.stream, q);
+        if (pair) hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, true, 1>), grid, dim3(THREADS), 0, d.stream, q);
+        else hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, false, 1>), grid, dim3(THREADS), 0, d.stream, q);
     } else {
-        if (pair) hipLaunchKernelGGL((matvec_q4k_mfma_resident_kernel<true, 2>), grid, dim3(THREADS), 0, d.stream, q);
-        else hipLaunchKernelGGL((matvec_q4k_mfma_resident_kernel<false, 2>), grid, dim3(THREADS), 0, d.stream, q);
+        if (pair) hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, true, 2>), grid, dim3(THREADS), 0, d.stream, q);
+        else hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, false, 2>), grid, dim3(THREADS), 0, d.stream, q);
     }
-    return check_launch(d, "matvec_q4_k");
+    return check_launch(d, F::name());
+}
+
+zhip_result launch_matvec_q4k_mfma_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) {
+    return launch_resident<ResQ4>(d, a, w_bytes, 0x03C003C0u, 0x4C004C00u);
+}
+
+// The same for matvec_q5_k (the arguments the Q4_K kernel accepts, rows of 176-byte blocks).
+bool matvec_q5k_mfma_resident_accepts(const MvArgs &a) { return matvec_q4k_mfma_resident_accepts(a) && a.row_bytes == a.k / 256u * 176u; }
+zhip_result launch_matvec_q5k_mfma_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) {
+    return launch_resident<ResQ5>(d, a, w_bytes, 0x01E001E0u, 0x50005000u);
 }
 
 }  // namespace zhip
