@@ -472,8 +472,9 @@ def test_matvec_q8_0_mfma_variant_prologues(ctx, rows, n, k, prologue):
     (7, 8232, 1024, 0, 0, True, "norm"),
     (3, 96, 3072, 0, 0, False, None),          # k the kernel does not take: the default variant's
 ])
-def test_matvec_q6_k_mfma_variant(ctx, rows, n, k, col0, pad, accumulate, prologue):
-    """matvec_q6_k on the matrix-core variant id (a wave per sixteen rows): the weights are read
+@pytest.mark.parametrize("t", [TensorType.q6_k, TensorType.q3_k])
+def test_matvec_q6_k_mfma_variant(ctx, t, rows, n, k, col0, pad, accumulate, prologue):
+    """matvec_q6_k and matvec_q3_k on the matrix-core variant id (a wave per sixteen rows): the weights are read
     once for all tokens of the step, the tokens split beforehand (with the RMSNorm and
     silu(x / act_div) prologues of src/kernels/matvec_quant.wgsl.hbs:73-89 where the step has
     them). 1e-5 against float64; columns outside the launch untouched; each token bitwise equal
@@ -484,9 +485,9 @@ def test_matvec_q6_k_mfma_variant(ctx, rows, n, k, col0, pad, accumulate, prolog
     x = c.random(rows * k, 3).reshape(rows, k)
     x[0] *= np.float32(1e-4)
     nw = c.random(k, 1.5)
-    raw, values = quant_rows(c, TensorType.q6_k, n, k)
+    raw, values = quant_rows(c, t, n, k)
     init = c.random(rows * stride, 2).reshape(rows, stride)
-    xa, wa, na = c.upload(x), c.gpu_weights(TensorType.q6_k, raw, k), c.upload(nw)
+    xa, wa, na = c.upload(x), c.gpu_weights(t, raw, k), c.upload(nw)
     x64 = np.stack([norm_row(r, nw if prologue else None, eps) for r in x])
     if div:
         x64 = (x64 / div) * sigmoid64(x64 / div)
@@ -494,7 +495,7 @@ def test_matvec_q6_k_mfma_variant(ctx, rows, n, k, col0, pad, accumulate, prolog
     want = prod + (init[:, col0 : col0 + n] if accumulate else 0)
     p = lambda: P.MatvecBf16(n=n, k=k, col0=col0, out_stride=stride, eps=eps, norm=prologue is not None, accumulate=accumulate)
     variant = K.MatvecVariant(MFMA_VARIANT.wg, MFMA_VARIANT.lanes, MFMA_VARIANT.rows, div)
-    pipeline = c.set.matvec(c.rec, Kernel.matvec_q6_k, variant)
+    pipeline = c.set.matvec(c.rec, K.weight_kernel("matvec", t), variant)
     grid_x = K.div_ceil(n, variant.group_rows())
     out = c.upload(init)
     c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, na], (grid_x, rows, 1))

@@ -229,6 +229,8 @@ zhip_result launch_matvec_q5k_mfma_resident(const Dispatch &d, const MvArgs &a, 
 // matvec_q6_k on the matrix cores for k of 1024, 2048 or 4096 (matvec_q6k_mfma_stream.hip).
 bool matvec_q6k_mfma_stream_accepts(const MvArgs &a);
 zhip_result launch_matvec_q6k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
+bool matvec_q3k_mfma_stream_accepts(const MvArgs &a);
+zhip_result launch_matvec_q3k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
 // Matrices from this size on take it: below, its fixed costs (the split of the tokens, a
 // workgroup's first tile) outweigh the general kernel's per-token work at two to four tokens
 // (8 MB, k = 1024: 6.4 / 6.8 / 7.8 us at 2 / 4 / 8 tokens against 4.7 / 6.2 / 9.3).
@@ -324,7 +326,8 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
         return launch_matvec_bf16_mfma_stream(d, a, d.bind[2].size);
 
     // MatvecVariant (wg 512, lanes 64, rows 16) names the matrix-core variants: a wave per sixteen rows.
-    const bool matrix_cores = quant && v.lanes == 64u && v.rows == 16u && (D::CHUNK == 4 || D::CHUNK == 8 || D::CHUNK == 6 || D::CHUNK == 5);
+    const bool matrix_cores = quant && v.lanes == 64u && v.rows == 16u && (D::CHUNK == 4 || D::CHUNK == 8 || D::CHUNK == 6 || D::CHUNK == 5 || D::CHUNK == 3);
+    if (D::CHUNK == 3 && matrix_cores && matvec_q3k_mfma_stream_accepts(a)) return launch_matvec_q3k_mfma_stream(d, a, d.bind[2].size);
     // (matvec_q5_k: the Q4_K kernel for k of 2048 or 4096 with the fifth bits; other shapes run the default variant)
     if (D::CHUNK == 5 && matrix_cores && matvec_q5k_mfma_resident_accepts(a)) return launch_matvec_q5k_mfma_resident(d, a, d.bind[2].size);
     // (matvec_q6_k: a launch of its own splits the tokens, prologue included, for the multiply)

@@ -1,9 +1,12 @@
-// matvec_q6_k, matrix-core variant (MatvecVariant wg 512, lanes 64, rows 16) for steps of up to
+// matvec_q6_k and matvec_q3_k, matrix-core variant (MatvecVariant wg 512, lanes 64, rows 16) for steps of up to
 // eight tokens and k = 1024, 2048 or 4096: the weight stream is read once for all tokens of the step
 // and the per-weight work is done once. Contract as the default variant's
 // (src/kernels/matvec_quant.wgsl.hbs with the decoder of src/kernels/quant/q6_k_dot.wgsl; block
 // formula src/ref/tensor.zig:118-140): out[t][col0 + j] (+)= sum over 16-weight sub-blocks of
-// d * scale * sum((q - 32) * x), q the 6-bit value of ql and qh.
+// d * scale * sum((q - 32) * x), q the 6-bit value of ql and qh; Q3_K (the rows repacked at
+// load, src/kernels/repack_q3_k.wgsl; src/ref/tensor.zig:141-160): d * (scale - 32) * sum((q - 4) * x),
+// q the two low bits and the third bit. What follows describes Q6_K; Q3_K has 128-byte blocks
+// (a unit is four lines a row, all eight waves load it) and its own unpacking.
 //
 // Arithmetic. v_mfma_f32_32x32x16_f16 multiplies 32 rows of inputs by 32 weight rows over one
 // sub-block. The weights enter as the exact f16 integers q - 32 (the byte dropped into the
@@ -51,14 +54,30 @@ typedef uint32_t qu32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t qu32x4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t THREADS = 512, WAVES = 8;
-constexpr uint32_t ROW_UNIT = 4u * 224u;        // a unit's bytes of one row: seven lines
-constexpr uint32_t UNIT = 32u * ROW_UNIT;       // a unit in LDS
 constexpr int SLOTS = 4;                        // ring slots: three units in flight behind the one multiplied
-constexpr int LOADS = 4;                        // wave-wide loads of a unit a wave issues (28 of 1 KB: seven waves' worth; the eighth asks for nothing)
 constexpr uint32_t PART_BYTES = 2u * WAVES * 256u * 4u;  // [tile parity][wave][token of the lane's four][lane]
 constexpr uint32_t KEPT = 16;                   // tiles whose outputs wait in LDS for one burst of stores
-constexpr uint32_t LDS_BYTES = PART_BYTES + SLOTS * UNIT + KEPT * 1024u + 64u + 1024u;  // (the last KB: where the eighth wave's loads of nothing land)
-static_assert(LDS_BYTES <= 160u * 1024u - 64u, "the ring must fit the CU's LDS");
+
+// The formats. A unit is four 256-weight blocks of each of a tile's 32 rows: whole lines of every row.
+struct FmtQ6 {  // 224-byte padded blocks: ql[128], qh[64], sixteen signed scales, d
+    static constexpr uint32_t BLOCK = 224, ROW_LINES = 7;  // a row's part of a unit: seven lines
+    static constexpr int LOADS = 4;                        // wave-wide loads of a unit a wave issues
+    static constexpr uint32_t LOADERS = 7;                 // 28 KB: seven waves' worth; the eighth asks for nothing
+    static constexpr float OFFSET = -1056.0f;              // 1024 + byte -> q - 32
+    static const char *name() { return "matvec_q6_k"; }
+};
+struct FmtQ3 {  // blocks repacked at load into eight self-contained 16-byte units (src/kernels/repack_q3_k.wgsl)
+    static constexpr uint32_t BLOCK = 128, ROW_LINES = 4;
+    static constexpr int LOADS = 2;
+    static constexpr uint32_t LOADERS = 8;
+    static constexpr float OFFSET = -1028.0f;              // 1024 + byte -> q - 4
+    static const char *name() { return "matvec_q3_k"; }
+};
+template <class F> constexpr uint32_t row_unit() { return 4u * F::BLOCK; }        // a unit's bytes of one row
+template <class F> constexpr uint32_t unit_bytes() { return 32u * row_unit<F>(); }  // a unit in LDS
+// (the last KB: where the loads of nothing land)
+template <class F> constexpr uint32_t lds_bytes() { return PART_BYTES + SLOTS * unit_bytes<F>() + KEPT * 1024u + 64u + 1024u; }
+static_assert(lds_bytes<FmtQ6>() <= 160u * 1024u - 64u, "the ring must fit the CU's LDS");
 
 struct Q6Args {
     MvArgs a;
@@ -97,9 +116,10 @@ __device__ __forceinline__ void load_lds_b128(__amdgpu_buffer_rsrc_t buf, uint32
     __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)(uintptr_t)dst, 16, voffset, 0, 0, 0);
 }
 
-// Eight 6-bit values, a byte each in two words, as the exact f16 values q - 32 in position order.
+// Eight quants, a byte each in two words, as the exact f16 values q - 32 (Q6_K) or q - 4 (Q3_K) in position order.
+template <class F>
 __device__ __forceinline__ qf16x8 weights_f16(qu32x2 q, uint32_t bias) {
-    const qf16x2 off = {(_Float16)-1056.0f, (_Float16)-1056.0f};
+    const qf16x2 off = {(_Float16)F::OFFSET, (_Float16)F::OFFSET};
     qu32x4 r;
 #pragma unroll
     for (int i = 0; i < 2; i++) {
@@ -154,8 +174,10 @@ __global__ __launch_bounds__(256) void matvec_q6k_split_kernel(MvArgs a, uint2 *
 }
 
 // NU: units of a tile (k = 1024 NU).
-template <int NU>
-__global__ __launch_bounds__(THREADS) void matvec_q6k_mfma_stream_kernel(Q6Args q) {
+template <class F, int NU>
+__global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Args q) {
+    constexpr uint32_t ROW_UNIT = row_unit<F>(), UNIT = unit_bytes<F>();
+    constexpr int LOADS = F::LOADS;
     const MvArgs &a = q.a;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     float *lds_part = reinterpret_cast<float *>(lds);
@@ -186,7 +208,7 @@ __global__ __launch_bounds__(THREADS) void matvec_q6k_mfma_stream_kernel(Q6Args 
     uint32_t woff[LOADS];
 #pragma unroll
     for (int j = 0; j < LOADS; j++) {
-        const uint32_t line = 8u * (LOADS * wave + j) + (lane >> 3), row = line / 7u, in_row = line % 7u;
+        const uint32_t line = 8u * (LOADS * wave + j) + (lane >> 3), row = line / F::ROW_LINES, in_row = line % F::ROW_LINES;
         woff[j] = row * a.row_bytes + 128u * in_row + 16u * ((lane & 7u) ^ (row & 7u));
     }
     // Unit v of the run: unit v % NU of tile v / NU. Past the run's end the loads still run, so
@@ -194,16 +216,16 @@ __global__ __launch_bounds__(THREADS) void matvec_q6k_mfma_stream_kernel(Q6Args 
     // and nothing is fetched.
     auto issue = [&](uint32_t v, uint32_t slot) __attribute__((always_inline)) {
         const uint32_t p = v / NU, u = v % NU;
-        const bool real = p < count && wave < 7u;
+        const bool real = p < count && wave < F::LOADERS;
         const uint32_t base = (real ? first_row(p) : 0u) * a.row_bytes + ROW_UNIT * u, rows = rows_of(p);
         // (a load against the empty buffer still lands zeros: the eighth wave's in a spare KB)
-        const uint32_t dst = wave < 7u ? ring0 + slot * UNIT + 1024u * (LOADS * wave) : ring0 + SLOTS * UNIT + KEPT * 1024u + 64u;
+        const uint32_t dst = wave < F::LOADERS ? ring0 + slot * UNIT + 1024u * (LOADS * wave) : ring0 + SLOTS * UNIT + KEPT * 1024u + 64u;
 #pragma unroll
         for (int j = 0; j < LOADS; j++) {
             // (lines of rows the workgroup's share of the last rows does not have are not fetched;
             // what the matrix instructions make of the zeros there is never stored)
-            const uint32_t first_line_row = (8u * (LOADS * wave + j)) / 7u;
-            load_lds_b128(real && first_line_row < rows ? wbuf : nobuf, wave < 7u ? dst + 1024u * j : dst, woff[j] + base);
+            const uint32_t first_line_row = (8u * (LOADS * wave + j)) / F::ROW_LINES;
+            load_lds_b128(real && first_line_row < rows ? wbuf : nobuf, wave < F::LOADERS ? dst + 1024u * j : dst, woff[j] + base);
         }
     };
 
@@ -236,47 +258,81 @@ __global__ __launch_bounds__(THREADS) void matvec_q6k_mfma_stream_kernel(Q6Args 
     // bytes at 224 (wave / 2). Byte o of a row's unit sits at 896 rho + 128 (o / 128) +
     // 16 ((o / 16 % 8) ^ (rho % 8)) + o % 16.
     auto at_byte = [&](uint32_t o) { return ROW_UNIT * rho + (o & ~127u) + 16u * (((o >> 4) & 7u) ^ (rho & 7u)) + (o & 15u); };
-    uint32_t at_ql[4], at_qh[2];  // ql: [which 32 of the half's 64][which 16]; qh: [which 16]
+    constexpr bool Q3 = F::BLOCK == 128u;
+    uint32_t at_ql[4], at_qh[2];  // Q6_K ql: [which 32 of the half's 64][which 16]; qh: [which 16]; Q3_K: at_ql = the half's four units
+    uint32_t at_sc = 0, at_d = 0;
+    if constexpr (Q3) {
 #pragma unroll
-    for (uint32_t i = 0; i < 4; i++) at_ql[i] = at_byte(224u * blk + 64u * half + 32u * (i >> 1) + 16u * (i & 1u) + 8u * kap);
+        for (uint32_t i = 0; i < 4; i++) at_ql[i] = at_byte(128u * blk + 64u * half + 16u * i);
+        at_qh[0] = at_qh[1] = 0;
+    } else {
 #pragma unroll
-    for (uint32_t i = 0; i < 2; i++) at_qh[i] = at_byte(224u * blk + 128u + 32u * half + 16u * i + 8u * kap);
-    const uint32_t at_sc = at_byte(224u * blk + 192u + 8u * half), at_d = at_byte(224u * blk + 208u);
+        for (uint32_t i = 0; i < 4; i++) at_ql[i] = at_byte(224u * blk + 64u * half + 32u * (i >> 1) + 16u * (i & 1u) + 8u * kap);
+#pragma unroll
+        for (uint32_t i = 0; i < 2; i++) at_qh[i] = at_byte(224u * blk + 128u + 32u * half + 16u * i + 8u * kap);
+        at_sc = at_byte(224u * blk + 192u + 8u * half);
+        at_d = at_byte(224u * blk + 208u);
+    }
 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};  // tokens 4 (lane / 32) + i, matrix row rho of the tile, this wave's blocks
+    // One sub-block: its eight quants of the lane (a byte each), d * scale, and the operand index.
+    auto sub_block = [&](qu32x2 v, float dsc, int s) __attribute__((always_inline)) {
+        qf32x16 zero;
+#pragma unroll
+        for (int e = 0; e < 16; e++) zero[e] = 0.f;
+        const qf32x16 r = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[s], weights_f16<F>(v, bias), zero, 0, 0, 0);
+#pragma unroll
+        for (int i = 0; i < 4; i++) acc[i] = fmaf(dsc, fmaf(r[4 + i], 1.0f / 2048.0f, r[i]), acc[i]);
+        // (a sub-block's results are used up before the next sub-block's matrix
+        // instruction: eight of them in flight would not fit the registers)
+        asm volatile("" : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]));
+    };
     auto multiply = [&](auto unit, uint32_t slot) __attribute__((always_inline)) {
         constexpr int U = decltype(unit)::value;
         const uint8_t *t = ring + slot * UNIT;
-        const qu32x2 sc = *reinterpret_cast<const qu32x2 *>(t + at_sc);
-        const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(t + at_d));
+        if constexpr (Q3) {
+            // Unit i of the half: 32 weights as two words of 2-bit values (byte b, bit pair e:
+            // position 4 e + b; the second word 16 further), a word of third bits (byte b, bit e:
+            // position 4 e + b), scale - 32 of each sixteen as signed bytes, d. The lane's eight
+            // positions of a sixteen are 8 kap ..: bit pairs 2 kap and 2 kap + 1 of the four bytes.
 #pragma unroll
-        for (uint32_t h16 = 0; h16 < 2; h16++) {
-            const qu32x2 qh = *reinterpret_cast<const qu32x2 *>(t + at_qh[h16]);
+            for (uint32_t i = 0; i < 4; i++) {
+                const qu32x4 u = *reinterpret_cast<const qu32x4 *>(t + at_ql[i]);
+                const float d = half_bits_to_float(u.w >> 16);
 #pragma unroll
-            for (uint32_t qp = 0; qp < 2; qp++) {
-                const qu32x2 ql = *reinterpret_cast<const qu32x2 *>(t + at_ql[2u * qp + h16]);
-#pragma unroll
-                for (uint32_t up = 0; up < 2; up++) {
-                    // Quadrant qd of the half: weights 32 qd + 16 h16 + 8 kap ... of its 128, sub-block 2 qd + h16 of its eight.
-                    const uint32_t qd = qp + 2u * up, s = 2u * qd + h16;
+                for (uint32_t h16 = 0; h16 < 2; h16++) {
+                    const uint32_t word = h16 ? u.y : u.x, third = u.z >> (4u * h16 + 2u * kap);
                     qu32x2 v;
+                    v[0] = ((word >> (4u * kap)) & 0x03030303u) | ((third & 0x01010101u) << 2);
+                    v[1] = ((word >> (4u * kap + 2u)) & 0x03030303u) | (((third >> 1) & 0x01010101u) << 2);
+                    const float dsc = d * (float)(int8_t)((u.w >> (8u * h16)) & 0xffu);
+                    sub_block(v, dsc, 8 * U + 2 * (int)i + (int)h16);
+                }
+            }
+        } else {
+            const qu32x2 sc = *reinterpret_cast<const qu32x2 *>(t + at_sc);
+            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(t + at_d));
 #pragma unroll
-                    for (int w = 0; w < 2; w++) {
-                        const uint32_t nib = up ? (ql[w] >> 4) & 0x0f0f0f0fu : ql[w] & 0x0f0f0f0fu;
-                        const uint32_t two = (qd ? qh[w] >> (2u * qd) : qh[w]) & 0x03030303u;
-                        v[w] = nib | (two << 4);
+            for (uint32_t h16 = 0; h16 < 2; h16++) {
+                const qu32x2 qh = *reinterpret_cast<const qu32x2 *>(t + at_qh[h16]);
+#pragma unroll
+                for (uint32_t qp = 0; qp < 2; qp++) {
+                    const qu32x2 ql = *reinterpret_cast<const qu32x2 *>(t + at_ql[2u * qp + h16]);
+#pragma unroll
+                    for (uint32_t up = 0; up < 2; up++) {
+                        // Quadrant qd of the half: weights 32 qd + 16 h16 + 8 kap ... of its 128, sub-block 2 qd + h16 of its eight.
+                        const uint32_t qd = qp + 2u * up, s = 2u * qd + h16;
+                        qu32x2 v;
+#pragma unroll
+                        for (int w = 0; w < 2; w++) {
+                            const uint32_t nib = up ? (ql[w] >> 4) & 0x0f0f0f0fu : ql[w] & 0x0f0f0f0fu;
+                            const uint32_t two = (qd ? qh[w] >> (2u * qd) : qh[w]) & 0x03030303u;
+                            v[w] = nib | (two << 4);
+                        }
+                        const uint32_t word = s < 4u ? sc.x : sc.y;
+                        const float dsc = d * (float)(int8_t)((word >> (8u * (s & 3u))) & 0xffu);
+                        sub_block(v, dsc, 8 * U + (int)s);
                     }
-                    const uint32_t word = s < 4u ? sc.x : sc.y;
-                    const float dsc = d * (float)(int8_t)((word >> (8u * (s & 3u))) & 0xffu);
-                    qf32x16 zero;
-#pragma unroll
-                    for (int e = 0; e < 16; e++) zero[e] = 0.f;
-                    const qf32x16 r = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[8 * U + s], weights_f16(v, bias), zero, 0, 0, 0);
-#pragma unroll
-                    for (int i = 0; i < 4; i++) acc[i] = fmaf(dsc, fmaf(r[4 + i], 1.0f / 2048.0f, r[i]), acc[i]);
-                    // (a sub-block's results are used up before the next sub-block's matrix
-                    // instruction: eight of them in flight would not fit the registers)
-                    asm volatile("" : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]));
                 }
             }
         }
@@ -350,39 +406,33 @@ __global__ __launch_bounds__(THREADS) void matvec_q6k_mfma_stream_kernel(Q6Args 
     }
 }
 
-template <int NU>
+template <class F, int NU>
 zhip_result launch_blocks(const Dispatch &d, const Q6Args &q, dim3 grid) {
-    auto kernel = matvec_q6k_mfma_stream_kernel<NU>;
+    auto kernel = matvec_kquant_mfma_stream_kernel<F, NU>;
+    constexpr uint32_t bytes = lds_bytes<F>();
     static bool configured = false;
     if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
             (void)hipGetLastError();
-            return fail(d, ZHIP_E_GPU, "matvec_q6_k: cannot reserve %u bytes of LDS", LDS_BYTES);
+            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", F::name(), bytes);
         }
         configured = true;
     }
-    hipLaunchKernelGGL(kernel, grid, dim3(THREADS), LDS_BYTES, d.stream, q);
-    return check_launch(d, "matvec_q6_k");
+    hipLaunchKernelGGL(kernel, grid, dim3(THREADS), bytes, d.stream, q);
+    return check_launch(d, F::name());
 }
 
-}  // namespace
-
-// Whether this kernel can run the (already validated) arguments: k of whole units, no pair.
-bool matvec_q6k_mfma_stream_accepts(const MvArgs &a) {
-    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && !(a.flags & FLAG_SILU_PAIR) && a.rows >= 1 && a.xr % 4u == 0 &&
-           (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == a.k / 256u * 224u;
-}
-
-zhip_result launch_matvec_q6k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) {
+template <class F>
+zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) {
     // 32-bit byte offsets, a tile past the last row.
     const uint64_t used = (uint64_t)a.rows * a.row_bytes;
-    if (used + 64ull * a.row_bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "matvec_q6_k: weights of 4 GiB or more");
-    if (!d.work) return fail(d, ZHIP_E_GPU, "matvec_q6_k: no workspace");
+    if (used + 64ull * a.row_bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "%s: weights of 4 GiB or more", F::name());
+    if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", F::name());
     const uint64_t plane_bytes = 4ull * a.m * a.k;
     if (zhip_result r = d.work->reserve(d, plane_bytes + 64u)) return r;
     float *inverse = reinterpret_cast<float *>(d.work->data + plane_bytes);
     hipLaunchKernelGGL(matvec_q6k_split_kernel, dim3(a.m), dim3(256), 0, d.stream, a, reinterpret_cast<uint2 *>(d.work->data), inverse);
-    if (zhip_result r = check_launch(d, "matvec_q6_k")) return r;
+    if (zhip_result r = check_launch(d, F::name())) return r;
 
     const uint32_t cus = (uint32_t)d.dev->compute_units;
     const uint32_t units = (a.rows + 7u) / 8u;
@@ -394,7 +444,20 @@ zhip_result launch_matvec_q6k_mfma_stream(const Dispatch &d, const MvArgs &a, ui
     q.a.norm_w = nullptr;
     q.a.act_div = 0.f;
     const dim3 grid(groups);
-    return a.k == 1024u ? launch_blocks<1>(d, q, grid) : a.k == 2048u ? launch_blocks<2>(d, q, grid) : launch_blocks<4>(d, q, grid);
+    return a.k == 1024u ? launch_blocks<F, 1>(d, q, grid) : a.k == 2048u ? launch_blocks<F, 2>(d, q, grid) : launch_blocks<F, 4>(d, q, grid);
 }
+
+bool stream_accepts(const MvArgs &a, uint32_t block_bytes) {
+    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && !(a.flags & FLAG_SILU_PAIR) && a.rows >= 1 && a.xr % 4u == 0 &&
+           (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == a.k / 256u * block_bytes;
+}
+
+}  // namespace
+
+// Whether these kernels can run the (already validated) arguments: k of whole units, no pair.
+bool matvec_q6k_mfma_stream_accepts(const MvArgs &a) { return stream_accepts(a, FmtQ6::BLOCK); }
+zhip_result launch_matvec_q6k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) { return launch_stream<FmtQ6>(d, a, w_bytes); }
+bool matvec_q3k_mfma_stream_accepts(const MvArgs &a) { return stream_accepts(a, FmtQ3::BLOCK); }
+zhip_result launch_matvec_q3k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) { return launch_stream<FmtQ3>(d, a, w_bytes); }
 
 }  // namespace zhip
