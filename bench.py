@@ -516,6 +516,23 @@ def bench_formats(env):
         nbytes = n * (k // e) * bb + m * 4 * k + m * 4 * n
         res[tag] = env["hbm_entry"](f"q8_0 decode matvec M={m} K={k} N={n}" + (", matrix-core variant" if variant else ""), nbytes, wall, gpu_s, steps,
                                     {"copies": len(launches), "max_err_over_max_want": rel})
+    # The K formats at eight tokens: default variant and matrix-core variant.
+    for name, ot in (("q6_k", oracle.Q6_K), ("q5_k", oracle.Q5_K), ("q3_k", oracle.Q3_K)):
+        t = TensorType[name]
+        raw = synth.random_blocks(synth.rng(0xF1), name, n, k)
+        w = oracle.dequantize(ot, raw, n * k).reshape(n, k)
+        e, bb = K.LAYOUT[t]
+        m = 8
+        xm = synth.activations(synth.rng(0xF8 + m), m, k)
+        want = xm.astype(np.float64) @ w.astype(np.float64).T
+        for variant, tag in ((None, f"{name}_m8"), (mc, f"{name}_m8_matrix_cores")):
+            launches, out = env["matvec_workload"](t, raw, n, k, m, False, xm, variant)
+            wall, gpu_s, steps = env["protocol"](launches)
+            got = env["read"](out)[: m * n].reshape(m, n).astype(np.float64)
+            rel = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+            nbytes = n * (k // e) * bb + m * 4 * k + m * 4 * n
+            res[tag] = env["hbm_entry"](f"{name} decode matvec M={m} K={k} N={n}" + (", matrix-core variant" if variant else ""), nbytes, wall, gpu_s, steps,
+                                        {"copies": len(launches), "max_err_over_max_want": rel})
     return res
 
 
