@@ -338,7 +338,7 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     // round of loads, which the norm weights join (C3 at four tokens with the FFN launch's
     // RMSNorm: 22.6 us, 26.1 us with a pass of its own in front, 20.7 us without a prologue).
     const bool resident = D::CHUNK == 4 && matrix_cores && matvec_q4k_mfma_resident_accepts(a);
-    const bool q8_stream = D::CHUNK == 8 && matrix_cores && !pair && matvec_q8_mfma_stream_accepts(a);
+    const bool q8_stream = D::CHUNK == 8 && matrix_cores && matvec_q8_mfma_stream_accepts(a);
     // The Q4_K kernel for the other multiples of 1024 takes its inputs as they are: a step with
     // a prologue first writes the transformed tokens to the workspace, one workgroup a token
     // with the staging arithmetic of the default variant, and the multiply reads those.
@@ -361,8 +361,8 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     if (resident) return launch_matvec_q4k_mfma_resident(d, a, d.bind[2].size);
     if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && plain && matvec_q4k_mfma_accepts(a))
         return launch_matvec_q4k_mfma(d, a, x_bound, d.bind[2].size);
-    // The same id on matvec_q8_0, without pair (a one-token step too, so that a token's bits do
-    // not depend on the step it ran in); other shapes without a prologue: the prefill tiling.
+    // The same id on matvec_q8_0 (a one-token step too, so that a token's bits do not depend on
+    // the step it ran in); other shapes without a prologue or pair: the prefill tiling.
     if (q8_stream) return launch_matvec_q8_mfma_stream(d, a, d.bind[2].size);
     if (D::CHUNK == 8 && v.lanes == 64u && v.rows == 16u && plain && !pair && a.m <= 32u)
         return launch_matvec_q8_0_mfma(d, a);

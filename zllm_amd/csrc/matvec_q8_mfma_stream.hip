@@ -146,11 +146,16 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
     // tiles left over after whole rounds are at most half as many as the workgroups, two
     // workgroups share each: a whole tile more on half of the CUs would be the launch's tail).
     // Half tile u is half u % 2 of tile u / 2.
+    // With SILU_PAIR (src/kernels/matvec_quant.wgsl.hbs:110-125) an output tile is two weight
+    // tiles, the gate rows and then the up rows `half` further down: tile p of the run is weight
+    // tile p % per of output tile p / per.
+    const uint32_t per = (a.flags & FLAG_SILU_PAIR) ? 2u : 1u;
     const bool extra = blockIdx.x < (q.split ? 2u * q.left : q.left);
-    const uint32_t count = q.rounds + (extra ? 1u : 0u);
+    const uint32_t count = per * (q.rounds + (extra ? 1u : 0u));
     const uint32_t last_row = 16u * (q.rounds * gridDim.x + (q.split ? blockIdx.x >> 1 : blockIdx.x)) + (q.split ? 8u * (blockIdx.x & 1u) : 0u);
-    auto first_row = [&](uint32_t p) { return p < q.rounds ? 16u * (blockIdx.x + p * gridDim.x) : last_row; };
-    auto rows_of = [&](uint32_t p) { return (q.split && p >= q.rounds) ? 8u : 16u; };
+    auto out0 = [&](uint32_t p) { return p / per < q.rounds ? 16u * (blockIdx.x + (p / per) * gridDim.x) : last_row; };  // first output of tile p
+    auto first_row = [&](uint32_t p) { return out0(p) + ((p % per) ? a.half : 0u); };
+    auto rows_of = [&](uint32_t p) { return (q.split && p / per >= q.rounds) ? 8u : 16u; };
     // A half tile's loads. Weights: load i brings rows (64 / CHUNKS) i .. of the half's k range,
     // lane l row l / CHUNKS and the chunk that belongs at position l % CHUNKS: chunk c of row r
     // sits at position c ^ key(r), the key such that sixteen rows' reads of one chunk fall in
@@ -311,6 +316,7 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
             acc[1] = fmaf(ds, fmaf(r[3], 1.0f / 2048.0f, r[2]), acc[1]);
         }
     };
+    float held = 0.f;
     auto finish = [&](uint32_t p) __attribute__((always_inline)) {
         float *part = lds_part + (p & 1u) * (WAVES * 128u);
         *reinterpret_cast<float2 *>(part + wave * 128u + 2u * lane) = float2{acc[0], acc[1]};
@@ -319,16 +325,21 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
         // Buffer p % 2 is written again in step p + 2, after the barrier of step p + 1, which a
         // wave passes only when it has read what it needs here. The 128 outputs of a tile are
         // summed by one pair of waves, a different pair from one tile to the next.
-        if ((tid >> 7) == (p & 3u)) {
+        if ((tid >> 7) == ((p / per) & 3u)) {
             const uint32_t row = tid & 15u, tk = (tid >> 4) & 7u;
             const float *src = part + 2u * ((tk >> 1) * 16u + row) + (tk & 1u);
             float sum = src[0];
 #pragma unroll
             for (uint32_t wv = 1; wv < WAVES; wv++) sum += src[wv * 128u];
             sum *= lds_inverse[tk];
-            if (tk < a.m && row < rows_of(p)) {
-                float *o = a.out + (size_t)tk * a.out_stride + a.col0 + first_row(p) + row;
-                store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + sum : sum);
+            if (per == 2u && !(p & 1u)) {
+                held = sum;  // the gate tile's result, until the up tile's arrives
+            } else {
+                const float v = per == 2u ? silu_f(held) * sum : sum;
+                if (tk < a.m && row < rows_of(p)) {
+                    float *o = a.out + (size_t)tk * a.out_stride + a.col0 + out0(p) + row;
+                    store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + v : v);
+                }
             }
         }
     };
@@ -367,9 +378,9 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
 }  // namespace
 
 // Whether this kernel can run the (already validated) arguments: whole tiles, k split into 4, 8
-// or 16 blocks a wave, no pair.
+// or 16 blocks a wave.
 bool matvec_q8_mfma_stream_accepts(const MvArgs &a) {
-    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && !(a.flags & FLAG_SILU_PAIR) && a.rows % 16u == 0 &&
+    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && (!(a.flags & FLAG_SILU_PAIR) || a.half % 16u == 0) && a.rows % 16u == 0 &&
            a.xr % 4u == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0;
 }
 
@@ -390,7 +401,8 @@ static zhip_result launch_blocks(const Dispatch &d, const StreamArgs &q, dim3 gr
 
 zhip_result launch_matvec_q8_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) {
     // 32-bit byte offsets, a tile past the last row.
-    if (w_bytes >= 0xfffffff0ull || ((uint64_t)a.rows + 16u) * a.row_bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "matvec_q8_0: operands of 4 GiB or more");
+    const uint64_t reach = ((uint64_t)((a.flags & FLAG_SILU_PAIR) ? a.half : 0u) + a.rows + 16u) * a.row_bytes;
+    if (w_bytes >= 0xfffffff0ull || reach >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "matvec_q8_0: operands of 4 GiB or more");
     const uint32_t cus = (uint32_t)d.dev->compute_units, tiles = a.rows / 16u;
     const uint32_t groups = tiles < cus ? (2u * tiles <= cus ? 2u * tiles : tiles) : cus;
     const uint32_t left = tiles % groups;
