@@ -85,16 +85,16 @@ def test_matvec_bf16_norm_accumulate(ctx, half):
     assert matvec_case(ctx, 1000, 37, True, half) <= 1e-5
 
 
-def bf16_tokens_case(c, m, n, k, col0=0, pad=0, accumulate=False, norm=False, x=None):
+def bf16_tokens_case(c, m, n, k, col0=0, pad=0, accumulate=False, norm=False, x=None, half="bf16"):
     """A matvec_bf16 step of m tokens over n x k weights, writing columns col0 .. col0 + n of
     rows n + col0 + pad wide; returns (got, want in float64, the launch's inputs)."""
     eps, stride = 1e-6, col0 + n + pad
     x = c.random(m * k, 3).reshape(m, k) if x is None else x
     nw = c.random(k, 1)
-    bits, values = random_half(c, n * k, 1)
+    bits, values = random_half(c, n * k, 1, half)
     init = c.random(m * stride, 4).reshape(m, stride)
     out = c.upload(init)
-    c.launcher().launch(Kernel.matvec_bf16, P.MatvecBf16(n=n, k=k, col0=col0, out_stride=stride, eps=eps, norm=norm, accumulate=accumulate),
+    c.launcher().launch(Kernel["matvec_" + half], P.MatvecBf16(n=n, k=k, col0=col0, out_stride=stride, eps=eps, norm=norm, accumulate=accumulate),
                         [c.upload(x), c.upload(bits), out, c.upload(nw)], (K.div_ceil(n, K.matvec_rows), m, 1))
     got = c.read(out).reshape(m, stride)
     want = init.astype(np.float64).copy()
@@ -120,8 +120,9 @@ def bf16_tokens_case(c, m, n, k, col0=0, pad=0, accumulate=False, norm=False, x=
     (19, 2052, 4096, 8, 0, True, False),
     (3, 100, 1024, 0, 0, False, False),        # a small matrix: the general kernel
 ])
-def test_matvec_bf16_several_tokens(ctx, m, n, k, col0, pad, accumulate, norm):
-    got, want, _ = bf16_tokens_case(ctx, m, n, k, col0, pad, accumulate, norm)
+@pytest.mark.parametrize("half", HALVES)
+def test_matvec_bf16_several_tokens(ctx, half, m, n, k, col0, pad, accumulate, norm):
+    got, want, _ = bf16_tokens_case(ctx, m, n, k, col0, pad, accumulate, norm, half=half)
     assert rel_err(got, want) <= 1e-5
     # Columns outside the launch's keep their contents bit for bit.
     keep = np.ones(got.shape[1], dtype=bool)
@@ -144,19 +145,20 @@ def test_matvec_bf16_several_tokens_many_rows(ctx):
     assert rel_err(got, want) <= 1e-5
 
 
-def test_matvec_bf16_several_tokens_keep_token_bits(ctx):
+@pytest.mark.parametrize("half", HALVES)
+def test_matvec_bf16_several_tokens_keep_token_bits(ctx, half):
     """A token's outputs do not depend on how many tokens share the step (from two tokens
     up), nor on where the step's columns start."""
     c = ctx
     m, n, k = 13, 4500, 2048
     x = c.random(m * k, 3).reshape(m, k)
-    bits, _ = random_half(c, n * k, 1)
+    bits, _ = random_half(c, n * k, 1, half)
     wa = c.upload(bits)
 
     def run(tokens, rows0, rows):
         out = c.output(len(tokens) * rows)
         wpart = c.upload(bits.reshape(n, k)[rows0 : rows0 + rows])
-        c.launcher().launch(Kernel.matvec_bf16, P.MatvecBf16(n=rows, k=k, col0=0, out_stride=rows, eps=1e-6),
+        c.launcher().launch(Kernel["matvec_" + half], P.MatvecBf16(n=rows, k=k, col0=0, out_stride=rows, eps=1e-6),
                             [c.upload(x[tokens]), wpart, out, c.upload(np.ones(k, dtype=np.float32))], (K.div_ceil(rows, K.matvec_rows), len(tokens), 1))
         return c.read(out).reshape(len(tokens), rows)
 

@@ -223,7 +223,7 @@ bool matvec_q8_mfma_stream_accepts(const MvArgs &a);
 zhip_result launch_matvec_q8_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
 // matvec_bf16 on the matrix cores, the weights read once for all tokens (matvec_bf16_mfma_stream.hip).
 bool matvec_bf16_mfma_stream_accepts(const MvArgs &a);
-zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
+zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes, bool f16);
 bool matvec_q5k_mfma_resident_accepts(const MvArgs &a);
 zhip_result launch_matvec_q5k_mfma_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
 // matvec_q6_k on the matrix cores for k of 1024, 2048 or 4096 (matvec_q6k_mfma_stream.hip).
@@ -319,11 +319,11 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     a.out = reinterpret_cast<float *>(d.bind[3].ptr);
     a.norm_w = norm ? reinterpret_cast<const float *>(d.bind[4].ptr) : nullptr;
 
-    // matvec_bf16 steps of several tokens over a matrix of some size go to the kernel that reads
+    // matvec_bf16 / matvec_f16 steps of several tokens over a matrix of some size go to the kernel that reads
     // the weights once for all of them (by the matrix, not by the step's width: a token's bits
     // are then the same at every width from two tokens up).
-    if (std::is_same<D, DecBF16>::value && a.m >= 2u && (uint64_t)a.rows * a.row_bytes >= kBf16StreamBytes && matvec_bf16_mfma_stream_accepts(a))
-        return launch_matvec_bf16_mfma_stream(d, a, d.bind[2].size);
+    if ((std::is_same<D, DecBF16>::value || std::is_same<D, DecF16>::value) && a.m >= 2u && (uint64_t)a.rows * a.row_bytes >= kBf16StreamBytes && matvec_bf16_mfma_stream_accepts(a))
+        return launch_matvec_bf16_mfma_stream(d, a, d.bind[2].size, std::is_same<D, DecF16>::value);
 
     // MatvecVariant (wg 512, lanes 64, rows 16) names the matrix-core variants: a wave per sixteen rows.
     const bool matrix_cores = quant && v.lanes == 64u && v.rows == 16u && (D::CHUNK == 4 || D::CHUNK == 8 || D::CHUNK == 6 || D::CHUNK == 5 || D::CHUNK == 3);

@@ -1,4 +1,4 @@
-// matvec_bf16 on the matrix cores for steps of several tokens and k = 1024 ... 4096 in steps of
+// matvec_bf16 (and matvec_f16) on the matrix cores for steps of several tokens and k = 1024 ... 4096 in steps of
 // 512: the weight stream is read once for all tokens of the step and nothing but partial sums
 // crosses LDS. Contract of src/kernels/matvec_half.wgsl:1-133 with the bf16 decoder of
 // src/kernels/half/bf16.wgsl:3-9: out[t][col0 + j] (+)= sum_i x[t][i] * w[j][i], the inputs
@@ -43,6 +43,8 @@ namespace zhip {
 namespace {
 
 typedef __bf16 hbf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 hf16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 hf16x4 __attribute__((ext_vector_type(4)));
 typedef float hf32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t hu32x4 __attribute__((ext_vector_type(4)));
 
@@ -53,7 +55,7 @@ constexpr uint32_t SLOT = 32u * 128u;
 constexpr uint32_t PART_BYTES = 2u * WAVES * 256u * 4u;  // [tile parity][wave][token of the lane's four][lane]
 constexpr uint32_t KEPT = 40;                            // tiles whose outputs wait in LDS for one burst of stores
 constexpr uint32_t RING_BYTES = WAVES * DEPTH * SLOT;
-constexpr uint32_t LDS_BYTES = PART_BYTES + RING_BYTES + KEPT * 1024u;
+constexpr uint32_t LDS_BYTES = PART_BYTES + RING_BYTES + KEPT * 1024u + 64u;  // (the last 64: f16 tokens' inverse scales)
 static_assert(LDS_BYTES <= 160u * 1024u - 64u, "the rings must fit the CU's LDS");
 
 struct StreamArgs {
@@ -67,6 +69,7 @@ struct StreamArgs {
     const uint8_t *planes;
     uint32_t plane_tokens;  // tokens a plane holds
     uint32_t t0;            // the launch's first token in the planes
+    const float *inverse;   // F16 kernels: one over each token's scale
 };
 
 // A barrier that waits for this wave's LDS traffic only: the weight loads of the pieces ahead
@@ -123,12 +126,21 @@ __device__ __forceinline__ uint32_t upper_halves(uint32_t lo, uint32_t hi) { ret
 // operations a value on it, four lanes on the same value (the lanes of the three pieces and of
 // the zero rows): 1.5 us of a launch at k = 1024, less than another launch costs, but 12 us at
 // k = 4096.
-template <int NP, bool SPLIT>
+// F16 (matvec_f16: the weights are f16 and the matrix instruction v_mfma_f32_32x32x16_f16): a
+// token enters as two f16 rows, the rounding of its inputs and the rounding of what that left
+// times 2^11, after a power of two has put its largest magnitude at 2^14 (an input keeps 22
+// bits); the planes come from matvec_f16_split_kernel, and a token's sums are multiplied by one
+// over its scale.
+template <int NP, bool SPLIT, bool F16>
 __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(StreamArgs q) {
+    static_assert(SPLIT || !F16, "f16 tokens are always split beforehand");
+    constexpr uint32_t PIECES = F16 ? 2u : 3u;
     const MvArgs &a = q.a;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     float *lds_part = reinterpret_cast<float *>(lds);
     float *lds_kept = reinterpret_cast<float *>(lds + PART_BYTES + RING_BYTES);  // [tile % KEPT][token][row]
+    float *lds_inverse = lds_kept + KEPT * 256u;                                 // [token], read behind the tiles' barriers
+    if (F16 && threadIdx.x < 8u) lds_inverse[threadIdx.x] = threadIdx.x < a.m ? q.inverse[q.t0 + threadIdx.x] : 1.0f;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     uint8_t *ring = lds + PART_BYTES + wave * (DEPTH * SLOT);
@@ -178,19 +190,19 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
     // lane's loads go out together.
     const uint32_t rho = lane & 31u, kap = lane >> 5;
     const uint32_t tok = 4u * ((rho >> 2) & 1u) + (rho & 3u), piece = rho >> 3;
-    const bool live = tok < a.m && piece < 3u;
+    const bool live = tok < a.m && piece < PIECES;
     // (masks, so that picking the lane's piece is two instructions a value and not a branch)
     uint32_t m0 = live && piece == 0u ? ~0u : 0u, m1 = live && piece == 1u ? ~0u : 0u, m2 = live && piece == 2u ? ~0u : 0u;
     asm volatile("" : "+v"(m0), "+v"(m1), "+v"(m2));
     const float *xt = a.x + (size_t)(tok < a.m ? tok : a.m - 1u) * a.xr + 64u * NP * wave + 8u * kap;
-    hbf16x8 xf[4 * NP];
+    hu32x4 xf[4 * NP];
     if constexpr (SPLIT) {
         // Every step's operand is sixteen bytes of a plane; the lanes of absent tokens and of
         // the zero rows ask past the buffer's end and get zeros.
-        const __amdgpu_buffer_rsrc_t pbuf = make_buffer(q.planes, 3u * q.plane_tokens * a.k * 2u);
+        const __amdgpu_buffer_rsrc_t pbuf = make_buffer(q.planes, PIECES * q.plane_tokens * a.k * 2u);
         const uint32_t at = live ? ((piece * q.plane_tokens + q.t0 + tok) * a.k + 64u * NP * wave + 8u * kap) * 2u : 0xfffffff0u;
 #pragma unroll
-        for (int s = 0; s < 4 * NP; s++) xf[s] = __builtin_bit_cast(hbf16x8, __builtin_amdgcn_raw_buffer_load_b128(pbuf, live ? at + 32u * s : at, 0, 0));
+        for (int s = 0; s < 4 * NP; s++) xf[s] = __builtin_bit_cast(hu32x4, __builtin_amdgcn_raw_buffer_load_b128(pbuf, live ? at + 32u * s : at, 0, 0));
         issue();
     } else
 #pragma unroll
@@ -213,7 +225,7 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
             for (int e = 0; e < 4; e++) {
                 words[e] = upper_halves(piece_bits(x[2 * e], m0, m1, m2), piece_bits(x[2 * e + 1], m0, m1, m2));
             }
-            xf[s0 + s] = __builtin_bit_cast(hbf16x8, words);
+            xf[s0 + s] = words;
         }
         // (a batch's loads are not to be requested before the batch before is in its operands:
         // all of them at once would need more registers than a lane has)
@@ -230,7 +242,7 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
     auto finish = [&](uint32_t p, const hf32x16 &sum) __attribute__((always_inline)) {
         float *part = lds_part + (p & 1u) * (WAVES * 256u);
 #pragma unroll
-        for (int i = 0; i < 4; i++) part[wave * 256u + 64u * i + lane] = (sum[i] + sum[4 + i]) + sum[8 + i];
+        for (int i = 0; i < 4; i++) part[wave * 256u + 64u * i + lane] = F16 ? fmaf(sum[4 + i], 1.0f / 2048.0f, sum[i]) : (sum[i] + sum[4 + i]) + sum[8 + i];
         lds_barrier();
         // Buffer p % 2 is written again in step p + 2, after the barrier of step p + 1, which a
         // wave passes only when it has read what it needs here. The 256 outputs of a tile are
@@ -242,6 +254,7 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
             float total = src[0];
 #pragma unroll
             for (uint32_t wv = 1; wv < WAVES; wv++) total += src[wv * 256u];
+            if (F16) total *= lds_inverse[tk];
             lds_kept[256u * (p % KEPT) + 32u * tk + row] = total;
         }
     };
@@ -280,8 +293,9 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
             const uint8_t *t = ring + slot * SLOT;
 #pragma unroll
             for (int s = 0; s < 4; s++) {
-                const hbf16x8 w = *reinterpret_cast<const hbf16x8 *>(t + r_at[s]);
-                sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(xf[4 * i + s], w, sum, 0, 0, 0);
+                const hu32x4 w = *reinterpret_cast<const hu32x4 *>(t + r_at[s]);
+                if constexpr (F16) sum = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(hf16x8, xf[4 * i + s]), __builtin_bit_cast(hf16x8, w), sum, 0, 0, 0);
+                else sum = __builtin_amdgcn_mfma_f32_32x32x16_bf16(__builtin_bit_cast(hbf16x8, xf[4 * i + s]), __builtin_bit_cast(hbf16x8, w), sum, 0, 0, 0);
             }
             // (the piece's matrix instructions belong here, not after the last piece's wait, where
             // the compiler would otherwise collect them with all their operands held in registers)
@@ -317,19 +331,59 @@ __global__ __launch_bounds__(256) void matvec_bf16_split_kernel(MvArgs a, uint2 
     }
 }
 
-template <int NP, bool SPLIT>
+// The same for matvec_f16: the token scaled by the power of two that puts its largest
+// magnitude in [2^14, 2^15) and split into its f16 rounding and what that left times 2^11
+// (planes [2][tokens][k]), and one over the scale.
+__global__ __launch_bounds__(256) void matvec_f16_split_kernel(MvArgs a, uint2 *planes, float *inverse) {
+    __shared__ float red[4];
+    __shared__ float4 staged[1024];
+    stage_token(a, blockIdx.x, staged, red);
+    __syncthreads();
+    const uint32_t tid = threadIdx.x, k4 = a.k / 4u;
+    float big = 0.f;
+    for (uint32_t i = tid; i < k4; i += 256u) {
+        const float4 v = staged[i];
+        big = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fmaxf(fabsf(v.z), fabsf(v.w)), big));
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) big = fmaxf(big, __shfl_xor(big, off, 64));
+    if ((tid & 63u) == 0) red[tid >> 6] = big;
+    __syncthreads();
+    big = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    const int e = (int)((__float_as_uint(big) >> 23) & 0xffu);  // biased exponent; 0 for zero and subnormals
+    int se = 127 + 14 - (e - 127);                               // scale = 2^(14 - (e - 127)), kept normal both ways
+    se = se < 1 ? 1 : se > 253 ? 253 : se;
+    const bool unit = e == 0 || e == 255;
+    const float scale = unit ? 1.0f : __uint_as_float((uint32_t)se << 23);
+    if (tid == 0) inverse[blockIdx.x] = unit ? 1.0f : __uint_as_float((uint32_t)(254 - se) << 23);
+    for (uint32_t i = tid; i < k4; i += 256u) {
+        const float4 v = staged[i];
+        const float x[4] = {v.x, v.y, v.z, v.w};
+        _Float16 hi[4], lo[4];
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            // The scale is a power of two, so x * scale - hi in one fused operation is exact.
+            hi[j] = (_Float16)(x[j] * scale);
+            lo[j] = (_Float16)(fmaf(x[j], scale, -(float)hi[j]) * 2048.0f);
+        }
+        planes[(size_t)blockIdx.x * k4 + i] = __builtin_bit_cast(uint2, hf16x4{hi[0], hi[1], hi[2], hi[3]});
+        planes[(size_t)(gridDim.x + blockIdx.x) * k4 + i] = __builtin_bit_cast(uint2, hf16x4{lo[0], lo[1], lo[2], lo[3]});
+    }
+}
+
+template <int NP, bool SPLIT, bool F16>
 zhip_result launch_blocks(const Dispatch &d, const StreamArgs &q, dim3 grid) {
-    auto kernel = matvec_bf16_mfma_stream_kernel<NP, SPLIT>;
+    auto kernel = matvec_bf16_mfma_stream_kernel<NP, SPLIT, F16>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess) {
             (void)hipGetLastError();
-            return fail(d, ZHIP_E_GPU, "matvec_bf16: cannot reserve %u bytes of LDS", LDS_BYTES);
+            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", F16 ? "matvec_f16" : "matvec_bf16", LDS_BYTES);
         }
         configured = true;
     }
     hipLaunchKernelGGL(kernel, grid, dim3(THREADS), LDS_BYTES, d.stream, q);
-    return check_launch(d, "matvec_bf16");
+    return check_launch(d, F16 ? "matvec_f16" : "matvec_bf16");
 }
 
 }  // namespace
@@ -341,43 +395,49 @@ bool matvec_bf16_mfma_stream_accepts(const MvArgs &a) {
            a.xr % 4u == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == 2u * a.k;
 }
 
-template <bool SPLIT>
+template <bool SPLIT, bool F16>
 static zhip_result launch_for_k(const Dispatch &d, const StreamArgs &q, dim3 grid) {
     switch (q.a.k / 512u) {
-    case 2: return launch_blocks<2, SPLIT>(d, q, grid);
-    case 3: return launch_blocks<3, SPLIT>(d, q, grid);
-    case 4: return launch_blocks<4, SPLIT>(d, q, grid);
-    case 5: return launch_blocks<5, SPLIT>(d, q, grid);
-    case 6: return launch_blocks<6, SPLIT>(d, q, grid);
-    case 7: return launch_blocks<7, SPLIT>(d, q, grid);
-    default: return launch_blocks<8, SPLIT>(d, q, grid);
+    case 2: return launch_blocks<2, SPLIT, F16>(d, q, grid);
+    case 3: return launch_blocks<3, SPLIT, F16>(d, q, grid);
+    case 4: return launch_blocks<4, SPLIT, F16>(d, q, grid);
+    case 5: return launch_blocks<5, SPLIT, F16>(d, q, grid);
+    case 6: return launch_blocks<6, SPLIT, F16>(d, q, grid);
+    case 7: return launch_blocks<7, SPLIT, F16>(d, q, grid);
+    default: return launch_blocks<8, SPLIT, F16>(d, q, grid);
     }
 }
 
-zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) {
+// f16: the weights are f16 (matvec_f16), bf16 otherwise.
+zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes, bool f16) {
+    const char *name = f16 ? "matvec_f16" : "matvec_bf16";
     // 32-bit byte offsets, a tile past the last row.
     const uint64_t used = (uint64_t)a.rows * a.row_bytes;
-    if (used + 64ull * a.row_bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "matvec_bf16: weights of 4 GiB or more");
+    if (used + 64ull * a.row_bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "%s: weights of 4 GiB or more", name);
     const uint32_t cus = (uint32_t)d.dev->compute_units;
     const uint32_t units = (a.rows + 7u) / 8u;
     const uint32_t groups = units < cus ? units : cus;
     const uint32_t rounds = (a.rows / 32u) / groups;
     const uint32_t tail = (a.rows - 32u * rounds * groups + 7u) / 8u;
-    StreamArgs q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, nullptr, 0u, 0u};
+    StreamArgs q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, nullptr, 0u, 0u, nullptr};
     // The tokens are split (and normalised) by a launch of their own where that is cheaper than
     // every workgroup splitting them again, and wherever the step carries the RMSNorm prologue
     // (the workgroups computing the norm themselves at k = 1024 measured the same: 151936 x 1024
-    // at 2 / 4 / 8 tokens 53.3 / 54.1 / 56.3 us against 54.2 / 54.2 / 55.5 us this way).
-    const bool split = (a.flags & FLAG_NORM) || a.k >= 2048u;
+    // at 2 / 4 / 8 tokens 53.3 / 54.1 / 56.3 us against 54.2 / 54.2 / 55.5 us this way). f16
+    // tokens, which need their scales first, always.
+    const bool split = f16 || (a.flags & FLAG_NORM) || a.k >= 2048u;
     if (split) {
-        const uint64_t bytes = 6ull * a.m * a.k;
-        if (!d.work) return fail(d, ZHIP_E_GPU, "matvec_bf16: no workspace");
-        if (bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "matvec_bf16: a step of %u tokens", a.m);
-        if (zhip_result r = d.work->reserve(d, bytes)) return r;
-        hipLaunchKernelGGL(matvec_bf16_split_kernel, dim3(a.m), dim3(256), 0, d.stream, a, reinterpret_cast<uint2 *>(d.work->data));
-        if (zhip_result r = check_launch(d, "matvec_bf16")) return r;
+        const uint64_t bytes = (f16 ? 4ull : 6ull) * a.m * a.k;
+        if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", name);
+        if (bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "%s: a step of %u tokens", name, a.m);
+        if (zhip_result r = d.work->reserve(d, bytes + 4ull * a.m + 64u)) return r;
+        float *inverse = reinterpret_cast<float *>(d.work->data + bytes);
+        if (f16) hipLaunchKernelGGL(matvec_f16_split_kernel, dim3(a.m), dim3(256), 0, d.stream, a, reinterpret_cast<uint2 *>(d.work->data), inverse);
+        else hipLaunchKernelGGL(matvec_bf16_split_kernel, dim3(a.m), dim3(256), 0, d.stream, a, reinterpret_cast<uint2 *>(d.work->data));
+        if (zhip_result r = check_launch(d, name)) return r;
         q.planes = d.work->data;
         q.plane_tokens = a.m;
+        q.inverse = inverse;
         q.a.flags &= ~FLAG_NORM;
         q.a.norm_w = nullptr;
     }
@@ -387,7 +447,7 @@ zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, u
         q.a.out = a.out + (size_t)t0 * a.out_stride;
         q.a.m = a.m - t0 < 8u ? a.m - t0 : 8u;
         q.t0 = t0;
-        if (zhip_result r = split ? launch_for_k<true>(d, q, grid) : launch_for_k<false>(d, q, grid)) return r;
+        if (zhip_result r = f16 ? launch_for_k<true, true>(d, q, grid) : split ? launch_for_k<true, false>(d, q, grid) : launch_for_k<false, false>(d, q, grid)) return r;
     }
     return ZHIP_OK;
 }
