@@ -431,8 +431,9 @@ def test_matvec_q8_0_mfma_variant(ctx, rows, n, k, col0, pad, accumulate):
 
 @pytest.mark.parametrize("norm", [False, True])
 @pytest.mark.parametrize("rows,n,k", [(8, 4128, 4096), (3, 64, 2048), (5, 3072, 1024), (2, 4104, 1024)])
-def test_matvec_q8_0_mfma_variant_silu_pair(ctx, rows, n, k, norm):
-    """The matrix-core variant of matvec_q8_0 on the fused gate / up step (SILU_PAIR: gate rows,
+@pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q6_k, TensorType.q3_k])
+def test_matvec_q8_0_mfma_variant_silu_pair(ctx, t, rows, n, k, norm):
+    """The matrix-core variant of matvec_q8_0, matvec_q6_k and matvec_q3_k on the fused gate / up step (SILU_PAIR: gate rows,
     then the up rows `half` further down; with the RMSNorm the planner's FFN launch carries):
     silu(gate) * up within 1e-5 of float64 row by row, each token bitwise equal to its lone
     launch. (4104 outputs: 513 eight-row units, the last tile shared by two workgroups.)"""
@@ -441,14 +442,14 @@ def test_matvec_q8_0_mfma_variant_silu_pair(ctx, rows, n, k, norm):
     x = c.random(rows * k, 3).reshape(rows, k)
     x[0] *= np.float32(1e-3)
     nw = c.random(k, 1.5)
-    raw, values = quant_rows(c, TensorType.q8_0, 2 * n, k)
-    xa, wa, na = c.upload(x), c.gpu_weights(TensorType.q8_0, raw, k), c.upload(nw)
+    raw, values = quant_rows(c, t, 2 * n, k)
+    xa, wa, na = c.upload(x), c.gpu_weights(t, raw, k), c.upload(nw)
     x64 = np.stack([norm_row(r, nw if norm else None, eps) for r in x])
     v64 = values.astype(np.float64)
     g, u = x64 @ v64[:n].T, x64 @ v64[n:].T
     want = g * sigmoid64(g) * u
     p = lambda: P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, eps=eps, norm=norm, silu_pair=True, half=n)
-    pipeline = c.set.matvec(c.rec, Kernel.matvec_q8_0, MFMA_VARIANT)
+    pipeline = c.set.matvec(c.rec, K.weight_kernel("matvec", t), MFMA_VARIANT)
     grid_x = K.div_ceil(n, MFMA_VARIANT.group_rows())
     out = c.output(rows * n)
     c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, na], (grid_x, rows, 1))

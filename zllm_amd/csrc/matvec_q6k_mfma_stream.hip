@@ -196,9 +196,15 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     const uint32_t b = q.by_die ? (blockIdx.x & 7u) * (G >> 3) + (blockIdx.x >> 3) : blockIdx.x;
     const uint32_t tail_units = q.tail_base + (b < q.tail_rem ? 1u : 0u);
     const uint32_t tail_row = 32u * q.rounds * G + 8u * (b * q.tail_base + (b < q.tail_rem ? b : q.tail_rem));
-    const uint32_t count = q.rounds + (tail_units ? 1u : 0u);
-    auto first_row = [&](uint32_t p) { return p < q.rounds ? 32u * (b + p * G) : tail_row; };
-    auto rows_of = [&](uint32_t p) { return p < q.rounds ? 32u : 8u * tail_units; };
+    // With SILU_PAIR (src/kernels/matvec_quant.wgsl.hbs:110-125) an output tile is two weight
+    // tiles, the gate rows and then the up rows `half` further down: tile p of the run is weight
+    // tile p % per of output tile p / per.
+    const uint32_t per = (a.flags & FLAG_SILU_PAIR) ? 2u : 1u;
+    const uint32_t count = per * (q.rounds + (tail_units ? 1u : 0u));
+    auto out_row = [&](uint32_t po) { return po < q.rounds ? 32u * (b + po * G) : tail_row; };  // first output of output tile po
+    auto out_rows = [&](uint32_t po) { return po < q.rounds ? 32u : 8u * tail_units; };
+    auto first_row = [&](uint32_t p) { return out_row(p / per) + ((p % per) ? a.half : 0u); };
+    auto rows_of = [&](uint32_t p) { return out_rows(p / per); };
 
     // A unit's loads. The unit is 224 lines, row after row; load g = 4 wave + j brings lines
     // 8 g .. 8 g + 7 (the eighth wave's four would be past the unit's end: they go against an
@@ -347,26 +353,30 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
         }
     };
     // (a wave sums tokens i and 4 + i, whose partial sums lie side by side: no two lanes on a bank)
+    float held = 0.f;  // the gate tile's result, until the up tile's arrives
     auto sum_up = [&](uint32_t p) __attribute__((always_inline)) {
-        if ((tid >> 8) != (p & 1u)) return;
+        const uint32_t po = p / per;
+        if ((tid >> 8) != (po & 1u)) return;  // (the same half of the workgroup for an output tile's two weight tiles)
         const float *part = lds_part + (p & 1u) * (WAVES * 256u);
         const uint32_t row = tid & 31u, tk = 4u * ((tid >> 5) & 1u) + ((tid >> 6) & 3u);
         const float *src = part + 64u * (tk & 3u) + 32u * (tk >> 2) + row;
         float total = src[0];
 #pragma unroll
         for (uint32_t wv = 1; wv < WAVES; wv++) total += src[wv * 256u];
-        lds_kept[256u * (p % KEPT) + 32u * tk + row] = total * lds_inverse[tk];
+        total *= lds_inverse[tk];
+        if (per == 2u && !(p & 1u)) held = total;
+        else lds_kept[256u * (po % KEPT) + 32u * tk + row] = per == 2u ? silu_f(held) * total : total;
     };
-    // The outputs of tiles first .. first + n - 1, from LDS to memory in one burst: 128 contiguous
-    // bytes a token and tile.
+    // The outputs of output tiles first .. first + n - 1, from LDS to memory in one burst: 128
+    // contiguous bytes a token and tile.
     auto store_kept = [&](uint32_t first, uint32_t n) __attribute__((always_inline)) {
         lds_barrier();
-        for (uint32_t p = first + (tid >> 8); p < first + n; p += 2u) {
+        for (uint32_t po = first + (tid >> 8); po < first + n; po += 2u) {
             const uint32_t row = tid & 31u, tk = (tid >> 5) & 7u;
-            const uint32_t j = first_row(p) + row;
-            if (tk < a.m && row < rows_of(p) && j < a.rows) {
+            const uint32_t j = out_row(po) + row;
+            if (tk < a.m && row < out_rows(po) && j < a.rows) {
                 float *o = a.out + (size_t)tk * a.out_stride + a.col0 + j;
-                const float total = lds_kept[256u * (p % KEPT) + (tid & 255u)];
+                const float total = lds_kept[256u * (po % KEPT) + (tid & 255u)];
                 store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + total : total);
             }
         }
@@ -385,7 +395,7 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
             sum_up(p - 1u);
             // (the next tile's sums are kept only behind a later barrier, which no thread passes
             // before it has stored what it stores here)
-            if (p % KEPT == 0u) store_kept(p - KEPT, KEPT);
+            if (p % (per * KEPT) == 0u) store_kept(p / per - KEPT, KEPT);
         }
         multiply(unit, v % SLOTS);
     };
@@ -402,7 +412,8 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     if (count > 0u) {
         lds_barrier();
         sum_up(count - 1u);
-        store_kept((count - 1u) - (count - 1u) % KEPT, (count - 1u) % KEPT + 1u);
+        const uint32_t last = count / per - 1u;  // the run's last output tile
+        store_kept(last - last % KEPT, last % KEPT + 1u);
     }
 }
 
@@ -425,7 +436,7 @@ zhip_result launch_blocks(const Dispatch &d, const Q6Args &q, dim3 grid) {
 template <class F>
 zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) {
     // 32-bit byte offsets, a tile past the last row.
-    const uint64_t used = (uint64_t)a.rows * a.row_bytes;
+    const uint64_t used = ((uint64_t)((a.flags & FLAG_SILU_PAIR) ? a.half : 0u) + a.rows) * a.row_bytes;
     if (used + 64ull * a.row_bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "%s: weights of 4 GiB or more", F::name());
     if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", F::name());
     const uint64_t plane_bytes = 4ull * a.m * a.k;
@@ -448,13 +459,13 @@ zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) 
 }
 
 bool stream_accepts(const MvArgs &a, uint32_t block_bytes) {
-    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && !(a.flags & FLAG_SILU_PAIR) && a.rows >= 1 && a.xr % 4u == 0 &&
+    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && a.rows >= 1 && a.xr % 4u == 0 &&
            (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == a.k / 256u * block_bytes;
 }
 
 }  // namespace
 
-// Whether these kernels can run the (already validated) arguments: k of whole units, no pair.
+// Whether these kernels can run the (already validated) arguments: k of whole units.
 bool matvec_q6k_mfma_stream_accepts(const MvArgs &a) { return stream_accepts(a, FmtQ6::BLOCK); }
 zhip_result launch_matvec_q6k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) { return launch_stream<FmtQ6>(d, a, w_bytes); }
 bool matvec_q3k_mfma_stream_accepts(const MvArgs &a) { return stream_accepts(a, FmtQ3::BLOCK); }
