@@ -177,7 +177,16 @@ zhip_result zhip_force_loss(zhip_context *context);
  * (MatvecVariant.id, src/kernels/kernels.zig:328-333). Returns the length
  * written (without the NUL), or 0 when this backend does not implement the
  * kernel, which the caller records as an empty artifact
- * (src/kernels/kernels.zig:776-783). */
+ * (src/kernels/kernels.zig:776-783).
+ *
+ * Every MatvecVariant id is accepted and keeps the reference's results bit
+ * for bit. Two things go beyond the reference's contract: decode multiplies
+ * take 5..8 token rows (the reference stops at 4,
+ * shaders/matvec_quant.wgsl.hbs:64-65), and on matvec_q3_k, matvec_q4_k,
+ * matvec_q5_k, matvec_q6_k and matvec_q8_0 the id 0x00104010 (wg 512, lanes 64,
+ * rows 16, a geometry no reference tuning emits) selects matrix-core kernels
+ * for steps of 2..8 tokens that read the weights once; their sums round
+ * differently from the reference's (within 2e-3 of the row's scale). */
 size_t zhip_kernel_artifact(const char *name, uint32_t variant, char *out, size_t capacity);
 /* Replaces the backend arm of kernels.backendSource (src/kernels/kernels.zig:
  * 914-922): bytes that change whenever the kernel's implementation changes
