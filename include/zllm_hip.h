@@ -182,7 +182,7 @@ zhip_result zhip_force_loss(zhip_context *context);
  * Every MatvecVariant id is accepted and keeps the reference's results bit
  * for bit. Two things go beyond the reference's contract: decode multiplies
  * take 5..8 token rows (the reference stops at 4,
- * shaders/matvec_quant.wgsl.hbs:64-65), and on matvec_q3_k, matvec_q4_k,
+ * src/kernels/matvec_quant.wgsl.hbs:64-65), and on matvec_q3_k, matvec_q4_k,
  * matvec_q5_k, matvec_q6_k and matvec_q8_0 the id 0x00104010 (wg 512, lanes 64,
  * rows 16, a geometry no reference tuning emits) selects matrix-core kernels
  * for steps of 2..8 tokens that read the weights once; their sums round
