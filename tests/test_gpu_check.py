@@ -510,9 +510,9 @@ def test_matvec_q8_0_mfma_variant_prologues(ctx, rows, n, k, prologue):
 @pytest.mark.parametrize("t", [TensorType.q6_k, TensorType.q3_k])
 def test_matvec_q6_k_mfma_variant(ctx, t, rows, n, k, col0, pad, accumulate, prologue):
     """matvec_q6_k and matvec_q3_k on the matrix-core variant id (a wave per sixteen rows): the weights are read
-    once for all tokens of the step, the tokens split beforehand (with the RMSNorm and
-    silu(x / act_div) prologues of src/kernels/matvec_quant.wgsl.hbs:73-89 where the step has
-    them). 1e-5 against float64; columns outside the launch untouched; each token bitwise equal
+    once for all tokens of the step, the tokens split into two f16 rows by every workgroup (with
+    the RMSNorm and silu(x / act_div) prologues of src/kernels/matvec_quant.wgsl.hbs:73-89 where
+    the step has them). 1e-5 against float64; columns outside the launch untouched; each token bitwise equal
     to its lone launch."""
     c = ctx
     stride = col0 + n + pad

@@ -17,24 +17,34 @@
 // tokens fill sixteen of the 32 operand rows; the others are zeros. A token's rows meet no other
 // token's: its results do not depend on how many tokens share the launch.
 //
-// Layout of the work. A launch of its own (matvec_q6k_split_kernel, one workgroup a token, the
-// default variant's staging arithmetic for the RMSNorm and silu(x / act_div) prologues) writes
-// the tokens' two f16 planes and inverse scales to the workspace once. In the multiply a
-// 512-thread workgroup is eight waves; its tiles are 32 matrix rows, taken as units of four
-// 256-weight blocks a row (896 bytes = seven whole lines of each row), wave w multiplying half
-// w % 2 of block w / 2 of the unit. A unit travels as a flat copy through a ring of four LDS
-// slots: the waves load it by wave-wide direct loads of whole lines (four each for seven of
-// them), each wave waits for its own and one barrier a unit tells everyone that all of it has
-// landed; the loads of the unit three ahead go out behind that barrier, so three units are in
-// flight while one is multiplied (two slots of twice the size, one unit in flight, measured the
-// same 94 us on 128256 x 4096: per 16-weight sub-block and wave the kernel issues 24 vector
-// instructions and a matrix instruction that do not overlap, 0.85 us a unit and SIMD against
-// the 1.1 us the unit's bytes need at full rate, and the two overlap only in part: with the
-// multiplies switched off the same launch takes 80 us, 6.1 TB/s). Chunk c (16 bytes) of a line of row r sits at position
-// c ^ (r % 8), which keeps the 32 rows' reads of one piece of a block to four lanes a bank. The
-// waves' partial sums meet in LDS behind the same barrier, are added in the order of the blocks
-// and wait there for one burst of stores when the workgroup's run ends. Workgroups are numbered
-// die by die and share the rows left after whole rounds in units of eight.
+// Layout of the work. A 512-thread workgroup is eight waves; its tiles are 32 matrix rows, taken
+// as units of four 256-weight blocks a row (896 bytes = seven whole lines of each row), wave w
+// multiplying half w % 2 of block w / 2 of the unit. Every workgroup builds the tokens' operands
+// for itself, each wave those of its own positions (the RMSNorm and silu(x / act_div) prologues
+// in the default variant's arithmetic; the waves' sums of squares and largest magnitudes meet in
+// LDS), while the first unit of weights is on its way: a launch of its own that wrote them to
+// memory once took 4.6 us, 1.5 us more than this costs. A unit travels as a flat copy through a
+// ring of four LDS slots: the waves load it by wave-wide direct loads of whole lines (four each
+// for seven of them), each wave waits for its own and one barrier a unit tells everyone that
+// all of it has landed; a wave reads the unit after the one it multiplies into registers behind
+// that barrier and sends the loads of the unit four ahead into the slot this frees. Chunk c (16
+// bytes) of a line of row r sits at position c ^ (r % 8), which keeps the 32 rows' reads of one
+// piece of a block to four lanes a bank. The waves' partial sums meet in LDS behind the same
+// barrier, are added in the order of the blocks and wait there for one burst of stores when the
+// workgroup's run ends. Workgroups are numbered die by die and share the rows left after whole
+// rounds in units of eight.
+//
+// What bounds it. Per 16-weight sub-block and wave the kernel issues about 28 vector instructions
+// and one matrix instruction. On this machine a vector instruction in a 32-bit encoding with
+// register or literal operands costs a SIMD 1.1 - 1.2 ns, one in a 64-bit encoding (v_perm_b32,
+// v_pk_add_f16, v_and_or_b32, v_lshl_or_b32, the SDWA conversions) or with a scalar-register
+// operand 1.9 - 2.0 ns (measured with two and four waves a SIMD): 43 ns a sub-block, 0.7 us a
+// unit and SIMD, against the 1.1 us (Q6_K) or 0.6 us (Q3_K) a unit's bytes need at full rate.
+// The matrix instruction hides behind the vector work once the next sub-block's unpacking is
+// put between it and the additions that wait for it. Measured on 14336 x 4096 at eight tokens:
+// Q6_K 19.2 us (21.8 us before the operands were built in the kernel, the next unit was read
+// ahead and the sub-blocks overlapped), Q3_K 16.8 us (20.3 us); Q6_K on 128256 x 4096 87 us
+// (94 - 99 us), and 80 us with the multiplies switched off.
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -54,7 +64,7 @@ typedef uint32_t qu32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t qu32x4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t THREADS = 512, WAVES = 8;
-constexpr int SLOTS = 4;                        // ring slots: three units in flight behind the one multiplied
+constexpr int SLOTS = 4;                        // ring slots: the unit being read ahead and three in flight
 constexpr uint32_t PART_BYTES = 2u * WAVES * 256u * 4u;  // [tile parity][wave][token of the lane's four][lane]
 constexpr uint32_t KEPT = 16;                   // tiles whose outputs wait in LDS for one burst of stores
 
@@ -76,8 +86,15 @@ struct FmtQ3 {  // blocks repacked at load into eight self-contained 16-byte uni
 template <class F> constexpr uint32_t row_unit() { return 4u * F::BLOCK; }        // a unit's bytes of one row
 template <class F> constexpr uint32_t unit_bytes() { return 32u * row_unit<F>(); }  // a unit in LDS
 // (the last KB: where the loads of nothing land)
-template <class F> constexpr uint32_t lds_bytes() { return PART_BYTES + SLOTS * unit_bytes<F>() + KEPT * 1024u + 64u + 1024u; }
+template <class F> constexpr uint32_t lds_bytes() { return PART_BYTES + SLOTS * unit_bytes<F>() + KEPT * 1024u + 64u + 1024u + 512u; }
 static_assert(lds_bytes<FmtQ6>() <= 160u * 1024u - 64u, "the ring must fit the CU's LDS");
+
+// What a lane reads of a unit in LDS for its wave's half block: Q6_K the low nibbles of its
+// positions in the four quadrants' pairs, their two-bit words, the half's scales and d; Q3_K
+// the half's four sixteen-byte units.
+template <bool Q3> struct Fetched;
+template <> struct Fetched<true> { qu32x4 u[4]; };
+template <> struct Fetched<false> { qu32x2 ql[4], qh[2], sc; uint32_t d; };
 
 struct Q6Args {
     MvArgs a;
@@ -88,8 +105,6 @@ struct Q6Args {
     uint32_t by_die;     // workgroups renumbered die by die (the grid is a multiple of eight)
     uint32_t bias;       // 0x64646464: the bytes of two f16 1024.0 exponents, as a kernel argument
                          // so that the byte shuffles stay one instruction each
-    const uint8_t *planes;  // [2][tokens][k] f16: the tokens' roundings and remainders
-    const float *inverse;   // [tokens]: one over each token's scale
 };
 
 __device__ __forceinline__ void lds_barrier() {
@@ -129,48 +144,6 @@ __device__ __forceinline__ qf16x8 weights_f16(qu32x2 q, uint32_t bias) {
         r[2 * i + 1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(qf16x2, hi) + off);
     }
     return __builtin_bit_cast(qf16x8, r);
-}
-
-// Token blockIdx.x as the multiply sees it (src/kernels/matvec_quant.wgsl.hbs:73-89: RMSNorm
-// times the norm weights and / or silu(x / act_div)), scaled by the power of two that puts its
-// largest magnitude in [2^14, 2^15) and split into the f16 rounding and what that left times
-// 2^11: planes [2][tokens][k], and one over the scale.
-__global__ __launch_bounds__(256) void matvec_q6k_split_kernel(MvArgs a, uint2 *planes, float *inverse) {
-    __shared__ float red[4];
-    __shared__ float4 staged[1024];
-    stage_token(a, blockIdx.x, staged, red);
-    __syncthreads();
-    const uint32_t tid = threadIdx.x, k4 = a.k / 4u;
-    float big = 0.f;
-    for (uint32_t i = tid; i < k4; i += 256u) {
-        const float4 v = staged[i];
-        big = fmaxf(fmaxf(fabsf(v.x), fabsf(v.y)), fmaxf(fmaxf(fabsf(v.z), fabsf(v.w)), big));
-    }
-#pragma unroll
-    for (int off = 32; off > 0; off >>= 1) big = fmaxf(big, __shfl_xor(big, off, 64));
-    if ((tid & 63u) == 0) red[tid >> 6] = big;
-    __syncthreads();
-    big = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    const int e = (int)((__float_as_uint(big) >> 23) & 0xffu);  // biased exponent; 0 for zero and subnormals
-    int se = 127 + 14 - (e - 127);                               // scale = 2^(14 - (e - 127)), kept normal both ways
-    se = se < 1 ? 1 : se > 253 ? 253 : se;
-    const bool unit = e == 0 || e == 255;
-    const float scale = unit ? 1.0f : __uint_as_float((uint32_t)se << 23);
-    if (tid == 0) inverse[blockIdx.x] = unit ? 1.0f : __uint_as_float((uint32_t)(254 - se) << 23);
-    for (uint32_t i = tid; i < k4; i += 256u) {
-        const float4 v = staged[i];
-        const float x[4] = {v.x, v.y, v.z, v.w};
-        _Float16 hi[4], lo[4];
-#pragma unroll
-        for (int j = 0; j < 4; j++) {
-            // The scale is a power of two, so x * scale - hi in one fused operation is exact.
-            hi[j] = (_Float16)(x[j] * scale);
-            lo[j] = (_Float16)(fmaf(x[j], scale, -(float)hi[j]) * 2048.0f);
-        }
-        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
-        planes[(size_t)blockIdx.x * k4 + i] = __builtin_bit_cast(uint2, h4{hi[0], hi[1], hi[2], hi[3]});
-        planes[(size_t)(gridDim.x + blockIdx.x) * k4 + i] = __builtin_bit_cast(uint2, h4{lo[0], lo[1], lo[2], lo[3]});
-    }
 }
 
 // NU: units of a tile (k = 1024 NU).
@@ -235,34 +208,137 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
         }
     };
 
-    // The tokens' operands, ready-made in the planes. Operand row r of the matrix instruction is
-    // piece r / 8 of token 4 (r / 4 % 2) + r % 4 (rows 16 .. 31 are zeros), so that a lane's
-    // results are its weight row times both pieces of four tokens; the lane's eight positions of
-    // sub-block s of its wave's block are 16 s + 8 (lane / 32) ... The lanes of absent tokens and
-    // of the zero rows ask past the buffer's end and get zeros.
+    // The tokens' operands. Wave w multiplies half w % 2 (sub-blocks 8 (w % 2) .. + 7, 128
+    // positions) of block w / 2 of every unit: positions 1024 u + 128 w ... of the tokens, which
+    // the wave prepares for itself with every lane at work (token lane / 8, sixteen bytes a lane
+    // and step). What has to be known before anything can be rounded comes first: with the
+    // RMSNorm prologue the tokens' sums of squares, then each token's largest magnitude as the
+    // multiply sees it (src/kernels/matvec_quant.wgsl.hbs:73-89: RMSNorm times the norm weights
+    // and / or silu(x / act_div), in the default variant's arithmetic); the waves' parts meet in
+    // LDS and are combined in the order of the waves. The first unit's loads go out between the
+    // inputs' loads and this arithmetic (loads complete in order within a wave), the next three
+    // once the inputs are in: all four at once would hold up the other waves' inputs in the
+    // CU's one address pipeline (+0.7 us).
+    const bool norm = (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
+    float *lds_max = lds_inverse + 16 + 256, *lds_ss = lds_max + 64;  // [wave][token], behind the spare KB
+    // Operand row r of the matrix instruction is piece r / 8 of token 4 (r / 4 % 2) + r % 4 (rows
+    // 16 .. 31 are zeros), so that a lane's results are its weight row times both pieces of four
+    // tokens: piece 0 the f16 rounding of the scaled inputs, piece 1 what that left times 2^11.
+    // The lane's eight positions of sub-block s of its wave's half block are 16 s + 8 (lane / 32) ...
     const uint32_t rho = lane & 31u, kap = lane >> 5;
     const uint32_t tok = 4u * ((rho >> 2) & 1u) + (rho & 3u), piece = rho >> 3;
     const bool live = tok < a.m && piece < 2u;
-    // Wave w multiplies half w % 2 (sub-blocks 8 (w % 2) .. + 7, 128 positions) of block w / 2 of
-    // every unit.
-    const uint32_t blk = wave >> 1, half = wave & 1u;
     qf16x8 xf[8 * NU];
     {
-        const __amdgpu_buffer_rsrc_t pbuf = make_buffer(q.planes, 2u * a.m * a.k * 2u);
-        const uint32_t at = live ? ((piece * a.m + tok) * a.k + 256u * blk + 128u * half + 8u * kap) * 2u : 0xfffffff0u;
+        // (an absent token's lanes ask past the buffer's end: zeros, and nothing is fetched)
+        const uint32_t t1 = lane >> 3, l8 = lane & 7u, t1c = t1 < a.m ? t1 : a.m - 1u;
+        float4 r1[4 * NU], g1[4 * NU];
+        const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.x, ((a.m - 1u) * a.xr + a.k) * 4u);
+        const uint32_t x1 = (t1 * a.xr + 128u * wave + 4u * l8) * 4u;
 #pragma unroll
         for (int u = 0; u < NU; u++)
 #pragma unroll
-            for (int s = 0; s < 8; s++)
-                xf[8 * u + s] = __builtin_bit_cast(qf16x8, __builtin_amdgcn_raw_buffer_load_b128(pbuf, live ? at + 2u * (1024u * u + 16u * s) : at, 0, 0));
-    }
-    if (tid < 8u) lds_inverse[tid] = tid < a.m ? q.inverse[tid] : 1.0f;  // read behind later barriers
+            for (int i = 0; i < 4; i++)
+                r1[4 * u + i] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(xbuf, t1 < a.m ? x1 + 4u * (1024u * u + 32u * i) : 0xfffffff0u, 0, 0));
+        if (norm) {
+            const float *gp = a.norm_w + 128u * wave + 4u * l8;
 #pragma unroll
-    for (int v = 0; v < SLOTS - 1; v++) issue(v, v);
+            for (int u = 0; u < NU; u++)
+#pragma unroll
+                for (int i = 0; i < 4; i++) g1[4 * u + i] = *reinterpret_cast<const float4 *>(gp + 1024 * u + 32 * i);
+        }
+        issue(0, 0);
+        if (norm) {
+            float ss = 0.f;
+#pragma unroll
+            for (int i = 0; i < 4 * NU; i++) ss += r1[i].x * r1[i].x + r1[i].y * r1[i].y + r1[i].z * r1[i].z + r1[i].w * r1[i].w;
+            ss += __shfl_xor(ss, 1, 64);
+            ss += __shfl_xor(ss, 2, 64);
+            ss += __shfl_xor(ss, 4, 64);
+            if (l8 == 0u) lds_ss[8u * wave + t1] = ss;
+            lds_barrier();
+            float total = lds_ss[t1];
+#pragma unroll
+            for (uint32_t wv = 1; wv < WAVES; wv++) total += lds_ss[8u * wv + t1];
+            const float rs = 1.0f / sqrtf(total / (float)a.k + a.eps);
+#pragma unroll
+            for (int i = 0; i < 4 * NU; i++) {
+                r1[i].x = r1[i].x * rs * g1[i].x; r1[i].y = r1[i].y * rs * g1[i].y;
+                r1[i].z = r1[i].z * rs * g1[i].z; r1[i].w = r1[i].w * rs * g1[i].w;
+            }
+        }
+        if (act) {
+#pragma unroll
+            for (int i = 0; i < 4 * NU; i++) {
+                r1[i].x = silu_f(r1[i].x / a.act_div); r1[i].y = silu_f(r1[i].y / a.act_div);
+                r1[i].z = silu_f(r1[i].z / a.act_div); r1[i].w = silu_f(r1[i].w / a.act_div);
+            }
+        }
+        float big = 0.f;
+#pragma unroll
+        for (int i = 0; i < 4 * NU; i++) big = fmaxf(fmaxf(fabsf(r1[i].x), fabsf(r1[i].y)), fmaxf(fmaxf(fabsf(r1[i].z), fabsf(r1[i].w)), big));
+        big = fmaxf(big, __shfl_xor(big, 1, 64));
+        big = fmaxf(big, __shfl_xor(big, 2, 64));
+        big = fmaxf(big, __shfl_xor(big, 4, 64));
+        if (l8 == 0u) lds_max[8u * wave + t1] = big;
+        lds_barrier();
+#pragma unroll
+        for (int v = 1; v < SLOTS; v++) issue(v, v);
+        // Each token's scale: the power of two that puts its largest magnitude in [2^14, 2^15).
+        auto scale_of = [&](uint32_t t, bool inverse) {
+            float most = lds_max[t];
+#pragma unroll
+            for (uint32_t wv = 1; wv < WAVES; wv++) most = fmaxf(most, lds_max[8u * wv + t]);
+            const int e = (int)((__float_as_uint(most) >> 23) & 0xffu);  // biased exponent; 0 for zero and subnormals
+            int se = 127 + 14 - (e - 127);                                // scale = 2^(14 - (e - 127)), kept normal both ways
+            se = se < 1 ? 1 : se > 253 ? 253 : se;
+            if (e == 0 || e == 255) return 1.0f;
+            return __uint_as_float((uint32_t)(inverse ? 254 - se : se) << 23);
+        };
+        if (tid < 8u) lds_inverse[tid] = tid < a.m ? scale_of(tid, true) : 1.0f;  // read behind later barriers
+        const float scale = scale_of(t1c, false);
+        // From this layout to the operands' through 4 KB of LDS a wave, a unit's 128 positions at
+        // a time: [piece][token][position] f16 (the space of the partial sums and of the kept
+        // outputs, neither in use yet). A wave's LDS operations complete in order, and nobody
+        // else touches its 4 KB: no barrier.
+        uint8_t *stage = wave < 4u ? lds + 4096u * wave : reinterpret_cast<uint8_t *>(lds_kept) + 4096u * (wave - 4u);
+        // (sixteen-byte chunk c of row r sits at position c ^ r: the sixteen rows' reads of one chunk fall on sixteen different banks)
+        const uint32_t row = (piece & 1u) * 8u + tok;
+        const uint32_t present = t1 < a.m ? 0xffffffffu : 0u;
+        typedef _Float16 h4 __attribute__((ext_vector_type(4)));
+#pragma unroll
+        for (int u = 0; u < NU; u++) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                const float x[4] = {r1[4 * u + i].x, r1[4 * u + i].y, r1[4 * u + i].z, r1[4 * u + i].w};
+                _Float16 hi[4], lo[4];
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    // The scale is a power of two, so x * scale - hi in one fused operation is exact.
+                    hi[e] = (_Float16)(x[e] * scale);
+                    lo[e] = (_Float16)(fmaf(x[e], scale, -(float)hi[e]) * 2048.0f);
+                }
+                qu32x2 h2 = __builtin_bit_cast(qu32x2, h4{hi[0], hi[1], hi[2], hi[3]}), l2 = __builtin_bit_cast(qu32x2, h4{lo[0], lo[1], lo[2], lo[3]});
+                h2.x &= present; h2.y &= present; l2.x &= present; l2.y &= present;
+                const uint32_t chunk = (l8 >> 1) + 4u * i, within = 8u * (l8 & 1u);
+                *reinterpret_cast<qu32x2 *>(stage + t1 * 256u + 16u * (chunk ^ t1) + within) = h2;
+                *reinterpret_cast<qu32x2 *>(stage + (8u + t1) * 256u + 16u * (chunk ^ (8u + t1)) + within) = l2;
+            }
+            asm volatile("" ::: "memory");
+#pragma unroll
+            for (int s = 0; s < 8; s++) {
+                qu32x4 v = *reinterpret_cast<const qu32x4 *>(stage + row * 256u + 16u * ((2u * s + kap) ^ row));
+                if (!live) v = qu32x4{0u, 0u, 0u, 0u};
+                xf[8 * u + s] = __builtin_bit_cast(qf16x8, v);
+            }
+            asm volatile("" ::: "memory");
+        }
+    }
 
     // The lane's reads of its wave's half block of a unit: row rho of the flat copy, the block's
     // bytes at 224 (wave / 2). Byte o of a row's unit sits at 896 rho + 128 (o / 128) +
     // 16 ((o / 16 % 8) ^ (rho % 8)) + o % 16.
+    const uint32_t blk = wave >> 1, half = wave & 1u;
     auto at_byte = [&](uint32_t o) { return ROW_UNIT * rho + (o & ~127u) + 16u * (((o >> 4) & 7u) ^ (rho & 7u)) + (o & 15u); };
     constexpr bool Q3 = F::BLOCK == 128u;
     uint32_t at_ql[4], at_qh[2];  // Q6_K ql: [which 32 of the half's 64][which 16]; qh: [which 16]; Q3_K: at_ql = the half's four units
@@ -281,66 +357,84 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     }
 
     float acc[4] = {0.f, 0.f, 0.f, 0.f};  // tokens 4 (lane / 32) + i, matrix row rho of the tile, this wave's blocks
-    // One sub-block: its eight quants of the lane (a byte each), d * scale, and the operand index.
-    auto sub_block = [&](qu32x2 v, float dsc, int s) __attribute__((always_inline)) {
-        qf32x16 zero;
-#pragma unroll
-        for (int e = 0; e < 16; e++) zero[e] = 0.f;
-        const qf32x16 r = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[s], weights_f16<F>(v, bias), zero, 0, 0, 0);
-#pragma unroll
-        for (int i = 0; i < 4; i++) acc[i] = fmaf(dsc, fmaf(r[4 + i], 1.0f / 2048.0f, r[i]), acc[i]);
-        // (a sub-block's results are used up before the next sub-block's matrix
-        // instruction: eight of them in flight would not fit the registers)
-        asm volatile("" : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]));
-    };
-    auto multiply = [&](auto unit, uint32_t slot) __attribute__((always_inline)) {
-        constexpr int U = decltype(unit)::value;
+    // The lane's part of the unit in `slot`, from LDS to registers.
+    auto fetch = [&](uint32_t slot) __attribute__((always_inline)) {
         const uint8_t *t = ring + slot * UNIT;
+        Fetched<Q3> f;
+        if constexpr (Q3) {
+#pragma unroll
+            for (uint32_t i = 0; i < 4; i++) f.u[i] = *reinterpret_cast<const qu32x4 *>(t + at_ql[i]);
+        } else {
+#pragma unroll
+            for (uint32_t i = 0; i < 4; i++) f.ql[i] = *reinterpret_cast<const qu32x2 *>(t + at_ql[i]);
+#pragma unroll
+            for (uint32_t i = 0; i < 2; i++) f.qh[i] = *reinterpret_cast<const qu32x2 *>(t + at_qh[i]);
+            f.sc = *reinterpret_cast<const qu32x2 *>(t + at_sc);
+            f.d = *reinterpret_cast<const uint16_t *>(t + at_d);
+        }
+        return f;
+    };
+    // Sub-block s (of the eight of the wave's half block) of a fetched unit, made ready for the
+    // matrix instruction: the lane's eight quants as f16, and d * scale.
+    auto prepare = [&](const Fetched<Q3> &f, int s, qf16x8 &wf, float &dsc) __attribute__((always_inline)) {
+        qu32x2 v;
         if constexpr (Q3) {
             // Unit i of the half: 32 weights as two words of 2-bit values (byte b, bit pair e:
             // position 4 e + b; the second word 16 further), a word of third bits (byte b, bit e:
             // position 4 e + b), scale - 32 of each sixteen as signed bytes, d. The lane's eight
             // positions of a sixteen are 8 kap ..: bit pairs 2 kap and 2 kap + 1 of the four bytes.
-#pragma unroll
-            for (uint32_t i = 0; i < 4; i++) {
-                const qu32x4 u = *reinterpret_cast<const qu32x4 *>(t + at_ql[i]);
-                const float d = half_bits_to_float(u.w >> 16);
-#pragma unroll
-                for (uint32_t h16 = 0; h16 < 2; h16++) {
-                    const uint32_t word = h16 ? u.y : u.x, third = u.z >> (4u * h16 + 2u * kap);
-                    qu32x2 v;
-                    v[0] = ((word >> (4u * kap)) & 0x03030303u) | ((third & 0x01010101u) << 2);
-                    v[1] = ((word >> (4u * kap + 2u)) & 0x03030303u) | (((third >> 1) & 0x01010101u) << 2);
-                    const float dsc = d * (float)(int8_t)((u.w >> (8u * h16)) & 0xffu);
-                    sub_block(v, dsc, 8 * U + 2 * (int)i + (int)h16);
-                }
-            }
+            const uint32_t h16 = (uint32_t)s & 1u;
+            const qu32x4 u = f.u[s >> 1];
+            const uint32_t word = h16 ? u.y : u.x, third = u.z >> (4u * h16 + 2u * kap);
+            v[0] = ((word >> (4u * kap)) & 0x03030303u) | ((third & 0x01010101u) << 2);
+            v[1] = ((word >> (4u * kap + 2u)) & 0x03030303u) | (((third >> 1) & 0x01010101u) << 2);
+            dsc = half_bits_to_float(u.w >> 16) * (float)(int8_t)((u.w >> (8u * h16)) & 0xffu);
         } else {
-            const qu32x2 sc = *reinterpret_cast<const qu32x2 *>(t + at_sc);
-            const float d = half_bits_to_float(*reinterpret_cast<const uint16_t *>(t + at_d));
+            // Quadrant qd of the half: weights 32 qd + 16 h16 + 8 kap ... of its 128; s = 2 qd + h16.
+            const uint32_t h16 = (uint32_t)s & 1u, qd = (uint32_t)s >> 1, qp = qd & 1u, up = qd >> 1;
+            const qu32x2 ql = f.ql[2u * qp + h16], qh = f.qh[h16];
 #pragma unroll
-            for (uint32_t h16 = 0; h16 < 2; h16++) {
-                const qu32x2 qh = *reinterpret_cast<const qu32x2 *>(t + at_qh[h16]);
-#pragma unroll
-                for (uint32_t qp = 0; qp < 2; qp++) {
-                    const qu32x2 ql = *reinterpret_cast<const qu32x2 *>(t + at_ql[2u * qp + h16]);
-#pragma unroll
-                    for (uint32_t up = 0; up < 2; up++) {
-                        // Quadrant qd of the half: weights 32 qd + 16 h16 + 8 kap ... of its 128, sub-block 2 qd + h16 of its eight.
-                        const uint32_t qd = qp + 2u * up, s = 2u * qd + h16;
-                        qu32x2 v;
-#pragma unroll
-                        for (int w = 0; w < 2; w++) {
-                            const uint32_t nib = up ? (ql[w] >> 4) & 0x0f0f0f0fu : ql[w] & 0x0f0f0f0fu;
-                            const uint32_t two = (qd ? qh[w] >> (2u * qd) : qh[w]) & 0x03030303u;
-                            v[w] = nib | (two << 4);
-                        }
-                        const uint32_t word = s < 4u ? sc.x : sc.y;
-                        const float dsc = d * (float)(int8_t)((word >> (8u * (s & 3u))) & 0xffu);
-                        sub_block(v, dsc, 8 * U + (int)s);
-                    }
-                }
+            for (int w = 0; w < 2; w++) {
+                const uint32_t nib = up ? (ql[w] >> 4) & 0x0f0f0f0fu : ql[w] & 0x0f0f0f0fu;
+                const uint32_t two = (qd ? qh[w] >> (2u * qd) : qh[w]) & 0x03030303u;
+                v[w] = nib | (two << 4);
             }
+            const uint32_t word = s < 4 ? f.sc.x : f.sc.y;
+            dsc = half_bits_to_float(f.d) * (float)(int8_t)((word >> (8u * ((uint32_t)s & 3u))) & 0xffu);
+        }
+        wf = weights_f16<F>(v, bias);
+    };
+    // A unit's eight matrix instructions. The vector work of a sub-block is made to surround the
+    // matrix instruction of the one before it: while that runs, the next sub-block is unpacked
+    // (the last one's successor is the first of the unit after, which is in registers by then),
+    // and only then are its results scaled and added. The scheduler is kept from moving anything
+    // across these lines: left to itself it puts each matrix instruction right before the
+    // additions that wait for it.
+    qf16x8 wf;
+    float dsc;
+    auto multiply = [&](auto unit, const Fetched<Q3> &f, const Fetched<Q3> &after) __attribute__((always_inline)) {
+        constexpr int U = decltype(unit)::value;
+        qf32x16 zero;
+#pragma unroll
+        for (int e = 0; e < 16; e++) zero[e] = 0.f;
+#pragma unroll
+        for (int s = 0; s < 8; s++) {
+            const qu32x4 running = __builtin_bit_cast(qu32x4, wf);
+            const qf32x16 r = __builtin_amdgcn_mfma_f32_32x32x16_f16(xf[8 * U + s], wf, zero, 0, 0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            const float scale = dsc;
+            if (s < 7) prepare(f, s + 1, wf, dsc);
+            else prepare(after, 0, wf, dsc);
+            // (the running instruction's operand and all sixteen of its results stay where they
+            // are: a write to any of them would have to wait for the matrix core)
+            asm volatile("" ::"v"(running), "v"(r));
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 4; i++) acc[i] = fmaf(scale, fmaf(r[4 + i], 1.0f / 2048.0f, r[i]), acc[i]);
+            // (and a sub-block's results are used up before the next matrix instruction: eight of
+            // them in flight would not fit the registers)
+            asm volatile("" : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]));
+            __builtin_amdgcn_sched_barrier(0);
         }
     };
     // A finished tile's partial sums into LDS; they are added behind the next barrier.
@@ -382,23 +476,33 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
         }
     };
 
-    // One barrier a unit: behind it all of unit v has landed (every wave has waited for its own
-    // loads of it; those of the two units after it stay in flight), nobody still reads the slot
-    // that is refilled next, and the tile before's partial sums are in LDS.
+    // One barrier a unit: behind the barrier of unit v's step all of unit v + 1 has landed (every
+    // wave has waited for its own loads of it; those of the two units after it stay in flight),
+    // every wave has unit v in registers, so its slot takes the loads of unit v + 4, and the
+    // tile before's partial sums are in LDS. A wave reads unit v + 1 into registers while it
+    // multiplies unit v: no multiply waits for LDS.
+    Fetched<Q3> cur;
     auto step = [&](uint32_t p, auto unit) __attribute__((always_inline)) {
         constexpr int U = decltype(unit)::value;
         const uint32_t v = NU * p + U;
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SLOTS - 2) * LOADS) : "memory");
         lds_barrier();
-        issue(v + (SLOTS - 1), (v + (SLOTS - 1)) % SLOTS);
+        issue(v + SLOTS, v % SLOTS);
+        const Fetched<Q3> next = fetch((v + 1u) % SLOTS);
+        asm volatile("" ::: "memory");  // (the reads go out here, not where the next step uses them)
         if (U == 0 && p > 0u) {
             sum_up(p - 1u);
             // (the next tile's sums are kept only behind a later barrier, which no thread passes
             // before it has stored what it stores here)
             if (p % (per * KEPT) == 0u) store_kept(p / per - KEPT, KEPT);
         }
-        multiply(unit, v % SLOTS);
+        multiply(unit, cur, next);
+        cur = next;
     };
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SLOTS - 1) * LOADS) : "memory");
+    lds_barrier();
+    cur = fetch(0);
+    prepare(cur, 0, wf, dsc);
     for (uint32_t p = 0; p < count; p++) {
         step(p, std::integral_constant<int, 0>{});
         if constexpr (NU >= 2) step(p, std::integral_constant<int, 1>{});
@@ -438,22 +542,12 @@ zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) 
     // 32-bit byte offsets, a tile past the last row.
     const uint64_t used = ((uint64_t)((a.flags & FLAG_SILU_PAIR) ? a.half : 0u) + a.rows) * a.row_bytes;
     if (used + 64ull * a.row_bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "%s: weights of 4 GiB or more", F::name());
-    if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", F::name());
-    const uint64_t plane_bytes = 4ull * a.m * a.k;
-    if (zhip_result r = d.work->reserve(d, plane_bytes + 64u)) return r;
-    float *inverse = reinterpret_cast<float *>(d.work->data + plane_bytes);
-    hipLaunchKernelGGL(matvec_q6k_split_kernel, dim3(a.m), dim3(256), 0, d.stream, a, reinterpret_cast<uint2 *>(d.work->data), inverse);
-    if (zhip_result r = check_launch(d, F::name())) return r;
-
     const uint32_t cus = (uint32_t)d.dev->compute_units;
     const uint32_t units = (a.rows + 7u) / 8u;
     const uint32_t groups = units < cus ? units : cus;
     const uint32_t rounds = (a.rows / 32u) / groups;
     const uint32_t tail = (a.rows - 32u * rounds * groups + 7u) / 8u;
-    Q6Args q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, 0x64646464u, d.work->data, inverse};
-    q.a.flags &= ~FLAG_NORM;
-    q.a.norm_w = nullptr;
-    q.a.act_div = 0.f;
+    Q6Args q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, 0x64646464u};
     const dim3 grid(groups);
     return a.k == 1024u ? launch_blocks<F, 1>(d, q, grid) : a.k == 2048u ? launch_blocks<F, 2>(d, q, grid) : launch_blocks<F, 4>(d, q, grid);
 }
