@@ -14,8 +14,10 @@
 // rows, the f16 rounding of its inputs and the f16 rounding of what that left times 2^11, after
 // a power of two has put its largest magnitude at 2^14 (an input keeps 22 bits, every product is
 // exact in the f32 accumulator); the sub-block's d * scale multiplies its sum afterwards. Eight
-// tokens fill sixteen of the 32 operand rows; the others are zeros. A token's rows meet no other
-// token's: its results do not depend on how many tokens share the launch.
+// tokens fill sixteen of the 32 operand rows; the others are zeros. Up to four tokens take a
+// layout of their own (eight rows, a lane's results are one piece of four tokens: four
+// multiply-adds a sub-block instead of eight). A token's rows meet no other token's: its results
+// do not depend on how many tokens share the launch.
 //
 // Layout of the work. A 512-thread workgroup is eight waves; its tiles are 32 matrix rows, taken
 // as units of four 256-weight blocks a row (896 bytes = seven whole lines of each row), wave w
@@ -41,10 +43,11 @@
 // operand 1.9 - 2.0 ns (measured with two and four waves a SIMD): 43 ns a sub-block, 0.7 us a
 // unit and SIMD, against the 1.1 us (Q6_K) or 0.6 us (Q3_K) a unit's bytes need at full rate.
 // The matrix instruction hides behind the vector work once the next sub-block's unpacking is
-// put between it and the additions that wait for it. Measured on 14336 x 4096 at eight tokens:
-// Q6_K 19.2 us (21.8 us before the operands were built in the kernel, the next unit was read
-// ahead and the sub-blocks overlapped), Q3_K 16.8 us (20.3 us); Q6_K on 128256 x 4096 87 us
-// (94 - 99 us), and 80 us with the multiplies switched off.
+// put between it and the additions that wait for it. Measured on 14336 x 4096 at four / eight
+// tokens: Q6_K 16.5 / 17.9 us (21.8 us before the operands were built in the kernel, the next
+// unit was read ahead and the sub-blocks overlapped), Q3_K 14.3 / 15.6 us (20.3 us); Q6_K on
+// 128256 x 4096 80 / 87 us (94 - 99 us; 80 us with the multiplies switched off, 80.7 us for
+// one token on the default variant).
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -147,7 +150,8 @@ __device__ __forceinline__ qf16x8 weights_f16(qu32x2 q, uint32_t bias) {
 }
 
 // NU: units of a tile (k = 1024 NU).
-template <class F, int NU>
+// FEW: at most four tokens, whose eight rows then leave every lane four results instead of eight.
+template <class F, int NU, bool FEW>
 __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Args q) {
     constexpr uint32_t ROW_UNIT = row_unit<F>(), UNIT = unit_bytes<F>();
     constexpr int LOADS = F::LOADS;
@@ -224,9 +228,14 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     // Operand row r of the matrix instruction is piece r / 8 of token 4 (r / 4 % 2) + r % 4 (rows
     // 16 .. 31 are zeros), so that a lane's results are its weight row times both pieces of four
     // tokens: piece 0 the f16 rounding of the scaled inputs, piece 1 what that left times 2^11.
-    // The lane's eight positions of sub-block s of its wave's half block are 16 s + 8 (lane / 32) ...
+    // With at most four tokens row r is piece r / 4 of token r % 4 (rows 8 .. 31 are zeros): the
+    // lower half of the lanes gets its weight row times the tokens' first pieces, the upper half
+    // times their second pieces. Either way a piece's sums are accumulated apart and a wave's
+    // two meet once a tile, by the same operations: a token's result does not depend on which
+    // of the two layouts its launch used. The lane's eight positions of sub-block s of its
+    // wave's half block are 16 s + 8 (lane / 32) ...
     const uint32_t rho = lane & 31u, kap = lane >> 5;
-    const uint32_t tok = 4u * ((rho >> 2) & 1u) + (rho & 3u), piece = rho >> 3;
+    const uint32_t tok = FEW ? rho & 3u : 4u * ((rho >> 2) & 1u) + (rho & 3u), piece = FEW ? rho >> 2 : rho >> 3;
     const bool live = tok < a.m && piece < 2u;
     qf16x8 xf[8 * NU];
     {
@@ -304,7 +313,6 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
         uint8_t *stage = wave < 4u ? lds + 4096u * wave : reinterpret_cast<uint8_t *>(lds_kept) + 4096u * (wave - 4u);
         // (sixteen-byte chunk c of row r sits at position c ^ r: the sixteen rows' reads of one chunk fall on sixteen different banks)
         const uint32_t row = (piece & 1u) * 8u + tok;
-        const uint32_t present = t1 < a.m ? 0xffffffffu : 0u;
         typedef _Float16 h4 __attribute__((ext_vector_type(4)));
 #pragma unroll
         for (int u = 0; u < NU; u++) {
@@ -318,18 +326,19 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
                     hi[e] = (_Float16)(x[e] * scale);
                     lo[e] = (_Float16)(fmaf(x[e], scale, -(float)hi[e]) * 2048.0f);
                 }
-                qu32x2 h2 = __builtin_bit_cast(qu32x2, h4{hi[0], hi[1], hi[2], hi[3]}), l2 = __builtin_bit_cast(qu32x2, h4{lo[0], lo[1], lo[2], lo[3]});
-                h2.x &= present; h2.y &= present; l2.x &= present; l2.y &= present;
+                // (an absent token's inputs are zeros, or what its lanes make of them: its rows of the layout are never read)
+                const qu32x2 h2 = __builtin_bit_cast(qu32x2, h4{hi[0], hi[1], hi[2], hi[3]}), l2 = __builtin_bit_cast(qu32x2, h4{lo[0], lo[1], lo[2], lo[3]});
                 const uint32_t chunk = (l8 >> 1) + 4u * i, within = 8u * (l8 & 1u);
                 *reinterpret_cast<qu32x2 *>(stage + t1 * 256u + 16u * (chunk ^ t1) + within) = h2;
                 *reinterpret_cast<qu32x2 *>(stage + (8u + t1) * 256u + 16u * (chunk ^ (8u + t1)) + within) = l2;
             }
             asm volatile("" ::: "memory");
 #pragma unroll
-            for (int s = 0; s < 8; s++) {
-                qu32x4 v = *reinterpret_cast<const qu32x4 *>(stage + row * 256u + 16u * ((2u * s + kap) ^ row));
-                if (!live) v = qu32x4{0u, 0u, 0u, 0u};
-                xf[8 * u + s] = __builtin_bit_cast(qf16x8, v);
+            for (int s = 0; s < 8; s++) xf[8 * u + s] = qf16x8{0, 0, 0, 0, 0, 0, 0, 0};
+            if (live) {  // (the other lanes stay out of the reads: half of the LDS traffic)
+#pragma unroll
+                for (int s = 0; s < 8; s++)
+                    xf[8 * u + s] = __builtin_bit_cast(qf16x8, *reinterpret_cast<const qu32x4 *>(stage + row * 256u + 16u * ((2u * s + kap) ^ row)));
             }
             asm volatile("" ::: "memory");
         }
@@ -356,7 +365,9 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
         at_d = at_byte(224u * blk + 208u);
     }
 
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};  // tokens 4 (lane / 32) + i, matrix row rho of the tile, this wave's blocks
+    // Matrix row rho of the tile, this wave's blocks: piece 0 (acc) and piece 1 (acc_lo) of tokens
+    // 4 (lane / 32) + i; with at most four tokens piece lane / 32 of token i in acc.
+    float acc[4] = {0.f, 0.f, 0.f, 0.f}, acc_lo[4] = {0.f, 0.f, 0.f, 0.f};
     // The lane's part of the unit in `slot`, from LDS to registers.
     auto fetch = [&](uint32_t slot) __attribute__((always_inline)) {
         const uint8_t *t = ring + slot * UNIT;
@@ -430,10 +441,14 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
             asm volatile("" ::"v"(running), "v"(r));
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-            for (int i = 0; i < 4; i++) acc[i] = fmaf(scale, fmaf(r[4 + i], 1.0f / 2048.0f, r[i]), acc[i]);
+            for (int i = 0; i < 4; i++) {
+                acc[i] = fmaf(scale, r[i], acc[i]);
+                if (!FEW) acc_lo[i] = fmaf(scale, r[4 + i], acc_lo[i]);
+            }
             // (and a sub-block's results are used up before the next matrix instruction: eight of
             // them in flight would not fit the registers)
             asm volatile("" : "+v"(acc[0]), "+v"(acc[1]), "+v"(acc[2]), "+v"(acc[3]));
+            if (!FEW) asm volatile("" : "+v"(acc_lo[0]), "+v"(acc_lo[1]), "+v"(acc_lo[2]), "+v"(acc_lo[3]));
             __builtin_amdgcn_sched_barrier(0);
         }
     };
@@ -442,8 +457,8 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
         float *part = lds_part + (p & 1u) * (WAVES * 256u);
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            part[wave * 256u + 64u * i + lane] = acc[i];
-            acc[i] = 0.f;
+            part[wave * 256u + 64u * i + lane] = FEW ? acc[i] : fmaf(acc_lo[i], 1.0f / 2048.0f, acc[i]);
+            acc[i] = acc_lo[i] = 0.f;
         }
     };
     // (a wave sums tokens i and 4 + i, whose partial sums lie side by side: no two lanes on a bank)
@@ -453,10 +468,13 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
         if ((tid >> 8) != (po & 1u)) return;  // (the same half of the workgroup for an output tile's two weight tiles)
         const float *part = lds_part + (p & 1u) * (WAVES * 256u);
         const uint32_t row = tid & 31u, tk = 4u * ((tid >> 5) & 1u) + ((tid >> 6) & 3u);
+        if (FEW && tk >= 4u) return;
         const float *src = part + 64u * (tk & 3u) + 32u * (tk >> 2) + row;
-        float total = src[0];
+        // (with at most four tokens a wave's two pieces still lie apart, 32 floats from each other)
+        auto of_wave = [&](uint32_t wv) { return FEW ? fmaf(src[wv * 256u + 32u], 1.0f / 2048.0f, src[wv * 256u]) : src[wv * 256u]; };
+        float total = of_wave(0);
 #pragma unroll
-        for (uint32_t wv = 1; wv < WAVES; wv++) total += src[wv * 256u];
+        for (uint32_t wv = 1; wv < WAVES; wv++) total += of_wave(wv);
         total *= lds_inverse[tk];
         if (per == 2u && !(p & 1u)) held = total;
         else lds_kept[256u * (po % KEPT) + 32u * tk + row] = per == 2u ? silu_f(held) * total : total;
@@ -521,9 +539,9 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     }
 }
 
-template <class F, int NU>
+template <class F, int NU, bool FEW>
 zhip_result launch_blocks(const Dispatch &d, const Q6Args &q, dim3 grid) {
-    auto kernel = matvec_kquant_mfma_stream_kernel<F, NU>;
+    auto kernel = matvec_kquant_mfma_stream_kernel<F, NU, FEW>;
     constexpr uint32_t bytes = lds_bytes<F>();
     static bool configured = false;
     if (!configured) {
@@ -549,7 +567,8 @@ zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) 
     const uint32_t tail = (a.rows - 32u * rounds * groups + 7u) / 8u;
     Q6Args q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, 0x64646464u};
     const dim3 grid(groups);
-    return a.k == 1024u ? launch_blocks<F, 1>(d, q, grid) : a.k == 2048u ? launch_blocks<F, 2>(d, q, grid) : launch_blocks<F, 4>(d, q, grid);
+    if (a.m <= 4u) return a.k == 1024u ? launch_blocks<F, 1, true>(d, q, grid) : a.k == 2048u ? launch_blocks<F, 2, true>(d, q, grid) : launch_blocks<F, 4, true>(d, q, grid);
+    return a.k == 1024u ? launch_blocks<F, 1, false>(d, q, grid) : a.k == 2048u ? launch_blocks<F, 2, false>(d, q, grid) : launch_blocks<F, 4, false>(d, q, grid);
 }
 
 bool stream_accepts(const MvArgs &a, uint32_t block_bytes) {
