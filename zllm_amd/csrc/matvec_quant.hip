@@ -105,6 +105,7 @@ __device__ __forceinline__ float dot_bytes(uint32_t word, const float4 &x, float
 // no minimum, so the input sums go unused.
 struct KQ8 {
     static constexpr int NSUM = 2;
+    static constexpr int STAGE2 = 0, STAGE4 = 1;  // tokens whose inputs are loaded at once
     static constexpr bool DEFER = false;
     static const char *name() { return "matvec_q8_0"; }
     struct Raw {
@@ -161,6 +162,7 @@ struct KQ8 {
 struct KQ3 {
     static constexpr uint32_t BLOCK_BYTES = 128;
     static constexpr int NSUM = 4;
+    static constexpr int STAGE2 = 2, STAGE4 = 2;  // tokens whose inputs are loaded at once
     static constexpr bool DEFER = true;
     static const char *name() { return "matvec_q3_k"; }
     struct Raw {
@@ -233,6 +235,7 @@ struct KQ3 {
 struct KQ4 {
     static constexpr uint32_t BLOCK_BYTES = 144;
     static constexpr int NSUM = 2;
+    static constexpr int STAGE2 = 2, STAGE4 = 1;  // tokens whose inputs are loaded at once
     static constexpr bool DEFER = true;
     static const char *name() { return "matvec_q4_k"; }
     struct Raw {
@@ -296,6 +299,7 @@ struct KQ4 {
 struct KQ5 {
     static constexpr uint32_t BLOCK_BYTES = 176;
     static constexpr int NSUM = 2;
+    static constexpr int STAGE2 = 0, STAGE4 = 1;  // tokens whose inputs are loaded at once
     static constexpr bool DEFER = true;
     static const char *name() { return "matvec_q5_k"; }
     struct Raw {
@@ -365,6 +369,7 @@ struct KQ5 {
 struct KQ6 {
     static constexpr uint32_t BLOCK_BYTES = 224;
     static constexpr int NSUM = 4;
+    static constexpr int STAGE2 = 2, STAGE4 = 1;  // tokens whose inputs are loaded at once
     static constexpr bool DEFER = false;
     static const char *name() { return "matvec_q6_k"; }
     struct Raw {
@@ -473,7 +478,7 @@ template <class P, int MT, bool PAIR, bool XREG>
 __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     const MvArgs &a = q.a;
     extern __shared__ float4 lds4[];
-    __shared__ float red[4];
+    __shared__ float red[8];
     constexpr int NSUM = P::NSUM, RUN = 64 / NSUM;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t tasks = q.tasks;
@@ -529,17 +534,35 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     // are fetched. kDepth positions stay in flight ahead of the one multiplied
     // (deeper queues cost registers, hence occupancy, and measured no faster).
     constexpr int kDepth = 1;
-    // One-token steps load the token's inputs first (up to four vectors a thread: k <= 4096):
-    // loads complete in order within a wave, so behind the weights they would wait for them.
-    float4 xv[4], gv[4];
-    if (XREG) {
-        const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)q.t0 * a.xr);
-        const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
+    // Rows of up to 4096 weights: the tokens' inputs are loaded first (up to four vectors a
+    // thread and token), all of them at once: loads complete in order within a wave, so behind
+    // the weights they would wait for them, and token after token each would wait for a trip
+    // to memory of its own.
+    // How many tokens' vectors are in flight at once is the format's choice (STAGE2 for passes
+    // of two tokens, STAGE4 for passes of four; 0: none, the tokens are staged one after the
+    // other by stage_token): each token more raises the register count of the whole kernel, and
+    // past 256 the multiply loses its second wave a SIMD.
+    constexpr int STAGE = MT == 1 ? 1 : MT == 2 ? P::STAGE2 : P::STAGE4;
+    constexpr int TG = STAGE > 0 ? STAGE : 1;
+    const bool early = XREG || (STAGE > 0 && a.k <= 4096u);
+    float4 xv[TG][4], gv[4];
+    auto load_tokens = [&](int first) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < 4; j++) {
             const uint32_t i = tid + 256u * j;
-            xv[j] = i < a.k / 4u ? xrow[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-            if (a.flags & FLAG_NORM) gv[j] = i < a.k / 4u ? nw[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+            for (int t = 0; t < TG; t++) {
+                const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)(q.t0 + ((uint32_t)(first + t) < q.mt ? first + t : 0)) * a.xr);
+                xv[t][j] = i < a.k / 4u ? xrow[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            }
+        }
+    };
+    if (early) {
+        const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
+        load_tokens(0);
+        if (a.flags & FLAG_NORM) {
+#pragma unroll
+            for (int j = 0; j < 4; j++) gv[j] = tid + 256u * j < a.k / 4u ? nw[tid + 256u * j] : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
     typename P::Raw buf[kDepth + 1][kRows];
@@ -556,37 +579,59 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     float xsum[NSUM];
     // Stage the pass's tokens in task order, padded per task (coalesced loads;
     // a lane's own 64 inputs are 256 bytes apart from its neighbour's).
-    if (XREG) {
-        // The arithmetic of stage_token on the vectors already loaded, in the same order.
+    if (early) {
+        // The arithmetic of stage_token on the vectors already loaded, in the same order, the
+        // tokens' sums of squares meeting in LDS together.
         const uint32_t k4 = a.k / 4u;
-        float scale = 1.0f;
-        if (a.flags & FLAG_NORM) {
-            float ss = 0.f;
 #pragma unroll
-            for (int j = 0; j < 4; j++)
-                if (tid + 256u * j < k4) ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w;
-            ss = wave_sum(ss);
-            __syncthreads();
-            if (lane == 0) red[wave] = ss;
-            __syncthreads();
-            ss = (red[0] + red[1]) + (red[2] + red[3]);
-            scale = 1.0f / sqrtf(ss / (float)a.k + a.eps);
-        }
+        for (int first = 0; first < MT; first += TG) {
+            if (first > 0) load_tokens(first);
+            float scale[TG];
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint32_t i = tid + 256u * j;
-            if (i >= k4) continue;
-            float4 v = xv[j];
+            for (int t = 0; t < TG; t++) scale[t] = 1.0f;
             if (a.flags & FLAG_NORM) {
-                v.x = v.x * scale * gv[j].x; v.y = v.y * scale * gv[j].y;
-                v.z = v.z * scale * gv[j].z; v.w = v.w * scale * gv[j].w;
+                float ss[TG];
+#pragma unroll
+                for (int t = 0; t < TG; t++) {
+                    ss[t] = 0.f;
+#pragma unroll
+                    for (int j = 0; j < 4; j++)
+                        if (tid + 256u * j < k4) ss[t] += xv[t][j].x * xv[t][j].x + xv[t][j].y * xv[t][j].y + xv[t][j].z * xv[t][j].z + xv[t][j].w * xv[t][j].w;
+                    ss[t] = wave_sum(ss[t]);
+                }
+                __syncthreads();
+                if (lane == 0) {
+#pragma unroll
+                    for (int t = 0; t < TG; t++) red[4 * t + wave] = ss[t];
+                }
+                __syncthreads();
+#pragma unroll
+                for (int t = 0; t < TG; t++) {
+                    const float total = (red[4 * t] + red[4 * t + 1]) + (red[4 * t + 2] + red[4 * t + 3]);
+                    scale[t] = 1.0f / sqrtf(total / (float)a.k + a.eps);
+                }
             }
-            if (a.act_div > 0.f) {
-                v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
-                v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+#pragma unroll
+            for (int t = 0; t < TG; t++) {
+                float4 *dst = lds4 + (size_t)(first + t) * tok_stride4;
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint32_t i = tid + 256u * j;
+                    if (i >= k4) continue;
+                    float4 v = xv[t][j];
+                    if (a.flags & FLAG_NORM) {
+                        v.x = v.x * scale[t] * gv[j].x; v.y = v.y * scale[t] * gv[j].y;
+                        v.z = v.z * scale[t] * gv[j].z; v.w = v.w * scale[t] * gv[j].w;
+                    }
+                    if (a.act_div > 0.f) {
+                        v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
+                        v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+                    }
+                    if ((uint32_t)(first + t) >= q.mt) v = make_float4(0.f, 0.f, 0.f, 0.f);  // (a pass of fewer tokens than it has room for)
+                    const uint32_t p = P::stage_index(i);
+                    dst[p + (p >> 4)] = v;
+                }
             }
-            const uint32_t p = P::stage_index(i);
-            lds4[p + (p >> 4)] = v;
         }
     } else
     for (uint32_t t = 0; t < (uint32_t)MT; t++) {
