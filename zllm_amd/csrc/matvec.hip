@@ -29,11 +29,12 @@ namespace zhip {
 // odd ones behind them, so that each read covers consecutive vectors.
 template <class D> constexpr bool kSplitInputs = std::is_same<D, DecBF16>::value || std::is_same<D, DecF16>::value;
 
-template <class D, int MT>
+// DEPTH: positions of the 16-bit formats' walk whose loads are in flight behind the one multiplied.
+template <class D, int MT, int DEPTH>
 __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
     extern __shared__ float4 xs4[];
     float *xs = reinterpret_cast<float *>(xs4);
-    __shared__ float red[4];
+    __shared__ float red[16];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t gwave = blockIdx.x * 4u + wave, nwaves = gridDim.x * 4u;
     const bool pair = (a.flags & FLAG_SILU_PAIR) != 0;
@@ -46,22 +47,40 @@ __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
     for (uint32_t t0 = 0; t0 < a.m; t0 += MT) {
         const uint32_t mt = min((uint32_t)MT, a.m - t0);
         __syncthreads();
-        for (uint32_t t = 0; t < (uint32_t)MT; t++) {
-            float4 *dst = xs4 + (size_t)t * k4;
-            if (t >= mt) {
-                for (uint32_t i = tid; i < k4; i += 256u) dst[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-                continue;
-            }
-            if constexpr (kSplitInputs<D>) stage_token(a, t0 + t, dst, red, [k4](uint32_t i) { return (i & 1u) * (k4 / 2u) + (i >> 1); });
-            else stage_token(a, t0 + t, dst, red);
-        }
-        __syncthreads();
-
         if constexpr (kSplitInputs<D>) {
-            // The 16-bit formats: a wave walks (group, 64-task slice) positions with the next
-            // position's two 16-byte loads in flight while it multiplies the current one (past
-            // its last position the loads are clamped to a valid one and their data unused).
+            // The 16-bit formats. With rows of up to 4096 weights the pass's inputs are loaded
+            // first (up to four vectors a thread and token, four tokens at a time), then the
+            // wave's first weights, and only then are the inputs staged: the one trip to memory
+            // serves both, where staging token after token and then starting on the weights
+            // took one for every token and one more (loads complete in order within a wave).
+            // A wave walks (group, 64-task slice) positions with the loads of the next DEPTH
+            // positions in flight while it multiplies the current one (past its last position
+            // the loads are clamped to a valid one and their data unused).
+            constexpr int TG = MT < 4 ? MT : 4;
+            // (a lone token on short rows measured no faster that way: 3072 x 1024, 4.2 against 4.5 us)
+            const bool early = a.k <= 4096u && (MT > 1 || DEPTH > 1);
             const uint32_t iters = (tasks + 63u) / 64u;
+            auto place = [k4](uint32_t i) { return (i & 1u) * (k4 / 2u) + (i >> 1); };
+            float4 xv[TG][4], gv[4];
+            auto load_tokens = [&](uint32_t first) __attribute__((always_inline)) {
+#pragma unroll
+                for (int j = 0; j < 4; j++) {
+                    const uint32_t i = tid + 256u * j;
+#pragma unroll
+                    for (int t = 0; t < TG; t++) {
+                        const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)(t0 + (first + t < mt ? first + t : 0u)) * a.xr);
+                        xv[t][j] = i < k4 ? xrow[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+                    }
+                }
+            };
+            if (early) {
+                load_tokens(0);
+                if (a.flags & FLAG_NORM) {
+                    const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
+#pragma unroll
+                    for (int j = 0; j < 4; j++) gv[j] = tid + 256u * j < k4 ? nw[tid + 256u * j] : make_float4(0.f, 0.f, 0.f, 0.f);
+                }
+            }
             auto rows_of = [&](uint32_t g, uint32_t &j0, uint32_t &r1, bool &has1) {
                 j0 = pair ? g : 2u * g;
                 r1 = pair ? a.half + g : j0 + 1u;
@@ -75,80 +94,161 @@ __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
                 q0 = *reinterpret_cast<const uint4 *>(a.w + (size_t)j0 * a.row_bytes + 16u * tk);
                 q1 = *reinterpret_cast<const uint4 *>(a.w + (size_t)(has1 ? r1 : j0) * a.row_bytes + 16u * tk);
             };
+            auto advance = [&](uint32_t &g, uint32_t &it) {
+                if (++it == iters) {
+                    it = 0;
+                    g += nwaves;
+                }
+            };
+            uint4 b0[DEPTH], b1[DEPTH];
+            uint32_t lg = gwave, lit = 0;
+#pragma unroll
+            for (int s = 0; s < DEPTH; s++) {
+                load_at(lg, lit, b0[s], b1[s]);
+                advance(lg, lit);
+            }
+            if (early) {
+                // The arithmetic of stage_token on the vectors already loaded, in the same
+                // order, the tokens' sums of squares meeting in LDS together.
+#pragma unroll
+                for (int first = 0; first < MT; first += TG) {
+                    if (first > 0) load_tokens(first);
+                    float scale[TG];
+#pragma unroll
+                    for (int t = 0; t < TG; t++) scale[t] = 1.0f;
+                    if (a.flags & FLAG_NORM) {
+                        float ss[TG];
+#pragma unroll
+                        for (int t = 0; t < TG; t++) {
+                            ss[t] = 0.f;
+#pragma unroll
+                            for (int j = 0; j < 4; j++)
+                                if (tid + 256u * j < k4) ss[t] += xv[t][j].x * xv[t][j].x + xv[t][j].y * xv[t][j].y + xv[t][j].z * xv[t][j].z + xv[t][j].w * xv[t][j].w;
+                            ss[t] = wave_sum(ss[t]);
+                        }
+                        __syncthreads();
+                        if (lane == 0) {
+#pragma unroll
+                            for (int t = 0; t < TG; t++) red[4 * t + wave] = ss[t];
+                        }
+                        __syncthreads();
+#pragma unroll
+                        for (int t = 0; t < TG; t++) {
+                            const float total = (red[4 * t] + red[4 * t + 1]) + (red[4 * t + 2] + red[4 * t + 3]);
+                            scale[t] = 1.0f / sqrtf(total / (float)a.k + a.eps);
+                        }
+                    }
+#pragma unroll
+                    for (int t = 0; t < TG; t++) {
+                        float4 *dst = xs4 + (size_t)(first + t) * k4;
+#pragma unroll
+                        for (int j = 0; j < 4; j++) {
+                            const uint32_t i = tid + 256u * j;
+                            if (i >= k4) continue;
+                            float4 v = xv[t][j];
+                            if (a.flags & FLAG_NORM) {
+                                v.x = v.x * scale[t] * gv[j].x; v.y = v.y * scale[t] * gv[j].y;
+                                v.z = v.z * scale[t] * gv[j].z; v.w = v.w * scale[t] * gv[j].w;
+                            }
+                            if (a.act_div > 0.f) {
+                                v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
+                                v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+                            }
+                            if ((uint32_t)(first + t) >= mt) v = make_float4(0.f, 0.f, 0.f, 0.f);  // (a pass of fewer tokens than it has room for)
+                            dst[place(i)] = v;
+                        }
+                    }
+                }
+            } else {
+                for (uint32_t t = 0; t < (uint32_t)MT; t++) {
+                    float4 *dst = xs4 + (size_t)t * k4;
+                    if (t >= mt) {
+                        for (uint32_t i = tid; i < k4; i += 256u) dst[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                        continue;
+                    }
+                    stage_token(a, t0 + t, dst, red, place);
+                }
+            }
+            __syncthreads();
+
             float acc0[MT], acc1[MT];
 #pragma unroll
             for (int t = 0; t < MT; t++) acc0[t] = acc1[t] = 0.f;
             uint32_t g = gwave, it = 0;
-            uint4 c0, c1;
-            load_at(g, it, c0, c1);
             while (g < groups) {
-                uint32_t ng = g, nit = it + 1u;
-                if (nit == iters) {
-                    nit = 0;
-                    ng = g + nwaves;
-                }
-                uint4 n0, n1;
-                load_at(ng, nit, n0, n1);
-                const uint32_t task = lane + 64u * it;
-                if (task < tasks) {
-                    float w0[D::E], w1[D::E];
-                    D::expand(c0, w0);
-                    D::expand(c1, w1);
 #pragma unroll
-                    for (int t = 0; t < MT; t++) {
-                        const float *xt = xs + (size_t)t * a.k;
-                        float s0 = 0.f, s1 = 0.f;
+                for (int s = 0; s < DEPTH; s++) {
+                    if (g >= groups) break;
+                    const uint4 c0 = b0[s], c1 = b1[s];
+                    load_at(lg, lit, b0[s], b1[s]);
+                    advance(lg, lit);
+                    const uint32_t task = lane + 64u * it;
+                    if (task < tasks) {
+                        float w0[D::E], w1[D::E];
+                        D::expand(c0, w0);
+                        D::expand(c1, w1);
 #pragma unroll
-                        for (int h = 0; h < 2; h++) {
-                            const float4 v = *reinterpret_cast<const float4 *>(xt + 4u * ((uint32_t)h * (k4 / 2u) + task));
-                            const int b = 4 * h;
-                            s0 = fmaf(w0[b + 0], v.x, s0); s1 = fmaf(w1[b + 0], v.x, s1);
-                            s0 = fmaf(w0[b + 1], v.y, s0); s1 = fmaf(w1[b + 1], v.y, s1);
-                            s0 = fmaf(w0[b + 2], v.z, s0); s1 = fmaf(w1[b + 2], v.z, s1);
-                            s0 = fmaf(w0[b + 3], v.w, s0); s1 = fmaf(w1[b + 3], v.w, s1);
+                        for (int t = 0; t < MT; t++) {
+                            const float *xt = xs + (size_t)t * a.k;
+                            float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+                            for (int h = 0; h < 2; h++) {
+                                const float4 v = *reinterpret_cast<const float4 *>(xt + 4u * ((uint32_t)h * (k4 / 2u) + task));
+                                const int b = 4 * h;
+                                s0 = fmaf(w0[b + 0], v.x, s0); s1 = fmaf(w1[b + 0], v.x, s1);
+                                s0 = fmaf(w0[b + 1], v.y, s0); s1 = fmaf(w1[b + 1], v.y, s1);
+                                s0 = fmaf(w0[b + 2], v.z, s0); s1 = fmaf(w1[b + 2], v.z, s1);
+                                s0 = fmaf(w0[b + 3], v.w, s0); s1 = fmaf(w1[b + 3], v.w, s1);
+                            }
+                            acc0[t] += s0;
+                            acc1[t] += s1;
                         }
-                        acc0[t] += s0;
-                        acc1[t] += s1;
                     }
-                }
-                if (it + 1u == iters) {
-                    uint32_t j0, r1;
-                    bool has1;
-                    rows_of(g, j0, r1, has1);
+                    if (it + 1u == iters) {
+                        uint32_t j0, r1;
+                        bool has1;
+                        rows_of(g, j0, r1, has1);
 #pragma unroll
-                    for (int t = 0; t < MT; t++) {
-                        acc0[t] = wave_sum(acc0[t]);
-                        acc1[t] = wave_sum(acc1[t]);
-                    }
-                    if (lane == 0) {
-                        for (uint32_t t = 0; t < mt; t++) {
-                            const size_t o = (size_t)(t0 + t) * a.out_stride + a.col0 + j0;
-                            if (pair) {
-                                float v = silu_f(acc0[t]) * acc1[t];
-                                if (a.flags & FLAG_ACCUMULATE) v += a.out[o];
-                                a.out[o] = v;
-                            } else {
-                                float v = acc0[t];
-                                if (a.flags & FLAG_ACCUMULATE) v += a.out[o];
-                                a.out[o] = v;
-                                if (has1) {
-                                    float u = acc1[t];
-                                    if (a.flags & FLAG_ACCUMULATE) u += a.out[o + 1];
-                                    a.out[o + 1] = u;
+                        for (int t = 0; t < MT; t++) {
+                            acc0[t] = wave_sum(acc0[t]);
+                            acc1[t] = wave_sum(acc1[t]);
+                        }
+                        if (lane == 0) {
+                            for (uint32_t t = 0; t < mt; t++) {
+                                const size_t o = (size_t)(t0 + t) * a.out_stride + a.col0 + j0;
+                                if (pair) {
+                                    float v = silu_f(acc0[t]) * acc1[t];
+                                    if (a.flags & FLAG_ACCUMULATE) v += a.out[o];
+                                    a.out[o] = v;
+                                } else {
+                                    float v = acc0[t];
+                                    if (a.flags & FLAG_ACCUMULATE) v += a.out[o];
+                                    a.out[o] = v;
+                                    if (has1) {
+                                        float u = acc1[t];
+                                        if (a.flags & FLAG_ACCUMULATE) u += a.out[o + 1];
+                                        a.out[o + 1] = u;
+                                    }
                                 }
                             }
                         }
-                    }
 #pragma unroll
-                    for (int t = 0; t < MT; t++) acc0[t] = acc1[t] = 0.f;
+                        for (int t = 0; t < MT; t++) acc0[t] = acc1[t] = 0.f;
+                    }
+                    advance(g, it);
                 }
-                c0 = n0;
-                c1 = n1;
-                g = ng;
-                it = nit;
             }
             continue;
         }
+        for (uint32_t t = 0; t < (uint32_t)MT; t++) {
+            float4 *dst = xs4 + (size_t)t * k4;
+            if (t >= mt) {
+                for (uint32_t i = tid; i < k4; i += 256u) dst[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+                continue;
+            }
+            stage_token(a, t0 + t, dst, red);
+        }
+        __syncthreads();
         for (uint32_t g = gwave; g < groups; g += nwaves) {
             // The group's two weight rows and whether each exists.
             const uint32_t j0 = pair ? g : 2u * g;
@@ -249,14 +349,18 @@ __global__ __launch_bounds__(256) void matvec_prologue_kernel(MvArgs a, float4 *
 
 template <class D, int MT>
 static zhip_result run(const Dispatch &d, const MvArgs &a, uint32_t lds_bytes) {
-    static int configured_device = -1;  // dynamic LDS above 64 KiB needs opting in once
-    auto kernel = matvec_kernel<D, MT>;
-    if (lds_bytes > 65536u && configured_device != 1) {
+    static bool configured[2] = {false, false};  // dynamic LDS above 64 KiB needs opting in once, kernel by kernel
+    // Long rows of a matrix of few rows: a wave has few positions, each a trip to memory; four
+    // in flight instead of one (1024 x 3072 bf16, one token: 6.3 -> 5.1 us). Elsewhere the
+    // registers that takes cost more than it gains (151936 x 1024: 52 -> 62 us).
+    const bool deep = kSplitInputs<D> && a.k >= 2048u && (uint64_t)a.rows * a.row_bytes <= (64ull << 20);
+    auto kernel = deep ? matvec_kernel<D, MT, kSplitInputs<D> ? 4 : 1> : matvec_kernel<D, MT, 1>;
+    if (lds_bytes > 65536u && !configured[deep]) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
             (void)hipGetLastError();
             return fail(d, ZHIP_E_BAD_COMMAND, "decode multiply: k = %u with %d tokens does not fit workgroup memory", a.k, MT);
         }
-        configured_device = 1;
+        configured[deep] = true;
     }
     const uint32_t per_group = (a.flags & FLAG_SILU_PAIR) ? 1u : 2u;
     const uint32_t groups = (a.rows + per_group - 1u) / per_group;
@@ -265,7 +369,7 @@ static zhip_result run(const Dispatch &d, const MvArgs &a, uint32_t lds_bytes) {
     // one's traffic, enough of them to keep every CU's SIMDs busy.
     const uint32_t cap = (uint32_t)d.dev->compute_units * (lds_bytes > 32768u ? 2u : 4u);
     const uint32_t blocks = want < cap ? want : cap;
-    hipLaunchKernelGGL((matvec_kernel<D, MT>), dim3(blocks ? blocks : 1), dim3(256), lds_bytes, d.stream, a);
+    hipLaunchKernelGGL(kernel, dim3(blocks ? blocks : 1), dim3(256), lds_bytes, d.stream, a);
     return check_launch(d, D::name());
 }
 
