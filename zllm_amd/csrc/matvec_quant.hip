@@ -474,7 +474,8 @@ struct KArgs {
     uint32_t defer;     // finished rows' outputs wait in registers for one store at the end of the wave's walk
 };
 
-template <class P, int MT, bool PAIR, bool XREG>
+// STG: tokens whose inputs are loaded at once ahead of the weights (0: none, staged by stage_token).
+template <class P, int MT, bool PAIR, bool XREG, int STG>
 __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     const MvArgs &a = q.a;
     extern __shared__ float4 lds4[];
@@ -538,13 +539,11 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     // thread and token), all of them at once: loads complete in order within a wave, so behind
     // the weights they would wait for them, and token after token each would wait for a trip
     // to memory of its own.
-    // How many tokens' vectors are in flight at once is the format's choice (STAGE2 for passes
-    // of two tokens, STAGE4 for passes of four; 0: none, the tokens are staged one after the
-    // other by stage_token): each token more raises the register count of the whole kernel, and
-    // past 256 the multiply loses its second wave a SIMD.
-    constexpr int STAGE = MT == 1 ? 1 : MT == 2 ? P::STAGE2 : P::STAGE4;
-    constexpr int TG = STAGE > 0 ? STAGE : 1;
-    const bool early = XREG || (STAGE > 0 && a.k <= 4096u);
+    // How many tokens' vectors are in flight at once (STG) is the launch's choice: each token
+    // more raises the register count of the whole kernel, and past 256 the multiply loses its
+    // second wave a SIMD, which a large matrix pays for and a small one does not.
+    constexpr int TG = STG > 0 ? STG : 1;
+    const bool early = XREG || (STG > 0 && a.k <= 4096u);
     float4 xv[TG][4], gv[4];
     auto load_tokens = [&](int first) __attribute__((always_inline)) {
 #pragma unroll
@@ -768,17 +767,17 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     if (P::DEFER && XREG && q.defer) flush_kept();
 }
 
-template <class P, int MT, bool PAIR, bool XREG>
+template <class P, int MT, bool PAIR, bool XREG, int STG>
 static zhip_result run_quant(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
     static bool configured = false;  // dynamic LDS above 64 KiB needs opting in once
     if (lds > 65536u && !configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_quant_kernel<P, MT, PAIR, XREG>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_quant_kernel<P, MT, PAIR, XREG, STG>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
             (void)hipGetLastError();
             return fail(d, ZHIP_E_BAD_COMMAND, "%s: k = %u with %d tokens does not fit workgroup memory", P::name(), q.a.k, MT);
         }
         configured = true;
     }
-    hipLaunchKernelGGL((matvec_quant_kernel<P, MT, PAIR, XREG>), dim3(blocks), dim3(256), lds, d.stream, q);
+    hipLaunchKernelGGL((matvec_quant_kernel<P, MT, PAIR, XREG, STG>), dim3(blocks), dim3(256), lds, d.stream, q);
     return check_launch(d, P::name());
 }
 
@@ -814,10 +813,18 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
         const uint32_t blocks = want < cap ? want : cap;
         q.defer = (P::DEFER && xreg && q.seg_log2 == 6u) ? 1u : 0u;
         zhip_result r;
-        if (xreg) r = pair ? run_quant<P, 1, true, true>(d, q, lds, blocks) : run_quant<P, 1, false, true>(d, q, lds, blocks);
-        else if (mt == 1u) r = pair ? run_quant<P, 1, true, false>(d, q, lds, blocks) : run_quant<P, 1, false, false>(d, q, lds, blocks);
-        else if (mt == 2u) r = pair ? run_quant<P, 2, true, false>(d, q, lds, blocks) : run_quant<P, 2, false, false>(d, q, lds, blocks);
-        else r = pair ? run_quant<P, 4, true, false>(d, q, lds, blocks) : run_quant<P, 4, false, false>(d, q, lds, blocks);
+        // A small matrix's launch is a chain of trips to memory, and all of the pass's tokens go
+        // in one; a large one keeps what the format's registers allow (STAGE2, STAGE4).
+        const bool small = (uint64_t)a.rows * a.row_bytes <= (16ull << 20);
+        if (xreg) r = pair ? run_quant<P, 1, true, true, 1>(d, q, lds, blocks) : run_quant<P, 1, false, true, 1>(d, q, lds, blocks);
+        else if (mt == 1u) r = pair ? run_quant<P, 1, true, false, 1>(d, q, lds, blocks) : run_quant<P, 1, false, false, 1>(d, q, lds, blocks);
+        else if (mt == 2u) {
+            if (small && P::STAGE2 != 2) r = pair ? run_quant<P, 2, true, false, 2>(d, q, lds, blocks) : run_quant<P, 2, false, false, 2>(d, q, lds, blocks);
+            else r = pair ? run_quant<P, 2, true, false, P::STAGE2>(d, q, lds, blocks) : run_quant<P, 2, false, false, P::STAGE2>(d, q, lds, blocks);
+        } else {
+            if (small && P::STAGE4 != 4) r = pair ? run_quant<P, 4, true, false, 4>(d, q, lds, blocks) : run_quant<P, 4, false, false, 4>(d, q, lds, blocks);
+            else r = pair ? run_quant<P, 4, true, false, P::STAGE4>(d, q, lds, blocks) : run_quant<P, 4, false, false, P::STAGE4>(d, q, lds, blocks);
+        }
         if (r != ZHIP_OK) return r;
         t0 += q.mt;
     }
