@@ -770,49 +770,59 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
 // Steps of several tokens over rows too long for the tokens' inputs to fit the workgroup's LDS
 // together (k above ~4800 for four tokens, ~9600 for two; the FFN-down shapes): the kernel
 // above would take such a step token by token, reading the weights once for each. Here a
-// workgroup takes a batch of rows (B units a wave) through the row tile by tile, a tile being
-// the 64 tasks of one step of the lanes' walk (4096 weights): the tile's inputs of all the pass's
-// tokens are staged, every wave multiplies its rows' slice of the tile, and the sums stay in
-// registers until the row ends. A lane adds its tasks in the order of the kernel above, and a
-// task's dot product and the lanes' reduction are the same code: the same bits. The inputs are
-// staged once a batch (from L2: 4 B x k x tokens for 8 B rows), the weights are read once.
-template <class P, int MT, bool PAIR, int B>
-__global__ __launch_bounds__(256) void matvec_quant_long_kernel(KArgs q) {
+// workgroup of eight waves takes a batch of rows (a unit a wave) through the row tile by tile,
+// a tile being the 64 tasks of one step of the lanes' walk (4096 weights): the tile's inputs of
+// all the pass's tokens are staged, every wave multiplies its rows' slice of the tile, and the
+// sums stay in registers until the row ends. The next tile's inputs and weights are asked for
+// before the current tile is multiplied: the weights wait in registers, the inputs land in LDS
+// as they are (wave-wide direct loads: no registers, which the multiply has none to spare) and
+// are normalised, activated and put in task order from there. A lane adds its tasks in the
+// order of the kernel above, and a task's dot product and the lanes' reduction are the same
+// code: the same bits. The inputs are staged once a batch (from L2: 4 B x k x tokens for
+// sixteen rows), the weights are read once.
+typedef __attribute__((address_space(3))) void *long_lds_ptr;
+template <class P, int MT, bool PAIR>
+__global__ __launch_bounds__(512) void matvec_quant_long_kernel(KArgs q) {
     const MvArgs &a = q.a;
-    extern __shared__ float4 lds4[];
+    extern __shared__ float4 lds4[];  // [token][tile in task order, padded]; the runs' sums; [token][tile as loaded]
     __shared__ float red[4 * MT];
     constexpr int NSUM = P::NSUM, RUN = 64 / NSUM, kRows = 2;
     constexpr uint32_t tile4 = 64u * (kTaskStride / 4u);  // float4s of one token's tile
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t tasks = q.tasks, k4 = a.k / 4u, tiles = (tasks + 63u) / 64u;
     float *sums_lds = reinterpret_cast<float *>(lds4 + (size_t)MT * tile4);  // [token][task of the tile][run]
+    float4 *raw4 = lds4 + (size_t)MT * tile4 + MT * 16u * NSUM;              // [token][1024 vectors]
     const Masks nm = q.nm;
     const uint32_t per_unit = PAIR ? 1u : 2u;
     const uint32_t units = (a.rows + per_unit - 1u) / per_unit;
-    const uint32_t batches = (units + 4u * B - 1u) / (4u * B);
+    const uint32_t batches = (units + 7u) / 8u;
     const bool norm = (a.flags & FLAG_NORM) != 0;
+    const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
 
-    // The RMSNorm prologue's scales (src/kernels/matvec_quant.wgsl.hbs:73-89), summed as stage_token sums them.
+    // The RMSNorm prologue's scales (src/kernels/matvec_quant.wgsl.hbs:73-89), summed as
+    // stage_token sums them: by 256 threads, vector i to thread i % 256, four waves.
     float scale[MT];
 #pragma unroll
     for (int t = 0; t < MT; t++) scale[t] = 1.0f;
     if (norm) {
-        float ss[MT];
+        if (tid < 256u) {
+            float ss[MT];
 #pragma unroll
-        for (int t = 0; t < MT; t++) {
-            ss[t] = 0.f;
-            if ((uint32_t)t < q.mt) {
-                const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)(q.t0 + t) * a.xr);
-                for (uint32_t i = tid; i < k4; i += 256u) {
-                    const float4 v = xrow[i];
-                    ss[t] += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+            for (int t = 0; t < MT; t++) {
+                ss[t] = 0.f;
+                if ((uint32_t)t < q.mt) {
+                    const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)(q.t0 + t) * a.xr);
+                    for (uint32_t i = tid; i < k4; i += 256u) {
+                        const float4 v = xrow[i];
+                        ss[t] += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                    }
                 }
+                ss[t] = wave_sum(ss[t]);
             }
-            ss[t] = wave_sum(ss[t]);
-        }
-        if (lane == 0) {
+            if (lane == 0) {
 #pragma unroll
-            for (int t = 0; t < MT; t++) red[4 * t + wave] = ss[t];
+                for (int t = 0; t < MT; t++) red[4 * t + wave] = ss[t];
+            }
         }
         __syncthreads();
 #pragma unroll
@@ -822,119 +832,129 @@ __global__ __launch_bounds__(256) void matvec_quant_long_kernel(KArgs q) {
         }
     }
 
-    for (uint32_t batch = blockIdx.x; batch < batches; batch += gridDim.x) {
-        // The wave's units: outputs j0 (and j0 + 1), or the gate row j0 and the up row half +
-        // j0. Units and rows past the end are clamped for the loads and skipped at the store.
-        uint32_t j0[B], ra[B], rb[B];
-        bool there[B];
+    // A tile's inputs: two vectors a thread and token, from memory straight into LDS (a wave's
+    // load lands 64 consecutive vectors; vectors past the row's end land as zeros) ...
+    const uint32_t raw0 = (uint32_t)(uintptr_t)raw4;
+    auto fetch_inputs = [&](uint32_t i) __attribute__((always_inline)) {
 #pragma unroll
-        for (int b = 0; b < B; b++) {
-            const uint32_t unit = (batch * 4u + wave) * B + b;
-            there[b] = unit < units;
-            const uint32_t u = there[b] ? unit : units - 1u;
-            j0[b] = PAIR ? u : 2u * u;
-            ra[b] = j0[b];
-            rb[b] = PAIR ? a.half + j0[b] : (j0[b] + 1u < a.rows ? j0[b] + 1u : j0[b]);
+        for (int t = 0; t < MT; t++) {
+            const float *xrow = a.x + (size_t)(q.t0 + ((uint32_t)t < q.mt ? t : 0)) * a.xr;
+            const __amdgpu_buffer_rsrc_t xbuf = __builtin_amdgcn_make_buffer_rsrc(const_cast<float *>(xrow), 0, (int)(a.k * 4u), 0x00020000);
+#pragma unroll
+            for (int j = 0; j < 2; j++) {
+                uint32_t dst = raw0 + 16u * ((uint32_t)t * 1024u + 512u * j + 64u * __builtin_amdgcn_readfirstlane(wave));
+                asm volatile("" : "+s"(dst));
+                __builtin_amdgcn_raw_ptr_buffer_load_lds(xbuf, (long_lds_ptr)(uintptr_t)dst, 16, 16u * (1024u * i + tid + 512u * j), 0, 0, 0);
+            }
         }
-        float acc[B][kRows][MT];
+    };
+    // ... and, normalised and activated as the step asks, into LDS in task order, padded per
+    // task as above; then the runs' input sums, added in the order of the kernel above.
+    auto stage_inputs = [&](uint32_t i) __attribute__((always_inline)) {
 #pragma unroll
-        for (int b = 0; b < B; b++)
+        for (int t = 0; t < MT; t++) {
 #pragma unroll
-            for (int j = 0; j < kRows; j++)
-#pragma unroll
-                for (int t = 0; t < MT; t++) acc[b][j][t] = 0.f;
-        typename P::Raw cur[B][kRows], next[B][kRows];
-        auto load_tile = [&](uint32_t i, typename P::Raw (&dst)[B][kRows]) __attribute__((always_inline)) {
-            const uint32_t task = lane + 64u * i, tk = task < tasks ? task : 0u;
-#pragma unroll
-            for (int b = 0; b < B; b++) {
-                dst[b][0] = P::load(a.w + (size_t)ra[b] * a.row_bytes, a.k, tk);
-                dst[b][1] = P::load(a.w + (size_t)rb[b] * a.row_bytes, a.k, tk);
-            }
-        };
-        load_tile(0, cur);
-        for (uint32_t i = 0; i < tiles; i++) {
-            __syncthreads();  // nobody still reads the tile before
-            // The tile's inputs of every token, in task order and padded per task as above.
-#pragma unroll
-            for (int t = 0; t < MT; t++) {
-                const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)(q.t0 + ((uint32_t)t < q.mt ? t : 0)) * a.xr);
-                const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
-#pragma unroll
-                for (int j = 0; j < 4; j++) {
-                    const uint32_t gi = 1024u * i + tid + 256u * j;
-                    if (gi >= k4) continue;
-                    float4 v = xrow[gi];
-                    if (norm) {
-                        const float4 g = nw[gi];
-                        v.x = v.x * scale[t] * g.x; v.y = v.y * scale[t] * g.y;
-                        v.z = v.z * scale[t] * g.z; v.w = v.w * scale[t] * g.w;
-                    }
-                    if (a.act_div > 0.f) {
-                        v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
-                        v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
-                    }
-                    if ((uint32_t)t >= q.mt) v = make_float4(0.f, 0.f, 0.f, 0.f);  // (a pass of fewer tokens than it has room for)
-                    const uint32_t p = P::stage_index(gi) - 1024u * i;
-                    lds4[(size_t)t * tile4 + p + (p >> 4)] = v;
+            for (int j = 0; j < 2; j++) {
+                const uint32_t gi = 1024u * i + tid + 512u * j;
+                if (gi >= k4) continue;
+                float4 v = raw4[(size_t)t * 1024u + tid + 512u * j];
+                if (norm) {
+                    const float4 g = nw[gi];
+                    v.x = v.x * scale[t] * g.x; v.y = v.y * scale[t] * g.y;
+                    v.z = v.z * scale[t] * g.z; v.w = v.w * scale[t] * g.w;
                 }
+                if (a.act_div > 0.f) {
+                    v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
+                    v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+                }
+                if ((uint32_t)t >= q.mt) v = make_float4(0.f, 0.f, 0.f, 0.f);  // (a pass of fewer tokens than it has room for)
+                const uint32_t p = P::stage_index(gi) - 1024u * i;
+                lds4[(size_t)t * tile4 + p + (p >> 4)] = v;
             }
-            __syncthreads();
-            // The runs' input sums, added in the order of the kernel above.
-            const uint32_t live = tasks - 64u * i < 64u ? tasks - 64u * i : 64u;  // tasks of this tile
-            for (uint32_t idx = tid; idx < (uint32_t)MT * 64u * NSUM; idx += 256u) {
-                const uint32_t t = idx / (64u * NSUM), rem = idx % (64u * NSUM);
-                if (rem / NSUM >= live) continue;
-                const float *src = reinterpret_cast<const float *>(lds4 + (size_t)t * tile4) + (rem / NSUM) * kTaskStride + (rem % NSUM) * RUN;
-                float sum = 0.f;
+        }
+        __syncthreads();
+        const uint32_t live = tasks - 64u * i < 64u ? tasks - 64u * i : 64u;  // tasks of this tile
+        for (uint32_t idx = tid; idx < (uint32_t)MT * 64u * NSUM; idx += 512u) {
+            const uint32_t t = idx / (64u * NSUM), rem = idx % (64u * NSUM);
+            if (rem / NSUM >= live) continue;
+            const float *src = reinterpret_cast<const float *>(lds4 + (size_t)t * tile4) + (rem / NSUM) * kTaskStride + (rem % NSUM) * RUN;
+            float sum = 0.f;
 #pragma unroll
-                for (int e = 0; e < RUN; e++) sum += src[e];
-                sums_lds[idx] = sum;
+            for (int e = 0; e < RUN; e++) sum += src[e];
+            sums_lds[idx] = sum;
+        }
+        __syncthreads();
+    };
+
+    for (uint32_t batch = blockIdx.x; batch < batches; batch += gridDim.x) {
+        // The wave's unit: outputs j0 (and j0 + 1), or the gate row j0 and the up row half + j0.
+        // A unit or row past the end is clamped for the loads and skipped at the store.
+        const uint32_t unit = batch * 8u + wave;
+        const bool there = unit < units;
+        const uint32_t u = there ? unit : units - 1u;
+        const uint32_t j0 = PAIR ? u : 2u * u;
+        const uint32_t ra = j0, rb = PAIR ? a.half + j0 : (j0 + 1u < a.rows ? j0 + 1u : j0);
+        float acc[kRows][MT];
+#pragma unroll
+        for (int j = 0; j < kRows; j++)
+#pragma unroll
+            for (int t = 0; t < MT; t++) acc[j][t] = 0.f;
+        typename P::Raw cur[kRows], next[kRows];
+        auto load_tile = [&](uint32_t i, typename P::Raw (&dst)[kRows]) __attribute__((always_inline)) {
+            const uint32_t task = lane + 64u * i, tk = task < tasks ? task : 0u;
+            dst[0] = P::load(a.w + (size_t)ra * a.row_bytes, a.k, tk);
+            dst[1] = P::load(a.w + (size_t)rb * a.row_bytes, a.k, tk);
+        };
+        __syncthreads();  // nobody still reads the batch before's last tile
+        fetch_inputs(0);
+        load_tile(0, cur);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();  // every wave's part of the tile has landed
+        stage_inputs(0);
+        for (uint32_t i = 0; i < tiles; i++) {
+            const bool more = i + 1u < tiles;
+            if (more) {
+                fetch_inputs(i + 1u);
+                load_tile(i + 1u, next);
             }
-            __syncthreads();
-            if (i + 1u < tiles) load_tile(i + 1u, next);
             const uint32_t task = lane + 64u * i;
             if (task < tasks) {
                 const float4 *xt = lds4 + lane * (kTaskStride / 4u);
                 const float *st = sums_lds + NSUM * lane;
+                float v[kRows][MT];
+                P::template dot<MT, kRows>(cur, task & 3u, nm,
+                    [&](int t, int vi) { return xt[(size_t)t * tile4 + vi]; },
+                    [&](int t, int sr) { return st[(size_t)t * 64u * NSUM + sr]; }, v);
 #pragma unroll
-                for (int b = 0; b < B; b++) {
-                    float v[kRows][MT];
-                    P::template dot<MT, kRows>(cur[b], task & 3u, nm,
-                        [&](int t, int vi) { return xt[(size_t)t * tile4 + vi]; },
-                        [&](int t, int sr) { return st[(size_t)t * 64u * NSUM + sr]; }, v);
+                for (int j = 0; j < kRows; j++)
 #pragma unroll
-                    for (int j = 0; j < kRows; j++)
-#pragma unroll
-                        for (int t = 0; t < MT; t++) acc[b][j][t] += v[j][t];
-                }
+                    for (int t = 0; t < MT; t++) acc[j][t] += v[j][t];
             }
-#pragma unroll
-            for (int b = 0; b < B; b++) {
-                cur[b][0] = next[b][0];
-                cur[b][1] = next[b][1];
+            if (more) {
+                asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+                __syncthreads();  // nobody still reads this tile, and every wave's part of the next has landed
+                stage_inputs(i + 1u);
+                cur[0] = next[0];
+                cur[1] = next[1];
             }
         }
 #pragma unroll
-        for (int b = 0; b < B; b++) {
-#pragma unroll
-            for (int t = 0; t < MT; t++) {
-                const float s0 = segment_sum(acc[b][0][t], 6u), s1 = segment_sum(acc[b][1][t], 6u);
-                if (lane == 63u && there[b] && (uint32_t)t < q.mt && j0[b] < a.rows) {
-                    const size_t o = (size_t)(q.t0 + t) * a.out_stride + a.col0 + j0[b];
-                    if (PAIR) {
-                        float r = silu_f(s0) * s1;
-                        if (a.flags & FLAG_ACCUMULATE) r += a.out[o];
-                        a.out[o] = r;
-                    } else {
-                        float r = s0;
-                        if (a.flags & FLAG_ACCUMULATE) r += a.out[o];
-                        a.out[o] = r;
-                        if (j0[b] + 1u < a.rows) {
-                            float r1 = s1;
-                            if (a.flags & FLAG_ACCUMULATE) r1 += a.out[o + 1];
-                            a.out[o + 1] = r1;
-                        }
+        for (int t = 0; t < MT; t++) {
+            const float s0 = segment_sum(acc[0][t], 6u), s1 = segment_sum(acc[1][t], 6u);
+            if (lane == 63u && there && (uint32_t)t < q.mt && j0 < a.rows) {
+                const size_t o = (size_t)(q.t0 + t) * a.out_stride + a.col0 + j0;
+                if (PAIR) {
+                    float r = silu_f(s0) * s1;
+                    if (a.flags & FLAG_ACCUMULATE) r += a.out[o];
+                    a.out[o] = r;
+                } else {
+                    float r = s0;
+                    if (a.flags & FLAG_ACCUMULATE) r += a.out[o];
+                    a.out[o] = r;
+                    if (j0 + 1u < a.rows) {
+                        float r1 = s1;
+                        if (a.flags & FLAG_ACCUMULATE) r1 += a.out[o + 1];
+                        a.out[o + 1] = r1;
                     }
                 }
             }
@@ -942,18 +962,18 @@ __global__ __launch_bounds__(256) void matvec_quant_long_kernel(KArgs q) {
     }
 }
 
-template <class P, int MT, bool PAIR, int B>
+template <class P, int MT, bool PAIR>
 static zhip_result run_long(const Dispatch &d, const KArgs &q, uint32_t blocks) {
-    constexpr uint32_t lds = MT * 64u * kTaskStride * 4u + MT * 64u * P::NSUM * 4u;
+    constexpr uint32_t lds = MT * 64u * kTaskStride * 4u + MT * 64u * P::NSUM * 4u + MT * 16384u;
     static bool configured = false;  // dynamic LDS above 64 KiB needs opting in once
     if (lds > 65536u && !configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_quant_long_kernel<P, MT, PAIR, B>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_quant_long_kernel<P, MT, PAIR>), hipFuncAttributeMaxDynamicSharedMemorySize, lds) != hipSuccess) {
             (void)hipGetLastError();
             return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", P::name(), lds);
         }
         configured = true;
     }
-    hipLaunchKernelGGL((matvec_quant_long_kernel<P, MT, PAIR, B>), dim3(blocks), dim3(256), lds, d.stream, q);
+    hipLaunchKernelGGL((matvec_quant_long_kernel<P, MT, PAIR>), dim3(blocks), dim3(512), lds, d.stream, q);
     return check_launch(d, P::name());
 }
 
@@ -996,12 +1016,12 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
             q.mt = left < mt ? left : mt;
             const uint32_t units = pair ? a.rows : (a.rows + 1u) / 2u;
             const uint32_t cus = (uint32_t)d.dev->compute_units;
-            // (a unit a wave: two at once take more than the 256 registers that leave a SIMD two waves)
-            const uint32_t batches = (units + 3u) / 4u;
-            const uint32_t blocks = batches < 2u * cus ? batches : 2u * cus;
+            // (a workgroup of eight waves a CU: its registers leave room for no second one)
+            const uint32_t batches = (units + 7u) / 8u;
+            const uint32_t blocks = batches < cus ? batches : cus;
             zhip_result r;
-            if (mt == 2u) r = pair ? run_long<P, 2, true, 1>(d, q, blocks) : run_long<P, 2, false, 1>(d, q, blocks);
-            else r = pair ? run_long<P, 4, true, 1>(d, q, blocks) : run_long<P, 4, false, 1>(d, q, blocks);
+            if (mt == 2u) r = pair ? run_long<P, 2, true>(d, q, blocks) : run_long<P, 2, false>(d, q, blocks);
+            else r = pair ? run_long<P, 4, true>(d, q, blocks) : run_long<P, 4, false>(d, q, blocks);
             if (r != ZHIP_OK) return r;
             t0 += q.mt;
             continue;
