@@ -84,7 +84,6 @@ struct MfmaArgs {
     uint32_t row_bytes;
     uint32_t x_bytes, w_bytes;  // bytes the kernel may read behind x and w
     uint32_t x_plane;           // compensated rung: bytes from the activations' f16 values to their residuals
-    const float *token_scale;   // decode variant: what each token's sums are multiplied by at the end, or null
 };
 
 // Two floats to packed bf16, round to nearest even as the reference narrows
@@ -442,7 +441,6 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_kernel(MfmaArgs a) {
                 f32x4 v = (p[0] + p[2]) + (p[1] + p[3]);
                 const uint32_t col = j0 + 32u * wn + 16u * j + 4u * g;
                 if (t >= a.rows || col >= a.n) continue;
-                if (a.token_scale) v *= a.token_scale[t];
                 float *o = a.out + (size_t)z * a.slice_stride + (size_t)t * a.out_stride + a.col0 + col;
                 if (aligned && col + 3u < a.n) {
                     f32x4 *o4 = reinterpret_cast<f32x4 *>(o);
@@ -494,38 +492,6 @@ __global__ __launch_bounds__(256) void narrow_split_kernel(const f32x4 *src, u32
         }
         hi_out[i] = hi;
         lo_out[i] = lo;
-    }
-}
-
-// The decode variant's activations: one workgroup a token. The token is scaled by a power of
-// two that brings its largest magnitude to [2^13, 2^14) (exact, and no value leaves the f16
-// range whatever the token's scale), then split like the compensated rung's; the inverse power
-// goes to scale_out[token] and multiplies the token's sums at the end.
-__global__ __launch_bounds__(256) void narrow_split_scaled_kernel(const float *x, uint32_t x_stride, uint32_t k, uint16_t *hi_out, uint16_t *lo_out, float *scale_out) {
-    __shared__ float red[4];
-    const uint32_t t = blockIdx.x, tid = threadIdx.x;
-    const float *row = x + (size_t)t * x_stride;
-    float big = 0.f;
-    for (uint32_t i = tid; i < k; i += 256u) big = fmaxf(big, fabsf(row[i]));
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) big = fmaxf(big, __shfl_xor(big, o));
-    if ((tid & 63u) == 0u) red[tid >> 6] = big;
-    __syncthreads();
-    big = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    int e = 0;
-    if (big > 0.f && big < __builtin_inff()) {
-        int ex;
-        (void)frexpf(big, &ex);  // big = m 2^ex, m in [0.5, 1)
-        e = 14 - ex;
-        e = e > 100 ? 100 : e < -100 ? -100 : e;
-    }
-    const float up = ldexpf(1.0f, e);
-    if (tid == 0) scale_out[t] = ldexpf(1.0f, -e);
-    for (uint32_t i = tid; i < k; i += 256u) {
-        const float v = row[i] * up;
-        const _Float16 h = (_Float16)v;
-        hi_out[(size_t)t * k + i] = __builtin_bit_cast(uint16_t, h);
-        lo_out[(size_t)t * k + i] = __builtin_bit_cast(uint16_t, (_Float16)__fsub_rn(v, (float)h));
     }
 }
 
@@ -654,36 +620,5 @@ zhip_result launch_matmul_q8_0_float_f16(const Dispatch &d) { return launch_mfma
 zhip_result launch_matmul_bf16_f16c(const Dispatch &d) { return launch_mfma<WBf16, false, F16, true>(d, "matmul_bf16", false, false); }
 zhip_result launch_matmul_f16_f16c(const Dispatch &d) { return launch_mfma<WF16, false, F16, true>(d, "matmul_f16", false, false); }
 zhip_result launch_matmul_q8_0_float_f16c(const Dispatch &d) { return launch_mfma<WQ8_0, false, F16, true>(d, "matmul_q8_0_float", true, true); }
-
-// The matrix-core variant of matvec_q8_0 for steps of several tokens (a speculative verify
-// step): the compensated arithmetic above on tiles of 32 tokens, every token scaled by its own
-// power of two first, so that the per-weight work is done once for all tokens of the step.
-// Validated arguments; no NORM / activation prologue and no SiLU pair (matvec.hip routes those
-// to the default kernel).
-zhip_result launch_matvec_q8_0_mfma(const Dispatch &d, const MvArgs &v) {
-    const char *name = "matvec_q8_0";
-    MfmaArgs a{};
-    a.rows = v.m; a.n = v.rows; a.k = v.k; a.col0 = v.col0; a.out_stride = v.out_stride;
-    a.accumulate = (v.flags & FLAG_ACCUMULATE) ? 1u : 0u;
-    a.k_slice = v.k;
-    a.row_bytes = v.row_bytes;
-    a.w = v.w;
-    a.out = v.out;
-    const uint64_t x_bytes = (uint64_t)v.m * v.k * 2u, w_bytes = (uint64_t)v.rows * v.row_bytes;
-    const uint64_t plane = (x_bytes + 255u) & ~(uint64_t)255u;
-    if (2u * plane >= (1ull << 32) || w_bytes >= (1ull << 32)) return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
-    if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", name);
-    if (zhip_result r = d.work->reserve(d, 2u * plane + (uint64_t)v.m * 4u)) return r;
-    float *scales = reinterpret_cast<float *>(d.work->data + 2u * plane);
-    hipLaunchKernelGGL(narrow_split_scaled_kernel, dim3(v.m), dim3(256), 0, d.stream, v.x, v.xr, v.k,
-        reinterpret_cast<uint16_t *>(d.work->data), reinterpret_cast<uint16_t *>(d.work->data + plane), scales);
-    a.x = d.work->data;
-    a.x_plane = (uint32_t)plane;
-    a.x_bytes = (uint32_t)(plane + x_bytes);
-    a.w_bytes = (uint32_t)w_bytes;
-    a.token_scale = scales;
-    const bool ragged = a.k % BK != 0;
-    return ragged ? launch_kernel<WQ8_0, F16, 2, true, true>(d, name, a, 1u) : launch_kernel<WQ8_0, F16, 2, false, true>(d, name, a, 1u);
-}
 
 }  // namespace zhip

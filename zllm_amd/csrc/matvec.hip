@@ -313,9 +313,6 @@ __global__ __launch_bounds__(256) void matvec_kernel(MvArgs a) {
     }
 }
 
-// The matrix-core variant of matvec_q4_k (matvec_mfma.hip).
-bool matvec_q4k_mfma_accepts(const MvArgs &a);
-zhip_result launch_matvec_q4k_mfma(const Dispatch &d, const MvArgs &a, uint64_t x_bytes, uint64_t w_bytes);
 bool matvec_q4k_mfma_resident_accepts(const MvArgs &a);
 zhip_result launch_matvec_q4k_mfma_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
 // The matrix-core variant of matvec_q8_0 for k of 2048 or 4096 (matvec_q8_mfma_stream.hip).
@@ -335,17 +332,8 @@ zhip_result launch_matvec_q3k_mfma_stream(const Dispatch &d, const MvArgs &a, ui
 // workgroup's first tile) outweigh the general kernel's per-token work at two to four tokens
 // (8 MB, k = 1024: 6.4 / 6.8 / 7.8 us at 2 / 4 / 8 tokens against 4.7 / 6.2 / 9.3).
 constexpr uint64_t kBf16StreamBytes = 16ull << 20;
-// The matrix-core variant of matvec_q8_0 (matmul_mfma.hip).
-zhip_result launch_matvec_q8_0_mfma(const Dispatch &d, const MvArgs &a);
 // The tuned multiply (matvec_quant.hip): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
 zhip_result launch_matvec_quant(const Dispatch &d, const MvArgs &a, int type);
-
-// Token blockIdx.x as the multiplies will see it (RMSNorm times the norm weights and / or
-// silu(x / act_div)), written to dst + token * k / 4.
-__global__ __launch_bounds__(256) void matvec_prologue_kernel(MvArgs a, float4 *dst) {
-    __shared__ float red[4];
-    stage_token(a, blockIdx.x, dst + (size_t)blockIdx.x * (a.k / 4u), red);
-}
 
 template <class D, int MT>
 static zhip_result run(const Dispatch &d, const MvArgs &a, uint32_t lds_bytes) {
@@ -434,7 +422,7 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     if (D::CHUNK == 3 && matrix_cores && matvec_q3k_mfma_stream_accepts(a)) return launch_matvec_q3k_mfma_stream(d, a, d.bind[2].size);
     // (matvec_q5_k: the Q4_K kernel for k of 2048 or 4096 with the fifth bits; other shapes run the default variant)
     if (D::CHUNK == 5 && matrix_cores && matvec_q5k_mfma_resident_accepts(a)) return launch_matvec_q5k_mfma_resident(d, a, d.bind[2].size);
-    // (matvec_q6_k: a launch of its own splits the tokens, prologue included, for the multiply)
+    // (matvec_q6_k and matvec_q3_k: k of 1024, 2048 or 4096; every workgroup builds the tokens' operands, prologue included)
     if (D::CHUNK == 6 && matrix_cores && matvec_q6k_mfma_stream_accepts(a)) return launch_matvec_q6k_mfma_stream(d, a, d.bind[2].size);
     // The kernels that keep the tokens' operands in registers (k of 2048 or 4096, for Q8_0 also
     // 1024, and whole tiles) compute a step's prologue (RMSNorm, silu(x / act_div):
@@ -443,33 +431,14 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     // RMSNorm: 22.6 us, 26.1 us with a pass of its own in front, 20.7 us without a prologue).
     const bool resident = D::CHUNK == 4 && matrix_cores && matvec_q4k_mfma_resident_accepts(a);
     const bool q8_stream = D::CHUNK == 8 && matrix_cores && matvec_q8_mfma_stream_accepts(a);
-    // The Q4_K kernel for the other multiples of 1024 takes its inputs as they are: a step with
-    // a prologue first writes the transformed tokens to the workspace, one workgroup a token
-    // with the staging arithmetic of the default variant, and the multiply reads those.
-    uint64_t x_bound = d.bind[1].size;
-    if (D::CHUNK == 4 && matrix_cores && !resident && (norm || a.act_div > 0.f) && a.m <= 8u && p.k % 1024u == 0) {
-        if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", D::name());
-        const uint64_t bytes = (uint64_t)a.m * p.k * 4u;
-        if (zhip_result r = d.work->reserve(d, bytes)) return r;
-        hipLaunchKernelGGL(matvec_prologue_kernel, dim3(a.m), dim3(256), 0, d.stream, a, reinterpret_cast<float4 *>(d.work->data));
-        if (zhip_result r = check_launch(d, D::name())) return r;
-        a.x = reinterpret_cast<const float *>(d.work->data);
-        a.xr = p.k;
-        a.flags &= ~FLAG_NORM;
-        a.act_div = 0.f;
-        a.norm_w = nullptr;
-        x_bound = bytes;
-        v.act_div = 0u;
-    }
-    const bool plain = !(a.flags & FLAG_NORM) && a.act_div == 0.f;
     if (resident) return launch_matvec_q4k_mfma_resident(d, a, d.bind[2].size);
-    if (D::CHUNK == 4 && v.lanes == 64u && v.rows == 16u && plain && matvec_q4k_mfma_accepts(a))
-        return launch_matvec_q4k_mfma(d, a, x_bound, d.bind[2].size);
     // The same id on matvec_q8_0 (a one-token step too, so that a token's bits do not depend on
-    // the step it ran in); other shapes without a prologue or pair: the prefill tiling.
+    // the step it ran in).
     if (q8_stream) return launch_matvec_q8_mfma_stream(d, a, d.bind[2].size);
-    if (D::CHUNK == 8 && v.lanes == 64u && v.rows == 16u && plain && !pair && a.m <= 32u)
-        return launch_matvec_q8_0_mfma(d, a);
+    // Shapes these kernels do not take run the default variant under the id as well: the
+    // matrix-core kernels that once stood in for them (a k-sliced Q4_K kernel, the compensated
+    // prefill tiling for Q8_0) lost to it at two to four tokens on every shape measured
+    // (Q4_K 4096 x 14336 at four tokens: 71.7 against 21.9 us; 5120 x 5120: 28.0 against 21.2).
     // The tuned kernel takes rows of whole 64-weight tasks.
     if (D::CHUNK != 0 && p.k % 64u == 0) return launch_matvec_quant(d, a, D::CHUNK);
 

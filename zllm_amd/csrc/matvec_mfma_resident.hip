@@ -1,7 +1,12 @@
-// matvec_q4_k and matvec_q5_k, matrix-core variant for k = 2048 or 4096: the same arithmetic as
-// matvec_mfma.hip (weights as exact f16 values 16 + q, every token as two f16
-// rows, per-token power-of-two scale; see there), laid out so that nothing
-// is recomputed and nothing but partial results crosses LDS.
+// matvec_q4_k and matvec_q5_k, matrix-core variant (MatvecVariant wg 512, lanes 64, rows 16) for
+// k = 2048 or 4096 and steps of up to eight tokens. The per-weight work is done once for all
+// tokens: the weights enter v_mfma_f32_16x16x32_f16 as the exact f16 values 16 + q (the nibble
+// dropped into the mantissa of 16.0; Q5_K: 32 + q with the fifth bit), every token as two f16
+// rows, the rounding of its inputs and what that left times 2^11, under a per-token power of
+// two, so that every product is exact in the f32 accumulator and a token's rows meet no other
+// token's; a block's sum is d sc S - (16 d sc + dmin m) X with X from the same rows times a
+// column of ones (src/ref/tensor.zig:94-117). Nothing is recomputed and nothing but partial
+// results crosses LDS.
 //
 // A 512-thread workgroup is eight waves that split k eight ways (one or two
 // 256-weight blocks a wave). A wave builds its k range of all tokens' f16 rows
