@@ -977,6 +977,163 @@ static zhip_result run_long(const Dispatch &d, const KArgs &q, uint32_t blocks) 
     return check_launch(d, P::name());
 }
 
+// One-token steps over rows of 65 .. 256 tasks (k above 4096, up to 16384: the FFN-down shapes).
+// The kernel above walks such a row with one wave, a lane taking a task of every 64-task slice
+// in turn with its inputs read from LDS each time. Here a slice is a wave's for the whole
+// launch, so the lane's 64 inputs stay in registers as in the short-row case: the waves of a
+// group (two for two slices, four for three or four) multiply the same rows, R at a time, each
+// its own slice, leave the lanes' partial sums in LDS, and behind one barrier the group's waves
+// add them, each for its share of the R rows, in the order of the slices, which is the order
+// in which the lane of the kernel above adds its tasks; the lanes' reduction is the same code.
+// The same bits, and the arithmetic of a short row per weight.
+template <class P, bool PAIR>
+__global__ __launch_bounds__(256) void matvec_quant_sliced_kernel(KArgs q) {
+    const MvArgs &a = q.a;
+    extern __shared__ float4 lds4[];  // [wave]: its slice of the token in task order, padded per task; afterwards the partial sums
+    __shared__ float red[4];
+    constexpr int NSUM = P::NSUM, RUN = 64 / NSUM, kRows = PAIR ? 2 : 1, R = PAIR ? 4 : 8;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t tasks = q.tasks, slices = (tasks + 63u) / 64u;
+    const Masks nm = q.nm;
+    const uint32_t per_group = slices <= 2u ? 2u : 4u, groups_here = 4u / per_group;
+    const uint32_t grp = wave / per_group, slice = wave % per_group;
+    const uint32_t group = blockIdx.x * groups_here + grp, groups = gridDim.x * groups_here;
+    const uint32_t units = a.rows;  // a unit: an output (its row, or its gate row and up row)
+    const uint32_t task = lane + 64u * slice;
+    const bool active = task < tasks;
+
+    // Unit n of the group's walk (R consecutive units a round, the groups' rounds interleaved)
+    // and its rows; past the end the loads are clamped to a valid row and their results unused.
+    auto unit_of = [&](uint32_t n) { return ((n / R) * groups + group) * R + n % R; };
+    const uint32_t rounds = (units + groups * R - 1u) / (groups * R);  // the same for every group: the barriers below are the workgroup's
+    typename P::Raw cur[kRows], next[kRows];
+    auto load_unit = [&](uint32_t n, typename P::Raw (&dst)[kRows]) __attribute__((always_inline)) {
+        const uint32_t u = unit_of(n), j = u < units ? u : units - 1u, tk = active ? task : 0u;
+        dst[0] = P::load(a.w + (size_t)j * a.row_bytes, a.k, tk);
+        if (PAIR) dst[kRows - 1] = P::load(a.w + (size_t)(a.half + j) * a.row_bytes, a.k, tk);
+    };
+    load_unit(0, cur);  // (before the inputs: the stream starts while they are staged)
+
+    // A wave stages its own slice (64 tasks, 1024 vectors: sixteen a lane, asked for together)
+    // through its own part of LDS, in task order and padded per task as in the kernel above,
+    // and reads its lanes' tasks back; only the RMSNorm sum needs the other waves, and is added
+    // as stage_token adds it (vector i by thread i % 256, the waves' sums in order).
+    const uint32_t k4 = a.k / 4u;
+    const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)q.t0 * a.xr);
+    const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
+    const bool norm = (a.flags & FLAG_NORM) != 0;
+    float scale = 1.0f;
+    if (norm) {
+        float ss = 0.f;
+#pragma unroll 4
+        for (uint32_t i = tid; i < k4; i += 256u) {
+            const float4 v = xrow[i];
+            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+        }
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        ss = (red[0] + red[1]) + (red[2] + red[3]);
+        scale = 1.0f / sqrtf(ss / (float)a.k + a.eps);
+    }
+    float xr[64], xsum[NSUM];
+    {
+        float4 *mine4 = lds4 + wave * (64u * (kTaskStride / 4u));
+        float4 in[16], g[16];
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t gi = 1024u * slice + lane + 64u * j;
+            const bool have = gi < k4 && slice < slices;
+            in[j] = have ? xrow[gi] : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (norm) g[j] = have ? nw[gi] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int j = 0; j < 16; j++) {
+            const uint32_t gi = 1024u * slice + lane + 64u * j;
+            if (gi >= k4 || slice >= slices) continue;
+            float4 v = in[j];
+            if (norm) {
+                v.x = v.x * scale * g[j].x; v.y = v.y * scale * g[j].y;
+                v.z = v.z * scale * g[j].z; v.w = v.w * scale * g[j].w;
+            }
+            if (a.act_div > 0.f) {
+                v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
+                v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+            }
+            const uint32_t p = P::stage_index(gi) - 1024u * slice;
+            mine4[p + (p >> 4)] = v;
+        }
+        asm volatile("" ::: "memory");  // (a wave's LDS operations complete in order: its reads below see its writes above)
+        const float4 *src = mine4 + lane * (kTaskStride / 4u);
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const float4 f = src[v];
+            xr[4 * v] = f.x; xr[4 * v + 1] = f.y; xr[4 * v + 2] = f.z; xr[4 * v + 3] = f.w;
+        }
+#pragma unroll
+        for (int sr = 0; sr < NSUM; sr++) {
+            xsum[sr] = 0.f;
+#pragma unroll
+            for (int e = 0; e < RUN; e++) xsum[sr] += xr[sr * RUN + e];
+        }
+    }
+    __syncthreads();  // the token's space now takes the partial sums: [round parity][wave][unit of the round][row][lane]
+    float *part = reinterpret_cast<float *>(lds4);
+
+    for (uint32_t round = 0; round < rounds; round++) {
+        float *mine = part + (((round & 1u) * 4u + wave) * R) * kRows * 64u;
+#pragma unroll
+        for (int r = 0; r < R; r++) {
+            load_unit(round * R + r + 1u, next);
+            float v[kRows][1];
+            P::template dot<1, kRows>(cur, task & 3u, nm,
+                [&](int, int vi) { return make_float4(xr[4 * vi], xr[4 * vi + 1], xr[4 * vi + 2], xr[4 * vi + 3]); },
+                [&](int, int sr) { return xsum[sr]; }, v);
+#pragma unroll
+            for (int j = 0; j < kRows; j++) mine[(r * kRows + j) * 64u + lane] = v[j][0];
+#pragma unroll
+            for (int j = 0; j < kRows; j++) cur[j] = next[j];
+        }
+        __syncthreads();
+        // The group's waves share the round's units; a unit's slices are added in order, a lane
+        // leaving out the slice in which it has no task.
+        const float *theirs = part + (((round & 1u) * 4u + grp * per_group) * R) * kRows * 64u;
+        for (uint32_t r = slice; r < (uint32_t)R; r += per_group) {
+            float acc[kRows];
+#pragma unroll
+            for (int j = 0; j < kRows; j++) acc[j] = 0.f;
+            for (uint32_t sl = 0; sl < slices; sl++) {
+                if (lane + 64u * sl >= tasks) continue;
+#pragma unroll
+                for (int j = 0; j < kRows; j++) acc[j] += theirs[((sl * R + r) * kRows + j) * 64u + lane];
+            }
+            const float s0 = segment_sum(acc[0], 6u), s1 = PAIR ? segment_sum(acc[kRows - 1], 6u) : 0.f;
+            const uint32_t u = unit_of(round * R + r);
+            if (lane == 63u && u < units) {
+                const size_t o = (size_t)q.t0 * a.out_stride + a.col0 + u;
+                float res = PAIR ? silu_f(s0) * s1 : s0;
+                if (a.flags & FLAG_ACCUMULATE) res += a.out[o];
+                a.out[o] = res;
+            }
+        }
+        // (the other parity's space is written next; this one again only behind the next barrier)
+    }
+}
+
+template <class P, bool PAIR>
+static zhip_result run_sliced(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
+    static bool configured = false;  // dynamic LDS above 64 KiB needs opting in once
+    if (lds > 65536u && !configured) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_quant_sliced_kernel<P, PAIR>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
+            (void)hipGetLastError();
+            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", P::name(), lds);
+        }
+        configured = true;
+    }
+    hipLaunchKernelGGL((matvec_quant_sliced_kernel<P, PAIR>), dim3(blocks), dim3(256), lds, d.stream, q);
+    return check_launch(d, P::name());
+}
+
 template <class P, int MT, bool PAIR, bool XREG, int STG>
 static zhip_result run_quant(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
     static bool configured = false;  // dynamic LDS above 64 KiB needs opting in once
@@ -1030,6 +1187,18 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
         q.t0 = t0;
         q.mt = left < mt ? left : mt;
         const uint32_t lds = (uint32_t)(mt * tok_lds);
+        if (a.m == 1u && q.tasks > 64u && q.tasks <= 256u) {
+            // (the partial sums take the token's space: 2 x 4 waves x R units x rows x 64 lanes, 16 KB)
+            const uint32_t lds1 = 4u * 64u * kTaskStride * 4u;  // a slice's inputs a wave
+            const uint32_t groups_here = q.tasks <= 128u ? 2u : 1u, per_round = groups_here * (pair ? 4u : 8u);
+            const uint32_t want = (a.rows + per_round - 1u) / per_round;
+            const uint32_t fit = (160u * 1024u - 64u) / lds1;
+            const uint32_t cap = (uint32_t)d.dev->compute_units * (fit < 3u ? fit : 3u);
+            const uint32_t blocks = want < cap ? want : cap;
+            if (zhip_result r = pair ? run_sliced<P, true>(d, q, lds1, blocks) : run_sliced<P, false>(d, q, lds1, blocks)) return r;
+            t0 += q.mt;
+            continue;
+        }
         const bool xreg = a.m == 1u && q.tasks <= 64u;
         const uint32_t per_unit = pair ? rpi : rpi * (xreg ? 1u : 2u);
         const uint32_t units = (a.rows + per_unit - 1u) / per_unit;
