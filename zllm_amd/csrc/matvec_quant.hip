@@ -986,12 +986,12 @@ static zhip_result run_long(const Dispatch &d, const KArgs &q, uint32_t blocks) 
 // add them, each for its share of the R rows, in the order of the slices, which is the order
 // in which the lane of the kernel above adds its tasks; the lanes' reduction is the same code.
 // The same bits, and the arithmetic of a short row per weight.
-template <class P, bool PAIR>
+template <class P, bool PAIR, int R>
 __global__ __launch_bounds__(256) void matvec_quant_sliced_kernel(KArgs q) {
     const MvArgs &a = q.a;
     extern __shared__ float4 lds4[];  // [wave]: its slice of the token in task order, padded per task; afterwards the partial sums
     __shared__ float red[4];
-    constexpr int NSUM = P::NSUM, RUN = 64 / NSUM, kRows = PAIR ? 2 : 1, R = PAIR ? 4 : 8;
+    constexpr int NSUM = P::NSUM, RUN = 64 / NSUM, kRows = PAIR ? 2 : 1;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t tasks = q.tasks, slices = (tasks + 63u) / 64u;
     const Masks nm = q.nm;
@@ -1120,17 +1120,17 @@ __global__ __launch_bounds__(256) void matvec_quant_sliced_kernel(KArgs q) {
     }
 }
 
-template <class P, bool PAIR>
+template <class P, bool PAIR, int R>
 static zhip_result run_sliced(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
     static bool configured = false;  // dynamic LDS above 64 KiB needs opting in once
     if (lds > 65536u && !configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_quant_sliced_kernel<P, PAIR>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_quant_sliced_kernel<P, PAIR, R>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
             (void)hipGetLastError();
             return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", P::name(), lds);
         }
         configured = true;
     }
-    hipLaunchKernelGGL((matvec_quant_sliced_kernel<P, PAIR>), dim3(blocks), dim3(256), lds, d.stream, q);
+    hipLaunchKernelGGL((matvec_quant_sliced_kernel<P, PAIR, R>), dim3(blocks), dim3(256), lds, d.stream, q);
     return check_launch(d, P::name());
 }
 
@@ -1188,14 +1188,20 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
         q.mt = left < mt ? left : mt;
         const uint32_t lds = (uint32_t)(mt * tok_lds);
         if (a.m == 1u && q.tasks > 64u && q.tasks <= 256u) {
-            // (the partial sums take the token's space: 2 x 4 waves x R units x rows x 64 lanes, 16 KB)
+            // (the partial sums take the inputs' space: 2 x 4 waves x R units x rows x 64 lanes, 16 KB at most)
             const uint32_t lds1 = 4u * 64u * kTaskStride * 4u;  // a slice's inputs a wave
-            const uint32_t groups_here = q.tasks <= 128u ? 2u : 1u, per_round = groups_here * (pair ? 4u : 8u);
-            const uint32_t want = (a.rows + per_round - 1u) / per_round;
-            const uint32_t fit = (160u * 1024u - 64u) / lds1;
-            const uint32_t cap = (uint32_t)d.dev->compute_units * (fit < 3u ? fit : 3u);
+            const uint32_t groups_here = q.tasks <= 128u ? 2u : 1u;
+            const uint32_t cap = (uint32_t)d.dev->compute_units * 2u;  // two workgroups' LDS a CU
+            // Four units a round where that still gives every workgroup a round of its own
+            // (4096 x 8192: 9.8 -> 8.5 us), eight otherwise; the gate / up step always four.
+            const uint32_t want4 = (a.rows + groups_here * 4u - 1u) / (groups_here * 4u);
+            const bool eight = !pair && want4 > cap;
+            const uint32_t want = eight ? (want4 + 1u) / 2u : want4;
             const uint32_t blocks = want < cap ? want : cap;
-            if (zhip_result r = pair ? run_sliced<P, true>(d, q, lds1, blocks) : run_sliced<P, false>(d, q, lds1, blocks)) return r;
+            zhip_result r;
+            if (pair) r = run_sliced<P, true, 4>(d, q, lds1, blocks);
+            else r = eight ? run_sliced<P, false, 8>(d, q, lds1, blocks) : run_sliced<P, false, 4>(d, q, lds1, blocks);
+            if (r != ZHIP_OK) return r;
             t0 += q.mt;
             continue;
         }
