@@ -281,25 +281,77 @@ def test_quant_matvec(ctx, t, k, pair):
     assert worst <= 1e-5
 
 
-def test_quant_matvec_act_prologue(ctx):
+@pytest.mark.parametrize("t,k", [
+    (TensorType.q8_0, 256),     # the reference's case
+    (TensorType.q8_0, 8192),    # long rows: a step of three tokens goes tile by tile, a lone token slice by slice
+    (TensorType.q6_k, 12288),   # ... with the inputs staged permuted
+    (TensorType.q4_k, 14336),
+])
+def test_quant_matvec_act_prologue(ctx, t, k):
     """hc_act fused into the multiply after it: each input staged as
-    silu(x / 4), read from rows 264 floats apart (src/kernels/check.zig:1082-1116)."""
+    silu(x / 4), read from rows 8 floats further apart than their length (src/kernels/check.zig:1082-1116);
+    each token alone gives the same bits as in the three-token launch."""
     c = ctx
-    rows, n, k, div = 3, 100, 256, 4
+    rows, n, div = 3, 100, 4
     stride = k + 8
     x = c.random(rows * stride, 3).reshape(rows, stride)
-    raw, values = quant_rows(c, TensorType.q8_0, n, k)
-    xa, wa = c.upload(x), c.gpu_weights(TensorType.q8_0, raw, k)
+    raw, values = quant_rows(c, t, n, k)
+    xa, wa = c.upload(x), c.gpu_weights(t, raw, k)
     v = x[:, :k].astype(np.float64) / div
     want = (v * sigmoid64(v)) @ values.astype(np.float64).T
     worst = 0.0
     for cand in K.MatvecVariant.candidates:
+        if not cand.suits(t):
+            continue
         var = K.MatvecVariant(cand.wg, cand.lanes, cand.rows, div)
+        pipeline = c.set.matvec(c.rec, K.weight_kernel("matvec", t), var)
+        p = lambda: P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, x_stride=stride // 4)
         out = c.output(rows * n)
-        c.launcher().launch_pipeline(c.set.matvec(c.rec, Kernel.matvec_q8_0, var), P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, x_stride=stride // 4),
-                                     [xa, wa, out, wa], (K.div_ceil(n, var.group_rows()), rows, 1))
-        worst = max(worst, rel_err(c.read(out).reshape(rows, n), want))
+        c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, wa], (K.div_ceil(n, var.group_rows()), rows, 1))
+        got = c.read(out).reshape(rows, n)
+        worst = max(worst, rel_err(got, want))
+        for tk in range(rows):
+            single = c.output(n)
+            c.launcher().launch_pipeline(pipeline, p(), [c.upload(x[tk]), wa, single, wa], (K.div_ceil(n, var.group_rows()), 1, 1))
+            assert got[tk].tobytes() == c.read(single)[:n].tobytes(), "a token's sums differ between a lone launch and a multi-token launch"
     assert worst <= 1e-5
+
+
+@pytest.mark.parametrize("t,k,pair,rows,n", [
+    (TensorType.q4_k, 14336, False, 2, 37),   # two tokens whose inputs do not fit LDS together: the tile-by-tile kernel's two-token form
+    (TensorType.q8_0, 10240, True, 2, 19),
+    (TensorType.q5_k, 16384, False, 4, 9),    # 256 tasks: four whole slices, a batch of rows with units past the end
+    (TensorType.q3_k, 4352, False, 1, 3),     # 68 tasks: a second slice of four lanes, three rows
+    (TensorType.q6_k, 16640, False, 2, 21),   # 260 tasks: past the sliced kernel's four slices
+])
+def test_quant_matvec_long_rows(ctx, t, k, pair, rows, n):
+    """Rows of more than 4096 weights at the widths and edges test_quant_matvec leaves out:
+    within 1e-5 of float64, with the norm prologue and the accumulate epilogue (or the SiLU
+    pair), and each token bitwise equal to its lone launch."""
+    c = ctx
+    eps = 1e-6
+    x = c.random(rows * k, 3).reshape(rows, k)
+    nw = c.random(k, 1)
+    raw, values = quant_rows(c, t, 2 * n if pair else n, k)
+    init = c.random(rows * n, 0 if pair else 4).reshape(rows, n)
+    xa, wa, na = c.upload(x), c.gpu_weights(t, raw, k), c.upload(nw)
+    v64 = values.astype(np.float64)
+    want = np.empty((rows, n))
+    for tk in range(rows):
+        xn = norm_row(x[tk], nw, eps)
+        g = v64[:n] @ xn
+        want[tk] = g * sigmoid64(g) * (v64[n:] @ xn) if pair else init[tk] + g
+    v = K.MatvecVariant()
+    p = lambda: P.MatvecBf16(n=n, k=k, col0=0, out_stride=n, eps=eps, norm=True, accumulate=not pair, silu_pair=pair, half=n if pair else 0)
+    pipeline = c.set.matvec(c.rec, K.weight_kernel("matvec", t), v)
+    out = c.upload(init)
+    c.launcher().launch_pipeline(pipeline, p(), [xa, wa, out, na], (K.div_ceil(n, v.group_rows()), rows, 1))
+    got = c.read(out).reshape(rows, n)
+    assert rel_err(got, want) <= 1e-5
+    for tk in range(rows):
+        single = c.upload(init[tk])
+        c.launcher().launch_pipeline(pipeline, p(), [c.upload(x[tk]), wa, single, na], (K.div_ceil(n, v.group_rows()), 1, 1))
+        assert got[tk].tobytes() == c.read(single).tobytes(), "a token's sums differ between a lone launch and a multi-token launch"
 
 
 def test_quant_matvec_eight_rows(ctx):
