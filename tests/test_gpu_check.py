@@ -119,6 +119,9 @@ def bf16_tokens_case(c, m, n, k, col0=0, pad=0, accumulate=False, norm=False, x=
     (4, 8192, 1024, 0, 0, False, True),        # k = 1024 with the prologue: the tokens split beforehand
     (19, 2052, 4096, 8, 0, True, False),
     (3, 100, 1024, 0, 0, False, False),        # a small matrix: the general kernel
+    (4, 1100, 9728, 0, 0, False, False),       # rows longer than 4096: stretches of columns, each launch adding to the one before
+    (2, 800, 14336, 3, 5, True, False),        # ... onto what the output already holds
+    (3, 1000, 8704, 0, 0, False, True),        # with the RMSNorm prologue: the tokens are normalised and split once for all the stretches
 ])
 @pytest.mark.parametrize("half", HALVES)
 def test_matvec_bf16_several_tokens(ctx, half, m, n, k, col0, pad, accumulate, norm):

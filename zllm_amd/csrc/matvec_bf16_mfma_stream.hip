@@ -68,6 +68,8 @@ struct StreamArgs {
     // Inputs split beforehand (SPLIT kernels): three planes [piece][token][k] of bf16.
     const uint8_t *planes;
     uint32_t plane_tokens;  // tokens a plane holds
+    uint32_t plane_k;       // positions of a token in a plane (the whole row's, of which the launch may take a stretch)
+    uint32_t plane_first;   // the launch's first position
     uint32_t t0;            // the launch's first token in the planes
     const float *inverse;   // F16 kernels: one over each token's scale
 };
@@ -199,8 +201,8 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
     if constexpr (SPLIT) {
         // Every step's operand is sixteen bytes of a plane; the lanes of absent tokens and of
         // the zero rows ask past the buffer's end and get zeros.
-        const __amdgpu_buffer_rsrc_t pbuf = make_buffer(q.planes, PIECES * q.plane_tokens * a.k * 2u);
-        const uint32_t at = live ? ((piece * q.plane_tokens + q.t0 + tok) * a.k + 64u * NP * wave + 8u * kap) * 2u : 0xfffffff0u;
+        const __amdgpu_buffer_rsrc_t pbuf = make_buffer(q.planes, PIECES * q.plane_tokens * q.plane_k * 2u);
+        const uint32_t at = live ? ((piece * q.plane_tokens + q.t0 + tok) * q.plane_k + q.plane_first + 64u * NP * wave + 8u * kap) * 2u : 0xfffffff0u;
 #pragma unroll
         for (int s = 0; s < 4 * NP; s++) xf[s] = __builtin_bit_cast(hu32x4, __builtin_amdgcn_raw_buffer_load_b128(pbuf, live ? at + 32u * s : at, 0, 0));
         issue();
@@ -314,7 +316,7 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
 // src/kernels/matvec_half.wgsl:58-80), split into the three planes.
 __global__ __launch_bounds__(256) void matvec_bf16_split_kernel(MvArgs a, uint2 *planes) {
     __shared__ float red[4];
-    __shared__ float4 staged[1024];
+    extern __shared__ float4 staged[];  // the token: k / 4 vectors
     stage_token(a, blockIdx.x, staged, red);
     __syncthreads();
     const uint32_t k4 = a.k / 4u;
@@ -336,7 +338,7 @@ __global__ __launch_bounds__(256) void matvec_bf16_split_kernel(MvArgs a, uint2 
 // (planes [2][tokens][k]), and one over the scale.
 __global__ __launch_bounds__(256) void matvec_f16_split_kernel(MvArgs a, uint2 *planes, float *inverse) {
     __shared__ float red[4];
-    __shared__ float4 staged[1024];
+    extern __shared__ float4 staged[];  // the token: k / 4 vectors
     stage_token(a, blockIdx.x, staged, red);
     __syncthreads();
     const uint32_t tid = threadIdx.x, k4 = a.k / 4u;
@@ -390,8 +392,9 @@ zhip_result launch_blocks(const Dispatch &d, const StreamArgs &q, dim3 grid) {
 
 // Whether this kernel can run the (already validated) arguments: k split into whole lines a
 // wave, no pair.
+// (rows of more than 4096 weights are taken in stretches of columns, a launch each; up to 16384: the split launch stages a token in 64 KB of LDS)
 bool matvec_bf16_mfma_stream_accepts(const MvArgs &a) {
-    return a.m >= 1 && a.k >= 1024u && a.k <= 4096u && a.k % 512u == 0 && !(a.flags & FLAG_SILU_PAIR) && a.act_div == 0.f && a.rows >= 1 &&
+    return a.m >= 1 && a.k >= 1024u && a.k <= 16384u && a.k % 512u == 0 && !(a.flags & FLAG_SILU_PAIR) && a.act_div == 0.f && a.rows >= 1 &&
            a.xr % 4u == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == 2u * a.k;
 }
 
@@ -419,7 +422,7 @@ zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, u
     const uint32_t groups = units < cus ? units : cus;
     const uint32_t rounds = (a.rows / 32u) / groups;
     const uint32_t tail = (a.rows - 32u * rounds * groups + 7u) / 8u;
-    StreamArgs q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, nullptr, 0u, 0u, nullptr};
+    StreamArgs q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, nullptr, 0u, 0u, 0u, 0u, nullptr};
     // The tokens are split (and normalised) by a launch of their own where that is cheaper than
     // every workgroup splitting them again, and wherever the step carries the RMSNorm prologue
     // (the workgroups computing the norm themselves at k = 1024 measured the same: 151936 x 1024
@@ -432,22 +435,37 @@ zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, u
         if (bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "%s: a step of %u tokens", name, a.m);
         if (zhip_result r = d.work->reserve(d, bytes + 4ull * a.m + 64u)) return r;
         float *inverse = reinterpret_cast<float *>(d.work->data + bytes);
-        if (f16) hipLaunchKernelGGL(matvec_f16_split_kernel, dim3(a.m), dim3(256), 0, d.stream, a, reinterpret_cast<uint2 *>(d.work->data), inverse);
-        else hipLaunchKernelGGL(matvec_bf16_split_kernel, dim3(a.m), dim3(256), 0, d.stream, a, reinterpret_cast<uint2 *>(d.work->data));
+        if (f16) hipLaunchKernelGGL(matvec_f16_split_kernel, dim3(a.m), dim3(256), a.k * 4u, d.stream, a, reinterpret_cast<uint2 *>(d.work->data), inverse);
+        else hipLaunchKernelGGL(matvec_bf16_split_kernel, dim3(a.m), dim3(256), a.k * 4u, d.stream, a, reinterpret_cast<uint2 *>(d.work->data));
         if (zhip_result r = check_launch(d, name)) return r;
         q.planes = d.work->data;
         q.plane_tokens = a.m;
+        q.plane_k = a.k;
         q.inverse = inverse;
         q.a.flags &= ~FLAG_NORM;
         q.a.norm_w = nullptr;
     }
     const dim3 grid(groups);
+    // Rows of more than 4096 weights (the FFN-down shapes; the general kernel takes them token by
+    // token): stretches of up to 4096 columns, each a launch that adds to the one before; the
+    // tokens are split once, prologue included, for all of them.
+    const uint32_t pieces = a.k / 512u, launches = (a.k + 4095u) / 4096u;
     for (uint32_t t0 = 0; t0 < a.m; t0 += 8u) {
-        q.a.x = a.x + (size_t)t0 * a.xr;
-        q.a.out = a.out + (size_t)t0 * a.out_stride;
-        q.a.m = a.m - t0 < 8u ? a.m - t0 : 8u;
-        q.t0 = t0;
-        if (zhip_result r = f16 ? launch_for_k<true, true>(d, q, grid) : split ? launch_for_k<true, false>(d, q, grid) : launch_for_k<false, false>(d, q, grid)) return r;
+        uint32_t first = 0;
+        for (uint32_t c = 0; c < launches; c++) {
+            q.a.k = 512u * (pieces / launches + (c < pieces % launches ? 1u : 0u));
+            q.a.x = a.x + (size_t)t0 * a.xr + first;
+            q.a.w = a.w + 2u * (size_t)first;
+            q.w_bytes = (uint32_t)((used < w_bytes ? used : w_bytes) - 2u * (uint64_t)first);
+            q.a.out = a.out + (size_t)t0 * a.out_stride;
+            q.a.m = a.m - t0 < 8u ? a.m - t0 : 8u;
+            q.a.flags = (a.flags & ~FLAG_NORM & ~FLAG_ACCUMULATE) | ((c || (a.flags & FLAG_ACCUMULATE)) ? FLAG_ACCUMULATE : 0u);
+            if (!split) q.a.flags = a.flags;
+            q.t0 = t0;
+            q.plane_first = first;
+            if (zhip_result r = f16 ? launch_for_k<true, true>(d, q, grid) : split ? launch_for_k<true, false>(d, q, grid) : launch_for_k<false, false>(d, q, grid)) return r;
+            first += q.a.k;
+        }
     }
     return ZHIP_OK;
 }
