@@ -45,7 +45,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,c5,formats,replay,floor for the 'also' section; 'none' skips it")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,c5,formats,down,replay,floor for the 'also' section; 'none' skips it")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-replay", action="store_true",
                     help="launch every dispatch of a repeated submit instead of replaying it from a HIP graph (for runs under a kernel tracer, "
@@ -309,7 +309,7 @@ def main() -> int:
     only = [s for s in args.only.split(",") if s]
     also = {}
     if "none" not in only:
-        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c4_int8", bench_c4_int8), ("c5", bench_c5), ("formats", bench_formats), ("replay", bench_replay), ("floor", bench_floor)):
+        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c4_int8", bench_c4_int8), ("c5", bench_c5), ("formats", bench_formats), ("down", bench_down), ("replay", bench_replay), ("floor", bench_floor)):
             if not only or name in only:
                 try:
                     also[name] = fn(locals())
@@ -533,6 +533,30 @@ def bench_formats(env):
             nbytes = n * (k // e) * bb + m * 4 * k + m * 4 * n
             res[tag] = env["hbm_entry"](f"{name} decode matvec M={m} K={k} N={n}" + (", matrix-core variant" if variant else ""), nbytes, wall, gpu_s, steps,
                                         {"copies": len(launches), "max_err_over_max_want": rel})
+    return res
+
+
+def bench_down(env):
+    """The FFN-down multiply of the same model (K = 14336, N = 4096: rows longer than a step's
+    tokens can share workgroup memory for) at one, two and four tokens, Q4_K and Q8_0."""
+    synth, oracle, K, TensorType = env["synth"], env["oracle"], env["K"], env["TensorType"]
+    n, k = 4096, 14336
+    res = {}
+    for name, ot in (("q4_k", oracle.Q4_K), ("q8_0", oracle.Q8_0)):
+        t = TensorType[name]
+        raw = synth.random_blocks(synth.rng(0xD0), name, n, k)
+        w = oracle.dequantize(ot, raw, n * k).reshape(n, k)
+        e, bb = K.LAYOUT[t]
+        for m in (1, 2, 4):
+            xm = synth.activations(synth.rng(0xD8 + m), m, k)
+            launches, out = env["matvec_workload"](t, raw, n, k, m, False, xm)
+            wall, gpu_s, steps = env["protocol"](launches)
+            got = env["read"](out)[: m * n].reshape(m, n).astype(np.float64)
+            want = xm.astype(np.float64) @ w.astype(np.float64).T
+            rel = float(np.max(np.abs(got - want)) / np.max(np.abs(want)))
+            nbytes = n * (k // e) * bb + m * 4 * k + m * 4 * n
+            res[f"{name}_m{m}"] = env["hbm_entry"](f"{name} decode matvec M={m} K={k} N={n}", nbytes, wall, gpu_s, steps,
+                                                    {"copies": len(launches), "max_err_over_max_want": rel})
     return res
 
 
