@@ -522,8 +522,8 @@ def test_matvec_q8_0_mfma_variant_silu_pair(ctx, t, rows, n, k, norm):
 def test_matvec_q8_0_mfma_variant_prologues(ctx, rows, n, k, prologue):
     """The matrix-core variant of matvec_q8_0 on steps with the RMSNorm and silu(x / act_div)
     prologues (src/kernels/matvec_quant.wgsl.hbs:73-89), which the streaming kernel computes
-    as it builds the tokens' operands (200 rows: not whole tiles, the default variant's
-    kernel); 1e-5 against float64, each token bitwise equal to its lone launch."""
+    as it builds the tokens' operands (200 rows of 1024 weights: the kernel that takes a
+    tile's rows as one flat stretch, a workgroup's share of the last rows); 1e-5 against float64, each token bitwise equal to its lone launch."""
     c = ctx
     div, eps = 4 if prologue == "norm_act" else 0, 1e-6
     x = c.random(rows * k, 3).reshape(rows, k)

@@ -328,6 +328,9 @@ bool matvec_q6k_mfma_stream_accepts(const MvArgs &a);
 zhip_result launch_matvec_q6k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
 bool matvec_q3k_mfma_stream_accepts(const MvArgs &a);
 zhip_result launch_matvec_q3k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
+// matvec_q8_0 over rows of 1024 weights in the same kernel: a tile's rows as one flat stretch.
+bool matvec_q8_0_mfma_flat_accepts(const MvArgs &a);
+zhip_result launch_matvec_q8_0_mfma_flat(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
 // Matrices from this size on take it: below, its fixed costs (the split of the tokens, a
 // workgroup's first tile) outweigh the general kernel's per-token work at two to four tokens
 // (8 MB, k = 1024: 6.4 / 6.8 / 7.8 us at 2 / 4 / 8 tokens against 4.7 / 6.2 / 9.3).
@@ -429,6 +432,7 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     // src/kernels/matvec_quant.wgsl.hbs:73-89) themselves: their operands are built from one
     // round of loads, which the norm weights join (C3 at four tokens with the FFN launch's
     // RMSNorm: 22.6 us, 26.1 us with a pass of its own in front, 20.7 us without a prologue).
+    if (D::CHUNK == 8 && matrix_cores && matvec_q8_0_mfma_flat_accepts(a)) return launch_matvec_q8_0_mfma_flat(d, a, d.bind[2].size);
     const bool resident = D::CHUNK == 4 && matrix_cores && matvec_q4k_mfma_resident_accepts(a);
     const bool q8_stream = D::CHUNK == 8 && matrix_cores && matvec_q8_mfma_stream_accepts(a);
     if (resident) return launch_matvec_q4k_mfma_resident(d, a, d.bind[2].size);

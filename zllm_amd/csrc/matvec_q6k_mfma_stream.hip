@@ -6,7 +6,10 @@
 // d * scale * sum((q - 32) * x), q the 6-bit value of ql and qh; Q3_K (the rows repacked at
 // load, src/kernels/repack_q3_k.wgsl; src/ref/tensor.zig:141-160): d * (scale - 32) * sum((q - 4) * x),
 // q the two low bits and the third bit. What follows describes Q6_K; Q3_K has 128-byte blocks
-// (a unit is four lines a row, all eight waves load it) and its own unpacking.
+// (a unit is four lines a row, all eight waves load it) and its own unpacking. matvec_q8_0 over
+// rows of 1024 weights runs here too (split rows, src/kernels/repack_q8_0.wgsl: d * sum(q * x)
+// over 32-weight blocks): a row is 8.5 lines, so a tile's 32 rows travel as one stretch of 272
+// whole lines through a ring of three slots and are read from LDS where they fall.
 //
 // Arithmetic. v_mfma_f32_32x32x16_f16 multiplies 32 rows of inputs by 32 weight rows over one
 // sub-block. The weights enter as the exact f16 integers q - 32 (the byte dropped into the
@@ -47,7 +50,9 @@
 // tokens: Q6_K 16.5 / 17.9 us (21.8 us before the operands were built in the kernel, the next
 // unit was read ahead and the sub-blocks overlapped), Q3_K 14.3 / 15.6 us (20.3 us); Q6_K on
 // 128256 x 4096 80 / 87 us (94 - 99 us; 80 us with the multiplies switched off, 80.7 us for
-// one token on the default variant).
+// one token on the default variant). Q8_0 on 151936 x 1024 at two / four / eight tokens:
+// 33.9 / 32.9 / 35.6 us (41.7 us with the rows read line by line, row by row, by the kernel that
+// takes k = 2048 and 4096; the default variant 33.6 / 44.1 / 79.7 us).
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -67,12 +72,14 @@ typedef uint32_t qu32x2 __attribute__((ext_vector_type(2)));
 typedef uint32_t qu32x4 __attribute__((ext_vector_type(4)));
 
 constexpr uint32_t THREADS = 512, WAVES = 8;
-constexpr int SLOTS = 4;                        // ring slots: the unit being read ahead and three in flight
 constexpr uint32_t PART_BYTES = 2u * WAVES * 256u * 4u;  // [tile parity][wave][token of the lane's four][lane]
 constexpr uint32_t KEPT = 16;                   // tiles whose outputs wait in LDS for one burst of stores
 
-// The formats. A unit is four 256-weight blocks of each of a tile's 32 rows: whole lines of every row.
+// The formats. A unit is four 256-weight blocks of each of a tile's 32 rows: whole lines of every row
+// (Q6_K, Q3_K) or of the tile (Q8_0).
 struct FmtQ6 {  // 224-byte padded blocks: ql[128], qh[64], sixteen signed scales, d
+    static constexpr int KIND = 6, SLOTS = 4;              // ring slots: the unit being read ahead and three in flight
+    static constexpr bool FLAT = false;
     static constexpr uint32_t BLOCK = 224, ROW_LINES = 7;  // a row's part of a unit: seven lines
     static constexpr int LOADS = 4;                        // wave-wide loads of a unit a wave issues
     static constexpr uint32_t LOADERS = 7;                 // 28 KB: seven waves' worth; the eighth asks for nothing
@@ -80,24 +87,42 @@ struct FmtQ6 {  // 224-byte padded blocks: ql[128], qh[64], sixteen signed scale
     static const char *name() { return "matvec_q6_k"; }
 };
 struct FmtQ3 {  // blocks repacked at load into eight self-contained 16-byte units (src/kernels/repack_q3_k.wgsl)
+    static constexpr int KIND = 3, SLOTS = 4;
+    static constexpr bool FLAT = false;
     static constexpr uint32_t BLOCK = 128, ROW_LINES = 4;
     static constexpr int LOADS = 2;
     static constexpr uint32_t LOADERS = 8;
     static constexpr float OFFSET = -1028.0f;              // 1024 + byte -> q - 4
     static const char *name() { return "matvec_q3_k"; }
 };
+// Q8_0 rows of 1024 weights in split form (src/kernels/repack_q8_0.wgsl: 1024 signed bytes, then
+// 32 f16 scales: 1088 bytes, 8.5 lines). The unit is the whole row, so a tile's 32 rows are one
+// contiguous stretch of 272 whole lines and travel as a flat copy; the rows do not start on
+// lines, which LDS does not mind (read line by line from memory, every second row's stretch of
+// a wave straddles two lines and the stream runs at half its rate: 151936 x 1024, 42 us).
+struct FmtQ8 {
+    static constexpr int KIND = 8, SLOTS = 3;              // 34 KB a unit
+    static constexpr bool FLAT = true;
+    static constexpr uint32_t BLOCK = 272, ROW_LINES = 1;  // (BLOCK only so that a unit's bytes of a row are 4 BLOCK = 1088)
+    static constexpr int LOADS = 5;                        // 34 loads of eight lines: seven waves' five, the 35th asks for nothing
+    static constexpr uint32_t LOADERS = 7;
+    static constexpr float OFFSET = -1152.0f;              // 1024 + (byte ^ 0x80) -> q
+    static const char *name() { return "matvec_q8_0"; }
+};
 template <class F> constexpr uint32_t row_unit() { return 4u * F::BLOCK; }        // a unit's bytes of one row
 template <class F> constexpr uint32_t unit_bytes() { return 32u * row_unit<F>(); }  // a unit in LDS
 // (the last KB: where the loads of nothing land)
-template <class F> constexpr uint32_t lds_bytes() { return PART_BYTES + SLOTS * unit_bytes<F>() + KEPT * 1024u + 64u + 1024u + 512u; }
-static_assert(lds_bytes<FmtQ6>() <= 160u * 1024u - 64u, "the ring must fit the CU's LDS");
+template <class F> constexpr uint32_t lds_bytes() { return PART_BYTES + F::SLOTS * unit_bytes<F>() + KEPT * 1024u + 64u + 1024u + 512u; }
+static_assert(lds_bytes<FmtQ6>() <= 160u * 1024u - 64u && lds_bytes<FmtQ8>() <= 160u * 1024u - 64u, "the ring must fit the CU's LDS");
 
 // What a lane reads of a unit in LDS for its wave's half block: Q6_K the low nibbles of its
 // positions in the four quadrants' pairs, their two-bit words, the half's scales and d; Q3_K
 // the half's four sixteen-byte units.
-template <bool Q3> struct Fetched;
-template <> struct Fetched<true> { qu32x4 u[4]; };
-template <> struct Fetched<false> { qu32x2 ql[4], qh[2], sc; uint32_t d; };
+// Q8_0: the lane's eight quants of each of the half block's eight sub-blocks, and its four scales.
+template <int KIND> struct Fetched;
+template <> struct Fetched<3> { qu32x4 u[4]; };
+template <> struct Fetched<6> { qu32x2 ql[4], qh[2], sc; uint32_t d; };
+template <> struct Fetched<8> { qu32x2 q[8], sc; };
 
 struct Q6Args {
     MvArgs a;
@@ -154,7 +179,7 @@ __device__ __forceinline__ qf16x8 weights_f16(qu32x2 q, uint32_t bias) {
 template <class F, int NU, bool FEW>
 __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Args q) {
     constexpr uint32_t ROW_UNIT = row_unit<F>(), UNIT = unit_bytes<F>();
-    constexpr int LOADS = F::LOADS;
+    constexpr int LOADS = F::LOADS, SLOTS = F::SLOTS;
     const MvArgs &a = q.a;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     float *lds_part = reinterpret_cast<float *>(lds);
@@ -192,7 +217,8 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
 #pragma unroll
     for (int j = 0; j < LOADS; j++) {
         const uint32_t line = 8u * (LOADS * wave + j) + (lane >> 3), row = line / F::ROW_LINES, in_row = line % F::ROW_LINES;
-        woff[j] = row * a.row_bytes + 128u * in_row + 16u * ((lane & 7u) ^ (row & 7u));
+        // (a flat tile: line after line of the stretch, chunk c of line l at position c ^ (l % 8))
+        woff[j] = F::FLAT ? 128u * line + 16u * ((lane & 7u) ^ (line & 7u)) : row * a.row_bytes + 128u * in_row + 16u * ((lane & 7u) ^ (row & 7u));
     }
     // Unit v of the run: unit v % NU of tile v / NU. Past the run's end the loads still run, so
     // that the waits count the same loads every step, but against an empty buffer: zeros land
@@ -207,8 +233,10 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
         for (int j = 0; j < LOADS; j++) {
             // (lines of rows the workgroup's share of the last rows does not have are not fetched;
             // what the matrix instructions make of the zeros there is never stored)
-            const uint32_t first_line_row = (8u * (LOADS * wave + j)) / F::ROW_LINES;
-            load_lds_b128(real && first_line_row < rows ? wbuf : nobuf, wave < F::LOADERS ? dst + 1024u * j : dst, woff[j] + base);
+            const uint32_t g = LOADS * wave + j;
+            const uint32_t first_line_row = F::FLAT ? (1024u * g) / ROW_UNIT : (8u * g) / F::ROW_LINES;
+            const bool within = 1024u * g < UNIT;  // (the flat tile's last load slot is past its end)
+            load_lds_b128(real && within && first_line_row < rows ? wbuf : nobuf, wave < F::LOADERS && within ? dst + 1024u * j : ring0 + SLOTS * UNIT + KEPT * 1024u + 64u, woff[j] + base);
         }
     };
 
@@ -348,11 +376,22 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     // bytes at 224 (wave / 2). Byte o of a row's unit sits at 896 rho + 128 (o / 128) +
     // 16 ((o / 16 % 8) ^ (rho % 8)) + o % 16.
     const uint32_t blk = wave >> 1, half = wave & 1u;
-    auto at_byte = [&](uint32_t o) { return ROW_UNIT * rho + (o & ~127u) + 16u * (((o >> 4) & 7u) ^ (rho & 7u)) + (o & 15u); };
-    constexpr bool Q3 = F::BLOCK == 128u;
+    auto at_byte = [&](uint32_t o) {
+        const uint32_t f = ROW_UNIT * rho + o;  // (flat: the byte's place in the tile)
+        return F::FLAT ? (f & ~127u) + 16u * (((f >> 4) & 7u) ^ ((f >> 7) & 7u)) + (f & 15u)
+                       : ROW_UNIT * rho + (o & ~127u) + 16u * (((o >> 4) & 7u) ^ (rho & 7u)) + (o & 15u);
+    };
+    constexpr int KIND = F::KIND;
+    constexpr bool Q3 = KIND == 3;
     uint32_t at_ql[4], at_qh[2];  // Q6_K ql: [which 32 of the half's 64][which 16]; qh: [which 16]; Q3_K: at_ql = the half's four units
-    uint32_t at_sc = 0, at_d = 0;
-    if constexpr (Q3) {
+    uint32_t at_sc = 0, at_d = 0, at_q8[8];
+    if constexpr (KIND == 8) {
+        // (the wave's 128 positions are four blocks of 32: sub-block s lies in block 4 wave + s / 2)
+#pragma unroll
+        for (uint32_t i = 0; i < 8; i++) at_q8[i] = at_byte(128u * wave + 16u * i + 8u * kap);
+        at_sc = at_byte(1024u + 8u * wave);
+        at_ql[0] = at_qh[0] = 0;
+    } else if constexpr (Q3) {
 #pragma unroll
         for (uint32_t i = 0; i < 4; i++) at_ql[i] = at_byte(128u * blk + 64u * half + 16u * i);
         at_qh[0] = at_qh[1] = 0;
@@ -371,8 +410,12 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     // The lane's part of the unit in `slot`, from LDS to registers.
     auto fetch = [&](uint32_t slot) __attribute__((always_inline)) {
         const uint8_t *t = ring + slot * UNIT;
-        Fetched<Q3> f;
-        if constexpr (Q3) {
+        Fetched<KIND> f;
+        if constexpr (KIND == 8) {
+#pragma unroll
+            for (uint32_t i = 0; i < 8; i++) f.q[i] = *reinterpret_cast<const qu32x2 *>(t + at_q8[i]);
+            f.sc = *reinterpret_cast<const qu32x2 *>(t + at_sc);
+        } else if constexpr (Q3) {
 #pragma unroll
             for (uint32_t i = 0; i < 4; i++) f.u[i] = *reinterpret_cast<const qu32x4 *>(t + at_ql[i]);
         } else {
@@ -387,9 +430,15 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     };
     // Sub-block s (of the eight of the wave's half block) of a fetched unit, made ready for the
     // matrix instruction: the lane's eight quants as f16, and d * scale.
-    auto prepare = [&](const Fetched<Q3> &f, int s, qf16x8 &wf, float &dsc) __attribute__((always_inline)) {
+    auto prepare = [&](const Fetched<KIND> &f, int s, qf16x8 &wf, float &dsc) __attribute__((always_inline)) {
         qu32x2 v;
-        if constexpr (Q3) {
+        if constexpr (KIND == 8) {
+            // (signed bytes: with the top bit turned they are q + 128)
+            v[0] = f.q[s][0] ^ 0x80808080u;
+            v[1] = f.q[s][1] ^ 0x80808080u;
+            const uint32_t word = s < 4 ? f.sc.x : f.sc.y;
+            dsc = half_bits_to_float((s & 2) ? word >> 16 : word & 0xffffu);
+        } else if constexpr (Q3) {
             // Unit i of the half: 32 weights as two words of 2-bit values (byte b, bit pair e:
             // position 4 e + b; the second word 16 further), a word of third bits (byte b, bit e:
             // position 4 e + b), scale - 32 of each sixteen as signed bytes, d. The lane's eight
@@ -423,7 +472,7 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     // additions that wait for it.
     qf16x8 wf;
     float dsc;
-    auto multiply = [&](auto unit, const Fetched<Q3> &f, const Fetched<Q3> &after) __attribute__((always_inline)) {
+    auto multiply = [&](auto unit, const Fetched<KIND> &f, const Fetched<KIND> &after) __attribute__((always_inline)) {
         constexpr int U = decltype(unit)::value;
         qf32x16 zero;
 #pragma unroll
@@ -499,14 +548,14 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     // every wave has unit v in registers, so its slot takes the loads of unit v + 4, and the
     // tile before's partial sums are in LDS. A wave reads unit v + 1 into registers while it
     // multiplies unit v: no multiply waits for LDS.
-    Fetched<Q3> cur;
+    Fetched<KIND> cur;
     auto step = [&](uint32_t p, auto unit) __attribute__((always_inline)) {
         constexpr int U = decltype(unit)::value;
         const uint32_t v = NU * p + U;
         asm volatile("s_waitcnt vmcnt(%0)" ::"n"((SLOTS - 2) * LOADS) : "memory");
         lds_barrier();
         issue(v + SLOTS, v % SLOTS);
-        const Fetched<Q3> next = fetch((v + 1u) % SLOTS);
+        const Fetched<KIND> next = fetch((v + 1u) % SLOTS);
         asm volatile("" ::: "memory");  // (the reads go out here, not where the next step uses them)
         if (U == 0 && p > 0u) {
             sum_up(p - 1u);
@@ -567,8 +616,12 @@ zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) 
     const uint32_t tail = (a.rows - 32u * rounds * groups + 7u) / 8u;
     Q6Args q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, 0x64646464u};
     const dim3 grid(groups);
+    if constexpr (F::FLAT) {  // (the unit is the whole row: k = 1024 only)
+        return a.m <= 4u ? launch_blocks<F, 1, true>(d, q, grid) : launch_blocks<F, 1, false>(d, q, grid);
+    } else {
     if (a.m <= 4u) return a.k == 1024u ? launch_blocks<F, 1, true>(d, q, grid) : a.k == 2048u ? launch_blocks<F, 2, true>(d, q, grid) : launch_blocks<F, 4, true>(d, q, grid);
     return a.k == 1024u ? launch_blocks<F, 1, false>(d, q, grid) : a.k == 2048u ? launch_blocks<F, 2, false>(d, q, grid) : launch_blocks<F, 4, false>(d, q, grid);
+    }
 }
 
 bool stream_accepts(const MvArgs &a, uint32_t block_bytes) {
@@ -581,6 +634,9 @@ bool stream_accepts(const MvArgs &a, uint32_t block_bytes) {
 // Whether these kernels can run the (already validated) arguments: k of whole units.
 bool matvec_q6k_mfma_stream_accepts(const MvArgs &a) { return stream_accepts(a, FmtQ6::BLOCK); }
 zhip_result launch_matvec_q6k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) { return launch_stream<FmtQ6>(d, a, w_bytes); }
+// Q8_0: rows of 1024 weights only (longer ones stay with the kernels that keep a tile resident).
+bool matvec_q8_0_mfma_flat_accepts(const MvArgs &a) { return a.k == 1024u && stream_accepts(a, FmtQ8::BLOCK); }
+zhip_result launch_matvec_q8_0_mfma_flat(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) { return launch_stream<FmtQ8>(d, a, w_bytes); }
 bool matvec_q3k_mfma_stream_accepts(const MvArgs &a) { return stream_accepts(a, FmtQ3::BLOCK); }
 zhip_result launch_matvec_q3k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) { return launch_stream<FmtQ3>(d, a, w_bytes); }
 
