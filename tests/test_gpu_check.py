@@ -448,7 +448,7 @@ def test_quant_matvec_mfma_variant(ctx, t, pair, rows, n, k, prologue):
     (8, 4112, 4096, 0, 0, False),    # 257 sixteen-row tiles: the kernel that streams whole tiles, two tiles on one workgroup
     (7, 4112, 2048, 5, 7, True),     # the same with eight blocks a wave, unaligned outputs, accumulating
     (2, 1536, 4096, 0, 0, True),
-    (8, 4112, 1024, 0, 0, False),    # four blocks a wave
+    (8, 4112, 1024, 0, 0, False),    # rows of 1024 weights: the kernel that moves a tile's 32 rows as one flat stretch
     (3, 4128, 1024, 5, 7, True),
 ])
 def test_matvec_q8_0_mfma_variant(ctx, rows, n, k, col0, pad, accumulate):

@@ -427,8 +427,7 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     if (D::CHUNK == 5 && matrix_cores && matvec_q5k_mfma_resident_accepts(a)) return launch_matvec_q5k_mfma_resident(d, a, d.bind[2].size);
     // (matvec_q6_k and matvec_q3_k: k of 1024, 2048 or 4096; every workgroup builds the tokens' operands, prologue included)
     if (D::CHUNK == 6 && matrix_cores && matvec_q6k_mfma_stream_accepts(a)) return launch_matvec_q6k_mfma_stream(d, a, d.bind[2].size);
-    // The kernels that keep the tokens' operands in registers (k of 2048 or 4096, for Q8_0 also
-    // 1024, and whole tiles) compute a step's prologue (RMSNorm, silu(x / act_div):
+    // The kernels that keep the tokens' operands in registers (k of 2048 or 4096 and whole tiles) compute a step's prologue (RMSNorm, silu(x / act_div):
     // src/kernels/matvec_quant.wgsl.hbs:73-89) themselves: their operands are built from one
     // round of loads, which the norm weights join (C3 at four tokens with the FFN launch's
     // RMSNorm: 22.6 us, 26.1 us with a pass of its own in front, 20.7 us without a prologue).

@@ -1,4 +1,4 @@
-// matvec_q8_0, matrix-core variant for steps of up to eight tokens and k = 1024, 2048 or 4096: the
+// matvec_q8_0, matrix-core variant for steps of up to eight tokens and k = 2048 or 4096: the
 // weight stream is read once for all tokens of the step and nothing but partial sums crosses
 // LDS. Contract as the other variants (src/kernels/matvec_quant.wgsl.hbs with the decoder of
 // src/kernels/quant/q8_0_dot.wgsl:5-14): out[t][col0 + j] (+)= sum over 32-weight blocks of
@@ -27,10 +27,10 @@
 // different banks. The eight waves' partial sums meet in LDS, where 128 threads add the eight
 // for one output each in the order of the k ranges and store. One barrier a tile; no barrier
 // waits for the loads in flight.
-// (k = 1024: a row and its scales are 1088 bytes, so every other row starts in the middle of a
-// cache line and a wave's 128 bytes of it lie across two: 151936 x 1024 runs at 42 us for one
-// to eight tokens, 3.9 TB/s against 6.6 TB/s at k = 4096 - still ahead of the default variant
-// from five tokens up: 29 / 42 / 78 us there at 1 / 4 / 8 tokens.)
+// (k = 1024 is not taken here: a row and its scales are 1088 bytes, so every other row starts
+// in the middle of a cache line and a wave's 128 bytes of it lie across two; 151936 x 1024 ran
+// at 42 us, 3.9 TB/s against 6.6 TB/s at k = 4096. Such rows go to the kernel that moves a
+// tile's rows as one stretch of whole lines, matvec_q6k_mfma_stream.hip.)
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -115,11 +115,10 @@ __device__ __forceinline__ void load_lds_b32(__amdgpu_buffer_rsrc_t buf, uint32_
 }
 
 // NS: 32-weight blocks of a wave's k range (k = 256 NS). The ring moves half tiles: the first or
-// second NS / 2 blocks of the wave's range of a tile's sixteen rows (at k = 1024 the whole range:
-// it is one 128-byte line a row). A slot: sixteen lines, then 256 bytes for the scales' load
+// second NS / 2 blocks of the wave's range of a tile's sixteen rows. A slot: sixteen lines, then 256 bytes for the scales' load
 // (two bytes a block and row; zeros from idle lanes behind).
 constexpr int DEPTH = 4;  // ring slots a wave: three half tiles in flight behind the one multiplied
-template <int NS> constexpr uint32_t slot_bytes() { return 16u * 32u * (NS >= 8 ? NS / 2 : NS) + 256u; }
+template <int NS> constexpr uint32_t slot_bytes() { return 16u * 32u * (NS / 2) + 256u; }
 constexpr uint32_t PART_BYTES = 2u * WAVES * 128u * 4u, SCALE_BYTES = 576u;  // [8 waves][8 tokens] maxima, [8] inverse scales, [8 waves][8 tokens] sums of squares
 template <int NS> constexpr uint32_t lds_bytes() { return PART_BYTES + SCALE_BYTES + WAVES * DEPTH * slot_bytes<NS>(); }
 static_assert(lds_bytes<16>() <= 160u * 1024u, "the rings must fit the CU's LDS");
@@ -131,7 +130,8 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
     float *lds_part = reinterpret_cast<float *>(lds);                  // [tile parity][wave][2 lane + token of the lane's two]
     float *lds_max = reinterpret_cast<float *>(lds + PART_BYTES);      // [wave][token]: the largest magnitude in the wave's range
     float *lds_inverse = lds_max + 64;                                 // [token]: one over the token's scale
-    constexpr int PARTS = NS >= 8 ? 2 : 1;  // ring slots a wave's range of a tile takes (k = 1024: one 128-byte line a row already)
+    static_assert(NS >= 8, "a half tile is whole 128-byte lines of every row");
+    constexpr int PARTS = 2;  // ring slots a wave's range of a tile takes
     constexpr int HB = NS / PARTS;           // blocks of a half tile
     constexpr uint32_t SLOT = slot_bytes<NS>(), LINE = 32u * HB, CHUNKS = 2u * HB;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, l16 = lane & 15u, g = lane >> 4;
@@ -360,10 +360,7 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
             load_half(u + s + (DEPTH - 1), (s + DEPTH - 1) % DEPTH);
             wait_loads<(DEPTH - 1) * LOADS>();
             if (u + s < PARTS * count) {
-                if constexpr (PARTS == 1) {
-                    multiply(std::integral_constant<int, 0>{}, s);
-                    finish(u + s);
-                } else if (s & 1) {
+                if (s & 1) {
                     multiply(std::integral_constant<int, 1>{}, s);
                     finish((u + s) >> 1);
                 } else {
@@ -380,7 +377,7 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
 // Whether this kernel can run the (already validated) arguments: whole tiles, k split into 4, 8
 // or 16 blocks a wave.
 bool matvec_q8_mfma_stream_accepts(const MvArgs &a) {
-    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && (!(a.flags & FLAG_SILU_PAIR) || a.half % 16u == 0) && a.rows % 16u == 0 &&
+    return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u) && (!(a.flags & FLAG_SILU_PAIR) || a.half % 16u == 0) && a.rows % 16u == 0 &&
            a.xr % 4u == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0;
 }
 
@@ -409,7 +406,7 @@ zhip_result launch_matvec_q8_mfma_stream(const Dispatch &d, const MvArgs &a, uin
     StreamArgs q{a, (uint32_t)w_bytes, tiles / groups, left, (tiles < groups || 2u * left <= groups) ? 1u : 0u, 0x64646464u};
     if (tiles < groups) { q.rounds = 0; q.left = tiles; }
     const dim3 grid(groups);
-    return a.k == 1024u ? launch_blocks<4>(d, q, grid) : a.k == 2048u ? launch_blocks<8>(d, q, grid) : launch_blocks<16>(d, q, grid);
+    return a.k == 2048u ? launch_blocks<8>(d, q, grid) : launch_blocks<16>(d, q, grid);
 }
 
 }  // namespace zhip
