@@ -741,6 +741,23 @@ def bench_c5(env):
         wantm = oracle.matmul_f64(xm, w)
         res[f"m{m}"] = env["hbm_entry"](f"C5: bf16 lm_head matvec M={m} K=1024 N=151936", 2 * n * k + 4 * m * k + 4 * m * n, wall, gpu_s, steps,
                                         {"copies": len(launches), "max_err_over_max_want": float(np.max(np.abs(got - wantm)) / np.max(np.abs(wantm)))})
+    # The same projection with Q8_0 weights (rows of 1024 weights with their scales: 1088 bytes,
+    # 8.5 cache lines): the default variant, and the matrix-core variant at verify widths.
+    mc = K.MatvecVariant(wg=512, lanes=64, rows=16)
+    raw = synth.random_blocks(synth.rng(0xC8), "q8_0", n, k)
+    wq = oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k)
+    e, bb = K.LAYOUT[TensorType.q8_0]
+    for m, variant in ((1, None), (4, None), (4, mc), (8, mc)):
+        xm = synth.activations(synth.rng(0xC8 + m), m, k)
+        launches, out = env["matvec_workload"](TensorType.q8_0, raw, n, k, m, False, xm, variant)
+        wall, gpu_s, steps = env["protocol"](launches)
+        got = env["read"](out)[: m * n].reshape(m, n)
+        wantm = oracle.matmul_f64(xm, wq)
+        res[f"q8_0_m{m}" + ("_matrix_cores" if variant else "")] = env["hbm_entry"](
+            f"q8_0 lm_head matvec M={m} K=1024 N=151936" + (", matrix-core variant" if variant else ""),
+            n * (k // e) * bb + 4 * m * k + 4 * m * n, wall, gpu_s, steps,
+            {"copies": len(launches), "max_err_over_max_want": float(np.max(np.abs(got - wantm)) / np.max(np.abs(wantm)))})
+    del wq
     # M = 128: the prefill multiply on the bf16 MFMA rung.
     rows = 128
     x = synth.activations(g, rows, k, bf16=True)

@@ -450,6 +450,7 @@ def test_quant_matvec_mfma_variant(ctx, t, pair, rows, n, k, prologue):
     (2, 1536, 4096, 0, 0, True),
     (8, 4112, 1024, 0, 0, False),    # rows of 1024 weights: the kernel that moves a tile's 32 rows as one flat stretch
     (3, 4128, 1024, 5, 7, True),
+    (4, 5, 1024, 1, 2, True),        # fewer rows than a unit of eight
 ])
 def test_matvec_q8_0_mfma_variant(ctx, rows, n, k, col0, pad, accumulate):
     """The matrix-core variant of matvec_q8_0 (the id of a wave per sixteen rows): every
