@@ -103,13 +103,16 @@ def bf16_tokens_case(c, m, n, k, col0=0, pad=0, accumulate=False, norm=False, x=
     return got, want, (x, bits)
 
 
-# Steps of several tokens over k = 1024 ... 4096 in steps of 512 and 16 MB or more of weights run
-# on the matrix cores, the weights read once for all tokens; every other shape keeps the
-# one-token kernel's path.
+# Steps of several tokens over k = 1024 ... 16384 in steps of 512 and 16 MB or more of weights run
+# on the matrix cores, the weights read once for all tokens, from the width on at which that
+# pays for the matrix ((tokens - 1) x bytes of 32 MB at k = 1024, 64 MB up to k = 4096, 192 MB
+# or four tokens beyond; five tokens always); every other step keeps the one-token kernel's path.
 @pytest.mark.parametrize("m,n,k,col0,pad,accumulate,norm", [
-    (2, 8192, 1024, 0, 0, False, False),
+    (2, 16400, 1024, 0, 0, False, False),
+    (2, 8192, 1024, 0, 0, False, False),       # two tokens over 16.8 MB: the general kernel
     (8, 8300, 1024, 0, 0, False, False),       # a ragged last unit of rows
-    (3, 5501, 1536, 5, 3, True, False),        # unaligned columns, accumulate
+    (3, 11001, 1536, 5, 3, True, False),       # unaligned columns, accumulate
+    (3, 5501, 1536, 5, 3, True, False),        # ... through the general kernel
     (4, 8200, 2048, 0, 0, False, False),       # a tail on every workgroup
     (5, 9000, 2560, 0, 0, False, True),        # the RMSNorm prologue
     (7, 2741, 3072, 32, 0, True, True),
@@ -119,9 +122,12 @@ def bf16_tokens_case(c, m, n, k, col0=0, pad=0, accumulate=False, norm=False, x=
     (4, 8192, 1024, 0, 0, False, True),        # k = 1024 with the prologue: the tokens split beforehand
     (19, 2052, 4096, 8, 0, True, False),
     (3, 100, 1024, 0, 0, False, False),        # a small matrix: the general kernel
-    (4, 1100, 9728, 0, 0, False, False),       # rows longer than 4096: stretches of columns, each launch adding to the one before
-    (2, 800, 14336, 3, 5, True, False),        # ... onto what the output already holds
-    (3, 1000, 8704, 0, 0, False, True),        # with the RMSNorm prologue: the tokens are normalised and split once for all the stretches
+    (5, 1100, 9728, 0, 0, False, False),       # rows longer than 4096: stretches of columns, each launch adding to the one before
+    (6, 800, 14336, 3, 5, True, False),        # ... onto what the output already holds
+    (5, 1000, 8704, 0, 0, False, True),        # with the RMSNorm prologue: the tokens are normalised and split once for all the stretches
+    (3, 1100, 9728, 0, 0, False, False),       # the same rows at widths the general kernel keeps: passes of as many tokens as fit workgroup memory
+    (2, 800, 14336, 3, 5, True, False),
+    (3, 1000, 8704, 0, 0, False, True),
 ])
 @pytest.mark.parametrize("half", HALVES)
 def test_matvec_bf16_several_tokens(ctx, half, m, n, k, col0, pad, accumulate, norm):
@@ -150,8 +156,9 @@ def test_matvec_bf16_several_tokens_many_rows(ctx):
 
 @pytest.mark.parametrize("half", HALVES)
 def test_matvec_bf16_several_tokens_keep_token_bits(ctx, half):
-    """A token's outputs do not depend on how many tokens share the step (from two tokens
-    up), nor on where the step's columns start."""
+    """A token's outputs do not depend on how many tokens share the step, on either side of
+    the width at which the matrix's steps move to the matrix cores (18 MB of weights: five
+    tokens), nor on where the step's columns start."""
     c = ctx
     m, n, k = 13, 4500, 2048
     x = c.random(m * k, 3).reshape(m, k)
@@ -166,8 +173,13 @@ def test_matvec_bf16_several_tokens_keep_token_bits(ctx, half):
         return c.read(out).reshape(len(tokens), rows)
 
     whole = run(list(range(m)), 0, n)
-    assert np.array_equal(run([4, 9], 0, n), whole[[4, 9]])
+    assert np.array_equal(run([4, 9, 1, 2, 6, 8], 0, n), whole[[4, 9, 1, 2, 6, 8]])
     assert np.array_equal(run([12, 0, 5, 7, 3], 0, n), whole[[12, 0, 5, 7, 3]])
+    # Below that width: the one-token step's bits.
+    few = run([4, 9, 11], 0, n)
+    for i, t in enumerate([4, 9, 11]):
+        assert np.array_equal(few[i], run([t], 0, n)[0])
+    assert np.array_equal(run([9, 4], 0, n), few[[1, 0]])
     assert np.array_equal(run(list(range(8)), 404, 4096), whole[:8, 404:])
     del wa
 
