@@ -45,7 +45,7 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=2000)
     ap.add_argument("--warmup", type=int, default=200)
-    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,c5,formats,down,replay,floor for the 'also' section; 'none' skips it")
+    ap.add_argument("--only", default="", help="comma-separated subset of: c1,c3,c4,c4_int8,long,c5,formats,down,replay,floor for the 'also' section; 'none' skips it")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline")
     ap.add_argument("--no-replay", action="store_true",
                     help="launch every dispatch of a repeated submit instead of replaying it from a HIP graph (for runs under a kernel tracer, "
@@ -309,7 +309,7 @@ def main() -> int:
     only = [s for s in args.only.split(",") if s]
     also = {}
     if "none" not in only:
-        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c4_int8", bench_c4_int8), ("c5", bench_c5), ("formats", bench_formats), ("down", bench_down), ("replay", bench_replay), ("floor", bench_floor)):
+        for name, fn in (("c1", bench_c1), ("c3", bench_c3), ("c4", bench_c4), ("c4_int8", bench_c4_int8), ("long", bench_long), ("c5", bench_c5), ("formats", bench_formats), ("down", bench_down), ("replay", bench_replay), ("floor", bench_floor)):
             if not only or name in only:
                 try:
                     also[name] = fn(locals())
@@ -654,6 +654,46 @@ def bench_c4(env):
         "reference_ladder_f32_activations": ladder,
         "vendor_library_context": vendor,
     }
+
+
+def bench_long(env):
+    """Longer prefill steps of the same multiply (2048 tokens): the 256 x 128 tiling."""
+    synth, oracle, K, TensorType, P = env["synth"], env["oracle"], env["K"], env["TensorType"], env["P"]
+    rec, kset, b = env["rec"], env["kset"], env["b"]
+    res = {}
+    for rows, k, n in ((2048, 4096, 4096), (2048, 4096, 14336)):
+        g = synth.rng(0x10 + n)
+        raw = synth.q8_0_rows(g, n, k)
+        x = synth.activations(g, rows, k, bf16=True)
+        kset.select_prefill(rec, K.Prefill.bf16_mfma_xbf16)
+        src = env["upload"](raw)
+        xa = env["upload"](synth.to_bf16_bits(x))
+        rb = K.row_bytes(TensorType.q8_0, k)
+        out = env["output"](4 * rows * n)
+        launches = []
+        for _ in range(3):
+            wa = env["output"](n * rb)
+            K.Launcher(rec, kset).layout(TensorType.q8_0, src, wa, n, k)
+            p = P.MatmulQuant(rows=rows, n=n, k=k, col0=0, out_stride=n, k_slice=k)
+            launches.append(env["L"](b.add(K.Kernel.matmul_q8_0_float, p, [xa, wa, out], K.Grid.tiles_y(K.div_ceil(n, 64), 16)), rows))
+        b.finish()
+        env["flush"]()
+        wall, gpu_s, steps = env["protocol"](launches)
+        kset.select_prefill(rec, K.Prefill.scalar_f32)
+        # Checked on every 16th token (the whole product in float64 would take the CPU longer than the bench).
+        got = env["read"](out)[: rows * n].reshape(rows, n)[::16].astype(np.float64)
+        w = oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k)
+        want = x[::16].astype(np.float64) @ w.astype(np.float64).T
+        flops = 2 * rows * n * k
+        res[f"m{rows}_k{k}_n{n}"] = {
+            "workload": f"Q8_0 prefill matmul M={rows} K={k} N={n}, packed bf16 activations, bf16 MFMA, fp32 accumulate; 3 weight copies",
+            "flops_per_step": flops,
+            "us_per_launch_gpu": round(gpu_s / steps * 1e6, 3),
+            "TFLOPs_gpu": round(flops * steps / gpu_s / 1e12, 1),
+            "mfma_frac": round(flops * steps / gpu_s / 1e12 / MFMA_BF16_PEAK_TFLOPS, 4),
+            "max_err_over_max_want": float(np.max(np.abs(got - want)) / np.max(np.abs(want))),
+        }
+    return res
 
 
 def bench_c4_int8(env):
