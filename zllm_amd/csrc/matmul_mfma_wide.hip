@@ -13,11 +13,16 @@
 // pulls from L2 per flop.
 //
 // Tiling: 512 threads = eight wave64s as 4 (tokens) x 2 (outputs), each wave a
-// 64 x 64 quadrant of the 256 x 128 tile as 4 x 4 MFMA tiles of 16 x 16 x 32:
+// 64 x 64 quadrant of the 256 x 128 tile as 2 x 2 MFMA tiles of 32 x 32 x 16:
 // two waves per SIMD, so one wave's LDS waits, conversions and barrier hide
 // behind the other's MFMAs. k tiles are 64 deep and double buffered in LDS
 // (rows padded to 144 bytes: conflict-free 16-byte fragment reads); three k
-// tiles of global loads are kept in flight in registers.
+// tiles of global loads are kept in flight in registers. Vector and matrix
+// instructions share a SIMD's issue on this machine, so what a k tile costs in
+// vector instructions is paid in full: the loads are buffer loads whose lane
+// offsets never change and whose uniform offset is the tile's position (2048 x
+// 4096 x 4096: 86.8 -> 81.5 us from that alone; the 32 x 32 x 16 form of the
+// matrix instruction instead of 16 x 16 x 32 measured the same).
 //
 // The launcher picks this tiling only when its tiles fill the CUs; smaller
 // steps take the 128 x 64 tiling of matmul_mfma.hip.
@@ -32,9 +37,16 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
 namespace wide {
+
+// Range-checked loads: the address is a lane's offset plus a uniform one, so a k tile's loads
+// take no vector arithmetic, and rows past the step or the matrix read zeros.
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const uint8_t *base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, (int)bytes, 0x00020000);
+}
 
 constexpr int GM = 256, GN = 128, GK = 64, THREADS = 512;
 constexpr int ROW = GK * 2 + 16;                 // LDS bytes per tile row
@@ -57,9 +69,13 @@ __device__ __forceinline__ uint32_t pack_bf16(float lo, float hi) {
 // A thread stages 16 weights of one row per k tile: row = tid / 4, quarter = tid % 4.
 struct WQ8_0 {
     struct Regs { u32x4 q; uint32_t d; };
-    __device__ static void load(const uint8_t *row, uint32_t k, uint32_t kpos, Regs &r) {
-        r.q = *reinterpret_cast<const u32x4 *>(row + kpos);
-        r.d = *reinterpret_cast<const uint16_t *>(row + k + 2u * (kpos / 32u));
+    // The lane's offsets in the tile's rows: of the sixteen quants from position pos on and of their block's scale.
+    __device__ static uint32_t quant_offset(uint32_t row_off, uint32_t pos) { return row_off + pos; }
+    __device__ static uint32_t scale_offset(uint32_t row_off, uint32_t k, uint32_t pos) { return row_off + k + 2u * (pos / 32u); }
+    // (kpos: a uniform multiple of 64 positions added to the lane's)
+    __device__ static void load(__amdgpu_buffer_rsrc_t buf, uint32_t qoff, uint32_t doff, uint32_t kpos, Regs &r) {
+        r.q = __builtin_amdgcn_raw_buffer_load_b128(buf, qoff, kpos, 0);
+        r.d = __builtin_amdgcn_raw_buffer_load_b16(buf, doff, kpos / 32u * 2u, 0);
     }
     __device__ static void store(const Regs &r, u32x4 *dst) {
         const float d = half_bits_to_float(r.d);
@@ -81,10 +97,11 @@ struct WQ8_0 {
 
 struct WBf16 {
     struct Regs { u32x4 v[2]; };
-    __device__ static void load(const uint8_t *row, uint32_t, uint32_t kpos, Regs &r) {
-        const u32x4 *src = reinterpret_cast<const u32x4 *>(row + 2u * kpos);
-        r.v[0] = src[0];
-        r.v[1] = src[1];
+    __device__ static uint32_t quant_offset(uint32_t row_off, uint32_t pos) { return row_off + 2u * pos; }
+    __device__ static uint32_t scale_offset(uint32_t, uint32_t, uint32_t) { return 0u; }
+    __device__ static void load(__amdgpu_buffer_rsrc_t buf, uint32_t qoff, uint32_t, uint32_t kpos, Regs &r) {
+        r.v[0] = __builtin_amdgcn_raw_buffer_load_b128(buf, qoff, 2u * kpos, 0);
+        r.v[1] = __builtin_amdgcn_raw_buffer_load_b128(buf, qoff + 16u, 2u * kpos, 0);
     }
     __device__ static void store(const Regs &r, u32x4 *dst) {
         dst[0] = r.v[0];
@@ -113,36 +130,45 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_wide_kernel(Args a) {
     const uint32_t j0 = nt * GN, t0 = mt * GM;
     const uint32_t kb = 0, ke = a.k;
     const uint32_t wm = (wave >> 1) * 64u, wn = (wave & 1u) * 64u;
-    const uint32_t lrow = lane & 15u, lk = (lane >> 4) * 16u;
+    const uint32_t lrow = lane & 31u, lk = (lane >> 5) * 16u;
 
-    f32x4 acc[4][4];
+    f32x16 acc[2][2];
 #pragma unroll
-    for (int i = 0; i < 4; i++)
+    for (int i = 0; i < 2; i++)
 #pragma unroll
-        for (int j = 0; j < 4; j++) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+        for (int j = 0; j < 2; j++)
+#pragma unroll
+            for (int e = 0; e < 16; e++) acc[i][j][e] = 0.f;
 
-    // Staging assignments. Rows past the matrix or the step are clamped: their
-    // results are never stored.
+    // Staging assignments. The tile's rows of tokens and of weights are a buffer each: rows past
+    // the step or the matrix read zeros, and their results are never stored.
     const uint32_t wrow = tid >> 2, wq = tid & 3u;
-    const uint32_t wj = min(j0 + wrow, a.n - 1u);
-    const uint8_t *wsrc = a.w + (size_t)wj * a.row_bytes;
+    const uint32_t wrows = min((uint32_t)GN, a.n - j0), xrows = min((uint32_t)GM, a.rows - t0);
+    const __amdgpu_buffer_rsrc_t wbuf = make_buffer(a.w + (size_t)j0 * a.row_bytes, wrows * a.row_bytes);
+    const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.x + (size_t)t0 * a.k * 2u, xrows * a.k * 2u);
+    const uint32_t wqoff = W::quant_offset(wrow * a.row_bytes, 16u * wq), wdoff = W::scale_offset(wrow * a.row_bytes, a.k, 16u * wq);
     uint8_t *wdst = ws + wrow * ROW + 32u * wq;
     const uint32_t xr0 = tid >> 3, xpiece = tid & 7u;
-    const uint8_t *xsrc[4];
+    uint32_t xoff[4];
 #pragma unroll
-    for (int i = 0; i < 4; i++) xsrc[i] = a.x + (size_t)min(t0 + xr0 + 64u * i, a.rows - 1u) * a.k * 2u;
+    for (int i = 0; i < 4; i++) xoff[i] = (xr0 + 64u * i) * a.k * 2u + 16u * xpiece;
     uint8_t *xdst = xs + xr0 * ROW + 16u * xpiece;
-    const uint32_t wk_last = ke - 16u, xk_last = ke - 8u;
+    const uint32_t wk_last = ke - 16u;
 
-    // Loads are unconditional (positions clamped into the split) so no branch
-    // separates them from their use; a tile that straddles the end of the split
-    // zeroes its activations instead, which zeroes the products whatever finite
-    // weights the clamped loads brought.
+    // Loads are unconditional, so no branch separates them from their use; a tile that
+    // straddles the end of k zeroes its activations instead (a load past a row's end brings
+    // the next row's start), which zeroes the products whatever finite weights came: the
+    // weights' positions are clamped into the row there, so that a scale is a scale. Whole
+    // tiles take the tile's position as the loads' uniform offset: no vector arithmetic.
     auto fetch = [&](uint32_t k0, typename W::Regs &w, XRegs &x) __attribute__((always_inline)) {
-        W::load(wsrc, a.k, min(k0 + 16u * wq, wk_last), w);
-        const uint32_t xk = min(k0 + 8u * xpiece, xk_last);
+        if (RAGGED) {
+            const uint32_t pos = min(k0 + 16u * wq, wk_last);
+            W::load(wbuf, W::quant_offset(wrow * a.row_bytes, pos), W::scale_offset(wrow * a.row_bytes, a.k, pos), 0u, w);
+        } else {
+            W::load(wbuf, wqoff, wdoff, k0, w);
+        }
 #pragma unroll
-        for (int i = 0; i < 4; i++) x.v[i] = *reinterpret_cast<const u32x4 *>(xsrc[i] + 2u * xk);
+        for (int i = 0; i < 4; i++) x.v[i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, xoff[i], 2u * k0, 0);
     };
     auto commit = [&](uint32_t b, uint32_t k0, const typename W::Regs &w, XRegs &x) __attribute__((always_inline)) {
         if (RAGGED && k0 + 8u * xpiece >= ke) {
@@ -159,16 +185,16 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_wide_kernel(Args a) {
         const uint8_t *xb = xs + cur * XS + (wm + lrow) * ROW + lk;
         const uint8_t *wb = ws + cur * WS + (wn + lrow) * ROW + lk;
 #pragma unroll
-        for (int kk = 0; kk < GK / 32; kk++) {
-            bf16x8 af[4], bfr[4];
+        for (int kk = 0; kk < GK / 16; kk++) {
+            bf16x8 af[2], bfr[2];
 #pragma unroll
-            for (int i = 0; i < 4; i++) af[i] = *reinterpret_cast<const bf16x8 *>(xb + 16 * i * ROW + 64 * kk);
+            for (int i = 0; i < 2; i++) af[i] = *reinterpret_cast<const bf16x8 *>(xb + 32 * i * ROW + 32 * kk);
 #pragma unroll
-            for (int j = 0; j < 4; j++) bfr[j] = *reinterpret_cast<const bf16x8 *>(wb + 16 * j * ROW + 64 * kk);
+            for (int j = 0; j < 2; j++) bfr[j] = *reinterpret_cast<const bf16x8 *>(wb + 32 * j * ROW + 32 * kk);
 #pragma unroll
-            for (int i = 0; i < 4; i++)
+            for (int i = 0; i < 2; i++)
 #pragma unroll
-                for (int j = 0; j < 4; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
+                for (int j = 0; j < 2; j++) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
         }
         if (kc + GK < ke) commit(cur ^ 1u, kc + GK, wnext, xnext);
         __syncthreads();
@@ -197,26 +223,27 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_wide_kernel(Args a) {
     }
 
     // D[output][token] (the weights are the MFMA's first operand): the lane holds
-    // outputs 4 (lane / 16) .. + 3 of token lane % 16 in each 16 x 16 tile, sixteen
-    // contiguous bytes of the token's row.
+    // outputs 8 r + 4 (lane / 32) .. + 3, r = 0 .. 3, of token lane % 32 in each 32 x 32
+    // tile: sixteen contiguous bytes of the token's row four times.
     const bool aligned = ((a.out_stride | a.col0) & 3u) == 0u && (reinterpret_cast<uintptr_t>(a.out) & 15u) == 0u;
 #pragma unroll
-    for (int i = 0; i < 4; i++) {
-        const uint32_t t = t0 + wm + 16 * i + lrow;
+    for (int i = 0; i < 2; i++) {
+        const uint32_t t = t0 + wm + 32 * i + lrow;
 #pragma unroll
-        for (int j = 0; j < 4; j++) {
-            const uint32_t col = j0 + wn + 16 * j + 4 * (lane >> 4);
+        for (int jr = 0; jr < 8; jr++) {
+            const int j = jr >> 2, r = jr & 3;
+            const uint32_t col = j0 + wn + 32 * j + 8 * r + 4 * (lane >> 5);
             if (t >= a.rows || col >= a.n) continue;
             float *o = a.out + (size_t)t * a.out_stride + a.col0 + col;
-            f32x4 v = acc[i][j];
+            f32x4 v = f32x4{acc[i][j][4 * r], acc[i][j][4 * r + 1], acc[i][j][4 * r + 2], acc[i][j][4 * r + 3]};
             if (aligned && col + 3u < a.n) {
                 f32x4 *o4 = reinterpret_cast<f32x4 *>(o);
                 if (a.accumulate) v += *o4;
                 *o4 = v;
             } else {
 #pragma unroll
-                for (int r = 0; r < 4; r++)
-                    if (col + r < a.n) o[r] = a.accumulate ? o[r] + v[r] : v[r];
+                for (int e = 0; e < 4; e++)
+                    if (col + e < a.n) o[e] = a.accumulate ? o[e] + v[e] : v[e];
             }
         }
     }
