@@ -82,6 +82,55 @@ __device__ __forceinline__ KScales chunk_scales(const uint4 &h, uint32_t s16, bo
     return s;
 }
 
+// The same four values for a lane whose chunk never changes: what depends on the chunk alone
+// (which header bytes, which bit fields) is worked out once, and a header costs eight integer
+// operations instead of fourteen. Lower chunks (c < 2) take the low six bits of bytes 2c, 2c + 1
+// of the scale and of the min words; upper ones the nibbles of bytes 2c + 4, 2c + 5 of the
+// third word with the top two bits of the lower chunks' bytes above them.
+struct ChunkKeys {
+    uint32_t sel;     // v_perm_b32 selector: bytes 2 (c & 1), + 1 of the scale word, then of the min word
+    uint32_t shift;   // 16 (c & 1)
+    uint32_t six;     // 0x3f3f3f3f for lower chunks, else 0
+    uint32_t top;     // 0x30303030 for upper chunks, else 0
+    uint32_t lo, hi;  // 0x0f0f, 0xf0f0 for upper chunks, else 0
+    uint32_t c;       // the chunk
+};
+__device__ __forceinline__ ChunkKeys chunk_keys(uint32_t c) {
+    const bool upper = c >= 2u;
+    ChunkKeys k;
+    k.sel = (c & 1u) ? 0x07060302u : 0x05040100u;
+    k.shift = 16u * (c & 1u);
+    k.six = upper ? 0u : 0x3f3f3f3fu;
+    k.top = upper ? 0x30303030u : 0u;
+    k.lo = upper ? 0x0f0fu : 0u;
+    k.hi = upper ? 0xf0f0u : 0u;
+    k.c = c;
+    return k;
+}
+template <bool SIXTEENTH>
+__device__ __forceinline__ KScales chunk_scales(const uint4 &h, const ChunkKeys &k) {
+    const float d = half_bits_to_float(h.x & 0xffffu);
+    const float dmin = half_bits_to_float(h.x >> 16);
+    const uint32_t w = __builtin_amdgcn_perm(h.z, h.y, k.sel);  // scale bytes, min bytes
+    const uint32_t a2 = h.w >> k.shift;
+    uint32_t r = w & k.six;
+    r = ((w >> 2) & k.top) | r;
+    r = (a2 & k.lo) | r;
+    r = ((a2 & k.hi) << 12) | r;  // bytes: scale 2c, scale 2c + 1, min 2c, min 2c + 1
+    KScales s;
+    s.d1 = d * cvt_byte<0>(r);
+    s.d2 = SIXTEENTH ? d * cvt_byte<1>(r) * 0.0625f : d * cvt_byte<1>(r);
+    s.m1 = dmin * cvt_byte<2>(r);
+    s.m2 = dmin * cvt_byte<3>(r);
+    return s;
+}
+// (the form the kernels whose lanes change chunks call)
+template <bool SIXTEENTH>
+__device__ __forceinline__ KScales chunk_scales(const uint4 &h, uint32_t c) { return chunk_scales<SIXTEENTH>(h, 16u * (c & 1u), c >= 2u); }
+
+__device__ __forceinline__ uint32_t chunk_no(uint32_t c) { return c; }
+__device__ __forceinline__ uint32_t chunk_no(const ChunkKeys &k) { return k.c; }
+
 __device__ __forceinline__ uint32_t word_of(const uint4 &v, int i) { return i == 0 ? v.x : i == 1 ? v.y : i == 2 ? v.z : v.w; }
 
 // Four weights (the bytes of `word`) times four inputs, added to `sum`.
@@ -93,12 +142,18 @@ __device__ __forceinline__ float dot_bytes(uint32_t word, const float4 &x, float
     return sum;
 }
 
+// A buffer offset no binding reaches (bindings end below 2 GiB): a load there returns zeros
+// and moves nothing.
+constexpr uint32_t kNowhere = 0x80000000u;
+
 // ---- the formats ---------------------------------------------------------------------
 // A format names its task's vectors (Raw), loads them, says where a row's
 // inputs go in task order, and multiplies one task of one row (ROWS = 1) or of
 // the two rows of a pass (ROWS = 2) for MT tokens. x(t, v) gives inputs
 // 4v .. 4v + 3 of the task in task order for token t; sums(t, s) the sum of the
-// task's s-th run of 64 / NSUM inputs.
+// task's s-th run of 64 / NSUM inputs. where() gives the byte offsets of a task's vectors from
+// the start of a stretch of rows (base: the row's offset in the stretch) and fetch() loads them
+// through a range-checked buffer that begins at the stretch.
 
 // Q8_0 split rows (src/kernels/repack_q8_0.wgsl): k signed bytes, then k / 32
 // f16 scales. Task = 64 consecutive weights, two blocks of 32 with a scale each;
@@ -120,8 +175,22 @@ struct KQ8 {
         r.d = *reinterpret_cast<const uint32_t *>(row + k + 4u * task);
         return r;
     }
+    struct Where {
+        uint32_t q, d;
+    };
+    __device__ static Where where(uint32_t base, uint32_t k, uint32_t task) { return Where{base + 64u * task, base + k + 4u * task}; }
+    __device__ static Where nowhere() { return Where{kNowhere, kNowhere}; }
+    __device__ static Raw fetch(__amdgpu_buffer_rsrc_t w, const Where &at) {
+        Raw r;
+#pragma unroll
+        for (int i = 0; i < 4; i++) r.q[i] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.q + 16u * i, 0, 0));
+        r.d = __builtin_amdgcn_raw_buffer_load_b32(w, at.d, 0, 0);
+        return r;
+    }
     __device__ static uint32_t stage_index(uint32_t v) { return v; }
 
+    typedef uint32_t Keys;
+    __device__ static Keys keys(uint32_t c) { return c; }
     template <int MT, int ROWS, class XF, class SF>
     __device__ static void dot(const Raw (&r)[ROWS], uint32_t, Masks, XF x, SF, float (&out)[ROWS][MT]) {
         float s[ROWS][MT][2];
@@ -178,8 +247,21 @@ struct KQ3 {
         r.u[1] = *reinterpret_cast<const uint4 *>(block + 32u * c + 16u);
         return r;
     }
+    struct Where {
+        uint32_t u;
+    };
+    __device__ static Where where(uint32_t base, uint32_t, uint32_t task) { return Where{base + (task >> 2) * BLOCK_BYTES + 32u * (task & 3u)}; }
+    __device__ static Where nowhere() { return Where{kNowhere}; }
+    __device__ static Raw fetch(__amdgpu_buffer_rsrc_t w, const Where &at) {
+        Raw r;
+        r.u[0] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.u, 0, 0));
+        r.u[1] = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.u + 16u, 0, 0));
+        return r;
+    }
     __device__ static uint32_t stage_index(uint32_t v) { return v; }
 
+    typedef uint32_t Keys;
+    __device__ static Keys keys(uint32_t c) { return c; }
     template <int MT, int ROWS, class XF, class SF>
     __device__ static void dot(const Raw (&r)[ROWS], uint32_t, Masks nm, XF x, SF sums, float (&out)[ROWS][MT]) {
         float s[ROWS][MT][4];
@@ -253,10 +335,27 @@ struct KQ4 {
         r.q1 = *reinterpret_cast<const uint4 *>(block + 32u + 32u * c);
         return r;
     }
+    struct Where {
+        uint32_t h, q;
+    };
+    __device__ static Where where(uint32_t base, uint32_t, uint32_t task) {
+        const uint32_t block = base + (task >> 2) * BLOCK_BYTES;
+        return Where{block, block + 16u + 32u * (task & 3u)};
+    }
+    __device__ static Where nowhere() { return Where{kNowhere, kNowhere}; }
+    __device__ static Raw fetch(__amdgpu_buffer_rsrc_t w, const Where &at) {
+        Raw r;
+        r.h = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.h, 0, 0));
+        r.q0 = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.q, 0, 0));
+        r.q1 = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.q + 16u, 0, 0));
+        return r;
+    }
     __device__ static uint32_t stage_index(uint32_t v) { return v; }
 
-    template <int MT, int ROWS, class XF, class SF>
-    __device__ static void dot(const Raw (&r)[ROWS], uint32_t c, Masks nm, XF x, SF sums, float (&out)[ROWS][MT]) {
+    typedef ChunkKeys Keys;
+    __device__ static Keys keys(uint32_t c) { return chunk_keys(c); }
+    template <int MT, int ROWS, class C, class XF, class SF>
+    __device__ static void dot(const Raw (&r)[ROWS], const C &c, Masks nm, XF x, SF sums, float (&out)[ROWS][MT]) {
         float s_lo[ROWS][MT], s_hi[ROWS][MT];
 #pragma unroll
         for (int j = 0; j < ROWS; j++)
@@ -283,7 +382,7 @@ struct KQ4 {
         }
 #pragma unroll
         for (int j = 0; j < ROWS; j++) {
-            const KScales s = chunk_scales<true>(r[j].h, 16u * (c & 1u), c >= 2u);
+            const KScales s = chunk_scales<true>(r[j].h, c);
 #pragma unroll
             for (int t = 0; t < MT; t++) {
                 float v = s.d1 * s_lo[j][t];
@@ -320,10 +419,29 @@ struct KQ5 {
         r.q1 = *reinterpret_cast<const uint4 *>(block + 64u + 32u * c);
         return r;
     }
+    struct Where {
+        uint32_t h, q;
+    };
+    __device__ static Where where(uint32_t base, uint32_t, uint32_t task) {
+        const uint32_t block = base + (task >> 2) * BLOCK_BYTES;
+        return Where{block, block + 48u + 32u * (task & 3u)};
+    }
+    __device__ static Where nowhere() { return Where{kNowhere, kNowhere}; }
+    __device__ static Raw fetch(__amdgpu_buffer_rsrc_t w, const Where &at) {
+        Raw r;
+        r.h = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.h, 0, 0));
+        r.b0 = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.h + 16u, 0, 0));
+        r.b1 = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.h + 32u, 0, 0));
+        r.q0 = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.q, 0, 0));
+        r.q1 = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.q + 16u, 0, 0));
+        return r;
+    }
     __device__ static uint32_t stage_index(uint32_t v) { return v; }
 
-    template <int MT, int ROWS, class XF, class SF>
-    __device__ static void dot(const Raw (&r)[ROWS], uint32_t c, Masks nm, XF x, SF sums, float (&out)[ROWS][MT]) {
+    typedef ChunkKeys Keys;
+    __device__ static Keys keys(uint32_t c) { return chunk_keys(c); }
+    template <int MT, int ROWS, class C, class XF, class SF>
+    __device__ static void dot(const Raw (&r)[ROWS], const C &c, Masks nm, XF x, SF sums, float (&out)[ROWS][MT]) {
         float s_lo[ROWS][MT], s_hi[ROWS][MT];
 #pragma unroll
         for (int j = 0; j < ROWS; j++)
@@ -335,7 +453,7 @@ struct KQ5 {
 #pragma unroll
             for (int j = 0; j < ROWS; j++) {
                 const uint32_t word = word_of(e < 4 ? r[j].q0 : r[j].q1, e & 3);
-                const uint32_t bits = word_of(e < 4 ? r[j].b0 : r[j].b1, e & 3) >> (2u * c);
+                const uint32_t bits = word_of(e < 4 ? r[j].b0 : r[j].b1, e & 3) >> (2u * chunk_no(c));
                 lo[j] = ((bits & nm.one) << 4) | (word & nm.lo);
                 hi[j] = (((bits >> 1) & nm.one) << 4) | ((word >> 4) & nm.lo);
             }
@@ -351,7 +469,7 @@ struct KQ5 {
         }
 #pragma unroll
         for (int j = 0; j < ROWS; j++) {
-            const KScales s = chunk_scales<false>(r[j].h, 16u * (c & 1u), c >= 2u);
+            const KScales s = chunk_scales<false>(r[j].h, c);
 #pragma unroll
             for (int t = 0; t < MT; t++) {
                 float v = s.d1 * s_lo[j][t];
@@ -393,12 +511,31 @@ struct KQ6 {
         r.d = *reinterpret_cast<const uint32_t *>(block + 208u);
         return r;
     }
+    struct Where {
+        uint32_t l, h, sc, d;
+    };
+    __device__ static Where where(uint32_t base, uint32_t, uint32_t task) {
+        const uint32_t block = base + (task >> 2) * BLOCK_BYTES, n = (task >> 1) & 1u, lh = task & 1u;
+        return Where{block + 64u * n + 16u * lh, block + 128u + 32u * n + 16u * lh, block + 192u + 8u * n, block + 208u};
+    }
+    __device__ static Where nowhere() { return Where{kNowhere, kNowhere, kNowhere, kNowhere}; }
+    __device__ static Raw fetch(__amdgpu_buffer_rsrc_t w, const Where &at) {
+        Raw r;
+        r.l0 = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.l, 0, 0));
+        r.l1 = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.l + 32u, 0, 0));
+        r.hv = __builtin_bit_cast(uint4, __builtin_amdgcn_raw_buffer_load_b128(w, at.h, 0, 0));
+        r.sc = __builtin_bit_cast(uint2, __builtin_amdgcn_raw_buffer_load_b64(w, at.sc, 0, 0));
+        r.d = __builtin_amdgcn_raw_buffer_load_b32(w, at.d, 0, 0);
+        return r;
+    }
     // Vector v of a row (inputs 4v ..) is vector q of run r of task 4 blk + 2 n + lh.
     __device__ static uint32_t stage_index(uint32_t v) {
         const uint32_t blk = v >> 6, n = (v >> 5) & 1u, run = (v >> 3) & 3u, lh = (v >> 2) & 1u, q = v & 3u;
         return 64u * blk + 32u * n + 16u * lh + 4u * run + q;
     }
 
+    typedef uint32_t Keys;
+    __device__ static Keys keys(uint32_t c) { return c; }
     template <int MT, int ROWS, class XF, class SF>
     __device__ static void dot(const Raw (&r)[ROWS], uint32_t p, Masks nm, XF x, SF sums, float (&out)[ROWS][MT]) {
         float s[ROWS][MT][4];
@@ -460,8 +597,11 @@ __device__ __forceinline__ float segment_sum(float v, uint32_t seg_log2) {
     v = dpp_add<0x4E, 0xF>(v);   // quad_perm [2,3,0,1]
     v = dpp_add<0x141, 0xF>(v);  // row_half_mirror
     v = dpp_add<0x140, 0xF>(v);  // row_mirror: every lane holds its row of 16's sum
-    if (seg_log2 >= 5) v = dpp_add<0x142, 0xA>(v);  // row_bcast15 into rows 1 and 3
-    if (seg_log2 >= 6) v = dpp_add<0x143, 0xC>(v);  // row_bcast31 into rows 2 and 3
+    // (one instruction each: the rows the mask leaves out keep their value, where update_dpp's
+    // form adds a zero to it; the segments' last lanes, which hold the totals, are in rows the
+    // masks name. The s_nop covers the two wait states between a vector write and a DPP read.)
+    if (seg_log2 >= 5) asm("s_nop 1\n\tv_add_f32_dpp %0, %0, %0 row_bcast:15 row_mask:0xa" : "+v"(v));  // into rows 1 and 3
+    if (seg_log2 >= 6) asm("s_nop 1\n\tv_add_f32_dpp %0, %0, %0 row_bcast:31 row_mask:0xc" : "+v"(v));  // into rows 2 and 3
     return v;
 }
 
@@ -770,6 +910,181 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
         }
     }
     if (P::DEFER && XREG && q.defer) flush_kept();
+}
+
+// One-token steps over rows of at most 64 tasks: the kernel above with XREG, taken apart so that
+// the loop holds nothing but the weight stream's loads and the multiply. A wave's walk is wave
+// uniform here: pass u covers rows u * RPI .. + RPI - 1 (RPI = 64 >> SEG_LOG2 rows side by side
+// in the wave), so the pass's position lives in scalar registers, a lane's byte offsets within
+// the pass never change (P::Where, computed once), and a pass's loads go through a buffer that
+// begins at the pass's first row and ends with the matrix: rows past the end, lanes without a
+// task and the loads after a wave's last pass all fall outside it and return zeros, which the
+// multiply turns into a sum of zero; no address arithmetic, clamp or branch per lane is left.
+// The staging of the inputs, a task's dot product and the lanes' reduction are the code of the
+// kernel above, so the results are its bits.
+// Passes whose loads are in flight ahead of the one multiplied, and workgroups a CU. Measured on
+// 14336 x 4096 Q4_K (7.9 us with 1 and 3): two or three passes ahead 8.6 / 9.8 us, four or five
+// workgroups 8.2 / 9.3 us, one workgroup with three passes ahead 9.8 us.
+constexpr int kRowDepth = 1;
+constexpr uint32_t kRowWorkgroups = 3;
+template <class P, bool PAIR, int SEG_LOG2>
+__global__ __launch_bounds__(256) void matvec_quant_row_kernel(KArgs q) {
+    const MvArgs &a = q.a;
+    extern __shared__ float4 lds4[];
+    __shared__ float red[4];
+    constexpr int NSUM = P::NSUM, RUN = 64 / NSUM, kRows = PAIR ? 2 : 1;
+    constexpr uint32_t SEG = 1u << SEG_LOG2, RPI = 64u >> SEG_LOG2;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
+    const uint32_t tasks = q.tasks, k4 = a.k / 4u;
+    const uint32_t tsub = lane & (SEG - 1u), rsub = lane >> SEG_LOG2;
+    const uint32_t units = (a.rows + RPI - 1u) / RPI;
+    const uint32_t gwave = blockIdx.x * 4u + (uint32_t)__builtin_amdgcn_readfirstlane((int)wave), nwaves = gridDim.x * 4u;
+
+    // The token's inputs (and norm weights) are asked for first, then the first rows: loads
+    // complete in order within a wave.
+    const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)q.t0 * a.xr);
+    const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
+    float4 xv[4], gv[4];
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t i = tid + 256u * j;
+        xv[j] = i < k4 ? xrow[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    if (a.flags & FLAG_NORM) {
+#pragma unroll
+        for (int j = 0; j < 4; j++) gv[j] = tid + 256u * j < k4 ? nw[tid + 256u * j] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+
+    const typename P::Where at = tsub < tasks ? P::where(rsub * a.row_bytes, a.k, tsub) : P::nowhere();
+    const uint64_t span = (uint64_t)a.rows * a.row_bytes;  // bytes of the rows covered (and of their up rows)
+    const uint64_t pass_bytes = (uint64_t)RPI * a.row_bytes;
+    // Pass u's rows, and with PAIR the up rows of its outputs.
+    auto fetch = [&](uint32_t u, typename P::Raw (&dst)[kRows]) __attribute__((always_inline)) {
+        const bool live = u < units;
+        const uint64_t off = live ? u * pass_bytes : 0u;
+        const uint32_t left = live ? (uint32_t)(span - off) : 0u;
+        dst[0] = P::fetch(__builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a.w + off), 0, (int)left, 0x00020000), at);
+        if (PAIR) dst[kRows - 1] = P::fetch(__builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a.w + (size_t)a.half * a.row_bytes + off), 0, (int)left, 0x00020000), at);
+        __builtin_amdgcn_sched_barrier(0);  // (the loads stay ahead of the multiply that follows them in the source)
+    };
+    typename P::Raw buf[kRowDepth + 1][kRows];
+#pragma unroll
+    for (int dpt = 0; dpt < kRowDepth; dpt++) fetch(gwave + dpt * nwaves, buf[dpt]);
+
+    // stage_token's arithmetic on the vectors already loaded.
+    float scale = 1.0f;
+    if (a.flags & FLAG_NORM) {
+        float ss = 0.f;
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+            if (tid + 256u * j < k4) ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w;
+        ss = wave_sum(ss);
+        if (lane == 0) red[wave] = ss;
+        __syncthreads();
+        const float total = (red[0] + red[1]) + (red[2] + red[3]);
+        scale = 1.0f / sqrtf(total / (float)a.k + a.eps);
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++) {
+        const uint32_t i = tid + 256u * j;
+        if (i >= k4) continue;
+        float4 v = xv[j];
+        if (a.flags & FLAG_NORM) {
+            v.x = v.x * scale * gv[j].x; v.y = v.y * scale * gv[j].y;
+            v.z = v.z * scale * gv[j].z; v.w = v.w * scale * gv[j].w;
+        }
+        if (a.act_div > 0.f) {
+            v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
+            v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+        }
+        const uint32_t p = P::stage_index(i);
+        lds4[p + (p >> 4)] = v;
+    }
+    __syncthreads();
+    if (gwave >= units) return;
+
+    // The lane's task's inputs and their runs' sums, for the whole walk.
+    float xr[64], xsum[NSUM];
+    {
+        const float4 *src = lds4 + (tsub < tasks ? tsub : 0u) * (kTaskStride / 4u);
+#pragma unroll
+        for (int v = 0; v < 16; v++) {
+            const float4 f = tsub < tasks ? src[v] : make_float4(0.f, 0.f, 0.f, 0.f);
+            xr[4 * v] = f.x; xr[4 * v + 1] = f.y; xr[4 * v + 2] = f.z; xr[4 * v + 3] = f.w;
+        }
+#pragma unroll
+        for (int s = 0; s < NSUM; s++) {
+            xsum[s] = 0.f;
+#pragma unroll
+            for (int e = 0; e < RUN; e++) xsum[s] += xr[s * RUN + e];
+        }
+    }
+    const Masks nm = q.nm;
+    const typename P::Keys ch = P::keys(tsub & 3u);
+    const size_t out0 = (size_t)q.t0 * a.out_stride + a.col0;
+    const bool accumulate = (a.flags & FLAG_ACCUMULATE) != 0;
+
+    // Whole-wave rows (SEG = 64) of a format with DEFER keep their finished sums in the lane of
+    // their number (the gate's and the up row's apart) and are finished and stored together,
+    // 64 outputs at a time: stores between the loads of the stream cost more than their bytes,
+    // and the activation runs once for 64 outputs instead of once a row.
+    constexpr bool kKeep = P::DEFER && SEG == 64u;
+    float kept0 = 0.f, kept1 = 0.f;
+    uint32_t nkept = 0, kept_first = gwave;
+    auto flush_kept = [&]() __attribute__((always_inline)) {
+        const uint32_t j = kept_first + lane * nwaves;
+        if (lane < nkept && j < a.rows) {
+            float r = PAIR ? silu_f(kept0) * kept1 : kept0;
+            if (accumulate) r += a.out[out0 + j];
+            a.out[out0 + j] = r;
+        }
+        kept_first += nkept * nwaves;
+        nkept = 0;
+    };
+    auto multiply = [&](uint32_t u, const typename P::Raw (&rows)[kRows]) __attribute__((always_inline)) {
+        float v[kRows][1];
+        P::template dot<1, kRows>(rows, ch, nm,
+            [&](int, int vi) { return make_float4(xr[4 * vi], xr[4 * vi + 1], xr[4 * vi + 2], xr[4 * vi + 3]); },
+            [&](int, int s) { return xsum[s]; }, v);
+        // (0 + v: the kernel above adds a lane's tasks to a sum that starts at zero)
+        const float s0 = segment_sum(0.f + v[0][0], SEG_LOG2);
+        const float s1 = PAIR ? segment_sum(0.f + v[kRows - 1][0], SEG_LOG2) : 0.f;
+        if (kKeep) {
+            const float t0 = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(s0), 63));
+            kept0 = lane == nkept ? t0 : kept0;
+            if (PAIR) {
+                const float t1 = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(s1), 63));
+                kept1 = lane == nkept ? t1 : kept1;
+            }
+            nkept++;
+            if (nkept == 64u) flush_kept();
+        } else {
+            const uint32_t j = u * RPI + rsub;
+            if (tsub == SEG - 1u && j < a.rows) {
+                float r = PAIR ? silu_f(s0) * s1 : s0;
+                if (accumulate) r += a.out[out0 + j];
+                a.out[out0 + j] = r;
+            }
+        }
+    };
+
+    // kRowDepth passes' loads stay in flight ahead of the one multiplied; a trip of
+    // kRowDepth + 1 passes so that the buffers rotate by name.
+    for (uint32_t u = gwave;;) {
+        bool done = false;
+#pragma unroll
+        for (int ph = 0; ph <= kRowDepth; ph++) {
+            fetch(u + kRowDepth * nwaves, buf[(ph + kRowDepth) % (kRowDepth + 1)]);
+            multiply(u, buf[ph]);
+            u += nwaves;
+            if (u >= units) {
+                done = true;
+                break;
+            }
+        }
+        if (done) break;
+    }
+    if (kKeep) flush_kept();
 }
 
 // Steps of several tokens over rows too long for the tokens' inputs to fit the workgroup's LDS
@@ -1139,6 +1454,16 @@ static zhip_result run_sliced(const Dispatch &d, const KArgs &q, uint32_t lds, u
     return check_launch(d, P::name());
 }
 
+template <class P, bool PAIR>
+static zhip_result run_row(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
+    switch (q.seg_log2) {
+    case 4: hipLaunchKernelGGL((matvec_quant_row_kernel<P, PAIR, 4>), dim3(blocks), dim3(256), lds, d.stream, q); break;
+    case 5: hipLaunchKernelGGL((matvec_quant_row_kernel<P, PAIR, 5>), dim3(blocks), dim3(256), lds, d.stream, q); break;
+    default: hipLaunchKernelGGL((matvec_quant_row_kernel<P, PAIR, 6>), dim3(blocks), dim3(256), lds, d.stream, q); break;
+    }
+    return check_launch(d, P::name());
+}
+
 template <class P, int MT, bool PAIR, bool XREG, int STG>
 static zhip_result run_quant(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
     static bool configured = false;  // dynamic LDS above 64 KiB needs opting in once
@@ -1225,8 +1550,12 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
         // format keeps what leaves the multiply its second wave a SIMD (STAGE2, STAGE4; 4096 x
         // 4096 at four tokens with all at once: Q4_K 12.3 against 9.1 us, Q6_K 13.4 against 10.9).
         const bool small = want <= (uint32_t)d.dev->compute_units;
-        if (xreg) r = pair ? run_quant<P, 1, true, true, 1>(d, q, lds, blocks) : run_quant<P, 1, false, true, 1>(d, q, lds, blocks);
-        else if (mt == 1u) r = pair ? run_quant<P, 1, true, false, 1>(d, q, lds, blocks) : run_quant<P, 1, false, false, 1>(d, q, lds, blocks);
+        if (xreg) {
+            // (a pass of the row kernel is a wave's 64 / seg rows, or that many gate / up pairs)
+            const uint32_t passes = (a.rows + rpi - 1u) / rpi, row_want = (passes + 3u) / 4u;
+            const uint32_t cap = (uint32_t)d.dev->compute_units * kRowWorkgroups;
+            r = pair ? run_row<P, true>(d, q, q.tasks * kTaskStride * 4u, row_want < cap ? row_want : cap) : run_row<P, false>(d, q, q.tasks * kTaskStride * 4u, row_want < cap ? row_want : cap);
+        } else if (mt == 1u) r = pair ? run_quant<P, 1, true, false, 1>(d, q, lds, blocks) : run_quant<P, 1, false, false, 1>(d, q, lds, blocks);
         else if (mt == 2u) {
             if (small && P::STAGE2 != 2) r = pair ? run_quant<P, 2, true, false, 2>(d, q, lds, blocks) : run_quant<P, 2, false, false, 2>(d, q, lds, blocks);
             else r = pair ? run_quant<P, 2, true, false, P::STAGE2>(d, q, lds, blocks) : run_quant<P, 2, false, false, P::STAGE2>(d, q, lds, blocks);
