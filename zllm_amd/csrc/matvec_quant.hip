@@ -922,11 +922,9 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
 // multiply turns into a sum of zero; no address arithmetic, clamp or branch per lane is left.
 // The staging of the inputs, a task's dot product and the lanes' reduction are the code of the
 // kernel above, so the results are its bits.
-// Passes whose loads are in flight ahead of the one multiplied, and workgroups a CU. Measured on
-// 14336 x 4096 Q4_K (7.9 us with 1 and 3): two or three passes ahead 8.6 / 9.8 us, four or five
-// workgroups 8.2 / 9.3 us, one workgroup with three passes ahead 9.8 us.
+// Passes whose loads are in flight ahead of the one multiplied. Measured on 14336 x 4096 Q4_K
+// (7.9 us with one): two or three passes ahead 8.6 / 9.8 us, and no better with fewer workgroups.
 constexpr int kRowDepth = 1;
-constexpr uint32_t kRowWorkgroups = 3;
 template <class P, bool PAIR, int SEG_LOG2>
 __global__ __launch_bounds__(256) void matvec_quant_row_kernel(KArgs q) {
     const MvArgs &a = q.a;
@@ -1553,7 +1551,15 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
         if (xreg) {
             // (a pass of the row kernel is a wave's 64 / seg rows, or that many gate / up pairs)
             const uint32_t passes = (a.rows + rpi - 1u) / rpi, row_want = (passes + 3u) / 4u;
-            const uint32_t cap = (uint32_t)d.dev->compute_units * kRowWorkgroups;
+            // Workgroups a CU: every one stages the inputs and every wave reads all of them from
+            // LDS, so two unless the launch is long (four passes a wave or more at three) and its
+            // passes light (up to 3 KB a wave: Q4_K, Q5_K, Q3_K rows without a second row of a
+            // pair). 14336 x 4096 at three / two: Q4_K 7.9 / 8.0 us, Q3_K 8.2 / 8.6, Q5_K 9.7 /
+            // 9.8, Q6_K 10.9 / 10.8, Q8_0 12.05 / 11.7, gate / up pairs of Q4_K 14.4 / 13.9, of
+            // Q5_K 18.3 / 17.2; 4096 x 4096 Q4_K 4.9 / 4.2; 28672 x 2048 Q4_K 8.0 / 9.05.
+            const uint32_t cus = (uint32_t)d.dev->compute_units;
+            const bool three = !pair && (uint64_t)rpi * a.row_bytes <= 3072u && passes >= cus * 48u;
+            const uint32_t cap = cus * (three ? 3u : 2u);
             r = pair ? run_row<P, true>(d, q, q.tasks * kTaskStride * 4u, row_want < cap ? row_want : cap) : run_row<P, false>(d, q, q.tasks * kTaskStride * 4u, row_want < cap ? row_want : cap);
         } else if (mt == 1u) r = pair ? run_quant<P, 1, true, false, 1>(d, q, lds, blocks) : run_quant<P, 1, false, false, 1>(d, q, lds, blocks);
         else if (mt == 2u) {
