@@ -51,6 +51,17 @@ enum {
  * submit a sequence of plain launches. No counterpart in the reference: its
  * hosts record command lists per submit (src/agility/host.zig:520-548). */
 #define ZHIP_OPTION_NO_REPLAY 1u
+/* matvec_bf16 / matvec_f16 over 16 MB or more of weights (k = 1024 ... 16384 in
+ * steps of 512) read the weights once for all of a step's tokens on the matrix
+ * cores, at every width from one token on, so that a token's bits do not depend
+ * on the width of the step it ran in (src/sched/sched.zig:55-58,
+ * src/plan/qwen35.zig:380-381). For deployments that verify speculated tokens
+ * on these matrices: a step of 2..8 tokens then costs what one token does
+ * (151936 x 1024 bf16: 55 us at any width; without the flag 52 / 75 / 122 us at
+ * 1 / 4 / 8 tokens). Without the flag every width runs the kernel that takes the
+ * tokens one pass each, whose one-token step is ~6 % faster; either way the
+ * route depends on the matrix alone, never on the step. */
+#define ZHIP_OPTION_WIDE_DECODE 2u
 
 typedef struct zhip_options {
     uint32_t device_index; /* HIP device ordinal */
@@ -179,14 +190,19 @@ zhip_result zhip_force_loss(zhip_context *context);
  * kernel, which the caller records as an empty artifact
  * (src/kernels/kernels.zig:776-783).
  *
- * Every MatvecVariant id is accepted and keeps the reference's results bit
- * for bit. Two things go beyond the reference's contract: decode multiplies
+ * Every MatvecVariant id is accepted. What the ids guarantee is the
+ * reference's kernel check (src/kernels/check.zig:1019-1060): every output
+ * within 1e-5 of the exact product's scale, and a token's bits independent of
+ * how many tokens share its step and of the id's lane / row tunables (the
+ * backend runs one arithmetic for all of them); the bits themselves are this
+ * backend's, not the WGSL kernels'. Two things go beyond the reference's contract: decode multiplies
  * take 5..8 token rows (the reference stops at 4,
  * src/kernels/matvec_quant.wgsl.hbs:64-65), and on matvec_q3_k, matvec_q4_k,
  * matvec_q5_k, matvec_q6_k and matvec_q8_0 the id 0x00104010 (wg 512, lanes 64,
  * rows 16, a geometry no reference tuning emits) selects matrix-core kernels
- * for steps of 2..8 tokens that read the weights once; their sums round
- * differently from the reference's (within 2e-3 of the row's scale). */
+ * for steps of 1..8 tokens that read the weights once; their sums round
+ * differently from the default id's (both within 1e-5 of the output scale), the
+ * same at every width. */
 size_t zhip_kernel_artifact(const char *name, uint32_t variant, char *out, size_t capacity);
 /* Replaces the backend arm of kernels.backendSource (src/kernels/kernels.zig:
  * 914-922): bytes that change whenever the kernel's implementation changes

@@ -31,3 +31,16 @@ def ctx():
     c = Ctx(d)
     yield c
     d.deinit()
+
+
+@pytest.fixture()
+def ctx_wide():
+    """The same on a device opened with ZHIP_OPTION_WIDE_DECODE: large bf16 / f16 matrices
+    take the kernel that reads the weights once for all of a step's tokens."""
+    from gpucheck import Ctx
+    from zllm_amd import Device
+
+    d = Device.open(0, Device.WIDE_DECODE)
+    c = Ctx(d)
+    yield c
+    d.deinit()

@@ -157,9 +157,12 @@ def test_c5_lm_head_decode(ctx):
 
 
 @pytest.mark.parametrize("norm", [False, True])
-def test_c5_lm_head_verify_width(ctx, norm):
+@pytest.mark.parametrize("wide", [False, True])
+def test_c5_lm_head_verify_width(ctx, ctx_wide, wide, norm):
     """bf16 lm_head, K=1024, N=151936, M=8 (a speculative verify step through the decode multiply,
-    plain and with the final RMSNorm fused in): logits and every row's argmax."""
+    plain and with the final RMSNorm fused in; the general kernel, and in a context opened with
+    ZHIP_OPTION_WIDE_DECODE the kernel that reads the weights once): logits and every row's argmax."""
+    ctx = ctx_wide if wide else ctx
     n, k, m, eps = 151936, 1024, 8, 1e-6
     g = synth.rng(0xC5)
     wbits = synth.bf16_matrix(g, n, k, 0.02)

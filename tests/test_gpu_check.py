@@ -103,16 +103,18 @@ def bf16_tokens_case(c, m, n, k, col0=0, pad=0, accumulate=False, norm=False, x=
     return got, want, (x, bits)
 
 
-# Steps of several tokens over k = 1024 ... 16384 in steps of 512 and 16 MB or more of weights run
-# on the matrix cores, the weights read once for all tokens, from the width on at which that
-# pays for the matrix ((tokens - 1) x bytes of 32 MB at k = 1024, 64 MB up to k = 4096, 192 MB
-# or four tokens beyond; five tokens always); every other step keeps the one-token kernel's path.
+# In a context opened with ZHIP_OPTION_WIDE_DECODE, steps over k = 1024 ... 16384 in steps of 512
+# and 16 MB or more of weights run on the matrix cores, the weights read once for all tokens, at
+# every width from one token on; smaller matrices, and every matrix in a context without the
+# option, keep the general kernel. The cases run under both.
 @pytest.mark.parametrize("m,n,k,col0,pad,accumulate,norm", [
     (2, 16400, 1024, 0, 0, False, False),
-    (2, 8192, 1024, 0, 0, False, False),       # two tokens over 16.8 MB: the general kernel
+    (2, 8192, 1024, 0, 0, False, False),       # 16.8 MB: the smallest matrix the option moves
+    (1, 16400, 1024, 0, 0, False, False),      # one token
+    (1, 4100, 4096, 3, 1, True, True),
     (8, 8300, 1024, 0, 0, False, False),       # a ragged last unit of rows
     (3, 11001, 1536, 5, 3, True, False),       # unaligned columns, accumulate
-    (3, 5501, 1536, 5, 3, True, False),        # ... through the general kernel
+    (3, 5501, 1536, 5, 3, True, False),        # ... just above 16 MB
     (4, 8200, 2048, 0, 0, False, False),       # a tail on every workgroup
     (5, 9000, 2560, 0, 0, False, True),        # the RMSNorm prologue
     (7, 2741, 3072, 32, 0, True, True),
@@ -125,13 +127,14 @@ def bf16_tokens_case(c, m, n, k, col0=0, pad=0, accumulate=False, norm=False, x=
     (5, 1100, 9728, 0, 0, False, False),       # rows longer than 4096: stretches of columns, each launch adding to the one before
     (6, 800, 14336, 3, 5, True, False),        # ... onto what the output already holds
     (5, 1000, 8704, 0, 0, False, True),        # with the RMSNorm prologue: the tokens are normalised and split once for all the stretches
-    (3, 1100, 9728, 0, 0, False, False),       # the same rows at widths the general kernel keeps: passes of as many tokens as fit workgroup memory
+    (3, 1100, 9728, 0, 0, False, False),       # the same rows at fewer tokens (the general kernel: passes of as many tokens as fit workgroup memory)
     (2, 800, 14336, 3, 5, True, False),
     (3, 1000, 8704, 0, 0, False, True),
 ])
 @pytest.mark.parametrize("half", HALVES)
-def test_matvec_bf16_several_tokens(ctx, half, m, n, k, col0, pad, accumulate, norm):
-    got, want, _ = bf16_tokens_case(ctx, m, n, k, col0, pad, accumulate, norm, half=half)
+@pytest.mark.parametrize("wide", [False, True])
+def test_matvec_bf16_several_tokens(ctx, ctx_wide, wide, half, m, n, k, col0, pad, accumulate, norm):
+    got, want, _ = bf16_tokens_case(ctx_wide if wide else ctx, m, n, k, col0, pad, accumulate, norm, half=half)
     assert rel_err(got, want) <= 1e-5
     # Columns outside the launch's keep their contents bit for bit.
     keep = np.ones(got.shape[1], dtype=bool)
@@ -139,10 +142,10 @@ def test_matvec_bf16_several_tokens(ctx, half, m, n, k, col0, pad, accumulate, n
     assert np.array_equal(got[:, keep].astype(np.float32), want[:, keep].astype(np.float32))
 
 
-def test_matvec_bf16_several_tokens_many_rows(ctx):
+def test_matvec_bf16_several_tokens_many_rows(ctx_wide):
     """More than forty 32-row tiles on every workgroup: the outputs kept back in workgroup
     memory are stored in the middle of the run, not only at its end."""
-    c = ctx
+    c = ctx_wide
     m, n, k = 2, 41 * 32 * c.device.caps.compute_units + 50, 1024
     x = c.random(m * k, 3).reshape(m, k)
     bits = synth.to_bf16_bits(c.rand.standard_normal(n * k, dtype=np.float32))
@@ -155,15 +158,15 @@ def test_matvec_bf16_several_tokens_many_rows(ctx):
 
 
 @pytest.mark.parametrize("half", HALVES)
-def test_matvec_bf16_several_tokens_keep_token_bits(ctx, half):
-    """A token's outputs do not depend on how many tokens share the step, on either side of
-    the width at which the matrix's steps move to the matrix cores (18 MB of weights: five
-    tokens), nor on where the step's columns start."""
-    c = ctx
+@pytest.mark.parametrize("wide", [False, True])
+def test_matvec_bf16_several_tokens_keep_token_bits(ctx, ctx_wide, wide, half):
+    """A token's outputs do not depend on how many tokens share the step - the lone launch gives
+    the bits of every wider one (src/sched/sched.zig:55-58) - nor on where the step's columns
+    start; over 18 MB of weights, with and without ZHIP_OPTION_WIDE_DECODE."""
+    c = ctx_wide if wide else ctx
     m, n, k = 13, 4500, 2048
     x = c.random(m * k, 3).reshape(m, k)
     bits, _ = random_half(c, n * k, 1, half)
-    wa = c.upload(bits)
 
     def run(tokens, rows0, rows):
         out = c.output(len(tokens) * rows)
@@ -173,22 +176,20 @@ def test_matvec_bf16_several_tokens_keep_token_bits(ctx, half):
         return c.read(out).reshape(len(tokens), rows)
 
     whole = run(list(range(m)), 0, n)
-    assert np.array_equal(run([4, 9, 1, 2, 6, 8], 0, n), whole[[4, 9, 1, 2, 6, 8]])
-    assert np.array_equal(run([12, 0, 5, 7, 3], 0, n), whole[[12, 0, 5, 7, 3]])
-    # Below that width: the one-token step's bits.
-    few = run([4, 9, 11], 0, n)
-    for i, t in enumerate([4, 9, 11]):
-        assert np.array_equal(few[i], run([t], 0, n)[0])
-    assert np.array_equal(run([9, 4], 0, n), few[[1, 0]])
+    lone = np.stack([run([t], 0, n)[0] for t in range(m)])
+    assert np.array_equal(lone, whole)
+    for tokens in ([4, 9], [4, 9, 11], [12, 0, 5, 7], [12, 0, 5, 7, 3], [4, 9, 1, 2, 6, 8], list(range(8))):
+        assert np.array_equal(run(tokens, 0, n), whole[tokens])
+    # (4096 rows of 2048 weights: 16 MB, the smallest matrix the option moves)
     assert np.array_equal(run(list(range(8)), 404, 4096), whole[:8, 404:])
-    del wa
+    assert np.array_equal(run([5], 404, 4096)[0], whole[5, 404:])
 
 
-def test_matvec_bf16_several_tokens_special_values(ctx):
+def test_matvec_bf16_several_tokens_special_values(ctx_wide):
     """Inputs the three-way split must carry exactly: full 24-bit mantissas (integer inputs
     against weights of +-1, where every partial sum is an integer f32 holds, so the result is
     exact whatever the order of the additions), the largest finite value, infinities and NaNs."""
-    c = ctx
+    c = ctx_wide
     m, n, k = 4, 8192, 1024
     x = np.zeros((m, k), dtype=np.float32)
     r = c.rand.integers(0, 2000, size=k)
@@ -870,6 +871,49 @@ def test_matmul_q8_0_float_bf16_whole_steps_keep_token_bits(ctx, rung):
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
 
 
+@pytest.mark.parametrize("k", [512, 2048])
+@pytest.mark.parametrize("weights", ["q8_0", "bf16"])
+def test_matmul_bf16_rungs_keep_token_bits_over_prompt_splits(ctx, weights, k):
+    """The prefill kernels give the same result however a prompt is split into steps
+    (src/sched/sched.zig:84-90): on this backend's bf16 rungs a matrix wide enough that a
+    512-token step's 256 x 128 tiles would fill the CUs (n = 16400) keeps the tiling its short
+    steps take, so 512 tokens in one step equal a first chunk of 64 and a step of 448 bit for
+    bit; with k = 512 the matrix is one the streaming kernel takes, a pass per 128 tokens."""
+    c = ctx
+    rows, n = 512, 16400
+    x = c.random(rows * k, 1).reshape(rows, k)
+    if weights == "q8_0":
+        raw, values = quant_rows(c, TensorType.q8_0, n, k)
+        wa = c.gpu_weights(TensorType.q8_0, raw, k)
+    else:
+        bits, values = random_half(c, n * k, 1)
+        wa = c.upload(bits.reshape(n, k))
+    values = values.reshape(n, k)
+    for rung in (K.Prefill.bf16_mfma, K.Prefill.bf16_mfma_xbf16):
+        packed = rung == K.Prefill.bf16_mfma_xbf16
+        c.set.select_prefill(c.rec, rung)
+
+        def run(first, count):
+            xa = c.upload(synth.to_bf16_bits(x[first : first + count]) if packed else x[first : first + count])
+            out = c.output(count * n)
+            if weights == "q8_0":
+                c.launcher().launch(Kernel.matmul_q8_0_float, P.MatmulQuant(rows=count, n=n, k=k, col0=0, out_stride=n, k_slice=k), [xa, wa, out],
+                                    (K.div_ceil(n, 64), K.div_ceil(count, 16), 1))
+            else:
+                c.launcher().launch(Kernel.matmul_bf16, P.MatmulBf16(rows=count, n=n, k=k, col0=0, out_stride=n), [xa, wa, out],
+                                    (K.div_ceil(n, K.matmul_tile_n), K.div_ceil(count, K.matmul_tile_t), 1))
+            return c.read(out).reshape(count, n)
+
+        whole = run(0, rows)
+        assert whole[:64].tobytes() == run(0, 64).tobytes(), (rung, "the first chunk of 64")
+        assert whole[64:].tobytes() == run(64, 448).tobytes(), (rung, "the step of 448")
+        assert whole[504:].tobytes() == run(504, 8).tobytes(), (rung, "a tail of 8")
+        some = np.arange(0, rows, 37)
+        want = synth.bf16_round(x[some]).astype(np.float64) @ synth.bf16_round(values).astype(np.float64).T
+        assert rel_err(whole[some], want) <= 1e-5, rung
+    c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
+
+
 @pytest.mark.parametrize("rows,n,k,col0,pad,accumulate,packed", [
     (128, 16400, 1024, 0, 0, False, True),    # whole token tiles, vector stores
     (70, 16389, 768, 5, 9, True, False),      # ragged last weight tile, unaligned output: scalar stores
@@ -877,7 +921,7 @@ def test_matmul_q8_0_float_bf16_whole_steps_keep_token_bits(ctx, rung):
     (1, 20000, 512, 0, 0, False, False),
 ])
 def test_matmul_bf16_streamed_chunk(ctx, rows, n, k, col0, pad, accumulate, packed):
-    """A chunk of up to 128 tokens against a tall bf16 matrix with k <= 1024 (the
+    """A step against a tall bf16 matrix with k <= 1024 (the
     vocabulary projection of a prefill chunk) takes the kernel that streams the
     weights into registers: against the rung's operand contract, columns
     outside the chunk untouched, and every token's bits the same whether it runs

@@ -3,8 +3,11 @@ against the dispatch it is a variant of: matmul_q8_0_float in the bf16 rung with
 f32-bound activations through zhip_execute. Same inputs, bit for bit the same
 outputs, on two calls in a row of which the second is smaller, so that the
 fixed scratch array still holds the first call's activations when the second
-runs. The caller's own buffers come from the HIP runtime the library is linked
-against, loaded through ctypes; the call itself must not allocate.
+runs. The caller's own buffers come from the HIP runtime the library itself is
+linked against (found among the process's mappings once the library is loaded);
+the call must not allocate: the device's free memory is read before and after
+every call, the first one in the context included, and each call runs before the
+dispatch it is compared with, so nothing has warmed its kernels up.
 """
 import ctypes as C
 
@@ -23,8 +26,13 @@ class Runtime:
     """hipMalloc / hipMemcpy / hipFree for the test's own operands."""
 
     def __init__(self):
-        self.hip = C.CDLL("libamdhip64.so.7")
+        # The runtime libzllm_hip.so brought in, whatever its soname.
+        with open("/proc/self/maps") as maps:
+            paths = sorted({line.split()[-1] for line in maps if "libamdhip64.so" in line})
+        assert paths, "libzllm_hip.so is loaded, so its HIP runtime must be mapped"
+        self.hip = C.CDLL(paths[0])
         self.hip.hipMalloc.argtypes = [C.POINTER(C.c_void_p), C.c_size_t]
+        self.hip.hipMemGetInfo.argtypes = [C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)]
         self.hip.hipMemcpy.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_int]
         self.hip.hipFree.argtypes = [C.c_void_p]
         self.live = []
@@ -43,6 +51,13 @@ class Runtime:
         assert self.hip.hipMemcpy(out.ctypes.data, p, out.nbytes, 2) == 0
         return out
 
+    def free_bytes(self) -> int:
+        """The device's free memory once everything launched has finished."""
+        free, total = C.c_size_t(), C.c_size_t()
+        assert self.hip.hipDeviceSynchronize() == 0
+        assert self.hip.hipMemGetInfo(C.byref(free), C.byref(total)) == 0
+        return free.value
+
     def free(self):
         for p in self.live:
             self.hip.hipFree(p)
@@ -50,7 +65,8 @@ class Runtime:
 
 
 def through_execute(c: Ctx, x, raw, init, rows, n, k, col0, stride, accumulate):
-    """The existing entry point: one matmul_q8_0_float dispatch of variant 0xfffb0000."""
+    """The existing entry point: one matmul_q8_0_float dispatch of variant 0xfffb0000; also
+    returns the weights as repack_q8_0 laid them out on the GPU."""
     c.set.select_prefill(c.rec, K.Prefill.bf16_mfma)
     wa = c.gpu_weights(TensorType.q8_0, raw, k)
     out = c.upload(init)
@@ -69,6 +85,8 @@ CASES = [
 
 
 def test_no_alloc_entry_matches_the_dispatch_twice_in_a_row():
+    import oracle
+
     dev = Device.open(0)
     rt = Runtime()
     try:
@@ -78,15 +96,18 @@ def test_no_alloc_entry_matches_the_dispatch_twice_in_a_row():
             x = synth.activations(g, rows, k)
             raw = synth.q8_0_rows(g, n, k)
             init = synth.activations(g, rows, stride)
-            want, split_rows = through_execute(c, x, raw, init, rows, n, k, col0, stride, accumulate)
+            # The weights in split rows, laid out on the CPU: the new entry point runs first.
+            split_rows = oracle.repack_q8_0(raw, n, k)
             dx, dw, do = rt.upload(x), rt.upload(split_rows), rt.upload(init)
+            free_before = rt.free_bytes()
             r = _lib.lib.zhip_matmul_q8_0_float_no_alloc(dev.ctx, None, dx, dw, do, rows, n, k, col0, stride, accumulate)
             dev.check(r)
+            assert rt.free_bytes() == free_before, "the call changed the device's free memory"
             got = rt.download(do, rows * stride)
+            want, gpu_rows = through_execute(c, x, raw, init, rows, n, k, col0, stride, accumulate)
+            assert gpu_rows.tobytes() == np.ascontiguousarray(split_rows).view(np.uint8).reshape(-1)[: gpu_rows.size].tobytes()
             assert got.tobytes() == want.tobytes(), (rows, n, k)
             # And the dispatch itself is the rung's arithmetic: both operands rounded to bf16.
-            import oracle
-
             values = oracle.dequantize(oracle.Q8_0, raw, n * k).reshape(n, k)
             prod = synth.bf16_round(x).astype(np.float64) @ synth.bf16_round(values).astype(np.float64).T
             ref = prod + (init[:, col0 : col0 + n] if accumulate else 0)

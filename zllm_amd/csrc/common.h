@@ -51,6 +51,10 @@ struct MatvecVariant {
 // are this backend's extension for speculative-verify widths.
 constexpr uint32_t kMaxDecodeRows = 8;
 
+// A byte offset no binding reaches (a binding is at most 2 GiB): a range-checked buffer load
+// there returns zeros and moves nothing.
+constexpr uint32_t kNowhere = 0xF0000000u;
+
 struct Bind {
     uint8_t *ptr = nullptr;  // buffer base + binding offset
     uint64_t size = 0;       // bytes bound
@@ -60,6 +64,7 @@ struct Bind {
 struct DeviceInfo {
     int compute_units = 256;
     int max_lds = 65536;
+    bool wide_decode = false;  // ZHIP_OPTION_WIDE_DECODE
 };
 
 struct Dispatch;
@@ -124,6 +129,18 @@ zhip_result launch_embed_bf16(const Dispatch &);
 zhip_result launch_embed_f16(const Dispatch &);
 zhip_result launch_embed_iq4_xs(const Dispatch &);
 
+// Dynamic LDS above 64 KiB needs opting in once per kernel: done the first time this is called
+// for the kernel (or ahead of time, see prepare_no_alloc_kernels), remembered after.
+template <auto Kernel, int Bytes>
+inline bool lds_opt_in() {
+    static const bool ok = [] {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(Kernel), hipFuncAttributeMaxDynamicSharedMemorySize, Bytes) == hipSuccess) return true;
+        (void)hipGetLastError();
+        return false;
+    }();
+    return ok;
+}
+
 // Host-side helpers shared by the launchers.
 zhip_result fail(const Dispatch &d, zhip_result code, const char *fmt, ...);
 zhip_result check_launch(const Dispatch &d, const char *kernel);
@@ -131,6 +148,12 @@ zhip_result check_launch(const Dispatch &d, const char *kernel);
 // The entry point that allocates nothing (no_alloc.hip): its fixed scratch array's address is
 // looked up once per device, with that device current.
 zhip_result no_alloc_setup(int device, const DeviceInfo &info);
+// The one-time set-up of every kernel that entry point can launch (each file its own), so
+// that the call itself does none.
+bool matmul_mfma_prepare_no_alloc();
+bool matmul_mfma_wide_prepare_no_alloc();
+bool matmul_stream_prepare_no_alloc();
+bool matmul_q8_bf16_prepare_no_alloc();
 uint64_t no_alloc_capacity();
 zhip_result no_alloc_matmul_q8_0_float(int device, hipStream_t stream, const float *x, const void *w, float *out, uint32_t rows, uint32_t n,
     uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, char *err, size_t err_cap);

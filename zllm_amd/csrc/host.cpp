@@ -930,6 +930,7 @@ zhip_result zhip_create(const zhip_options *options, zhip_context **out_context)
     c->use_graphs = !(options && (options->flags & ZHIP_OPTION_NO_REPLAY)) && !getenv("ZHIP_NO_REPLAY");
     c->info.compute_units = prop.multiProcessorCount;
     c->info.max_lds = (int)prop.sharedMemPerBlock;
+    c->info.wide_decode = options && (options->flags & ZHIP_OPTION_WIDE_DECODE);
     c->caps.abi_version = ZHIP_ABI_VERSION;
     c->caps.compute_units = (uint32_t)prop.multiProcessorCount;
     c->caps.wavefront = (uint32_t)prop.warpSize;
@@ -963,6 +964,8 @@ zhip_result zhip_matmul_q8_0_float_no_alloc(zhip_context *c, void *stream, const
     uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate) {
     if (!c) return ZHIP_E_INVALID_ARGUMENT;
     if (c->lost) return set_error(c, ZHIP_E_DEVICE_LOST, "device lost");
+    // (the launches go to the current device: make it the context's)
+    if (zhip_result r = hip_check(c, hipSetDevice(c->device), "hipSetDevice")) return r;
     char err[384] = "";
     const zhip_result r = no_alloc_matmul_q8_0_float(c->device, static_cast<hipStream_t>(stream), x, weights, out, rows, n, k, col0, out_stride,
         accumulate, err, sizeof err);

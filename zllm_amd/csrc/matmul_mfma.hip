@@ -520,18 +520,15 @@ static zhip_result launch_kernel(const Dispatch &d, const char *name, const Mfma
     auto kernel = matmul_mfma_kernel<W, H, MT, RAGGED, COMP>;
     constexpr int bytes = lds_bytes<W, MT, COMP>();
     static_assert(bytes <= 160 * 1024, "three buffers must fit the CU's LDS");
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
-        }
-        configured = true;
-    }
+    if (!lds_opt_in<matmul_mfma_kernel<W, H, MT, RAGGED, COMP>, bytes>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
     const dim3 grid((a.n + BN - 1) / BN, (a.rows + 16 * MT - 1) / (16 * MT), slices);
     hipLaunchKernelGGL(kernel, grid, dim3(THREADS), bytes, d.stream, a);
     return check_launch(d, name);
 }
+
+// The longest step the reference's planner records (src/plan/plan.zig:129,
+// src/plan/qwen35.zig:335).
+constexpr uint32_t kPlannerStepCap = 512;
 
 // XPACKED: the activations are bound already packed in the operand format (an extension of
 // the contract, bf16 only); otherwise they are bound as f32 and narrowed first.
@@ -581,14 +578,19 @@ static zhip_result launch_mfma(const Dispatch &d, const char *name, bool sliced,
         a.x = d.work->data;
     }
     const uint32_t slices = sliced ? d.grid[2] : 1u;
-    // A chunk of up to 128 tokens against a tall matrix with a short k is one pass over the
-    // weights: the kernel that streams them into registers.
+    // Which tiling a step takes depends on the matrix, never on the step's length within the
+    // 512 tokens a planner records (src/plan/plan.zig:129): the tilings add k in different
+    // orders, and a token's bits must not depend on how its prompt was split into steps
+    // (src/sched/sched.zig:84-90).
+    // A tall matrix with a short k is a pass over the weights per chunk of up to 128 tokens: the
+    // kernel that streams them into registers.
     constexpr bool kBf16Rung = std::is_same<H, Bf16>::value && (std::is_same<W, WBf16>::value || std::is_same<W, WQ8_0>::value);
     if (kBf16Rung && slices == 1u && a.k_slice >= a.k && matmul_stream_accepts(d, q8_0, a.out, a.rows, a.n, a.k, a.col0, a.out_stride))
         return launch_matmul_stream(d, name, q8_0, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes);
-    // Long steps whose 256 x 128 tiles fill the CUs take that tiling: each
-    // weight is converted once per 256 tokens and half the bytes cross from L2.
-    if (kBf16Rung && slices == 1u && a.k_slice >= a.k && (uint64_t)((a.rows + 255u) / 256u) * ((a.n + 127u) / 128u) >= (uint64_t)d.dev->compute_units)
+    // Steps longer than any the planner records (callers of their own), whose 256 x 128 tiles
+    // fill the CUs, take that tiling: each weight is converted once per 256 tokens and half
+    // the bytes cross from L2.
+    if (kBf16Rung && slices == 1u && a.k_slice >= a.k && a.rows > kPlannerStepCap && (uint64_t)((a.rows + 255u) / 256u) * ((a.n + 127u) / 128u) >= (uint64_t)d.dev->compute_units)
         return launch_mfma_wide(d, name, q8_0, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes);
     if constexpr (std::is_same<W, WQ8_0>::value && !COMP) {
         if (matmul_q8_bf16_accepts(a.k, a.k_slice, slices))
@@ -606,6 +608,12 @@ static zhip_result launch_mfma(const Dispatch &d, const char *name, bool sliced,
     if (a.rows > 64u && 2u * tall > (uint64_t)d.dev->compute_units)
         return ragged ? launch_kernel<W, H, 8, true>(d, name, a, slices) : launch_kernel<W, H, 8, false>(d, name, a, slices);
     return ragged ? launch_kernel<W, H, 4, true>(d, name, a, slices) : launch_kernel<W, H, 4, false>(d, name, a, slices);
+}
+
+// (matmul_q8_0_float with f32-bound activations on the bf16 rung: both tile heights, whole and ragged k)
+bool matmul_mfma_prepare_no_alloc() {
+    return lds_opt_in<matmul_mfma_kernel<WQ8_0, Bf16, 8, false, false>, lds_bytes<WQ8_0, 8, false>()>() && lds_opt_in<matmul_mfma_kernel<WQ8_0, Bf16, 8, true, false>, lds_bytes<WQ8_0, 8, false>()>() &&
+           lds_opt_in<matmul_mfma_kernel<WQ8_0, Bf16, 4, false, false>, lds_bytes<WQ8_0, 4, false>()>() && lds_opt_in<matmul_mfma_kernel<WQ8_0, Bf16, 4, true, false>, lds_bytes<WQ8_0, 4, false>()>();
 }
 
 zhip_result launch_matmul_bf16_mfma(const Dispatch &d) { return launch_mfma<WBf16, false>(d, "matmul_bf16", false, false); }

@@ -165,10 +165,18 @@ __global__ __launch_bounds__(THREADS) void matmul_mfma_wide_kernel(Args a) {
             const uint32_t pos = min(k0 + 16u * wq, wk_last);
             W::load(wbuf, W::quant_offset(wrow * a.row_bytes, pos), W::scale_offset(wrow * a.row_bytes, a.k, pos), 0u, w);
         } else {
-            W::load(wbuf, wqoff, wdoff, k0, w);
+            // (a tile past the end of k, loaded ahead like the others and never used: from an
+            // offset no binding reaches, whether or not the range check covers the scalar offset)
+            const bool live = k0 < ke;
+            W::load(wbuf, live ? wqoff : kNowhere, live ? wdoff : kNowhere, live ? k0 : 0u, w);
         }
+        const bool xlive = k0 < ke;
 #pragma unroll
-        for (int i = 0; i < 4; i++) x.v[i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, xoff[i], 2u * k0, 0);
+        for (int i = 0; i < 4; i++) {
+            // (ragged k: the position joins the lane's offset, which the range check covers whatever it does with the scalar one)
+            if (RAGGED) x.v[i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, xoff[i] + 2u * k0, 0u, 0);
+            else x.v[i] = __builtin_amdgcn_raw_buffer_load_b128(xbuf, xlive ? xoff[i] : kNowhere, xlive ? 2u * k0 : 0u, 0);
+        }
     };
     auto commit = [&](uint32_t b, uint32_t k0, const typename W::Regs &w, XRegs &x) __attribute__((always_inline)) {
         if (RAGGED && k0 + 8u * xpiece >= ke) {
@@ -256,14 +264,8 @@ static zhip_result launch(const Dispatch &d, const char *name, Args a) {
     const uint32_t tiles = a.mtiles * a.ntiles;
     const bool ragged = a.k % GK != 0;
     auto kernel = ragged ? matmul_mfma_wide_kernel<W, true> : matmul_mfma_wide_kernel<W, false>;
-    static bool configured[2] = {false, false};
-    if (!configured[ragged]) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, LDS_BYTES);
-        }
-        configured[ragged] = true;
-    }
+    if (!(ragged ? lds_opt_in<matmul_mfma_wide_kernel<W, true>, LDS_BYTES>() : lds_opt_in<matmul_mfma_wide_kernel<W, false>, LDS_BYTES>()))
+        return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, LDS_BYTES);
     hipLaunchKernelGGL(kernel, dim3(tiles), dim3(THREADS), LDS_BYTES, d.stream, a);
     return check_launch(d, name);
 }
@@ -277,6 +279,10 @@ zhip_result launch_mfma_wide(const Dispatch &d, const char *name, bool q8_0, con
     a.x = x; a.w = w; a.out = out;
     a.rows = rows; a.n = n; a.k = k; a.col0 = col0; a.out_stride = out_stride; a.accumulate = accumulate; a.row_bytes = row_bytes;
     return q8_0 ? wide::launch<wide::WQ8_0>(d, name, a) : wide::launch<wide::WBf16>(d, name, a);
+}
+
+bool matmul_mfma_wide_prepare_no_alloc() {
+    return lds_opt_in<wide::matmul_mfma_wide_kernel<wide::WQ8_0, true>, wide::LDS_BYTES>() && lds_opt_in<wide::matmul_mfma_wide_kernel<wide::WQ8_0, false>, wide::LDS_BYTES>();
 }
 
 }  // namespace zhip

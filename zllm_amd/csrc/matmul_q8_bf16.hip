@@ -168,18 +168,28 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
         }
         // A step's scales of the producer's sixteen rows, 8 bytes a row; the upper half of the
         // wave asks past the buffer's end (reads zero) and fills the filler.
-        const uint32_t soff = lane < 32u ? (j0 + 16u * p + (lane >> 1)) * a.row_bytes + a.k + 4u * (lane & 1u) : 0xF0000000u;
+        const uint32_t soff = lane < 32u ? (j0 + 16u * p + (lane >> 1)) * a.row_bytes + a.k + 4u * (lane & 1u) : kNowhere;
+        // Steps past the end of k are loaded like the others, so that every wait counts the same
+        // loads, but from an offset no binding reaches (they land as zeros and move nothing;
+        // nothing reads them): the step's position travels in the loads' scalar offset, and
+        // whether the range check of a raw buffer covers that offset is not relied on.
         auto fetch = [&](uint32_t buf, uint32_t step) __attribute__((always_inline)) {
             uint8_t *base = lds + buf * BUF;
+            if (step < steps) {
 #pragma unroll
-            for (int i = 0; i < XL; i++) load_lds_b128(xbuf, base + xdst[i], xoff[i], 256u * step);
+                for (int i = 0; i < XL; i++) load_lds_b128(xbuf, base + xdst[i], xoff[i], 256u * step);
 #pragma unroll
-            for (int i = 0; i < 2; i++) load_lds_b128(wbuf, base + ABUF + 1024u * (2u * p + i), woff[i], 128u * step);
-            load_lds_b32(wbuf, base + ABUF + BN * 128 + 256u * p, soff, 8u * step);
+                for (int i = 0; i < 2; i++) load_lds_b128(wbuf, base + ABUF + 1024u * (2u * p + i), woff[i], 128u * step);
+                load_lds_b32(wbuf, base + ABUF + BN * 128 + 256u * p, soff, 8u * step);
+            } else {
+#pragma unroll
+                for (int i = 0; i < XL; i++) load_lds_b128(xbuf, base + xdst[i], kNowhere, 0u);
+#pragma unroll
+                for (int i = 0; i < 2; i++) load_lds_b128(wbuf, base + ABUF + 1024u * (2u * p + i), kNowhere, 0u);
+                load_lds_b32(wbuf, base + ABUF + BN * 128 + 256u * p, kNowhere, 0u);
+            }
         };
         constexpr int PER_STEP = XL + 3;
-        // Steps past the end of k are loaded like the others (zeros or whatever follows in the
-        // operands; nothing reads them), so that every wait counts the same loads.
         fetch(0, 0);
         fetch(1, 1);
         fetch(2, 2);
@@ -351,20 +361,17 @@ template <int TT, class H>
 zhip_result launch_tile(const Dispatch &d, const char *name, const Q8Args &a) {
     auto kernel = matmul_q8_bf16_kernel<TT, H>;
     constexpr int bytes = lds_bytes<TT>();
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
-        }
-        configured = true;
-    }
+    if (!lds_opt_in<matmul_q8_bf16_kernel<TT, H>, bytes>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
     const dim3 grid((a.n + BN - 1) / BN, (a.rows + 32 * TT - 1) / (32 * TT));
     hipLaunchKernelGGL(kernel, grid, dim3(THREADS), bytes, d.stream, a);
     return check_launch(d, name);
 }
 
 }  // namespace
+
+bool matmul_q8_bf16_prepare_no_alloc() {
+    return lds_opt_in<matmul_q8_bf16_kernel<2, AsBf16>, lds_bytes<2>()>() && lds_opt_in<matmul_q8_bf16_kernel<4, AsBf16>, lds_bytes<4>()>();
+}
 
 // Whole, unsliced k in 128-deep steps, operands the 32-bit offsets reach (the caller has
 // validated the bindings).

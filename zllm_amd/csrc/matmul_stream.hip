@@ -254,18 +254,14 @@ __global__ __launch_bounds__(THREADS) void matmul_stream_kernel(StreamArgs a) {
     }
 }
 
+template <int MT>
+constexpr int stream_lds_bytes() { return 2 * WAVES * MT * 64 * 16; }
+
 template <int MT, int KC, bool Q8>
 static zhip_result launch(const Dispatch &d, const char *name, const StreamArgs &a, uint32_t groups) {
     auto kernel = matmul_stream_kernel<MT, KC, Q8>;
-    constexpr int bytes = 2 * WAVES * MT * 64 * 16;
-    static bool configured = false;
-    if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
-        }
-        configured = true;
-    }
+    constexpr int bytes = stream_lds_bytes<MT>();
+    if (!lds_opt_in<matmul_stream_kernel<MT, KC, Q8>, bytes>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
     hipLaunchKernelGGL(kernel, dim3(groups), dim3(THREADS), bytes, d.stream, a);
     return check_launch(d, name);
 }
@@ -283,27 +279,39 @@ static zhip_result launch_k(const Dispatch &d, const char *name, const StreamArg
 
 }  // namespace
 
+bool matmul_stream_prepare_no_alloc() {
+    return lds_opt_in<matmul_stream_kernel<4, 2, true>, stream_lds_bytes<4>()>() && lds_opt_in<matmul_stream_kernel<4, 4, true>, stream_lds_bytes<4>()>() &&
+           lds_opt_in<matmul_stream_kernel<8, 2, true>, stream_lds_bytes<8>()>() && lds_opt_in<matmul_stream_kernel<8, 4, true>, stream_lds_bytes<8>()>();
+}
+
 // Whether the streaming kernel suits a (validated) step on the bf16 rung: few tokens, a
 // short k in whole chunks (Q8_0: two or four blocks a wave), enough whole weight tiles to
 // occupy every CU several times, and outputs that can be stored 16 bytes at a time.
 bool matmul_stream_accepts(const Dispatch &d, bool q8_0, const float *out, uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride) {
     const bool k_fits = q8_0 ? (k == 512u || k == 1024u) : (k >= 256u && k <= 1024u && k % 256u == 0);
-    return rows >= 1 && rows <= 128 && k_fits && (n + 15u) / 16u >= 4u * (uint32_t)d.dev->compute_units &&
+    return rows >= 1 && k_fits && (n + 15u) / 16u >= 4u * (uint32_t)d.dev->compute_units &&
            (uintptr_t)out % 16u == 0 && out_stride % 4u == 0 && col0 % 4u == 0 && n % 16u == 0;
 }
 
 zhip_result launch_matmul_stream(const Dispatch &d, const char *name, bool q8_0, const uint8_t *x, const uint8_t *w, float *out,
     uint32_t rows, uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, uint32_t row_bytes) {
-    const uint64_t x_bytes = (uint64_t)rows * k * 2u, w_bytes = (uint64_t)n * row_bytes;
+    const uint64_t w_bytes = (uint64_t)n * row_bytes;
     // 32-bit byte offsets, up to a tile of sixteen past the last token and row.
     if (w_bytes + 16ull * row_bytes >= 0xfffffff0ull - 256u) return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
-    StreamArgs a{};
-    a.x = x; a.w = w; a.out = out;
-    a.rows = rows; a.n = n; a.k = k; a.col0 = col0; a.out_stride = out_stride; a.accumulate = accumulate;
-    a.x_bytes = (uint32_t)x_bytes; a.w_bytes = (uint32_t)w_bytes; a.row_bytes = row_bytes;
-    a.tiles = (n + 15u) / 16u;
-    const uint32_t groups = a.tiles < (uint32_t)d.dev->compute_units ? a.tiles : (uint32_t)d.dev->compute_units;
-    return rows <= 64u ? launch_k<4>(d, name, a, groups, q8_0) : launch_k<8>(d, name, a, groups, q8_0);
+    // A chunk of up to 128 tokens a launch, each a pass over the weights: which kernel a matrix
+    // takes must not depend on the step's length (a token's bits are the same however a prompt
+    // is split into steps, src/sched/sched.zig:84-90), so longer steps stay here as well.
+    for (uint32_t t0 = 0; t0 < rows; t0 += 128u) {
+        const uint32_t chunk = rows - t0 < 128u ? rows - t0 : 128u;
+        StreamArgs a{};
+        a.x = x + (size_t)t0 * k * 2u; a.w = w; a.out = out + (size_t)t0 * out_stride;
+        a.rows = chunk; a.n = n; a.k = k; a.col0 = col0; a.out_stride = out_stride; a.accumulate = accumulate;
+        a.x_bytes = (uint32_t)((uint64_t)chunk * k * 2u); a.w_bytes = (uint32_t)w_bytes; a.row_bytes = row_bytes;
+        a.tiles = (n + 15u) / 16u;
+        const uint32_t groups = a.tiles < (uint32_t)d.dev->compute_units ? a.tiles : (uint32_t)d.dev->compute_units;
+        if (zhip_result r = chunk <= 64u ? launch_k<4>(d, name, a, groups, q8_0) : launch_k<8>(d, name, a, groups, q8_0)) return r;
+    }
+    return ZHIP_OK;
 }
 
 }  // namespace zhip

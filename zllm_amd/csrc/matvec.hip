@@ -331,29 +331,18 @@ zhip_result launch_matvec_q3k_mfma_stream(const Dispatch &d, const MvArgs &a, ui
 // matvec_q8_0 over rows of 1024 weights in the same kernel: a tile's rows as one flat stretch.
 bool matvec_q8_0_mfma_flat_accepts(const MvArgs &a);
 zhip_result launch_matvec_q8_0_mfma_flat(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
-// Which steps take it. Its time hardly depends on the step's width; the general kernel's grows
-// by a share of the matrix's bytes with every token. Below 16 MB its fixed costs (the split of
-// the tokens, a workgroup's first tile) outweigh that at every width the general kernel takes in
-// one pass (8 MB, k = 1024: 6.4 / 6.8 / 7.8 us at 2 / 4 / 8 tokens against 4.7 / 6.2 / 9.3);
-// above, the step's width decides with the matrix: (tokens - 1) x bytes from 64 MB on (4096 x
-// 4096, 33.5 MB, at 2 / 3 / 4 tokens: 13.6 / 13.9 / 14.4 us against 10.8 / 12.5 / 14.2; 14336 x
-// 4096 at 2 / 3: 26.0 / 26.3 against 26.6 / 30.3), from 32 MB on for rows of 1024 weights, where
-// the general kernel's rows are short (32768 x 1024 at 2 tokens: 14.0 against 20.4 us), and
-// from 192 MB on for rows beyond 4096 weights, which it takes in stretches, a launch each, while
-// the general kernel takes the tokens that do not fit workgroup memory together in passes
-// (4096 x 8192, 67 MB, at 2 / 4 tokens: 26.7 / 27.9 against 20.0 / 32.8 us; 8192 x 8192: 38.2 /
-// 39.6 against 31.7 / 53.5; 5120 x 5120 at 4: 22.2 against 29.0): such rows come here from
-// four tokens on whatever the matrix. Five tokens and more always take it. A token's bits are the
-// one-token step's wherever the general kernel runs and this kernel's own from the width on
-// at which the matrix's steps move here: the same at every width on either side.
+// Which matrices take it: 16 MB of weights or more (below, its fixed costs - the split of the
+// tokens, a workgroup's first tile - outweigh what it saves at every width: 8 MB, k = 1024: 6.4 /
+// 6.8 / 7.8 us at 2 / 4 / 8 tokens against 4.7 / 6.2 / 9.3) in contexts opened with
+// ZHIP_OPTION_WIDE_DECODE, and then at every width from one token on: the kernel sums in another
+// order than the general one, and a token's bits must not depend on the width of the step it
+// runs in (src/sched/sched.zig:55-58; src/plan/qwen35.zig:380-381), so the route is a property
+// of the matrix and of the context, never of the step. Its time hardly depends on the width
+// (151936 x 1024: 55 us at 1 ... 8 tokens; the general kernel 52 / 75 / 122 us at 1 / 4 / 8), so
+// a context pays ~6 % of a one-token step for verify steps at the one-token price.
 constexpr uint64_t kBf16StreamBytes = 16ull << 20;
-static bool bf16_stream_pays(const MvArgs &a) {
-    const uint64_t bytes = (uint64_t)a.rows * a.row_bytes;
-    if (a.m < 2u || bytes < kBf16StreamBytes) return false;
-    if (a.m >= 5u) return true;
-    if (a.k > 4096u && a.m >= 4u) return true;
-    const uint64_t from = a.k > 4096u ? (192ull << 20) : a.k <= 1024u ? (32ull << 20) : (64ull << 20);
-    return (uint64_t)(a.m - 1u) * bytes >= from;
+static bool bf16_stream_pays(const Dispatch &d, const MvArgs &a) {
+    return d.dev->wide_decode && (uint64_t)a.rows * a.row_bytes >= kBf16StreamBytes;
 }
 // The tuned multiply (matvec_quant.hip): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
 zhip_result launch_matvec_quant(const Dispatch &d, const MvArgs &a, int type);
@@ -434,9 +423,9 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     a.out = reinterpret_cast<float *>(d.bind[3].ptr);
     a.norm_w = norm ? reinterpret_cast<const float *>(d.bind[4].ptr) : nullptr;
 
-    // matvec_bf16 / matvec_f16 steps of several tokens over a matrix of some size go to the kernel that reads
-    // the weights once for all of them.
-    if ((std::is_same<D, DecBF16>::value || std::is_same<D, DecF16>::value) && bf16_stream_pays(a) && matvec_bf16_mfma_stream_accepts(a))
+    // matvec_bf16 / matvec_f16 over a matrix of some size, in a context that asked for it, go to
+    // the kernel that reads the weights once for all of a step's tokens.
+    if ((std::is_same<D, DecBF16>::value || std::is_same<D, DecF16>::value) && bf16_stream_pays(d, a) && matvec_bf16_mfma_stream_accepts(a))
         return launch_matvec_bf16_mfma_stream(d, a, d.bind[2].size, std::is_same<D, DecF16>::value);
 
     // MatvecVariant (wg 512, lanes 64, rows 16) names the matrix-core variants: a wave per sixteen rows.

@@ -142,10 +142,6 @@ __device__ __forceinline__ float dot_bytes(uint32_t word, const float4 &x, float
     return sum;
 }
 
-// A buffer offset no binding reaches (bindings end below 2 GiB): a load there returns zeros
-// and moves nothing.
-constexpr uint32_t kNowhere = 0x80000000u;
-
 // ---- the formats ---------------------------------------------------------------------
 // A format names its task's vectors (Raw), loads them, says where a row's
 // inputs go in task order, and multiplies one task of one row (ROWS = 1) or of

@@ -101,7 +101,8 @@ class Timings:
 class Device:
     """One MI355X (src/gpu/host.zig:48-135)."""
 
-    NO_REPLAY = 1  # ZHIP_OPTION_NO_REPLAY: never replay a repeated submit from a HIP graph
+    NO_REPLAY = 1    # ZHIP_OPTION_NO_REPLAY: never replay a repeated submit from a HIP graph
+    WIDE_DECODE = 2  # ZHIP_OPTION_WIDE_DECODE: large matvec_bf16 / matvec_f16 matrices read once for all of a step's tokens, at every width
 
     def __init__(self, index: int = 0, flags: int = 0) -> None:
         self.ctx = C.c_void_p()
