@@ -190,13 +190,43 @@ class MatvecVariant:
     def fits_rows(self, n: int) -> bool:
         return div_ceil(n, self.group_rows()) <= 65535
 
+    def fits(self, d: "DeviceLimits") -> bool:
+        """Whether the device runs it: threads per workgroup, and the WGSL kernel's workgroup
+        memory (src/kernels/kernels.zig:343-345)."""
+        return self.wg <= d.invocations and 2048 * 4 + 2 * self.wg * self.rows * 4 <= d.workgroup_storage
+
+    def is_matrix_cores(self) -> bool:
+        """The id that names this backend's matrix-core decode kernels (wg 512, lanes 64,
+        rows 16: a geometry no WGSL variant has)."""
+        return (self.wg, self.lanes, self.rows) == (512, 64, 16)
+
     def suits(self, t: TensorType) -> bool:
-        return self.lanes <= 32 or (t == TensorType.q8_0 and self.lanes == 64)
+        """src/kernels/kernels.zig:355-357, and with the edit the HIP backend asks for: the
+        matrix-core id suits every type its kernels take."""
+        return self.lanes <= 32 or (t == TensorType.q8_0 and self.lanes == 64) or \
+            (self.is_matrix_cores() and t in (TensorType.q8_0, TensorType.q3_k, TensorType.q4_k, TensorType.q5_k, TensorType.q6_k))
 
 
+@dataclass(frozen=True)
+class DeviceLimits:
+    """Device limits kernel variants are checked against (src/kernels/kernels.zig:390-393:
+    WebGPU's defaults); `hip()` is what the HIP backend reports (1024 threads a workgroup,
+    160 KB of workgroup memory a CU), under which the matrix-core id fits."""
+
+    invocations: int = 256
+    workgroup_storage: int = 16384
+
+    @classmethod
+    def hip(cls) -> "DeviceLimits":
+        return cls(invocations=1024, workgroup_storage=160 * 1024)
+
+
+# The reference's sweep (src/kernels/kernels.zig:372-381), and the HIP backend's: the same
+# sixteen and the matrix-core id.
 MatvecVariant.candidates = tuple(
     MatvecVariant(wg=wg, lanes=lanes, rows=rows) for wg in (256, 128) for lanes in (32, 16, 8, 64) for rows in (1, 2)
 )
+MatvecVariant.hip_candidates = MatvecVariant.candidates + (MatvecVariant(wg=512, lanes=64, rows=16),)
 
 
 # Reserved create_kernel variants of the prefill identities
