@@ -43,8 +43,8 @@ MFMA_BF16_PEAK_TFLOPS = 2500.0  # MI355X dense bf16, published
 MFMA_INT8_PEAK_TOPS = 5000.0    # MI355X dense int8, published
 ROTATE_BYTES = 640 << 20    # distinct weight bytes a rotation must exceed (L2 + Infinity Cache, with margin)
 # HBM bytes one launch of the headline kernel moves, from rocprofv3 FETCH_SIZE and
-# WRITE_SIZE counter runs scaled by a plain copy of known size (profiles/matvec_quant_kernel_q4k_c2.txt).
-C2_TRAFFIC_BYTES = 33_395_507
+# WRITE_SIZE counter runs scaled by a plain copy of known size (profiles/matvec_quant_row_kernel_q4k_c2.txt).
+C2_TRAFFIC_BYTES = 33_427_456
 
 
 def sig2(v: float) -> float:
