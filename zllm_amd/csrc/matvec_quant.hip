@@ -1003,8 +1003,13 @@ __global__ __launch_bounds__(256) void matvec_quant_row_kernel(KArgs q) {
         const float4 *src = lds4 + (tsub < tasks ? tsub : 0u) * (kTaskStride / 4u);
 #pragma unroll
         for (int v = 0; v < 16; v++) {
-            const float4 f = tsub < tasks ? src[v] : make_float4(0.f, 0.f, 0.f, 0.f);
+            const float4 f = src[v];
             xr[4 * v] = f.x; xr[4 * v + 1] = f.y; xr[4 * v + 2] = f.z; xr[4 * v + 3] = f.w;
+        }
+        // (a lane without a task multiplies zeros by zeros, whatever the inputs hold)
+        if (tsub >= tasks) {
+#pragma unroll
+            for (int e = 0; e < 64; e++) xr[e] = 0.f;
         }
 #pragma unroll
         for (int s = 0; s < NSUM; s++) {
