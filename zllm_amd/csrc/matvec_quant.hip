@@ -919,7 +919,9 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
 // The staging of the inputs, a task's dot product and the lanes' reduction are the code of the
 // kernel above, so the results are its bits.
 // Passes whose loads are in flight ahead of the one multiplied. Measured on 14336 x 4096 Q4_K
-// (7.9 us with one): two or three passes ahead 8.6 / 9.8 us, and no better with fewer workgroups.
+// (7.9 us with one): two or three passes ahead 8.6 / 9.8 us, and no better with fewer workgroups;
+// two passes asked for before the inputs are staged (instead of one) 8.7 us; the first pass
+// asked for only once the inputs have arrived 8.0 us.
 constexpr int kRowDepth = 1;
 template <class P, bool PAIR, int SEG_LOG2>
 __global__ __launch_bounds__(256) void matvec_quant_row_kernel(KArgs q) {
@@ -1297,97 +1299,115 @@ static zhip_result run_long(const Dispatch &d, const KArgs &q, uint32_t blocks) 
 }
 
 // One-token steps over rows of 65 .. 256 tasks (k above 4096, up to 16384: the FFN-down shapes).
-// The kernel above walks such a row with one wave, a lane taking a task of every 64-task slice
-// in turn with its inputs read from LDS each time. Here a slice is a wave's for the whole
+// matvec_quant_kernel walks such a row with one wave, a lane taking a task of every 64-task
+// slice in turn with its inputs read from LDS each time. Here a slice is a wave's for the whole
 // launch, so the lane's 64 inputs stay in registers as in the short-row case: the waves of a
-// group (two for two slices, four for three or four) multiply the same rows, R at a time, each
-// its own slice, leave the lanes' partial sums in LDS, and behind one barrier the group's waves
-// add them, each for its share of the R rows, in the order of the slices, which is the order
-// in which the lane of the kernel above adds its tasks; the lanes' reduction is the same code.
+// group (one a slice: two, three or four) multiply the same rows, R at a time, each its own
+// slice, leave the lanes' partial sums in LDS, and behind one barrier the group's waves add
+// them, each for its share of the R rows, in the order of the slices, which is the order in
+// which the lane of matvec_quant_kernel adds its tasks; the lanes' reduction is the same code.
 // The same bits, and the arithmetic of a short row per weight.
-template <class P, bool PAIR, int R>
-__global__ __launch_bounds__(256) void matvec_quant_sliced_kernel(KArgs q) {
+//
+// The walk is matvec_quant_row_kernel's: a workgroup of NW waves (a multiple of the slices)
+// stages the token once for all its groups, a unit's position lives in scalar registers and
+// its loads go through a buffer that is the unit's row (a unit past the end, or a lane without
+// a task, loads zeros). What the outputs hold, for a step that accumulates, is asked for before
+// the round's loads: loads complete in order within a wave, so behind them it would wait for
+// rows of the next round.
+template <class P, bool PAIR, int R, int NW>
+__global__ __launch_bounds__(64 * NW) void matvec_quant_slices_kernel(KArgs q) {
     const MvArgs &a = q.a;
-    extern __shared__ float4 lds4[];  // [wave]: its slice of the token in task order, padded per task; afterwards the partial sums
+    extern __shared__ float4 lds4[];  // the token in task order, padded per task; then the partial sums [parity][group][unit of the round][slice][row][lane]
     __shared__ float red[4];
     constexpr int NSUM = P::NSUM, RUN = 64 / NSUM, kRows = PAIR ? 2 : 1;
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
-    const uint32_t tasks = q.tasks, slices = (tasks + 63u) / 64u;
-    const Masks nm = q.nm;
-    const uint32_t per_group = slices <= 2u ? 2u : 4u, groups_here = 4u / per_group;
-    const uint32_t grp = wave / per_group, slice = wave % per_group;
+    constexpr uint32_t THREADS = 64u * NW;
+    constexpr int XV = (4096 + THREADS - 1) / THREADS;  // vectors of the token a thread stages (k <= 16384)
+    static_assert(R % 2 == 0, "the buffers alternate by name");
+    const uint32_t tid = threadIdx.x, lane = tid & 63u;
+    const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
+    const uint32_t tasks = q.tasks, slices = (tasks + 63u) / 64u, k4 = a.k / 4u;
+    const uint32_t groups_here = (uint32_t)NW / slices;
+    const uint32_t grp = wave / slices, slice = wave % slices;
     const uint32_t group = blockIdx.x * groups_here + grp, groups = gridDim.x * groups_here;
     const uint32_t units = a.rows;  // a unit: an output (its row, or its gate row and up row)
     const uint32_t task = lane + 64u * slice;
     const bool active = task < tasks;
+    const bool norm = (a.flags & FLAG_NORM) != 0, accumulate = (a.flags & FLAG_ACCUMULATE) != 0;
 
-    // Unit n of the group's walk (R consecutive units a round, the groups' rounds interleaved)
-    // and its rows; past the end the loads are clamped to a valid row and their results unused.
-    auto unit_of = [&](uint32_t n) { return ((n / R) * groups + group) * R + n % R; };
-    const uint32_t rounds = (units + groups * R - 1u) / (groups * R);  // the same for every group: the barriers below are the workgroup's
-    typename P::Raw cur[kRows], next[kRows];
-    auto load_unit = [&](uint32_t n, typename P::Raw (&dst)[kRows]) __attribute__((always_inline)) {
-        const uint32_t u = unit_of(n), j = u < units ? u : units - 1u, tk = active ? task : 0u;
-        dst[0] = P::load(a.w + (size_t)j * a.row_bytes, a.k, tk);
-        if (PAIR) dst[kRows - 1] = P::load(a.w + (size_t)(a.half + j) * a.row_bytes, a.k, tk);
-    };
-    load_unit(0, cur);  // (before the inputs: the stream starts while they are staged)
-
-    // A wave stages its own slice (64 tasks, 1024 vectors: sixteen a lane, asked for together)
-    // through its own part of LDS, in task order and padded per task as in the kernel above,
-    // and reads its lanes' tasks back; only the RMSNorm sum needs the other waves, and is added
-    // as stage_token adds it (vector i by thread i % 256, the waves' sums in order).
-    const uint32_t k4 = a.k / 4u;
+    // The token's inputs first, then the first rows (loads complete in order within a wave).
     const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)q.t0 * a.xr);
     const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
-    const bool norm = (a.flags & FLAG_NORM) != 0;
+    float4 xv[XV], gv[XV];
+#pragma unroll
+    for (int j = 0; j < XV; j++) {
+        const uint32_t i = tid + THREADS * j;
+        xv[j] = i < k4 ? xrow[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        if (norm) gv[j] = i < k4 ? nw[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+
+    // Unit n of the group's walk: R consecutive units a round, the groups' rounds interleaved.
+    auto unit_of = [&](uint32_t n) { return ((n / R) * groups + group) * R + n % R; };
+    const uint32_t rounds = (units + groups * R - 1u) / (groups * R);  // the same for every group: the barriers below are the workgroup's
+    const typename P::Where at = active && grp < groups_here ? P::where(0u, a.k, task) : P::nowhere();
+    auto fetch = [&](uint32_t n, typename P::Raw (&dst)[kRows]) __attribute__((always_inline)) {
+        const uint32_t u = unit_of(n);
+        const bool live = u < units;
+        const uint64_t off = live ? (uint64_t)u * a.row_bytes : 0u;
+        const uint32_t left = live ? a.row_bytes : 0u;
+        dst[0] = P::fetch(__builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a.w + off), 0, (int)left, 0x00020000), at);
+        if (PAIR) dst[kRows - 1] = P::fetch(__builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(a.w + (size_t)a.half * a.row_bytes + off), 0, (int)left, 0x00020000), at);
+        __builtin_amdgcn_sched_barrier(0);  // (the loads stay ahead of the multiply that follows them in the source)
+    };
+    typename P::Raw cur[kRows], nxt[kRows];
+    fetch(0, cur);
+
+    // stage_token's arithmetic: the RMSNorm sum by the first 256 threads, vector i by thread
+    // i % 256 and the four waves' sums in order; then every thread stages the vectors it loaded.
     float scale = 1.0f;
     if (norm) {
-        float ss = 0.f;
+        if (tid < 256u) {
+            float ss = 0.f;
 #pragma unroll 4
-        for (uint32_t i = tid; i < k4; i += 256u) {
-            const float4 v = xrow[i];
-            ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+            for (uint32_t i = tid; i < k4; i += 256u) {
+                const float4 v = xrow[i];
+                ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+            }
+            ss = wave_sum(ss);
+            if (lane == 0) red[wave] = ss;
         }
-        ss = wave_sum(ss);
-        if (lane == 0) red[wave] = ss;
         __syncthreads();
-        ss = (red[0] + red[1]) + (red[2] + red[3]);
-        scale = 1.0f / sqrtf(ss / (float)a.k + a.eps);
+        const float total = (red[0] + red[1]) + (red[2] + red[3]);
+        scale = 1.0f / sqrtf(total / (float)a.k + a.eps);
     }
+#pragma unroll
+    for (int j = 0; j < XV; j++) {
+        const uint32_t i = tid + THREADS * j;
+        if (i >= k4) continue;
+        float4 v = xv[j];
+        if (norm) {
+            v.x = v.x * scale * gv[j].x; v.y = v.y * scale * gv[j].y;
+            v.z = v.z * scale * gv[j].z; v.w = v.w * scale * gv[j].w;
+        }
+        if (a.act_div > 0.f) {
+            v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
+            v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+        }
+        const uint32_t p = P::stage_index(i);
+        lds4[p + (p >> 4)] = v;
+    }
+    __syncthreads();
+
     float xr[64], xsum[NSUM];
     {
-        float4 *mine4 = lds4 + wave * (64u * (kTaskStride / 4u));
-        float4 in[16], g[16];
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const uint32_t gi = 1024u * slice + lane + 64u * j;
-            const bool have = gi < k4 && slice < slices;
-            in[j] = have ? xrow[gi] : make_float4(0.f, 0.f, 0.f, 0.f);
-            if (norm) g[j] = have ? nw[gi] : make_float4(0.f, 0.f, 0.f, 0.f);
-        }
-#pragma unroll
-        for (int j = 0; j < 16; j++) {
-            const uint32_t gi = 1024u * slice + lane + 64u * j;
-            if (gi >= k4 || slice >= slices) continue;
-            float4 v = in[j];
-            if (norm) {
-                v.x = v.x * scale * g[j].x; v.y = v.y * scale * g[j].y;
-                v.z = v.z * scale * g[j].z; v.w = v.w * scale * g[j].w;
-            }
-            if (a.act_div > 0.f) {
-                v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
-                v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
-            }
-            const uint32_t p = P::stage_index(gi) - 1024u * slice;
-            mine4[p + (p >> 4)] = v;
-        }
-        asm volatile("" ::: "memory");  // (a wave's LDS operations complete in order: its reads below see its writes above)
-        const float4 *src = mine4 + lane * (kTaskStride / 4u);
+        const float4 *src = lds4 + (active ? task : 0u) * (kTaskStride / 4u);
 #pragma unroll
         for (int v = 0; v < 16; v++) {
             const float4 f = src[v];
             xr[4 * v] = f.x; xr[4 * v + 1] = f.y; xr[4 * v + 2] = f.z; xr[4 * v + 3] = f.w;
+        }
+        if (!active) {
+#pragma unroll
+            for (int e = 0; e < 64; e++) xr[e] = 0.f;
         }
 #pragma unroll
         for (int sr = 0; sr < NSUM; sr++) {
@@ -1396,60 +1416,77 @@ __global__ __launch_bounds__(256) void matvec_quant_sliced_kernel(KArgs q) {
             for (int e = 0; e < RUN; e++) xsum[sr] += xr[sr * RUN + e];
         }
     }
-    __syncthreads();  // the token's space now takes the partial sums: [round parity][wave][unit of the round][row][lane]
-    float *part = reinterpret_cast<float *>(lds4);
+    const Masks nm = q.nm;
+    const typename P::Keys ch = P::keys(task & 3u);
+    const size_t out0 = (size_t)q.t0 * a.out_stride + a.col0;
+    // (the partial sums lie behind the token: no barrier between reading the one and writing the other)
+    float *part = reinterpret_cast<float *>(lds4 + (size_t)tasks * (kTaskStride / 4u));
+    constexpr uint32_t kMine = 2;  // units of a round a wave finishes, at most: R <= 4 over two or more slices
 
     for (uint32_t round = 0; round < rounds; round++) {
-        float *mine = part + (((round & 1u) * 4u + wave) * R) * kRows * 64u;
+        float *mine = part + ((((round & 1u) * groups_here + grp) * R) * slices + 0u) * kRows * 64u;
+        // What the outputs hold, for the units this wave will finish: asked for before the
+        // round's loads, so that the wait for it is the wait for rows the wave needs anyway.
+        float held[kMine];
+        if (accumulate) {
+#pragma unroll
+            for (uint32_t i = 0; i < kMine; i++) {
+                const uint32_t r = slice + i * slices, u = unit_of(round * R + r);
+                held[i] = (lane == 63u && r < (uint32_t)R && u < units) ? a.out[out0 + u] : 0.f;
+            }
+        }
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            load_unit(round * R + r + 1u, next);
             float v[kRows][1];
-            P::template dot<1, kRows>(cur, task & 3u, nm,
-                [&](int, int vi) { return make_float4(xr[4 * vi], xr[4 * vi + 1], xr[4 * vi + 2], xr[4 * vi + 3]); },
-                [&](int, int sr) { return xsum[sr]; }, v);
+            if (r % 2 == 0) {
+                fetch(round * R + r + 1u, nxt);
+                P::template dot<1, kRows>(cur, ch, nm,
+                    [&](int, int vi) { return make_float4(xr[4 * vi], xr[4 * vi + 1], xr[4 * vi + 2], xr[4 * vi + 3]); },
+                    [&](int, int sr) { return xsum[sr]; }, v);
+            } else {
+                fetch(round * R + r + 1u, cur);
+                P::template dot<1, kRows>(nxt, ch, nm,
+                    [&](int, int vi) { return make_float4(xr[4 * vi], xr[4 * vi + 1], xr[4 * vi + 2], xr[4 * vi + 3]); },
+                    [&](int, int sr) { return xsum[sr]; }, v);
+            }
 #pragma unroll
-            for (int j = 0; j < kRows; j++) mine[(r * kRows + j) * 64u + lane] = v[j][0];
-#pragma unroll
-            for (int j = 0; j < kRows; j++) cur[j] = next[j];
+            for (int j = 0; j < kRows; j++) mine[((r * slices + slice) * kRows + j) * 64u + lane] = v[j][0];
         }
-        __syncthreads();
+        // (a barrier that leaves the next unit's loads in flight)
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
         // The group's waves share the round's units; a unit's slices are added in order, a lane
         // leaving out the slice in which it has no task.
-        const float *theirs = part + (((round & 1u) * 4u + grp * per_group) * R) * kRows * 64u;
-        for (uint32_t r = slice; r < (uint32_t)R; r += per_group) {
+#pragma unroll
+        for (uint32_t i = 0; i < kMine; i++) {
+            const uint32_t r = slice + i * slices;
+            if (r >= (uint32_t)R) break;
+            const float *theirs = mine + (r * slices) * kRows * 64u;
             float acc[kRows];
 #pragma unroll
             for (int j = 0; j < kRows; j++) acc[j] = 0.f;
             for (uint32_t sl = 0; sl < slices; sl++) {
                 if (lane + 64u * sl >= tasks) continue;
 #pragma unroll
-                for (int j = 0; j < kRows; j++) acc[j] += theirs[((sl * R + r) * kRows + j) * 64u + lane];
+                for (int j = 0; j < kRows; j++) acc[j] += theirs[(sl * kRows + j) * 64u + lane];
             }
             const float s0 = segment_sum(acc[0], 6u), s1 = PAIR ? segment_sum(acc[kRows - 1], 6u) : 0.f;
             const uint32_t u = unit_of(round * R + r);
             if (lane == 63u && u < units) {
-                const size_t o = (size_t)q.t0 * a.out_stride + a.col0 + u;
                 float res = PAIR ? silu_f(s0) * s1 : s0;
-                if (a.flags & FLAG_ACCUMULATE) res += a.out[o];
-                a.out[o] = res;
+                if (accumulate) res += held[i];
+                a.out[out0 + u] = res;
             }
         }
         // (the other parity's space is written next; this one again only behind the next barrier)
     }
 }
 
-template <class P, bool PAIR, int R>
-static zhip_result run_sliced(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
-    static bool configured = false;  // dynamic LDS above 64 KiB needs opting in once
-    if (lds > 65536u && !configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_quant_sliced_kernel<P, PAIR, R>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
-            (void)hipGetLastError();
-            return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", P::name(), lds);
-        }
-        configured = true;
-    }
-    hipLaunchKernelGGL((matvec_quant_sliced_kernel<P, PAIR, R>), dim3(blocks), dim3(256), lds, d.stream, q);
+template <class P, bool PAIR, int R, int NW>
+static zhip_result run_slices(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
+    if (!lds_opt_in<matvec_quant_slices_kernel<P, PAIR, R, NW>, 160 * 1024 - 64>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", P::name(), lds);
+    hipLaunchKernelGGL((matvec_quant_slices_kernel<P, PAIR, R, NW>), dim3(blocks), dim3(64 * NW), lds, d.stream, q);
     return check_launch(d, P::name());
 }
 
@@ -1517,19 +1554,30 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
         q.mt = left < mt ? left : mt;
         const uint32_t lds = (uint32_t)(mt * tok_lds);
         if (a.m == 1u && q.tasks > 64u && q.tasks <= 256u) {
-            // (the partial sums take the inputs' space: 2 x 4 waves x R units x rows x 64 lanes, 16 KB at most)
-            const uint32_t lds1 = 4u * 64u * kTaskStride * 4u;  // a slice's inputs a wave
-            const uint32_t groups_here = q.tasks <= 128u ? 2u : 1u;
-            const uint32_t cap = (uint32_t)d.dev->compute_units * 2u;  // two workgroups' LDS a CU
-            // Four units a round where that still gives every workgroup a round of its own
-            // (4096 x 8192: 9.8 -> 8.5 us), eight otherwise; the gate / up step always four.
-            const uint32_t want4 = (a.rows + groups_here * 4u - 1u) / (groups_here * 4u);
-            const bool eight = !pair && want4 > cap;
-            const uint32_t want = eight ? (want4 + 1u) / 2u : want4;
-            const uint32_t blocks = want < cap ? want : cap;
+            // Eight waves a workgroup (and CU) for rows of two or four slices, twelve for three.
+            // Measured, Q4_K 4096 x 14336: 9.9 us with eight, 10.4 with twelve, 14.6 with sixteen
+            // (their registers spill); 4096 x 11008 (three slices): 8.0 us with twelve, 8.9 / 9.3
+            // with nine / six. Two or four units a round, whichever leaves fewer empty places in
+            // the last round; of equal, four for light units and two for heavy ones (from 3.5 KB
+            // a wave and unit: Q8_0 rows, gate / up pairs): Q4_K 9.9 / 10.4 us at four / two,
+            // Q3_K 10.1 / 11.5, Q8_0 13.3 / 12.9, a Q4_K gate / up pair over 8192 28.2 / 25.0.
+            const uint32_t slices = (q.tasks + 63u) / 64u, nw = slices == 3u ? 12u : 8u, groups_here = nw / slices;
+            const uint32_t cus = (uint32_t)d.dev->compute_units;
+            const uint32_t want = (a.rows + groups_here * 2u - 1u) / (groups_here * 2u);
+            const uint32_t blocks = want < cus ? want : cus;
+            const uint32_t groups = blocks * groups_here;
+            const uint32_t slots4 = (a.rows + groups * 4u - 1u) / (groups * 4u) * 4u, slots2 = (a.rows + groups * 2u - 1u) / (groups * 2u) * 2u;
+            const bool heavy = (uint64_t)a.row_bytes * (pair ? 2u : 1u) / slices >= 3584u;
+            const bool two = slots2 < slots4 || (slots2 == slots4 && heavy);
+            const uint32_t lds1 = q.tasks * kTaskStride * 4u + 2u * nw * (two ? 2u : 4u) * (pair ? 2u : 1u) * 256u;
             zhip_result r;
-            if (pair) r = run_sliced<P, true, 4>(d, q, lds1, blocks);
-            else r = eight ? run_sliced<P, false, 8>(d, q, lds1, blocks) : run_sliced<P, false, 4>(d, q, lds1, blocks);
+            if (nw == 12u) {
+                if (pair) r = two ? run_slices<P, true, 2, 12>(d, q, lds1, blocks) : run_slices<P, true, 4, 12>(d, q, lds1, blocks);
+                else r = two ? run_slices<P, false, 2, 12>(d, q, lds1, blocks) : run_slices<P, false, 4, 12>(d, q, lds1, blocks);
+            } else {
+                if (pair) r = two ? run_slices<P, true, 2, 8>(d, q, lds1, blocks) : run_slices<P, true, 4, 8>(d, q, lds1, blocks);
+                else r = two ? run_slices<P, false, 2, 8>(d, q, lds1, blocks) : run_slices<P, false, 4, 8>(d, q, lds1, blocks);
+            }
             if (r != ZHIP_OK) return r;
             t0 += q.mt;
             continue;
