@@ -27,16 +27,17 @@
 // depend on how many tokens share the launch or on which variant below runs
 // it: the reference's bitwise split invariant (matvec_quant.wgsl.hbs:14-18).
 //
-// Variants. XREG (one token, at most one task per lane, i.e. k <= 4096): the
-// lane's 64 inputs never change from row to row, so they live in registers and
-// the loop touches nothing but the weight stream. Otherwise inputs are read
-// from a bank-conflict-free padded LDS copy kept in task order, once per task
-// for both rows of a pass (two outputs, or the gate and up rows of one output
-// with SILU_PAIR). In both, the next task's vectors are loaded before the
-// current one is multiplied. An XREG workgroup asks for the token's inputs (and
-// norm weights) before its first weights: loads complete in order within a
-// wave, so inputs requested behind a weight row would wait for that row's trip
-// to memory before the staging could start.
+// Kernels. matvec_quant_kernel (steps of one to four tokens, any row length): inputs are read
+// from a bank-conflict-free padded LDS copy kept in task order, once per task for both rows of
+// a pass (two outputs, or the gate and up rows of one output with SILU_PAIR), the next task's
+// vectors loaded before the current one is multiplied. matvec_quant_row_kernel (one token, at
+// most one task per lane, i.e. k <= 4096): the lane's 64 inputs never change from row to row,
+// so they live in registers and the loop touches nothing but the weight stream; it asks for the
+// token's inputs (and norm weights) before its first weights: loads complete in order within a
+// wave, so inputs requested behind a weight row would wait for that row's trip to memory before
+// the staging could start. matvec_quant_slices_kernel: the same for one token over longer rows,
+// a 64-task slice of the row a wave. matvec_quant_long_kernel: steps of several tokens over
+// rows too long for the tokens to share LDS, tile by tile.
 #include <hip/hip_runtime.h>
 
 #include "common.h"
@@ -612,11 +613,10 @@ struct KArgs {
     uint32_t seg_log2;  // lanes per row: 4, 5 or 6
     uint32_t tasks;     // k / 64
     Masks nm;
-    uint32_t defer;     // finished rows' outputs wait in registers for one store at the end of the wave's walk
 };
 
 // STG: tokens whose inputs are loaded at once ahead of the weights (0: none, staged by stage_token).
-template <class P, int MT, bool PAIR, bool XREG, int STG>
+template <class P, int MT, bool PAIR, int STG>
 __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     const MvArgs &a = q.a;
     extern __shared__ float4 lds4[];
@@ -628,9 +628,8 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     float *sums_lds = reinterpret_cast<float *>(lds4 + (size_t)MT * tok_stride4);
 
     // Rows a pass takes: the gate and up rows of an output, or two outputs so
-    // that one read of the inputs from LDS serves both; with the inputs in
-    // registers a pass is a single row.
-    constexpr int kRows = (PAIR || !XREG) ? 2 : 1;
+    // that one read of the inputs from LDS serves both.
+    constexpr int kRows = 2;
     const uint32_t gwave = blockIdx.x * 4u + wave, nwaves = gridDim.x * 4u;
     const uint32_t seg = 1u << q.seg_log2;
     const uint32_t tsub = lane & (seg - 1u), rsub = lane >> q.seg_log2, rpi = 64u >> q.seg_log2;
@@ -684,7 +683,7 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     // more raises the register count of the whole kernel, and past 256 the multiply loses its
     // second wave a SIMD, which a large matrix pays for and a small one does not.
     constexpr int TG = STG > 0 ? STG : 1;
-    const bool early = XREG || (STG > 0 && a.k <= 4096u);
+    const bool early = STG > 0 && a.k <= 4096u;
     float4 xv[TG][4], gv[4];
     auto load_tokens = [&](int first) __attribute__((always_inline)) {
 #pragma unroll
@@ -715,8 +714,6 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
         advance(lc);
     }
 
-    float xr[64];
-    float xsum[NSUM];
     // Stage the pass's tokens in task order, padded per task (coalesced loads;
     // a lane's own 64 inputs are 256 bytes apart from its neighbour's).
     if (early) {
@@ -783,24 +780,7 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
         }
     }
     __syncthreads();
-    if (XREG) {
-        // The lane's one task's inputs into registers, and their run sums in
-        // the same order the LDS pass below adds them.
-        if (gwave >= units) return;
-        const uint32_t task = tsub < tasks ? tsub : 0u;
-        const float4 *src = lds4 + task * (kTaskStride / 4u);
-#pragma unroll
-        for (int v = 0; v < 16; v++) {
-            const float4 f = src[v];
-            xr[4 * v] = f.x; xr[4 * v + 1] = f.y; xr[4 * v + 2] = f.z; xr[4 * v + 3] = f.w;
-        }
-#pragma unroll
-        for (int s = 0; s < NSUM; s++) {
-            xsum[s] = 0.f;
-#pragma unroll
-            for (int e = 0; e < RUN; e++) xsum[s] += xr[s * RUN + e];
-        }
-    } else {
+    {
         for (uint32_t idx = tid; idx < (uint32_t)MT * tasks * NSUM; idx += 256u) {
             const uint32_t t = idx / (tasks * NSUM), rem = idx % (tasks * NSUM);
             const float *src = reinterpret_cast<const float *>(lds4 + (size_t)t * tok_stride4) + (rem / NSUM) * kTaskStride + (rem % NSUM) * RUN;
@@ -819,22 +799,6 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
 #pragma unroll
         for (int t = 0; t < MT; t++) acc[j][t] = 0.f;
 
-    // One-token steps over rows of 4096 weights keep a finished row's output in the lane of
-    // its number and store them together when the wave's walk ends (a format's DEFER: stores
-    // between the loads of the stream cost 0.1 - 0.3 us of the 14336 x 4096 launch for Q4_K,
-    // Q5_K and Q3_K; Q6_K, whose multiply needs the most registers, lost 0.4 us and Q8_0 gained
-    // nothing, so they store row by row).
-    float kept = 0.f;
-    uint32_t nkept = 0, kept_first = gwave;
-    auto flush_kept = [&]() {
-        const uint32_t j = kept_first + lane * nwaves;
-        if (lane < nkept && j < a.rows) {
-            const size_t o = (size_t)q.t0 * a.out_stride + a.col0 + j;
-            a.out[o] = (a.flags & FLAG_ACCUMULATE) ? kept + a.out[o] : kept;
-        }
-        kept_first += nkept * nwaves;
-        nkept = 0;
-    };
     // Multiplies the position `c` from `cur`; at a unit's last slice reduces
     // and stores its outputs.
     auto compute = [&](const Cursor &c, const typename P::Raw (&cur)[kRows]) {
@@ -842,17 +806,11 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
         if (task < tasks) {
             const uint32_t ch = task & 3u;
             float v[kRows][MT];
-            if (XREG) {
-                P::template dot<MT, kRows>(cur, ch, q.nm,
-                    [&](int, int vi) { return make_float4(xr[4 * vi], xr[4 * vi + 1], xr[4 * vi + 2], xr[4 * vi + 3]); },
-                    [&](int, int s) { return xsum[s]; }, v);
-            } else {
-                const float4 *xt = lds4 + task * (kTaskStride / 4u);
-                const float *st = sums_lds + NSUM * task;
-                P::template dot<MT, kRows>(cur, ch, q.nm,
-                    [&](int t, int vi) { return xt[(size_t)t * tok_stride4 + vi]; },
-                    [&](int t, int s) { return st[(size_t)t * tasks * NSUM + s]; }, v);
-            }
+            const float4 *xt = lds4 + task * (kTaskStride / 4u);
+            const float *st = sums_lds + NSUM * task;
+            P::template dot<MT, kRows>(cur, ch, q.nm,
+                [&](int t, int vi) { return xt[(size_t)t * tok_stride4 + vi]; },
+                [&](int t, int s) { return st[(size_t)t * tasks * NSUM + s]; }, v);
 #pragma unroll
             for (int j = 0; j < kRows; j++)
 #pragma unroll
@@ -864,13 +822,6 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
                 const float s0 = segment_sum(acc[0][t], q.seg_log2);
                 const float s1 = kRows == 2 ? segment_sum(acc[kRows - 1][t], q.seg_log2) : 0.f;
                 acc[0][t] = acc[kRows - 1][t] = 0.f;
-                if (P::DEFER && XREG && q.defer) {
-                    const float r = PAIR ? silu_f(s0) * s1 : s0;
-                    const float total = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(r), 63));
-                    kept = lane == nkept ? total : kept;
-                    nkept++;
-                    if (nkept == 64u) flush_kept();
-                } else
                 if (writer && (uint32_t)t < q.mt && c.j0 < a.rows) {
                     const size_t o = (size_t)(q.t0 + t) * a.out_stride + a.col0 + c.j0;
                     if (PAIR) {
@@ -905,10 +856,9 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
             done = cc.u >= units;
         }
     }
-    if (P::DEFER && XREG && q.defer) flush_kept();
 }
 
-// One-token steps over rows of at most 64 tasks: the kernel above with XREG, taken apart so that
+// One-token steps over rows of at most 64 tasks, with the lane's inputs in registers, so that
 // the loop holds nothing but the weight stream's loads and the multiply. A wave's walk is wave
 // uniform here: pass u covers rows u * RPI .. + RPI - 1 (RPI = 64 >> SEG_LOG2 rows side by side
 // in the wave), so the pass's position lives in scalar registers, a lane's byte offsets within
@@ -1500,17 +1450,17 @@ static zhip_result run_row(const Dispatch &d, const KArgs &q, uint32_t lds, uint
     return check_launch(d, P::name());
 }
 
-template <class P, int MT, bool PAIR, bool XREG, int STG>
+template <class P, int MT, bool PAIR, int STG>
 static zhip_result run_quant(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
     static bool configured = false;  // dynamic LDS above 64 KiB needs opting in once
     if (lds > 65536u && !configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_quant_kernel<P, MT, PAIR, XREG, STG>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
+        if (hipFuncSetAttribute(reinterpret_cast<const void *>(matvec_quant_kernel<P, MT, PAIR, STG>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 64) != hipSuccess) {
             (void)hipGetLastError();
             return fail(d, ZHIP_E_BAD_COMMAND, "%s: k = %u with %d tokens does not fit workgroup memory", P::name(), q.a.k, MT);
         }
         configured = true;
     }
-    hipLaunchKernelGGL((matvec_quant_kernel<P, MT, PAIR, XREG, STG>), dim3(blocks), dim3(256), lds, d.stream, q);
+    hipLaunchKernelGGL((matvec_quant_kernel<P, MT, PAIR, STG>), dim3(blocks), dim3(256), lds, d.stream, q);
     return check_launch(d, P::name());
 }
 
@@ -1590,7 +1540,6 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
         // more of them repeat the input staging, fewer leave too few loads in flight.
         const uint32_t cap = (uint32_t)d.dev->compute_units * (xreg ? 3u : 2u);
         const uint32_t blocks = want < cap ? want : cap;
-        q.defer = (P::DEFER && xreg && q.seg_log2 == 6u) ? 1u : 0u;
         zhip_result r;
         // A launch of at most one workgroup a CU is a chain of trips to memory and has the CU's
         // registers to itself: all of the pass's tokens go in one. With more workgroups a CU the
@@ -1610,13 +1559,13 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
             const bool three = !pair && (uint64_t)rpi * a.row_bytes <= 3072u && passes >= cus * 48u;
             const uint32_t cap = cus * (three ? 3u : 2u);
             r = pair ? run_row<P, true>(d, q, q.tasks * kTaskStride * 4u, row_want < cap ? row_want : cap) : run_row<P, false>(d, q, q.tasks * kTaskStride * 4u, row_want < cap ? row_want : cap);
-        } else if (mt == 1u) r = pair ? run_quant<P, 1, true, false, 1>(d, q, lds, blocks) : run_quant<P, 1, false, false, 1>(d, q, lds, blocks);
+        } else if (mt == 1u) r = pair ? run_quant<P, 1, true, 1>(d, q, lds, blocks) : run_quant<P, 1, false, 1>(d, q, lds, blocks);
         else if (mt == 2u) {
-            if (small && P::STAGE2 != 2) r = pair ? run_quant<P, 2, true, false, 2>(d, q, lds, blocks) : run_quant<P, 2, false, false, 2>(d, q, lds, blocks);
-            else r = pair ? run_quant<P, 2, true, false, P::STAGE2>(d, q, lds, blocks) : run_quant<P, 2, false, false, P::STAGE2>(d, q, lds, blocks);
+            if (small && P::STAGE2 != 2) r = pair ? run_quant<P, 2, true, 2>(d, q, lds, blocks) : run_quant<P, 2, false, 2>(d, q, lds, blocks);
+            else r = pair ? run_quant<P, 2, true, P::STAGE2>(d, q, lds, blocks) : run_quant<P, 2, false, P::STAGE2>(d, q, lds, blocks);
         } else {
-            if (small && P::ALL4 && P::STAGE4 != 4) r = pair ? run_quant<P, 4, true, false, 4>(d, q, lds, blocks) : run_quant<P, 4, false, false, 4>(d, q, lds, blocks);
-            else r = pair ? run_quant<P, 4, true, false, P::STAGE4>(d, q, lds, blocks) : run_quant<P, 4, false, false, P::STAGE4>(d, q, lds, blocks);
+            if (small && P::ALL4 && P::STAGE4 != 4) r = pair ? run_quant<P, 4, true, 4>(d, q, lds, blocks) : run_quant<P, 4, false, 4>(d, q, lds, blocks);
+            else r = pair ? run_quant<P, 4, true, P::STAGE4>(d, q, lds, blocks) : run_quant<P, 4, false, P::STAGE4>(d, q, lds, blocks);
         }
         if (r != ZHIP_OK) return r;
         t0 += q.mt;
