@@ -160,6 +160,7 @@ struct KQ8 {
     static constexpr int STAGE2 = 0, STAGE4 = 1;  // tokens whose inputs are loaded at once
     static constexpr bool ALL4 = true;            // a launch of at most a workgroup a CU stages a pass of four at once
     static constexpr bool DEFER = false;
+    static constexpr bool PAIR2 = false;  // a two-token gate / up step with the inputs in registers leaves two waves a SIMD their registers
     static const char *name() { return "matvec_q8_0"; }
     struct Raw {
         uint4 q[4];
@@ -232,6 +233,7 @@ struct KQ3 {
     static constexpr int STAGE2 = 2, STAGE4 = 2;  // tokens whose inputs are loaded at once
     static constexpr bool ALL4 = false;           // (four at once measured slower on every shape: 1024 x 4096 7.7 against 7.1 us)
     static constexpr bool DEFER = true;
+    static constexpr bool PAIR2 = true;  // a two-token gate / up step with the inputs in registers leaves two waves a SIMD their registers
     static const char *name() { return "matvec_q3_k"; }
     struct Raw {
         uint4 u[2];
@@ -319,6 +321,7 @@ struct KQ4 {
     static constexpr int STAGE2 = 2, STAGE4 = 1;  // tokens whose inputs are loaded at once
     static constexpr bool ALL4 = true;            // a launch of at most a workgroup a CU stages a pass of four at once
     static constexpr bool DEFER = true;
+    static constexpr bool PAIR2 = true;  // a two-token gate / up step with the inputs in registers leaves two waves a SIMD their registers
     static const char *name() { return "matvec_q4_k"; }
     struct Raw {
         uint4 h, q0, q1;
@@ -401,6 +404,7 @@ struct KQ5 {
     static constexpr int STAGE2 = 0, STAGE4 = 4;  // tokens whose inputs are loaded at once
     static constexpr bool ALL4 = true;            // a launch of at most a workgroup a CU stages a pass of four at once
     static constexpr bool DEFER = true;
+    static constexpr bool PAIR2 = false;  // a two-token gate / up step with the inputs in registers leaves two waves a SIMD their registers
     static const char *name() { return "matvec_q5_k"; }
     struct Raw {
         uint4 h, b0, b1, q0, q1;
@@ -491,6 +495,7 @@ struct KQ6 {
     static constexpr int STAGE2 = 2, STAGE4 = 1;  // tokens whose inputs are loaded at once
     static constexpr bool ALL4 = true;            // a launch of at most a workgroup a CU stages a pass of four at once
     static constexpr bool DEFER = false;
+    static constexpr bool PAIR2 = false;  // a two-token gate / up step with the inputs in registers leaves two waves a SIMD their registers
     static const char *name() { return "matvec_q6_k"; }
     struct Raw {
         uint4 l0, l1, hv;
@@ -873,28 +878,32 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
 // two passes asked for before the inputs are staged (instead of one) 8.7 us; the first pass
 // asked for only once the inputs have arrived 8.0 us.
 constexpr int kRowDepth = 1;
-template <class P, bool PAIR, int SEG_LOG2>
+template <class P, int MT, bool PAIR, int SEG_LOG2>
 __global__ __launch_bounds__(256) void matvec_quant_row_kernel(KArgs q) {
     const MvArgs &a = q.a;
     extern __shared__ float4 lds4[];
-    __shared__ float red[4];
+    __shared__ float red[4 * MT];
     constexpr int NSUM = P::NSUM, RUN = 64 / NSUM, kRows = PAIR ? 2 : 1;
     constexpr uint32_t SEG = 1u << SEG_LOG2, RPI = 64u >> SEG_LOG2;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t tasks = q.tasks, k4 = a.k / 4u;
+    const uint32_t tok_stride4 = tasks * (kTaskStride / 4u);  // float4s per token
     const uint32_t tsub = lane & (SEG - 1u), rsub = lane >> SEG_LOG2;
     const uint32_t units = (a.rows + RPI - 1u) / RPI;
     const uint32_t gwave = blockIdx.x * 4u + (uint32_t)__builtin_amdgcn_readfirstlane((int)wave), nwaves = gridDim.x * 4u;
 
-    // The token's inputs (and norm weights) are asked for first, then the first rows: loads
+    // The tokens' inputs (and norm weights) are asked for first, then the first rows: loads
     // complete in order within a wave.
-    const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)q.t0 * a.xr);
     const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
-    float4 xv[4], gv[4];
+    float4 xv[MT][4], gv[4];
 #pragma unroll
     for (int j = 0; j < 4; j++) {
         const uint32_t i = tid + 256u * j;
-        xv[j] = i < k4 ? xrow[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)(q.t0 + t) * a.xr);
+            xv[t][j] = i < k4 ? xrow[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
     }
     if (a.flags & FLAG_NORM) {
 #pragma unroll
@@ -917,105 +926,142 @@ __global__ __launch_bounds__(256) void matvec_quant_row_kernel(KArgs q) {
 #pragma unroll
     for (int dpt = 0; dpt < kRowDepth; dpt++) fetch(gwave + dpt * nwaves, buf[dpt]);
 
-    // stage_token's arithmetic on the vectors already loaded.
-    float scale = 1.0f;
-    if (a.flags & FLAG_NORM) {
-        float ss = 0.f;
+    // stage_token's arithmetic on the vectors already loaded, the tokens' sums of squares
+    // meeting in LDS together.
+    float scale[MT];
 #pragma unroll
-        for (int j = 0; j < 4; j++)
-            if (tid + 256u * j < k4) ss += xv[j].x * xv[j].x + xv[j].y * xv[j].y + xv[j].z * xv[j].z + xv[j].w * xv[j].w;
-        ss = wave_sum(ss);
-        if (lane == 0) red[wave] = ss;
+    for (int t = 0; t < MT; t++) scale[t] = 1.0f;
+    if (a.flags & FLAG_NORM) {
+        float ss[MT];
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            ss[t] = 0.f;
+#pragma unroll
+            for (int j = 0; j < 4; j++)
+                if (tid + 256u * j < k4) ss[t] += xv[t][j].x * xv[t][j].x + xv[t][j].y * xv[t][j].y + xv[t][j].z * xv[t][j].z + xv[t][j].w * xv[t][j].w;
+            ss[t] = wave_sum(ss[t]);
+        }
+        if (lane == 0) {
+#pragma unroll
+            for (int t = 0; t < MT; t++) red[4 * t + wave] = ss[t];
+        }
         __syncthreads();
-        const float total = (red[0] + red[1]) + (red[2] + red[3]);
-        scale = 1.0f / sqrtf(total / (float)a.k + a.eps);
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            const float total = (red[4 * t] + red[4 * t + 1]) + (red[4 * t + 2] + red[4 * t + 3]);
+            scale[t] = 1.0f / sqrtf(total / (float)a.k + a.eps);
+        }
     }
 #pragma unroll
-    for (int j = 0; j < 4; j++) {
-        const uint32_t i = tid + 256u * j;
-        if (i >= k4) continue;
-        float4 v = xv[j];
-        if (a.flags & FLAG_NORM) {
-            v.x = v.x * scale * gv[j].x; v.y = v.y * scale * gv[j].y;
-            v.z = v.z * scale * gv[j].z; v.w = v.w * scale * gv[j].w;
+    for (int t = 0; t < MT; t++) {
+        float4 *dst = lds4 + (size_t)t * tok_stride4;
+#pragma unroll
+        for (int j = 0; j < 4; j++) {
+            const uint32_t i = tid + 256u * j;
+            if (i >= k4) continue;
+            float4 v = xv[t][j];
+            if (a.flags & FLAG_NORM) {
+                v.x = v.x * scale[t] * gv[j].x; v.y = v.y * scale[t] * gv[j].y;
+                v.z = v.z * scale[t] * gv[j].z; v.w = v.w * scale[t] * gv[j].w;
+            }
+            if (a.act_div > 0.f) {
+                v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
+                v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+            }
+            const uint32_t p = P::stage_index(i);
+            dst[p + (p >> 4)] = v;
         }
-        if (a.act_div > 0.f) {
-            v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
-            v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
-        }
-        const uint32_t p = P::stage_index(i);
-        lds4[p + (p >> 4)] = v;
     }
     __syncthreads();
     if (gwave >= units) return;
 
     // The lane's task's inputs and their runs' sums, for the whole walk.
-    float xr[64], xsum[NSUM];
-    {
-        const float4 *src = lds4 + (tsub < tasks ? tsub : 0u) * (kTaskStride / 4u);
+    float xr[MT][64], xsum[MT][NSUM];
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+        const float4 *src = lds4 + (size_t)t * tok_stride4 + (tsub < tasks ? tsub : 0u) * (kTaskStride / 4u);
 #pragma unroll
         for (int v = 0; v < 16; v++) {
             const float4 f = src[v];
-            xr[4 * v] = f.x; xr[4 * v + 1] = f.y; xr[4 * v + 2] = f.z; xr[4 * v + 3] = f.w;
+            xr[t][4 * v] = f.x; xr[t][4 * v + 1] = f.y; xr[t][4 * v + 2] = f.z; xr[t][4 * v + 3] = f.w;
         }
         // (a lane without a task multiplies zeros by zeros, whatever the inputs hold)
         if (tsub >= tasks) {
 #pragma unroll
-            for (int e = 0; e < 64; e++) xr[e] = 0.f;
+            for (int e = 0; e < 64; e++) xr[t][e] = 0.f;
         }
 #pragma unroll
         for (int s = 0; s < NSUM; s++) {
-            xsum[s] = 0.f;
+            xsum[t][s] = 0.f;
 #pragma unroll
-            for (int e = 0; e < RUN; e++) xsum[s] += xr[s * RUN + e];
+            for (int e = 0; e < RUN; e++) xsum[t][s] += xr[t][s * RUN + e];
         }
     }
     const Masks nm = q.nm;
     const typename P::Keys ch = P::keys(tsub & 3u);
-    const size_t out0 = (size_t)q.t0 * a.out_stride + a.col0;
     const bool accumulate = (a.flags & FLAG_ACCUMULATE) != 0;
+    auto out_at = [&](int t, uint32_t j) { return (size_t)(q.t0 + t) * a.out_stride + a.col0 + j; };
 
     // Whole-wave rows (SEG = 64) of a format with DEFER keep their finished sums in the lane of
     // their number (the gate's and the up row's apart) and are finished and stored together,
     // 64 outputs at a time: stores between the loads of the stream cost more than their bytes,
     // and the activation runs once for 64 outputs instead of once a row.
     constexpr bool kKeep = P::DEFER && SEG == 64u;
-    float kept0 = 0.f, kept1 = 0.f;
+    float kept0[MT], kept1[MT];
+#pragma unroll
+    for (int t = 0; t < MT; t++) kept0[t] = kept1[t] = 0.f;
     uint32_t nkept = 0, kept_first = gwave;
     auto flush_kept = [&]() __attribute__((always_inline)) {
         const uint32_t j = kept_first + lane * nwaves;
         if (lane < nkept && j < a.rows) {
-            float r = PAIR ? silu_f(kept0) * kept1 : kept0;
-            if (accumulate) r += a.out[out0 + j];
-            a.out[out0 + j] = r;
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                float r = PAIR ? silu_f(kept0[t]) * kept1[t] : kept0[t];
+                if (accumulate) r += a.out[out_at(t, j)];
+                a.out[out_at(t, j)] = r;
+            }
         }
         kept_first += nkept * nwaves;
         nkept = 0;
     };
     auto multiply = [&](uint32_t u, const typename P::Raw (&rows)[kRows]) __attribute__((always_inline)) {
-        float v[kRows][1];
-        P::template dot<1, kRows>(rows, ch, nm,
-            [&](int, int vi) { return make_float4(xr[4 * vi], xr[4 * vi + 1], xr[4 * vi + 2], xr[4 * vi + 3]); },
-            [&](int, int s) { return xsum[s]; }, v);
-        // (0 + v: the kernel above adds a lane's tasks to a sum that starts at zero)
-        const float s0 = segment_sum(0.f + v[0][0], SEG_LOG2);
-        const float s1 = PAIR ? segment_sum(0.f + v[kRows - 1][0], SEG_LOG2) : 0.f;
-        if (kKeep) {
-            const float t0 = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(s0), 63));
-            kept0 = lane == nkept ? t0 : kept0;
-            if (PAIR) {
-                const float t1 = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(s1), 63));
-                kept1 = lane == nkept ? t1 : kept1;
+        // (a row at a time: with the inputs in registers two rows share nothing, and one row's
+        // sums and words are fewer registers than two rows')
+        float v[kRows][MT];
+#pragma unroll
+        for (int j = 0; j < kRows; j++) {
+            const typename P::Raw(&one)[1] = reinterpret_cast<const typename P::Raw(&)[1]>(rows[j]);
+            float vj[1][MT];
+            P::template dot<MT, 1>(one, ch, nm,
+                [&](int t, int vi) { return make_float4(xr[t][4 * vi], xr[t][4 * vi + 1], xr[t][4 * vi + 2], xr[t][4 * vi + 3]); },
+                [&](int t, int s) { return xsum[t][s]; }, vj);
+#pragma unroll
+            for (int t = 0; t < MT; t++) v[j][t] = vj[0][t];
+        }
+#pragma unroll
+        for (int t = 0; t < MT; t++) {
+            // (0 + v: matvec_quant_kernel adds a lane's tasks to a sum that starts at zero)
+            const float s0 = segment_sum(0.f + v[0][t], SEG_LOG2);
+            const float s1 = PAIR ? segment_sum(0.f + v[kRows - 1][t], SEG_LOG2) : 0.f;
+            if (kKeep) {
+                const float t0 = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(s0), 63));
+                kept0[t] = lane == nkept ? t0 : kept0[t];
+                if (PAIR) {
+                    const float t1 = __uint_as_float(__builtin_amdgcn_readlane(__float_as_uint(s1), 63));
+                    kept1[t] = lane == nkept ? t1 : kept1[t];
+                }
+            } else {
+                const uint32_t j = u * RPI + rsub;
+                if (tsub == SEG - 1u && j < a.rows) {
+                    float r = PAIR ? silu_f(s0) * s1 : s0;
+                    if (accumulate) r += a.out[out_at(t, j)];
+                    a.out[out_at(t, j)] = r;
+                }
             }
+        }
+        if (kKeep) {
             nkept++;
             if (nkept == 64u) flush_kept();
-        } else {
-            const uint32_t j = u * RPI + rsub;
-            if (tsub == SEG - 1u && j < a.rows) {
-                float r = PAIR ? silu_f(s0) * s1 : s0;
-                if (accumulate) r += a.out[out0 + j];
-                a.out[out0 + j] = r;
-            }
         }
     };
 
@@ -1440,12 +1486,18 @@ static zhip_result run_slices(const Dispatch &d, const KArgs &q, uint32_t lds, u
     return check_launch(d, P::name());
 }
 
-template <class P, bool PAIR>
+template <class P, int MT, bool PAIR>
 static zhip_result run_row(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
+    if (lds > 65536u) {
+        const bool ok = q.seg_log2 == 4u ? lds_opt_in<matvec_quant_row_kernel<P, MT, PAIR, 4>, 160 * 1024 - 64>()
+                      : q.seg_log2 == 5u ? lds_opt_in<matvec_quant_row_kernel<P, MT, PAIR, 5>, 160 * 1024 - 64>()
+                                         : lds_opt_in<matvec_quant_row_kernel<P, MT, PAIR, 6>, 160 * 1024 - 64>();
+        if (!ok) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", P::name(), lds);
+    }
     switch (q.seg_log2) {
-    case 4: hipLaunchKernelGGL((matvec_quant_row_kernel<P, PAIR, 4>), dim3(blocks), dim3(256), lds, d.stream, q); break;
-    case 5: hipLaunchKernelGGL((matvec_quant_row_kernel<P, PAIR, 5>), dim3(blocks), dim3(256), lds, d.stream, q); break;
-    default: hipLaunchKernelGGL((matvec_quant_row_kernel<P, PAIR, 6>), dim3(blocks), dim3(256), lds, d.stream, q); break;
+    case 4: hipLaunchKernelGGL((matvec_quant_row_kernel<P, MT, PAIR, 4>), dim3(blocks), dim3(256), lds, d.stream, q); break;
+    case 5: hipLaunchKernelGGL((matvec_quant_row_kernel<P, MT, PAIR, 5>), dim3(blocks), dim3(256), lds, d.stream, q); break;
+    default: hipLaunchKernelGGL((matvec_quant_row_kernel<P, MT, PAIR, 6>), dim3(blocks), dim3(256), lds, d.stream, q); break;
     }
     return check_launch(d, P::name());
 }
@@ -1532,7 +1584,8 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
             t0 += q.mt;
             continue;
         }
-        const bool xreg = a.m == 1u && q.tasks <= 64u;
+        // Steps of one or two tokens over rows of up to 64 tasks keep the lanes' inputs in registers.
+        const bool xreg = (a.m == 1u || (a.m == 2u && (!pair || P::PAIR2))) && q.tasks <= 64u;
         const uint32_t per_unit = pair ? rpi : rpi * (xreg ? 1u : 2u);
         const uint32_t units = (a.rows + per_unit - 1u) / per_unit;
         const uint32_t want = (units + 3u) / 4u;
@@ -1556,9 +1609,13 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
             // 9.8, Q6_K 10.9 / 10.8, Q8_0 12.05 / 11.7, gate / up pairs of Q4_K 14.4 / 13.9, of
             // Q5_K 18.3 / 17.2; 4096 x 4096 Q4_K 4.9 / 4.2; 28672 x 2048 Q4_K 8.0 / 9.05.
             const uint32_t cus = (uint32_t)d.dev->compute_units;
-            const bool three = !pair && (uint64_t)rpi * a.row_bytes <= 3072u && passes >= cus * 48u;
-            const uint32_t cap = cus * (three ? 3u : 2u);
-            r = pair ? run_row<P, true>(d, q, q.tasks * kTaskStride * 4u, row_want < cap ? row_want : cap) : run_row<P, false>(d, q, q.tasks * kTaskStride * 4u, row_want < cap ? row_want : cap);
+            // (two tokens' inputs leave the registers for two waves a SIMD: two workgroups)
+            const bool three = a.m == 1u && !pair && (uint64_t)rpi * a.row_bytes <= 3072u && passes >= cus * 48u;
+            const uint32_t cap = cus * (three ? 3u : 2u), row_blocks = row_want < cap ? row_want : cap;
+            const uint32_t row_lds = a.m * q.tasks * kTaskStride * 4u;
+            if (a.m == 1u) r = pair ? run_row<P, 1, true>(d, q, row_lds, row_blocks) : run_row<P, 1, false>(d, q, row_lds, row_blocks);
+            else if (pair) r = P::PAIR2 ? run_row<P, 2, P::PAIR2>(d, q, row_lds, row_blocks) : ZHIP_E_GPU;
+            else r = run_row<P, 2, false>(d, q, row_lds, row_blocks);
         } else if (mt == 1u) r = pair ? run_quant<P, 1, true, 1>(d, q, lds, blocks) : run_quant<P, 1, false, 1>(d, q, lds, blocks);
         else if (mt == 2u) {
             if (small && P::STAGE2 != 2) r = pair ? run_quant<P, 2, true, 2>(d, q, lds, blocks) : run_quant<P, 2, false, 2>(d, q, lds, blocks);
