@@ -339,6 +339,15 @@ def test_quant_matvec_act_prologue(ctx, t, k):
     (TensorType.q5_k, 16384, False, 4, 9),    # 256 tasks: four whole slices, a batch of rows with units past the end
     (TensorType.q3_k, 4352, False, 1, 3),     # 68 tasks: a second slice of four lanes, three rows
     (TensorType.q6_k, 16640, False, 2, 21),   # 260 tasks: past the sliced kernel's four slices
+    (TensorType.q4_k, 11008, False, 2, 30),   # two tokens over three slices: a workgroup of six waves
+    (TensorType.q8_0, 8192, False, 2, 70),    # two tokens over two slices
+    # Steps of exactly two tokens over short rows keep both tokens' inputs in registers:
+    (TensorType.q4_k, 4096, True, 2, 100),
+    (TensorType.q3_k, 3072, True, 2, 21),     # 48 tasks: idle lanes
+    (TensorType.q5_k, 4096, True, 2, 40),     # (a format whose gate / up step of two tokens stays on the general kernel)
+    (TensorType.q8_0, 2048, False, 2, 50),    # two rows a wave pass
+    (TensorType.q6_k, 1024, False, 2, 33),    # four rows a wave pass, a ragged last pass
+    (TensorType.q5_k, 4096, False, 2, 64),
 ])
 def test_quant_matvec_long_rows(ctx, t, k, pair, rows, n):
     """Rows of more than 4096 weights at the widths and edges test_quant_matvec leaves out:

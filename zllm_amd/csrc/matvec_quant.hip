@@ -1310,18 +1310,19 @@ static zhip_result run_long(const Dispatch &d, const KArgs &q, uint32_t blocks) 
 // a task, loads zeros). What the outputs hold, for a step that accumulates, is asked for before
 // the round's loads: loads complete in order within a wave, so behind them it would wait for
 // rows of the next round.
-template <class P, bool PAIR, int R, int NW>
+template <class P, int MT, bool PAIR, int R, int NW>
 __global__ __launch_bounds__(64 * NW) void matvec_quant_slices_kernel(KArgs q) {
     const MvArgs &a = q.a;
-    extern __shared__ float4 lds4[];  // the token in task order, padded per task; then the partial sums [parity][group][unit of the round][slice][row][lane]
-    __shared__ float red[4];
+    extern __shared__ float4 lds4[];  // the tokens in task order, padded per task; then the partial sums [parity][group][unit of the round][slice][row][token][lane]
+    __shared__ float red[4 * MT];
     constexpr int NSUM = P::NSUM, RUN = 64 / NSUM, kRows = PAIR ? 2 : 1;
     constexpr uint32_t THREADS = 64u * NW;
-    constexpr int XV = (4096 + THREADS - 1) / THREADS;  // vectors of the token a thread stages (k <= 16384)
+    constexpr int XV = (4096 + THREADS - 1) / THREADS;  // vectors of a token a thread stages (k <= 16384)
     static_assert(R % 2 == 0, "the buffers alternate by name");
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
     const uint32_t tasks = q.tasks, slices = (tasks + 63u) / 64u, k4 = a.k / 4u;
+    const uint32_t tok_stride4 = tasks * (kTaskStride / 4u);  // float4s per token
     const uint32_t groups_here = (uint32_t)NW / slices;
     const uint32_t grp = wave / slices, slice = wave % slices;
     const uint32_t group = blockIdx.x * groups_here + grp, groups = gridDim.x * groups_here;
@@ -1329,22 +1330,13 @@ __global__ __launch_bounds__(64 * NW) void matvec_quant_slices_kernel(KArgs q) {
     const uint32_t task = lane + 64u * slice;
     const bool active = task < tasks;
     const bool norm = (a.flags & FLAG_NORM) != 0, accumulate = (a.flags & FLAG_ACCUMULATE) != 0;
-
-    // The token's inputs first, then the first rows (loads complete in order within a wave).
-    const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)q.t0 * a.xr);
     const float4 *nw = reinterpret_cast<const float4 *>(a.norm_w);
-    float4 xv[XV], gv[XV];
-#pragma unroll
-    for (int j = 0; j < XV; j++) {
-        const uint32_t i = tid + THREADS * j;
-        xv[j] = i < k4 ? xrow[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-        if (norm) gv[j] = i < k4 ? nw[i] : make_float4(0.f, 0.f, 0.f, 0.f);
-    }
+    auto token_row = [&](int t) { return reinterpret_cast<const float4 *>(a.x + (size_t)(q.t0 + t) * a.xr); };
 
     // Unit n of the group's walk: R consecutive units a round, the groups' rounds interleaved.
     auto unit_of = [&](uint32_t n) { return ((n / R) * groups + group) * R + n % R; };
     const uint32_t rounds = (units + groups * R - 1u) / (groups * R);  // the same for every group: the barriers below are the workgroup's
-    const typename P::Where at = active && grp < groups_here ? P::where(0u, a.k, task) : P::nowhere();
+    const typename P::Where at = active ? P::where(0u, a.k, task) : P::nowhere();
     auto fetch = [&](uint32_t n, typename P::Raw (&dst)[kRows]) __attribute__((always_inline)) {
         const uint32_t u = unit_of(n);
         const bool live = u < units;
@@ -1355,98 +1347,120 @@ __global__ __launch_bounds__(64 * NW) void matvec_quant_slices_kernel(KArgs q) {
         __builtin_amdgcn_sched_barrier(0);  // (the loads stay ahead of the multiply that follows them in the source)
     };
     typename P::Raw cur[kRows], nxt[kRows];
-    fetch(0, cur);
 
-    // stage_token's arithmetic: the RMSNorm sum by the first 256 threads, vector i by thread
-    // i % 256 and the four waves' sums in order; then every thread stages the vectors it loaded.
-    float scale = 1.0f;
-    if (norm) {
-        if (tid < 256u) {
-            float ss = 0.f;
-#pragma unroll 4
-            for (uint32_t i = tid; i < k4; i += 256u) {
-                const float4 v = xrow[i];
-                ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
-            }
-            ss = wave_sum(ss);
-            if (lane == 0) red[wave] = ss;
-        }
-        __syncthreads();
-        const float total = (red[0] + red[1]) + (red[2] + red[3]);
-        scale = 1.0f / sqrtf(total / (float)a.k + a.eps);
-    }
+    // A token at a time: its inputs first, then (with the first token) the first rows: loads
+    // complete in order within a wave. stage_token's arithmetic: the RMSNorm sum by the first
+    // 256 threads, vector i by thread i % 256 and the four waves' sums in order; then every
+    // thread stages the vectors it loaded.
 #pragma unroll
-    for (int j = 0; j < XV; j++) {
-        const uint32_t i = tid + THREADS * j;
-        if (i >= k4) continue;
-        float4 v = xv[j];
+    for (int t = 0; t < MT; t++) {
+        const float4 *xrow = token_row(t);
+        float4 xv[XV], gv[XV];
+#pragma unroll
+        for (int j = 0; j < XV; j++) {
+            const uint32_t i = tid + THREADS * j;
+            xv[j] = i < k4 ? xrow[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+            if (norm) gv[j] = i < k4 ? nw[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+        if (t == 0) fetch(0, cur);
+        float scale = 1.0f;
         if (norm) {
-            v.x = v.x * scale * gv[j].x; v.y = v.y * scale * gv[j].y;
-            v.z = v.z * scale * gv[j].z; v.w = v.w * scale * gv[j].w;
+            if (tid < 256u) {
+                float ss = 0.f;
+#pragma unroll 4
+                for (uint32_t i = tid; i < k4; i += 256u) {
+                    const float4 v = xrow[i];
+                    ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+                }
+                ss = wave_sum(ss);
+                if (lane == 0) red[4 * t + wave] = ss;
+            }
+            __syncthreads();
+            const float total = (red[4 * t] + red[4 * t + 1]) + (red[4 * t + 2] + red[4 * t + 3]);
+            scale = 1.0f / sqrtf(total / (float)a.k + a.eps);
         }
-        if (a.act_div > 0.f) {
-            v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
-            v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+        float4 *dst = lds4 + (size_t)t * tok_stride4;
+#pragma unroll
+        for (int j = 0; j < XV; j++) {
+            const uint32_t i = tid + THREADS * j;
+            if (i >= k4) continue;
+            float4 v = xv[j];
+            if (norm) {
+                v.x = v.x * scale * gv[j].x; v.y = v.y * scale * gv[j].y;
+                v.z = v.z * scale * gv[j].z; v.w = v.w * scale * gv[j].w;
+            }
+            if (a.act_div > 0.f) {
+                v.x = silu_f(v.x / a.act_div); v.y = silu_f(v.y / a.act_div);
+                v.z = silu_f(v.z / a.act_div); v.w = silu_f(v.w / a.act_div);
+            }
+            const uint32_t p = P::stage_index(i);
+            dst[p + (p >> 4)] = v;
         }
-        const uint32_t p = P::stage_index(i);
-        lds4[p + (p >> 4)] = v;
     }
     __syncthreads();
 
-    float xr[64], xsum[NSUM];
-    {
-        const float4 *src = lds4 + (active ? task : 0u) * (kTaskStride / 4u);
+    float xr[MT][64], xsum[MT][NSUM];
+#pragma unroll
+    for (int t = 0; t < MT; t++) {
+        const float4 *src = lds4 + (size_t)t * tok_stride4 + (active ? task : 0u) * (kTaskStride / 4u);
 #pragma unroll
         for (int v = 0; v < 16; v++) {
             const float4 f = src[v];
-            xr[4 * v] = f.x; xr[4 * v + 1] = f.y; xr[4 * v + 2] = f.z; xr[4 * v + 3] = f.w;
+            xr[t][4 * v] = f.x; xr[t][4 * v + 1] = f.y; xr[t][4 * v + 2] = f.z; xr[t][4 * v + 3] = f.w;
         }
         if (!active) {
 #pragma unroll
-            for (int e = 0; e < 64; e++) xr[e] = 0.f;
+            for (int e = 0; e < 64; e++) xr[t][e] = 0.f;
         }
 #pragma unroll
         for (int sr = 0; sr < NSUM; sr++) {
-            xsum[sr] = 0.f;
+            xsum[t][sr] = 0.f;
 #pragma unroll
-            for (int e = 0; e < RUN; e++) xsum[sr] += xr[sr * RUN + e];
+            for (int e = 0; e < RUN; e++) xsum[t][sr] += xr[t][sr * RUN + e];
         }
     }
     const Masks nm = q.nm;
     const typename P::Keys ch = P::keys(task & 3u);
-    const size_t out0 = (size_t)q.t0 * a.out_stride + a.col0;
-    // (the partial sums lie behind the token: no barrier between reading the one and writing the other)
-    float *part = reinterpret_cast<float *>(lds4 + (size_t)tasks * (kTaskStride / 4u));
+    auto out_at = [&](int t, uint32_t j) { return (size_t)(q.t0 + t) * a.out_stride + a.col0 + j; };
+    // (the partial sums lie behind the tokens: no barrier between reading the one and writing the other)
+    float *part = reinterpret_cast<float *>(lds4 + (size_t)MT * tok_stride4);
     constexpr uint32_t kMine = 2;  // units of a round a wave finishes, at most: R <= 4 over two or more slices
+    constexpr uint32_t kCell = kRows * MT * 64u;  // floats one wave leaves per unit
+    auto multiply = [&](const typename P::Raw (&rows)[kRows], float *to) __attribute__((always_inline)) {
+#pragma unroll
+        for (int j = 0; j < kRows; j++) {
+            const typename P::Raw(&one)[1] = reinterpret_cast<const typename P::Raw(&)[1]>(rows[j]);
+            float vj[1][MT];
+            P::template dot<MT, 1>(one, ch, nm,
+                [&](int t, int vi) { return make_float4(xr[t][4 * vi], xr[t][4 * vi + 1], xr[t][4 * vi + 2], xr[t][4 * vi + 3]); },
+                [&](int t, int sr) { return xsum[t][sr]; }, vj);
+#pragma unroll
+            for (int t = 0; t < MT; t++) to[(j * MT + t) * 64u + lane] = vj[0][t];
+        }
+    };
 
     for (uint32_t round = 0; round < rounds; round++) {
-        float *mine = part + ((((round & 1u) * groups_here + grp) * R) * slices + 0u) * kRows * 64u;
+        float *mine = part + (((round & 1u) * groups_here + grp) * R) * slices * kCell;
         // What the outputs hold, for the units this wave will finish: asked for before the
         // round's loads, so that the wait for it is the wait for rows the wave needs anyway.
-        float held[kMine];
+        float held[kMine][MT];
         if (accumulate) {
 #pragma unroll
             for (uint32_t i = 0; i < kMine; i++) {
                 const uint32_t r = slice + i * slices, u = unit_of(round * R + r);
-                held[i] = (lane == 63u && r < (uint32_t)R && u < units) ? a.out[out0 + u] : 0.f;
+#pragma unroll
+                for (int t = 0; t < MT; t++) held[i][t] = (lane == 63u && r < (uint32_t)R && u < units) ? a.out[out_at(t, u)] : 0.f;
             }
         }
 #pragma unroll
         for (int r = 0; r < R; r++) {
-            float v[kRows][1];
             if (r % 2 == 0) {
                 fetch(round * R + r + 1u, nxt);
-                P::template dot<1, kRows>(cur, ch, nm,
-                    [&](int, int vi) { return make_float4(xr[4 * vi], xr[4 * vi + 1], xr[4 * vi + 2], xr[4 * vi + 3]); },
-                    [&](int, int sr) { return xsum[sr]; }, v);
+                multiply(cur, mine + (r * slices + slice) * kCell);
             } else {
                 fetch(round * R + r + 1u, cur);
-                P::template dot<1, kRows>(nxt, ch, nm,
-                    [&](int, int vi) { return make_float4(xr[4 * vi], xr[4 * vi + 1], xr[4 * vi + 2], xr[4 * vi + 3]); },
-                    [&](int, int sr) { return xsum[sr]; }, v);
+                multiply(nxt, mine + (r * slices + slice) * kCell);
             }
-#pragma unroll
-            for (int j = 0; j < kRows; j++) mine[((r * slices + slice) * kRows + j) * 64u + lane] = v[j][0];
         }
         // (a barrier that leaves the next unit's loads in flight)
         asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -1458,31 +1472,34 @@ __global__ __launch_bounds__(64 * NW) void matvec_quant_slices_kernel(KArgs q) {
         for (uint32_t i = 0; i < kMine; i++) {
             const uint32_t r = slice + i * slices;
             if (r >= (uint32_t)R) break;
-            const float *theirs = mine + (r * slices) * kRows * 64u;
-            float acc[kRows];
-#pragma unroll
-            for (int j = 0; j < kRows; j++) acc[j] = 0.f;
-            for (uint32_t sl = 0; sl < slices; sl++) {
-                if (lane + 64u * sl >= tasks) continue;
-#pragma unroll
-                for (int j = 0; j < kRows; j++) acc[j] += theirs[(sl * kRows + j) * 64u + lane];
-            }
-            const float s0 = segment_sum(acc[0], 6u), s1 = PAIR ? segment_sum(acc[kRows - 1], 6u) : 0.f;
+            const float *theirs = mine + (r * slices) * kCell;
             const uint32_t u = unit_of(round * R + r);
-            if (lane == 63u && u < units) {
-                float res = PAIR ? silu_f(s0) * s1 : s0;
-                if (accumulate) res += held[i];
-                a.out[out0 + u] = res;
+#pragma unroll
+            for (int t = 0; t < MT; t++) {
+                float acc[kRows];
+#pragma unroll
+                for (int j = 0; j < kRows; j++) acc[j] = 0.f;
+                for (uint32_t sl = 0; sl < slices; sl++) {
+                    if (lane + 64u * sl >= tasks) continue;
+#pragma unroll
+                    for (int j = 0; j < kRows; j++) acc[j] += theirs[sl * kCell + (j * MT + t) * 64u + lane];
+                }
+                const float s0 = segment_sum(acc[0], 6u), s1 = PAIR ? segment_sum(acc[kRows - 1], 6u) : 0.f;
+                if (lane == 63u && u < units) {
+                    float res = PAIR ? silu_f(s0) * s1 : s0;
+                    if (accumulate) res += held[i][t];
+                    a.out[out_at(t, u)] = res;
+                }
             }
         }
         // (the other parity's space is written next; this one again only behind the next barrier)
     }
 }
 
-template <class P, bool PAIR, int R, int NW>
+template <class P, int MT, bool PAIR, int R, int NW>
 static zhip_result run_slices(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
-    if (!lds_opt_in<matvec_quant_slices_kernel<P, PAIR, R, NW>, 160 * 1024 - 64>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", P::name(), lds);
-    hipLaunchKernelGGL((matvec_quant_slices_kernel<P, PAIR, R, NW>), dim3(blocks), dim3(64 * NW), lds, d.stream, q);
+    if (!lds_opt_in<matvec_quant_slices_kernel<P, MT, PAIR, R, NW>, 160 * 1024 - 64>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", P::name(), lds);
+    hipLaunchKernelGGL((matvec_quant_slices_kernel<P, MT, PAIR, R, NW>), dim3(blocks), dim3(64 * NW), lds, d.stream, q);
     return check_launch(d, P::name());
 }
 
@@ -1533,6 +1550,21 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
     for (uint32_t t0 = 0; t0 < a.m;) {
         uint32_t left = a.m - t0;
         uint32_t mt = left >= 3u ? 4u : left;
+        // A step of exactly two tokens over rows of 65 .. 256 tasks keeps both tokens' slices in
+        // registers like the one-token step (Q4_K 4096 x 14336: 16.5 us tile by tile).
+        if (a.m == 2u && !pair && q.tasks > 64u && q.tasks <= 256u) {
+            q.t0 = 0;
+            q.mt = 2;
+            // (eight waves for two or four slices, six for three: twelve would spill)
+            const uint32_t slices = (q.tasks + 63u) / 64u, nw = slices == 3u ? 6u : 8u, groups_here = nw / slices;
+            const uint32_t cus = (uint32_t)d.dev->compute_units;
+            const uint32_t want = (a.rows + groups_here * 2u - 1u) / (groups_here * 2u);
+            const uint32_t blocks = want < cus ? want : cus;
+            const uint32_t lds2 = 2u * q.tasks * kTaskStride * 4u + 2u * nw * 2u * 2u * 256u;
+            const zhip_result r = nw == 6u ? run_slices<P, 2, false, 2, 6>(d, q, lds2, blocks) : run_slices<P, 2, false, 2, 8>(d, q, lds2, blocks);
+            if (r != ZHIP_OK) return r;
+            break;
+        }
         // Two workgroups a CU must fit their staged tokens in the 160 KB of LDS. Where the
         // pass's tokens do not, the rows are long (64 tasks or more) and the step is taken tile
         // by tile with all of them (matvec_quant_long_kernel).
@@ -1574,11 +1606,11 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
             const uint32_t lds1 = q.tasks * kTaskStride * 4u + 2u * nw * (two ? 2u : 4u) * (pair ? 2u : 1u) * 256u;
             zhip_result r;
             if (nw == 12u) {
-                if (pair) r = two ? run_slices<P, true, 2, 12>(d, q, lds1, blocks) : run_slices<P, true, 4, 12>(d, q, lds1, blocks);
-                else r = two ? run_slices<P, false, 2, 12>(d, q, lds1, blocks) : run_slices<P, false, 4, 12>(d, q, lds1, blocks);
+                if (pair) r = two ? run_slices<P, 1, true, 2, 12>(d, q, lds1, blocks) : run_slices<P, 1, true, 4, 12>(d, q, lds1, blocks);
+                else r = two ? run_slices<P, 1, false, 2, 12>(d, q, lds1, blocks) : run_slices<P, 1, false, 4, 12>(d, q, lds1, blocks);
             } else {
-                if (pair) r = two ? run_slices<P, true, 2, 8>(d, q, lds1, blocks) : run_slices<P, true, 4, 8>(d, q, lds1, blocks);
-                else r = two ? run_slices<P, false, 2, 8>(d, q, lds1, blocks) : run_slices<P, false, 4, 8>(d, q, lds1, blocks);
+                if (pair) r = two ? run_slices<P, 1, true, 2, 8>(d, q, lds1, blocks) : run_slices<P, 1, true, 4, 8>(d, q, lds1, blocks);
+                else r = two ? run_slices<P, 1, false, 2, 8>(d, q, lds1, blocks) : run_slices<P, 1, false, 4, 8>(d, q, lds1, blocks);
             }
             if (r != ZHIP_OK) return r;
             t0 += q.mt;
