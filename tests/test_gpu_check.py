@@ -848,14 +848,16 @@ def test_matmul_bf16_mfma_tilings(ctx, rows, n, k):
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
 
 
+@pytest.mark.parametrize("n", [2830, 8230])
 @pytest.mark.parametrize("rung", ["bf16_mfma", "fp16_single"])
-def test_matmul_q8_0_float_bf16_whole_steps_keep_token_bits(ctx, rung):
+def test_matmul_q8_0_float_bf16_whole_steps_keep_token_bits(ctx, rung, n):
     """Q8_0 weights on the bf16 rung and on the reference's fp16_single rung with k a multiple
-    of 128 take the kernel with producer waves and 32 x 32 x 16 MFMAs in 128- or 64-token
-    tiles: a token's sums are the same bits whichever tile height its step runs in and
+    of 128 take the kernels with producer waves and 32 x 32 x 16 MFMAs in 128- or 64-token
+    tiles (64 matrix rows a tile; 128 where the matrix has the rows to fill the CUs with those,
+    n = 8230): a token's sums are the same bits whichever tile height its step runs in and
     whichever tokens share the step; ragged rows and outputs, a column offset and a padded stride."""
     c = ctx
-    rows, n, k, col0, stride = 300, 2830, 384, 3, 2840
+    rows, k, col0, stride = 300, 384, 3, n + 10
     x = c.random(rows * k, 1).reshape(rows, k)
     raw, wq = quant_rows(c, TensorType.q8_0, n, k)
     wa = c.gpu_weights(TensorType.q8_0, raw, k)

@@ -55,6 +55,10 @@ constexpr uint32_t kMaxDecodeRows = 8;
 // there returns zeros and moves nothing.
 constexpr uint32_t kNowhere = 0xF0000000u;
 
+// The longest step the reference's planner records (src/plan/plan.zig:129,
+// src/plan/qwen35.zig:335).
+constexpr uint32_t kPlannerStepCap = 512;
+
 struct Bind {
     uint8_t *ptr = nullptr;  // buffer base + binding offset
     uint64_t size = 0;       // bytes bound
@@ -154,6 +158,7 @@ bool matmul_mfma_prepare_no_alloc();
 bool matmul_mfma_wide_prepare_no_alloc();
 bool matmul_stream_prepare_no_alloc();
 bool matmul_q8_bf16_prepare_no_alloc();
+bool matmul_q8_bf16_wide_prepare_no_alloc();
 uint64_t no_alloc_capacity();
 zhip_result no_alloc_matmul_q8_0_float(int device, hipStream_t stream, const float *x, const void *w, float *out, uint32_t rows, uint32_t n,
     uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, char *err, size_t err_cap);

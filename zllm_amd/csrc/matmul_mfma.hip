@@ -512,6 +512,10 @@ zhip_result launch_mfma_wide(const Dispatch &d, const char *name, bool q8_0, con
 
 // Q8_0 weights on the bf16 rung over whole 128-deep steps (matmul_q8_bf16.hip).
 bool matmul_q8_bf16_accepts(uint32_t k, uint32_t k_slice, uint32_t slices);
+// The same for matrices with enough rows for 128-row tiles (matmul_q8_bf16_wide.hip).
+bool matmul_q8_bf16_wide_accepts(const Dispatch &d, uint32_t n);
+zhip_result launch_matmul_q8_bf16_wide(const Dispatch &d, const char *name, bool f16, const uint8_t *x, const uint8_t *w, float *out, uint32_t rows,
+    uint32_t n, uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, uint32_t row_bytes, uint32_t x_bytes, uint32_t w_bytes);
 zhip_result launch_matmul_q8_bf16(const Dispatch &d, const char *name, bool f16, const uint8_t *x, const uint8_t *w, float *out, uint32_t rows, uint32_t n,
     uint32_t k, uint32_t col0, uint32_t out_stride, uint32_t accumulate, uint32_t row_bytes, uint32_t x_bytes, uint32_t w_bytes);
 
@@ -525,10 +529,6 @@ static zhip_result launch_kernel(const Dispatch &d, const char *name, const Mfma
     hipLaunchKernelGGL(kernel, grid, dim3(THREADS), bytes, d.stream, a);
     return check_launch(d, name);
 }
-
-// The longest step the reference's planner records (src/plan/plan.zig:129,
-// src/plan/qwen35.zig:335).
-constexpr uint32_t kPlannerStepCap = 512;
 
 // XPACKED: the activations are bound already packed in the operand format (an extension of
 // the contract, bf16 only); otherwise they are bound as f32 and narrowed first.
@@ -593,6 +593,9 @@ static zhip_result launch_mfma(const Dispatch &d, const char *name, bool sliced,
     if (kBf16Rung && slices == 1u && a.k_slice >= a.k && a.rows > kPlannerStepCap && (uint64_t)((a.rows + 255u) / 256u) * ((a.n + 127u) / 128u) >= (uint64_t)d.dev->compute_units)
         return launch_mfma_wide(d, name, q8_0, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes);
     if constexpr (std::is_same<W, WQ8_0>::value && !COMP) {
+        if (matmul_q8_bf16_accepts(a.k, a.k_slice, slices) && matmul_q8_bf16_wide_accepts(d, a.n))
+            return launch_matmul_q8_bf16_wide(d, name, std::is_same<H, F16>::value, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate,
+                a.row_bytes, a.x_bytes, a.w_bytes);
         if (matmul_q8_bf16_accepts(a.k, a.k_slice, slices))
             return launch_matmul_q8_bf16(d, name, std::is_same<H, F16>::value, a.x, a.w, a.out, a.rows, a.n, a.k, a.col0, a.out_stride, a.accumulate, a.row_bytes,
                 a.x_bytes, a.w_bytes);

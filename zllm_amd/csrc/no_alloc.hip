@@ -52,7 +52,7 @@ zhip_result no_alloc_setup(int device, const DeviceInfo &info) {
     }
     // Every kernel the entry point can launch opts in to its LDS now, so that the call itself
     // does no one-time set-up.
-    if (!(matmul_mfma_prepare_no_alloc() && matmul_mfma_wide_prepare_no_alloc() && matmul_stream_prepare_no_alloc() && matmul_q8_bf16_prepare_no_alloc())) return ZHIP_E_GPU;
+    if (!(matmul_mfma_prepare_no_alloc() && matmul_mfma_wide_prepare_no_alloc() && matmul_stream_prepare_no_alloc() && matmul_q8_bf16_prepare_no_alloc() && matmul_q8_bf16_wide_prepare_no_alloc())) return ZHIP_E_GPU;
     pd.info = info;
     pd.ptr = ptr;
     return ZHIP_OK;
