@@ -242,6 +242,7 @@ def main() -> int:
                     help="launch every dispatch of a repeated submit instead of replaying it from a HIP graph")
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="first run 4 plain elementwise copies (256 MiB read + 256 MiB written each) so a counter run has a kernel of known traffic to scale by")
+    ap.add_argument("--grid", default="", help="with prefill_grid: only these keys (comma-separated, e.g. m512_k4096_n14336), for a profile of one shape")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this path is built and measured on one GPU; --gpus above 1 is not supported "
@@ -267,7 +268,7 @@ def main() -> int:
     from zllm_amd import Device
 
     env = make_env(Device.NO_REPLAY if args.no_replay else 0)
-    env.update(vendor_c4=vendor_c4, torch_read=torch_read, make_env=make_env, Device=Device)
+    env.update(vendor_c4=vendor_c4, torch_read=torch_read, make_env=make_env, Device=Device, grid=[w for w in args.grid.split(",") if w])
     synth, K, TensorType = env["synth"], env["K"], env["TensorType"]
 
     # ---- headline: C2, Q4_K decode multiply M = 1, K = 4096, N = 14336 ----------------------
@@ -744,6 +745,8 @@ def bench_prefill_grid(env):
     for k, n in ((4096, 14336), (14336, 4096), (4096, 4096)):
         raw = synth.q8_0_rows(synth.rng(0x9D + n), n, k)
         for rows in (64, 128, 256, 512):
+            if env.get("grid") and f"m{rows}_k{k}_n{n}" not in env["grid"]:
+                continue
             flops = 2 * rows * n * k
             t, err, _ = _prefill_q8(env, rows, k, n, K.Prefill.bf16_mfma_xbf16, check_stride=8)
             ti, erri = _prefill_int8(env, TensorType.q8_0, oracle.Q8_0, raw, rows, k, n, check_stride=8)
