@@ -363,6 +363,10 @@ zhip_result launch_tile(const Dispatch &d, const char *name, const Q8Args &a) {
     constexpr int bytes = lds_bytes<TT>();
     if (!lds_opt_in<matmul_q8_bf16_kernel<TT, H>, bytes>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
     const dim3 grid((a.n + BN - 1) / BN, (a.rows + 32 * TT - 1) / (32 * TT));
+    if (grid.y > 65535u) return fail(d, ZHIP_E_BAD_COMMAND, "%s: grid too large", name);
+    // The kernel's 32-bit offsets also name the rows and tokens of partial tiles past the end.
+    if ((uint64_t)grid.x * BN * a.row_bytes >= (1ull << 32) || (uint64_t)grid.y * (32 * TT) * a.k * 2u >= (1ull << 32))
+        return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
     hipLaunchKernelGGL(kernel, grid, dim3(THREADS), bytes, d.stream, a);
     return check_launch(d, name);
 }

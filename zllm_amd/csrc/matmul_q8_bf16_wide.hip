@@ -338,8 +338,11 @@ zhip_result launch_tile(const Dispatch &d, const char *name, Q8Args a) {
     constexpr int bytes = lds_bytes<TT, RQ>();
     if (!lds_opt_in<matmul_q8_bf16_wide_kernel<TT, H, RQ>, bytes>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
     a.tiles_n = (a.n + 32 * RQ - 1) / (32 * RQ);
-    const uint64_t tiles = (uint64_t)a.tiles_n * ((a.rows + 32 * TT - 1) / (32 * TT));
+    const uint64_t tiles_t = (a.rows + 32 * TT - 1) / (32 * TT), tiles = (uint64_t)a.tiles_n * tiles_t;
     if (tiles >= (1ull << 31)) return fail(d, ZHIP_E_BAD_COMMAND, "%s: grid too large", name);
+    // The kernel's 32-bit offsets also name the rows and tokens of partial tiles past the end.
+    if ((uint64_t)a.tiles_n * (32 * RQ) * a.row_bytes >= (1ull << 32) || tiles_t * (32 * TT) * a.k * 2u >= (1ull << 32))
+        return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
     hipLaunchKernelGGL(kernel, dim3((uint32_t)tiles), dim3(threads<RQ>()), bytes, d.stream, a);
     return check_launch(d, name);
 }
