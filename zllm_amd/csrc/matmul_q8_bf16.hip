@@ -48,18 +48,19 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 
-constexpr int BN = 64, BK = 128;
-constexpr int CONSUMERS = 8, PRODUCERS = 4, THREADS = 64 * (CONSUMERS + PRODUCERS);
+constexpr int BK = 128, PRODUCERS = 4;
+// TT: 32-token tiles a workgroup covers (4: 128 tokens, 2: 64, 1: 32). RN: 32-row tiles of the
+// matrix it covers (2: 64 rows, 1: 32), each the work of four multiplying waves.
+template <int RN> constexpr int threads() { return 64 * (4 * RN + PRODUCERS); }
 // One step's weights in LDS: int8 [row][128 B], then per producer [16 rows][4 f16] and 128
 // bytes of filler (the upper half of its scale load).
-constexpr int WPART = BN * 128 + PRODUCERS * 256;
-// TT: 32-token tiles a workgroup covers (4: 128 tokens, 2: 64 tokens).
+template <int RN> constexpr int wpart_bytes() { return 32 * RN * 128 + PRODUCERS * 256; }
 template <int TT> constexpr int abuf_bytes() { return 2 * 32 * TT * 128; }  // activations of a step: [line][token][128 B]
-template <int TT> constexpr int buf_bytes() { return abuf_bytes<TT>() + WPART; }
-template <int TT> constexpr int lds_bytes() { return 3 * buf_bytes<TT>(); }
-static_assert(lds_bytes<4>() <= 160 * 1024, "three buffers must fit the CU's LDS");
-// The exchange of the k quarters reuses the buffers: 8 waves x 3 inboxes x TT KB.
-static_assert(lds_bytes<4>() >= 8 * 3 * 4 * 1024 && lds_bytes<2>() >= 8 * 3 * 2 * 1024, "the exchange must fit the buffers");
+template <int TT, int RN> constexpr int buf_bytes() { return abuf_bytes<TT>() + wpart_bytes<RN>(); }
+template <int TT, int RN> constexpr int lds_bytes() { return 3 * buf_bytes<TT, RN>(); }
+static_assert(lds_bytes<4, 2>() <= 160 * 1024, "three buffers must fit the CU's LDS");
+// The exchange of the k quarters reuses the buffers: 4 RN waves x 3 inboxes x TT KB.
+static_assert(lds_bytes<4, 2>() >= 8 * 3 * 4 * 1024 && lds_bytes<2, 2>() >= 8 * 3 * 2 * 1024 && lds_bytes<1, 1>() >= 4 * 3 * 1024, "the exchange must fit the buffers");
 
 struct Q8Args {
     const uint8_t *x;  // packed bf16 rows
@@ -136,11 +137,11 @@ __device__ __forceinline__ void convert(const WRaw &r, typename H::vec &w0, type
     w1 = __builtin_bit_cast(typename H::vec, hi);
 }
 
-template <int TT, class H>
-__global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
+template <int TT, class H, int RN>
+__global__ __launch_bounds__((threads<RN>())) void matmul_q8_bf16_kernel(Q8Args a) {
     typedef typename H::vec opvec;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
-    constexpr int BM = 32 * TT, ABUF = abuf_bytes<TT>(), BUF = buf_bytes<TT>();
+    constexpr int BM = 32 * TT, BN = 32 * RN, CONSUMERS = 4 * RN, ABUF = abuf_bytes<TT>(), BUF = buf_bytes<TT, RN>();
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t j0 = blockIdx.x * BN, t0 = blockIdx.y * BM;
@@ -148,13 +149,14 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
 
     if (wave >= CONSUMERS) {
         // Producers. Producer p loads a quarter of the step's activation lines (block b = p + 4 i:
-        // line b / (BM / 8), tokens 8 (b % (BM / 8)) .. + 7), matrix rows 16 p .. + 15 and their scales.
+        // line b / (BM / 8), tokens 8 (b % (BM / 8)) .. + 7), matrix rows 8 RN p .. + 8 RN - 1 and, while
+        // there are rows left, the scales of rows 16 p .. + 15.
         // 8 neighbouring lanes cover one 128-byte line; the lane at position q of a line asks
         // for chunk q ^ key(row), so that chunk c of a row sits at position c ^ key(row).
         const uint32_t p = wave - CONSUMERS;
         const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.x, a.x_bytes), wbuf = make_buffer(a.w, a.w_bytes);
         constexpr int XL = 2 * TT;  // activation loads a producer issues per step
-        uint32_t xoff[XL], xdst[XL], woff[2];
+        uint32_t xoff[XL], xdst[XL], woff[RN];
 #pragma unroll
         for (int i = 0; i < XL; i++) {
             const uint32_t b = p + 4u * i, line = b / (BM / 8), row = 8u * (b % (BM / 8)) + (lane >> 3);
@@ -162,13 +164,13 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
             xdst[i] = line * (BM * 128) + 1024u * (b % (BM / 8));
         }
 #pragma unroll
-        for (int i = 0; i < 2; i++) {
-            const uint32_t row = 8u * (2u * p + i) + (lane >> 3);
+        for (int i = 0; i < RN; i++) {
+            const uint32_t row = 8u * (RN * p + i) + (lane >> 3);
             woff[i] = (j0 + row) * a.row_bytes + 16u * ((lane & 7u) ^ line_key(row));
         }
         // A step's scales of the producer's sixteen rows, 8 bytes a row; the upper half of the
         // wave asks past the buffer's end (reads zero) and fills the filler.
-        const uint32_t soff = lane < 32u ? (j0 + 16u * p + (lane >> 1)) * a.row_bytes + a.k + 4u * (lane & 1u) : kNowhere;
+        const uint32_t soff = lane < 32u && 16u * p < (uint32_t)BN ? (j0 + 16u * p + (lane >> 1)) * a.row_bytes + a.k + 4u * (lane & 1u) : kNowhere;
         // Steps past the end of k are loaded like the others, so that every wait counts the same
         // loads, but from an offset no binding reaches (they land as zeros and move nothing;
         // nothing reads them): the step's position travels in the loads' scalar offset, and
@@ -179,17 +181,17 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
 #pragma unroll
                 for (int i = 0; i < XL; i++) load_lds_b128(xbuf, base + xdst[i], xoff[i], 256u * step);
 #pragma unroll
-                for (int i = 0; i < 2; i++) load_lds_b128(wbuf, base + ABUF + 1024u * (2u * p + i), woff[i], 128u * step);
+                for (int i = 0; i < RN; i++) load_lds_b128(wbuf, base + ABUF + 1024u * (RN * p + i), woff[i], 128u * step);
                 load_lds_b32(wbuf, base + ABUF + BN * 128 + 256u * p, soff, 8u * step);
             } else {
 #pragma unroll
                 for (int i = 0; i < XL; i++) load_lds_b128(xbuf, base + xdst[i], kNowhere, 0u);
 #pragma unroll
-                for (int i = 0; i < 2; i++) load_lds_b128(wbuf, base + ABUF + 1024u * (2u * p + i), kNowhere, 0u);
+                for (int i = 0; i < RN; i++) load_lds_b128(wbuf, base + ABUF + 1024u * (RN * p + i), kNowhere, 0u);
                 load_lds_b32(wbuf, base + ABUF + BN * 128 + 256u * p, kNowhere, 0u);
             }
         };
-        constexpr int PER_STEP = XL + 3;
+        constexpr int PER_STEP = XL + RN + 1;
         fetch(0, 0);
         fetch(1, 1);
         fetch(2, 2);
@@ -207,7 +209,7 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
         return;
     }
 
-    const uint32_t lrow = lane & 31u, h = lane >> 5, wn = wave & 1u, kq = wave >> 1;
+    const uint32_t lrow = lane & 31u, h = lane >> 5, wn = wave % RN, kq = wave / RN;
     f32x16 acc[TT];
 #pragma unroll
     for (int i = 0; i < TT; i++)
@@ -266,7 +268,7 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
         for (int i = 0; i < 2 * TT; i++) {
             __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
             __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            __builtin_amdgcn_sched_group_barrier(0x002, TT == 4 ? 6 : 11, 0);
+            __builtin_amdgcn_sched_group_barrier(0x002, TT == 4 ? 6 : TT == 2 ? 11 : 22, 0);
         }
         __builtin_amdgcn_sched_barrier(0);
         sync_after_reads();
@@ -292,14 +294,14 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
 
     // The four k quarters of a tile meet in LDS: the wave of quarter q keeps token tile q % TT
     // (with 64-token tiles, quarters q and q + 2 each keep half of tile q % 2: parts 2 (q / 2) and
-    // + 1 of the lane's four groups of sums) and hands the rest to their owners; sums are always
-    // (q0 + q2) + (q1 + q3).
+    // + 1 of the lane's four groups of sums; with one token tile, quarter q keeps group q) and
+    // hands the rest to their owners; sums are always (q0 + q2) + (q1 + q3).
     f32x4 *inbox = reinterpret_cast<f32x4 *>(lds);
-    constexpr int PARTS = TT;  // groups of four sums (of a tile's four) a quarter finishes
-    auto owner_of = [](int tt, int part) { return TT == 4 ? tt : tt + 2 * (part / 2); };
+    constexpr int PARTS = TT == 1 ? 1 : TT;  // groups of four sums (of a tile's four) a quarter finishes
+    auto owner_of = [](int tt, int part) { return TT == 4 ? tt : TT == 2 ? tt + 2 * (part / 2) : part; };
     auto slot = [&](uint32_t owner, uint32_t from, int part) {
         // owner: the quarter that finishes the sums; from != owner; part: which of the groups it finishes
-        return (((owner * 2u + wn) * 3u + ((from + 3u - owner) & 3u)) * PARTS + part) * 64u + lane;
+        return (((owner * RN + wn) * 3u + ((from + 3u - owner) & 3u)) * PARTS + part) * 64u + lane;
     };
     auto send = [&](auto quarter) __attribute__((always_inline)) {
         constexpr int Q = decltype(quarter)::value;
@@ -308,7 +310,7 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
 #pragma unroll
             for (int p = 0; p < 4; p++) {
                 if (owner_of(tt, p) == Q) continue;
-                inbox[slot(owner_of(tt, p), Q, TT == 4 ? p : p % 2)] = f32x4{acc[tt][4 * p], acc[tt][4 * p + 1], acc[tt][4 * p + 2], acc[tt][4 * p + 3]};
+                inbox[slot(owner_of(tt, p), Q, TT == 4 ? p : TT == 2 ? p % 2 : 0)] = f32x4{acc[tt][4 * p], acc[tt][4 * p + 1], acc[tt][4 * p + 2], acc[tt][4 * p + 3]};
             }
     };
     const bool aligned = ((a.out_stride | a.col0) & 3u) == 0u && (reinterpret_cast<uintptr_t>(a.out) & 15u) == 0u;
@@ -321,7 +323,7 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
         const uint32_t t = t0 + 32u * tile + lrow;
 #pragma unroll
         for (int i = 0; i < PARTS; i++) {
-            constexpr int first = TT == 4 ? 0 : 2 * (Q / 2);
+            constexpr int first = TT == 4 ? 0 : TT == 2 ? 2 * (Q / 2) : Q;
             const int p = first + i;
             f32x4 part[4];
 #pragma unroll
@@ -357,24 +359,38 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_bf16_kernel(Q8Args a) {
     }
 }
 
-template <int TT, class H>
+template <int TT, class H, int RN = 2>
 zhip_result launch_tile(const Dispatch &d, const char *name, const Q8Args &a) {
-    auto kernel = matmul_q8_bf16_kernel<TT, H>;
-    constexpr int bytes = lds_bytes<TT>();
-    if (!lds_opt_in<matmul_q8_bf16_kernel<TT, H>, bytes>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
+    auto kernel = matmul_q8_bf16_kernel<TT, H, RN>;
+    constexpr int bytes = lds_bytes<TT, RN>(), BN = 32 * RN;
+    if (!lds_opt_in<matmul_q8_bf16_kernel<TT, H, RN>, bytes>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
     const dim3 grid((a.n + BN - 1) / BN, (a.rows + 32 * TT - 1) / (32 * TT));
     if (grid.y > 65535u) return fail(d, ZHIP_E_BAD_COMMAND, "%s: grid too large", name);
     // The kernel's 32-bit offsets also name the rows and tokens of partial tiles past the end.
     if ((uint64_t)grid.x * BN * a.row_bytes >= (1ull << 32) || (uint64_t)grid.y * (32 * TT) * a.k * 2u >= (1ull << 32))
         return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
-    hipLaunchKernelGGL(kernel, grid, dim3(THREADS), bytes, d.stream, a);
+    hipLaunchKernelGGL(kernel, grid, dim3(threads<RN>()), bytes, d.stream, a);
     return check_launch(d, name);
+}
+
+template <class H>
+zhip_result launch_as(const Dispatch &d, const char *name, const Q8Args &a) {
+    // The largest tile that keeps more than half of the CUs busy: what a CU can have in flight
+    // from memory bounds its share of the loads, so a short step is faster in many small tiles
+    // than in few large ones. 128 tokens x 64 rows, 64 x 64 (every weight converted twice as
+    // often), 32 x 64, 32 x 32. A token's sums are the same bits in all of them.
+    const uint64_t cus = (uint64_t)d.dev->compute_units, columns = (a.n + 63u) / 64u;
+    if (a.rows > 64u && 2u * ((a.rows + 127u) / 128u) * columns > cus) return launch_tile<4, H, 2>(d, name, a);
+    if (a.rows > 32u && 2u * ((a.rows + 63u) / 64u) * columns > cus) return launch_tile<2, H, 2>(d, name, a);
+    if (2u * ((a.rows + 31u) / 32u) * columns > cus) return launch_tile<1, H, 2>(d, name, a);
+    return launch_tile<1, H, 1>(d, name, a);
 }
 
 }  // namespace
 
 bool matmul_q8_bf16_prepare_no_alloc() {
-    return lds_opt_in<matmul_q8_bf16_kernel<2, AsBf16>, lds_bytes<2>()>() && lds_opt_in<matmul_q8_bf16_kernel<4, AsBf16>, lds_bytes<4>()>();
+    return lds_opt_in<matmul_q8_bf16_kernel<4, AsBf16, 2>, lds_bytes<4, 2>()>() && lds_opt_in<matmul_q8_bf16_kernel<2, AsBf16, 2>, lds_bytes<2, 2>()>() &&
+           lds_opt_in<matmul_q8_bf16_kernel<1, AsBf16, 2>, lds_bytes<1, 2>()>() && lds_opt_in<matmul_q8_bf16_kernel<1, AsBf16, 1>, lds_bytes<1, 1>()>();
 }
 
 // Whole, unsliced k in 128-deep steps, operands the 32-bit offsets reach (the caller has
@@ -388,12 +404,7 @@ zhip_result launch_matmul_q8_bf16(const Dispatch &d, const char *name, bool f16,
     a.x = x; a.w = w; a.out = out;
     a.rows = rows; a.n = n; a.k = k; a.col0 = col0; a.out_stride = out_stride; a.accumulate = accumulate;
     a.row_bytes = row_bytes; a.x_bytes = x_bytes; a.w_bytes = w_bytes;
-    // 128-token tiles unless those leave half of the CUs idle: then 64-token tiles, which
-    // convert every weight twice as often but run in one round on twice the CUs.
-    const uint64_t tall = (uint64_t)((rows + 127u) / 128u) * ((n + BN - 1) / BN);
-    const bool high = rows > 64u && 2u * tall > (uint64_t)d.dev->compute_units;
-    if (f16) return high ? launch_tile<4, AsF16>(d, name, a) : launch_tile<2, AsF16>(d, name, a);
-    return high ? launch_tile<4, AsBf16>(d, name, a) : launch_tile<2, AsBf16>(d, name, a);
+    return f16 ? launch_as<AsF16>(d, name, a) : launch_as<AsBf16>(d, name, a);
 }
 
 }  // namespace zhip
