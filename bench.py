@@ -381,13 +381,14 @@ def vendor_c4_context():
         import torch
 
         tx = torch.randn(rows, k, device="cuda:0", dtype=torch.bfloat16)
-        tws = [torch.randn(n, k, device="cuda:0", dtype=torch.bfloat16) * 0.02 for _ in range(4)]
+        copies = -(-ROTATE_BYTES // (2 * n * k))  # (weights from HBM, like the kernel beside it)
+        tws = [torch.randn(n, k, device="cuda:0", dtype=torch.bfloat16) * 0.02 for _ in range(copies)]
         ev0, ev1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         ts = []
         for rep in range(3 + 7):
             ev0.record()
             for i in range(200):
-                torch.matmul(tx, tws[i % 4].t())
+                torch.matmul(tx, tws[i % copies].t())
             ev1.record()
             torch.cuda.synchronize()
             if rep >= 3:
@@ -606,8 +607,10 @@ def bench_c3(env):
     return {"headline": head, **rest}
 
 
-def _prefill_q8(env, rows, k, n, rung, copies=4, f32_x=False, check_stride=1):
-    """matmul_q8_0_float at rows x k x n on a prefill rung: (GPU seconds a step, err, err_bound)."""
+def _prefill_q8(env, rows, k, n, rung, copies=None, f32_x=False, check_stride=1):
+    """matmul_q8_0_float at rows x k x n on a prefill rung: (GPU seconds a step, err, err_bound).
+    The launches rotate over weight copies that together exceed L2 and the Infinity Cache (a
+    prefill step finds a layer's weights in HBM), unless `copies` says otherwise."""
     synth, oracle, K, TensorType, P = env["synth"], env["oracle"], env["K"], env["TensorType"], env["P"]
     rec, kset, b = env["rec"], env["kset"], env["b"]
     g = synth.rng(0xC4 if (rows, k, n) == (512, 4096, 4096) else 0x10 + n + rows)
@@ -619,7 +622,7 @@ def _prefill_q8(env, rows, k, n, rung, copies=4, f32_x=False, check_stride=1):
     rb = K.row_bytes(TensorType.q8_0, k)
     out = env["output"](4 * rows * n)
     held, launches = [src, xa, out], []
-    for _ in range(copies):
+    for _ in range(copies or env["rotation"](n * rb)):
         wa = env["output"](n * rb)
         held.append(wa)
         K.Launcher(rec, kset).layout(TensorType.q8_0, src, wa, n, k)
@@ -650,10 +653,11 @@ def _mfma_entry(t, flops, err=None, bound=None):
 
 def bench_c4(env):
     """Q8_0 prefill multiply M = 512, K = 4096, N = 4096 on the bf16 MFMA rung with the
-    activations bound as packed bf16 (4 weight copies, 71 MB: within the Infinity Cache - the
-    kernel is bound by the path into the CUs, not by HBM); then the reference's own ladder on
-    the same shape with f32-bound activations (its two f16 matrix-core rungs and the exact f32
-    rung), and the vendor library's bf16 multiply for context."""
+    activations bound as packed bf16, the weights from HBM (launches rotate over 36 copies,
+    641 MB) - `weights_in_cache` is the same with 4 copies, 71 MB, which the Infinity Cache
+    holds; then the reference's own ladder on the same shape with f32-bound activations (its
+    two f16 matrix-core rungs and the exact f32 rung), and the vendor library's bf16 multiply
+    for context, its weights rotating the same way."""
     K = env["K"]
     rows, k, n = 512, 4096, 4096
     flops = 2 * rows * n * k
@@ -664,7 +668,8 @@ def bench_c4(env):
     for rung in (K.Prefill.fp16_single, K.Prefill.fp16_compensated, K.Prefill.scalar_f32):
         rt, rerr, _ = _prefill_q8(env, rows, k, n, rung, f32_x=True)
         ladder[rung.name] = _mfma_entry(rt, flops, rerr)
-    return {"headline": head, "ladder_f32_activations": ladder, "vendor_library": env.get("vendor_c4")}
+    tw, errw, _ = _prefill_q8(env, rows, k, n, K.Prefill.bf16_mfma_xbf16, copies=4)
+    return {"headline": head, "weights_in_cache": _mfma_entry(tw, flops, errw), "ladder_f32_activations": ladder, "vendor_library": env.get("vendor_c4")}
 
 
 def bench_long(env):
@@ -691,7 +696,7 @@ def _prefill_int8(env, t, otype, raw, rows, k, n, check_stride=1):
     rb = K.row_bytes(t, k)
     qx, dx = env["output"](rows * k), env["output"](4 * rows * k // block)
     held, launches = [xa, out, src, qx, dx], []
-    for _ in range(4):
+    for _ in range(env["rotation"](n * rb)):
         wa = env["output"](n * rb)
         held.append(wa)
         if K.needs_layout(t):
