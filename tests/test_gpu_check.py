@@ -1194,6 +1194,47 @@ def test_quantize_q8_value_for_value(ctx, t):
     assert np.array_equal(got, oracle.round_like_llama(ORACLE_TYPE[t], x))
 
 
+@pytest.mark.parametrize("k", [1056, 2048, 4096, 14336])
+@pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q4_k])
+def test_quantize_q8_long_rows(ctx, t, k):
+    """Rows long enough that a wave takes two or four chunks of 256 values and a row several
+    workgroups (k = 14336: 56 chunks), and for Q8_0 a row whose last chunk is ragged
+    (k = 1056): integers and scales equal the oracle's, plain and behind the RMSNorm and
+    SiLU-pair prologues; ties between equal magnitudes across lanes and chunks. A few rows
+    (one chunk a wave) as well as many."""
+    c = ctx
+    block = K.act_block(t)
+    if k % block:
+        pytest.skip("k is not a multiple of the activation block")
+    rows = 130 if k > 4096 else 520  # (enough workgroups that a wave takes four chunks at once, or two)
+    x = c.random(rows * k, 3).reshape(rows, k)
+    x[1, k - 1] = -11.5      # a negative maximum in the last lane of the last chunk
+    x[2, 300] = 8.75         # +amax / -amax ties in different lanes and chunks
+    x[2, 301] = -8.75
+    x[2, k - 7] = -8.75
+    x[3] = 0
+    wq, wd = oracle.quantize_q8(x, block)
+    for count in (rows, 5):
+        qx, dx = quantize_x(c, t, c.upload(x[:count]), count, k)
+        q, d = read_q8(c, qx, dx, count, k)
+        assert np.array_equal(q, wq[:count])
+        assert np.array_equal(d[:, : k // block].view(np.uint32), wd[:count].view(np.uint32))
+    if block == 256:
+        eps, nw = 1e-6, c.random(k, 1)
+        qx, dx = quantize_x(c, t, c.upload(x), rows, k, mode=1, eps=eps, nw=c.upload(nw))
+        q, d = read_q8(c, qx, dx, rows, k)
+        wq, wd = oracle.quantize_q8(x, 256, mode=1, eps=eps, nw=nw)
+        assert np.array_equal(q, wq) and np.array_equal(d[:, : k // 256].view(np.uint32), wd.view(np.uint32))
+        pair = c.random(rows * 2 * k, 2).reshape(rows, 2 * k)
+        qx, dx = quantize_x(c, t, c.upload(pair), rows, k, mode=2)
+        q, d = read_q8(c, qx, dx, rows, k)
+        d = d[:, : k // 256]
+        g = pair[:, :k].astype(np.float64)
+        want = g * sigmoid64(g) * pair[:, k:]
+        step = np.repeat(np.abs(d), 256, axis=1).astype(np.float64)
+        assert np.max(np.abs(q.astype(np.float64) * np.repeat(d, 256, axis=1) - want) / (step / 2)) <= 1.0001
+
+
 def _llama_kats():
     import json
     import os
