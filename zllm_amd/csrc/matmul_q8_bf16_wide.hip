@@ -22,21 +22,14 @@
 #include <type_traits>
 
 #include "common.h"
+#include "matmul_q8_tiles.h"
 
 namespace zhip {
 
 namespace {
 
-typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
-typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
-typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
-typedef float f32x2 __attribute__((ext_vector_type(2)));
-typedef float f32x4 __attribute__((ext_vector_type(4)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
-typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+using namespace q8tiles;
 
-constexpr int BK = 128, PRODUCERS = 4;
 // TT: 32-token tiles a workgroup covers (4: 128 tokens, 2: 64 tokens). RQ: 32-row tiles of the
 // matrix it covers (4: 128 rows, 2: 64 rows), each the work of two multiplying waves.
 template <int RQ> constexpr int threads() { return 64 * (2 * RQ + PRODUCERS); }
@@ -48,90 +41,16 @@ template <int TT, int RQ> constexpr int lds_bytes() { return 3 * buf_bytes<TT, R
 static_assert(lds_bytes<4, 4>() <= 160 * 1024, "three buffers must fit the CU's LDS");
 // The exchange of the k halves reuses the buffers: 2 RQ waves x TT / 2 tiles x 4 KB.
 static_assert(lds_bytes<2, 2>() >= 4 * 2 * 4096 && lds_bytes<2, 4>() >= 8 * 2 * 4096, "the exchange must fit the buffers");
-struct Q8Args {
-    const uint8_t *x;  // packed bf16 rows
-    const uint8_t *w;  // split rows: k int8 values, k / 32 f16 scales, zero pad to 16 bytes
-    float *out;
-    uint32_t rows, n, k, col0, out_stride, accumulate, row_bytes;
-    uint32_t x_bytes, w_bytes;  // bytes the kernel may read behind x and w
-    uint32_t tiles_n;           // column tiles: workgroup b takes column tile b % tiles_n of token tile b / tiles_n
-};
-
-// The operand type of a rung: two floats rounded into one word, and the matrix instruction.
-struct AsBf16 {
-    typedef bf16x8 vec;
-    static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-        const f32x2 v = {lo, hi};
-        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, bf16x2));
-    }
-    static __device__ __forceinline__ f32x16 mfma(vec a, vec b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0); }
-};
-struct AsF16 {
-    typedef f16x8 vec;
-    static __device__ __forceinline__ uint32_t pack(float lo, float hi) {
-        const f32x2 v = {lo, hi};
-        return __builtin_bit_cast(uint32_t, __builtin_convertvector(v, f16x2));
-    }
-    static __device__ __forceinline__ f32x16 mfma(vec a, vec b, f32x16 c) { return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0); }
-};
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const uint8_t *base, uint32_t bytes) {
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<uint8_t *>(base), 0, (int)bytes, 0x00020000);
-}
-typedef __attribute__((address_space(3))) void *lds_ptr;
-// One wave-wide load straight into LDS: lane l's bytes land at dst + size * l.
-__device__ __forceinline__ void load_lds_b128(__amdgpu_buffer_rsrc_t buf, uint8_t *dst, uint32_t voff, uint32_t soff) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)dst, 16, voff, soff, 0, 0);
-}
-__device__ __forceinline__ void load_lds_b32(__amdgpu_buffer_rsrc_t buf, uint8_t *dst, uint32_t voff, uint32_t soff) {
-    __builtin_amdgcn_raw_ptr_buffer_load_lds(buf, (lds_ptr)dst, 4, voff, soff, 0, 0);
-}
-// A workgroup barrier that leaves loads into LDS in flight (__syncthreads() would wait for
-// every outstanding memory operation, the loads running steps ahead included).
-template <int LOADS_LEFT>
-__device__ __forceinline__ void sync_keeping_loads() {
-    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(LOADS_LEFT) : "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
-__device__ __forceinline__ void sync_after_reads() {
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-}
-// Rows are unpadded 128-byte lines whose 16-byte chunks are stored permuted: chunk c of row r
-// sits at position c ^ key(r). With this key the 32-row fragment reads run at the LDS's full
-// rate (measured; an unpermuted layout is ten times slower).
-__device__ __forceinline__ uint32_t line_key(uint32_t row) { return (row & 7u) ^ ((row >> 3) & 1u); }
-
-struct WRaw { u32x4 q; uint32_t d; };
-
-// Sixteen int8 weights times their block's scale (exact in f32), rounded once to the operand
-// type: the first operands of the lane's two MFMAs.
-template <class H>
-__device__ __forceinline__ void convert(const WRaw &r, typename H::vec &w0, typename H::vec &w1) {
-    const float d = (float)__builtin_bit_cast(_Float16, (uint16_t)r.d);
-    u32x4 lo, hi;
-#pragma unroll
-    for (int i = 0; i < 2; i++) {
-        const int32_t v = (int32_t)r.q[i];
-        lo[2 * i] = H::pack((float)(int8_t)(v) * d, (float)(int8_t)(v >> 8) * d);
-        lo[2 * i + 1] = H::pack((float)(int8_t)(v >> 16) * d, (float)(v >> 24) * d);
-        const int32_t u = (int32_t)r.q[2 + i];
-        hi[2 * i] = H::pack((float)(int8_t)(u) * d, (float)(int8_t)(u >> 8) * d);
-        hi[2 * i + 1] = H::pack((float)(int8_t)(u >> 16) * d, (float)(u >> 24) * d);
-    }
-    w0 = __builtin_bit_cast(typename H::vec, lo);
-    w1 = __builtin_bit_cast(typename H::vec, hi);
-}
 
 template <int TT, class H, int RQ>
-__global__ __launch_bounds__(threads<RQ>()) void matmul_q8_bf16_wide_kernel(Q8Args a) {
+__global__ __launch_bounds__(threads<RQ>()) void matmul_q8_bf16_wide_kernel(Q8Args a, uint32_t tiles_n) {
     typedef typename H::vec opvec;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int BM = 32 * TT, BN = 32 * RQ, CONSUMERS = 2 * RQ, ABUF = abuf_bytes<TT>(), BUF = buf_bytes<TT, RQ>();
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t j0 = (blockIdx.x % a.tiles_n) * BN, t0 = (blockIdx.x / a.tiles_n) * BM;
+    // Workgroup b takes column tile b % tiles_n of token tile b / tiles_n.
+    const uint32_t j0 = (blockIdx.x % tiles_n) * BN, t0 = (blockIdx.x / tiles_n) * BM;
     const uint32_t steps = a.k / BK;
 
     if (wave >= CONSUMERS) {
@@ -333,17 +252,17 @@ __global__ __launch_bounds__(threads<RQ>()) void matmul_q8_bf16_wide_kernel(Q8Ar
 }
 
 template <int TT, class H, int RQ>
-zhip_result launch_tile(const Dispatch &d, const char *name, Q8Args a) {
+zhip_result launch_tile(const Dispatch &d, const char *name, const Q8Args &a) {
     auto kernel = matmul_q8_bf16_wide_kernel<TT, H, RQ>;
     constexpr int bytes = lds_bytes<TT, RQ>();
     if (!lds_opt_in<matmul_q8_bf16_wide_kernel<TT, H, RQ>, bytes>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %d bytes of LDS", name, bytes);
-    a.tiles_n = (a.n + 32 * RQ - 1) / (32 * RQ);
-    const uint64_t tiles_t = (a.rows + 32 * TT - 1) / (32 * TT), tiles = (uint64_t)a.tiles_n * tiles_t;
+    const uint32_t tiles_n = (a.n + 32 * RQ - 1) / (32 * RQ);
+    const uint64_t tiles_t = (a.rows + 32 * TT - 1) / (32 * TT), tiles = (uint64_t)tiles_n * tiles_t;
     if (tiles >= (1ull << 31)) return fail(d, ZHIP_E_BAD_COMMAND, "%s: grid too large", name);
     // The kernel's 32-bit offsets also name the rows and tokens of partial tiles past the end.
-    if ((uint64_t)a.tiles_n * (32 * RQ) * a.row_bytes >= (1ull << 32) || tiles_t * (32 * TT) * a.k * 2u >= (1ull << 32))
+    if ((uint64_t)tiles_n * (32 * RQ) * a.row_bytes >= (1ull << 32) || tiles_t * (32 * TT) * a.k * 2u >= (1ull << 32))
         return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", name);
-    hipLaunchKernelGGL(kernel, dim3((uint32_t)tiles), dim3(threads<RQ>()), bytes, d.stream, a);
+    hipLaunchKernelGGL(kernel, dim3((uint32_t)tiles), dim3(threads<RQ>()), bytes, d.stream, a, tiles_n);
     return check_launch(d, name);
 }
 
