@@ -359,7 +359,7 @@ def main() -> int:
             r = fns[name](env)
         except Exception as e:  # a secondary workload must not lose the headline
             r = {"error": f"{type(e).__name__}: {e}"}
-        # The configurations the metric and BASELINE.json name go into `roofline`, beside the headline's.
+        # The other configurations the metric is quoted on go into `roofline`, beside the headline's.
         if name in ("c1", "c3", "c4", "c5") and "error" not in r:
             roofline[name] = r.pop("headline", None)
             if r:
