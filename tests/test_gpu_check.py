@@ -413,6 +413,11 @@ MFMA_VARIANT = K.MatvecVariant(wg=512, lanes=64, rows=16)
     (True, 8, 4128, 4096),    # gate and up tiles of 258 output tiles
     (True, 3, 64, 2048),      # one block a wave
     (False, 2, 48, 2048),
+    # rows of more than 4096 weights: workgroups that share a tile, 2048 columns each (steps
+    # with the RMSNorm prologue run the default variant)
+    (False, 8, 1296, 14336),  # seven parts, 81 tiles over 36 walkers: two rounds and nine tiles in halves
+    (True, 4, 528, 8192),     # four parts, gate and up, fewer tiles than walkers
+    (False, 5, 4096, 6144),   # three parts, 256 tiles over 85 walkers: one whole tile left over
 ])
 @pytest.mark.parametrize("prologue", ["plain", "norm", "norm_act"])
 @pytest.mark.parametrize("t", [TensorType.q4_k, TensorType.q5_k])

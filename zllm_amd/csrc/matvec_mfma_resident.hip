@@ -1,5 +1,5 @@
 // matvec_q4_k and matvec_q5_k, matrix-core variant (MatvecVariant wg 512, lanes 64, rows 16) for
-// k = 2048 or 4096 and steps of up to eight tokens. The per-weight work is done once for all
+// k = 2048 or 4096 (longer rows in parts, below) and steps of up to eight tokens. The per-weight work is done once for all
 // tokens: the weights enter v_mfma_f32_16x16x32_f16 as the exact f16 values 16 + q (the nibble
 // dropped into the mantissa of 16.0; Q5_K: 32 + q with the fifth bit), every token as two f16
 // rows, the rounding of its inputs and what that left times 2^11, under a per-token power of
@@ -28,6 +28,16 @@
 // epilogue and store. Each lane reads its row's header and nibbles back from
 // the copy (chunks XOR-permuted by row against bank conflicts) and multiplies.
 //
+// Rows of 6144 .. 16384 weights (a multiple of 2048; the FFN-down shapes) do not fit a
+// workgroup's registers: `parts` = k / 2048 workgroups share a walker's tiles, workgroup b taking
+// columns 2048 (b % parts) .. of the tiles of walker b / parts (one block a wave, the tile's
+// sixteen pieces of nine or eleven lines a whole row apart), each under its own per-token
+// scales, and store their sums per part; a second launch adds a tile's parts in the order of
+// their columns and applies the epilogue. Steps with the RMSNorm prologue, whose sum of squares
+// is no single workgroup's, stay with the default variant. Measured on Q4_K 4096 x 14336 at
+// one to eight tokens: 14.3 - 14.8 us (12.1 + the sums' launch) against 10.3 / 14.3 / 21.7 /
+// 21.6 / 40.9 us at one / two / three / four / eight tokens on the default variant.
+//
 // Contract as the other variants (src/kernels/matvec_quant.wgsl.hbs); a token's
 // result does not depend on how many tokens share the launch.
 #include <hip/hip_runtime.h>
@@ -47,7 +57,8 @@ typedef uint32_t ru32x2 __attribute__((ext_vector_type(2)));
 namespace {
 
 constexpr uint32_t THREADS = 512, WAVES = 8;
-constexpr int DEPTH = 3;  // ring slots: one tile multiplied, the others in flight (two slots: +0.3 us on the 2 x 14336 x 4096 pair, four: +0.8 us)
+constexpr int kLongDepth = 3;
+constexpr int kDepth = 3;  // ring slots: one tile multiplied, the others in flight (two slots: +0.3 us on the 2 x 14336 x 4096 pair, four: +0.8 us)
 // The formats: a 256-weight block is a 16-byte header (d, dmin, twelve bytes of 6-bit scales and
 // minimums) and 128 bytes of nibbles; Q5_K keeps a fifth bit of every weight in 32 bytes between
 // the two (src/ref/tensor.zig:100-117). A weight enters the matrix cores as the exact f16 value
@@ -78,6 +89,10 @@ struct ResArgs {
     uint32_t rounds;                // sixteen-output tiles every workgroup takes: tiles b, b + G, ...
     uint32_t left;                  // output tiles after those, fewer than G: one for each of the first workgroups,
     uint32_t split;                 // or (split) eight outputs of one for each of the first 2 * left
+    // Rows of more than 4096 weights: `parts` workgroups share a tile, each over 2048 of its
+    // columns, and leave their sums in `partial` ([part][gate, up][token of 8][output]).
+    uint32_t parts;
+    float *partial;
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void *base, uint32_t bytes) {
@@ -144,9 +159,13 @@ __device__ __forceinline__ rf16x8 nibbles(ru32x2 w, ru32x2 fifth, uint32_t mask,
     return __builtin_bit_cast(rf16x8, r);
 }
 
-// NB: 256-weight blocks of a wave's k range (k = 2048 NB).
-template <class F, bool PAIR, int NB>
+// NB: 256-weight blocks of a wave's k range (k = 2048 NB). LONG (NB = 1): k = 2048 q.parts;
+// workgroup b multiplies columns 2048 (b % parts) .. (part `kpart`) of the tiles that walker b / parts takes, and
+// matvec_kquant_mfma_parts_sum_kernel adds the parts in their order and applies the epilogue.
+template <class F, bool PAIR, int NB, bool LONG>
 __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_resident_kernel(ResArgs q) {
+    static_assert(!LONG || NB == 1, "parts of a long row are 2048 columns");
+    constexpr int DEPTH = LONG ? kLongDepth : kDepth;
     const MvArgs &a = q.a;
     __shared__ float lds_scale[16];               // [8 ..]: one over each token's scale
     __shared__ float lds_max[WAVES * 8];          // [wave][token]: the largest magnitude in the wave's range
@@ -160,14 +179,15 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_resident_kernel(Re
     // The workgroup's weight tiles: output tiles b, b + G, ...; with SILU_PAIR the gate tile
     // and then the up tile of each. Tile p of the run starts at matrix row:
     const uint32_t per = PAIR ? 2u : 1u;
+    const uint32_t kpart = LONG ? blockIdx.x % q.parts : 0u, walker = LONG ? blockIdx.x / q.parts : blockIdx.x, walkers = LONG ? gridDim.x / q.parts : gridDim.x;
     // When the output tiles left over after whole rounds are at most half as many as the
     // workgroups, two workgroups share each, eight rows apiece: a whole tile more on half of
     // the CUs would be the launch's tail.
-    const bool extra = blockIdx.x < (q.split ? 2u * q.left : q.left);
+    const bool extra = walker < (q.split ? 2u * q.left : q.left);
     const uint32_t mine = q.rounds + (extra ? 1u : 0u);
     const uint32_t count = per * mine;
-    const uint32_t last_out = 16u * (q.rounds * gridDim.x + (q.split ? blockIdx.x >> 1 : blockIdx.x)) + (q.split ? 8u * (blockIdx.x & 1u) : 0u);
-    auto out0 = [&](uint32_t p) { return p / per < q.rounds ? 16u * (blockIdx.x + (p / per) * gridDim.x) : last_out; };  // first output of tile p
+    const uint32_t last_out = 16u * (q.rounds * walkers + (q.split ? walker >> 1 : walker)) + (q.split ? 8u * (walker & 1u) : 0u);
+    auto out0 = [&](uint32_t p) { return p / per < q.rounds ? 16u * (walker + (p / per) * walkers) : last_out; };  // first output of tile p
     auto rows_of = [&](uint32_t p) { return (q.split && p / per >= q.rounds) ? 8u : 16u; };
     auto row0 = [&](uint32_t p) { return out0(p) + ((PAIR && (p & 1u)) ? a.half : 0u); };
 
@@ -188,7 +208,8 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_resident_kernel(Re
 #pragma unroll
     for (int j = 0; j < LOADS; j++) {
         const uint32_t line = 8u * (LOADS * wave + j) + (lane >> 3), row = line / ROW_LINES;
-        woff[j] = 128u * line + 16u * ((lane & 7u) ^ (row & 7u));
+        // (a part of a long row: the tile's rows lie a whole row apart)
+        woff[j] = (LONG ? row * a.row_bytes + 128u * (ROW_LINES * kpart + line % ROW_LINES) : 128u * line) + 16u * ((lane & 7u) ^ (row & 7u));
     }
     auto load_tile = [&](uint32_t p, uint32_t slot) __attribute__((always_inline)) {
         const bool real = p < count;
@@ -213,14 +234,15 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_resident_kernel(Re
     const uint32_t tok = l16 >> 1, sub = l16 & 1u, tsrc = tok < a.m ? tok : a.m - 1u;
     float4 raw[NB * 8];
     {
-        const float *xt = a.x + (size_t)tsrc * a.xr + NB * 256u * wave + 8u * g + 4u * sub;
+        const float *xt = a.x + (size_t)tsrc * a.xr + 2048u * kpart + NB * 256u * wave + 8u * g + 4u * sub;
 #pragma unroll
         for (int s = 0; s < NB * 8; s++) raw[s] = *reinterpret_cast<const float4 *>(xt + 32 * s);
     }
     // A step's prologue (src/kernels/matvec_quant.wgsl.hbs:73-89) on the same registers, in the
     // default variant's arithmetic: RMSNorm times the norm weights (the wave ranges' sums of
     // squares meet in LDS, added in the order of the ranges) and / or silu(x / act_div).
-    const bool norm = (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
+    // (the sum of squares of a long row is not any one workgroup's: such steps run other kernels)
+    const bool norm = !LONG && (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
     float4 gw[NB * 8];
     if (norm) {
         const float *gt = a.norm_w + NB * 256u * wave + 8u * g + 4u * sub;
@@ -381,7 +403,9 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_resident_kernel(Re
 #pragma unroll
         for (uint32_t wv = 1; wv < WAVES; wv++) sum += src[wv * 128u];
         sum *= lds_scale[8 + t];
-        if (PAIR && !(p & 1u)) {
+        if (LONG) {
+            if (t < a.m && row < rows_of(p)) store_apart(q.partial + ((size_t)(per * kpart + (PAIR ? p & 1u : 0u)) * 8u + t) * a.rows + out0(p) + row, sum);
+        } else if (PAIR && !(p & 1u)) {
             held = sum;
         } else {
             const float v = PAIR ? silu_f(held) * sum : sum;
@@ -417,13 +441,47 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_resident_kernel(Re
     wait_loads<0>();  // nothing may still land in LDS once the workgroup is gone
 }
 
+constexpr uint32_t kMaxParts = 8;  // rows of up to 16384 weights
+
+// The outputs of a step over long rows: the parts' sums added in the order of their columns,
+// then the SILU_PAIR / ACCUMULATE epilogue. One thread an output.
+template <bool PAIR>
+__global__ __launch_bounds__(256) void matvec_kquant_mfma_parts_sum_kernel(MvArgs a, const float *partial, uint32_t parts) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x, row = i % a.rows, t = i / a.rows;
+    if (t >= a.m) return;
+    constexpr uint32_t per = PAIR ? 2u : 1u;
+    const float *src = partial + (size_t)t * a.rows + row;
+    const size_t plane = (size_t)8u * a.rows;
+    float *o = a.out + (size_t)t * a.out_stride + a.col0 + row;
+    // Every load first: the parts were written by other workgroups and come from memory.
+    float first[kMaxParts], second[kMaxParts];
+#pragma unroll
+    for (uint32_t p = 0; p < kMaxParts; p++) {
+        first[p] = p < parts ? src[per * p * plane] : 0.f;
+        second[p] = (PAIR && p < parts) ? src[(per * p + 1u) * plane] : 0.f;
+    }
+    const float before = (a.flags & FLAG_ACCUMULATE) ? *o : 0.f;
+    float sum = first[0], up = second[0];
+#pragma unroll
+    for (uint32_t p = 1; p < kMaxParts; p++) {
+        if (p < parts) {
+            sum += first[p];
+            up += second[p];
+        }
+    }
+    const float v = PAIR ? silu_f(sum) * up : sum;
+    *o = (a.flags & FLAG_ACCUMULATE) ? before + v : v;
+}
+
 }  // namespace
 
 // Whether this kernel can run the (already validated) arguments: whole tiles, k split into
-// one or two blocks a wave.
+// one or two blocks a wave, or rows of 6144 .. 16384 weights in parts of 2048 (without the
+// RMSNorm prologue).
 bool matvec_q4k_mfma_resident_accepts(const MvArgs &a) {
     const bool pair = a.flags & FLAG_SILU_PAIR;
-    return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u) && a.rows % 16u == 0 && (!pair || a.half % 16u == 0);
+    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMaxParts && !(a.flags & FLAG_NORM);
+    return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u || parts) && a.rows % 16u == 0 && (!pair || a.half % 16u == 0);
 }
 
 template <class F>
@@ -432,18 +490,34 @@ static zhip_result launch_resident(const Dispatch &d, const MvArgs &a, uint64_t 
     // 32-bit byte offsets.
     const uint64_t reach = ((uint64_t)(pair ? a.half : 0u) + a.rows + 16u) * a.row_bytes;
     if (w_bytes >= 0xfffffff0ull || reach >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "%s: operands of 4 GiB or more", F::name());
+    // The workgroups that walk the tiles: one a CU, or (rows of more than 4096 weights) one for
+    // every `parts` CUs, each of them `parts` workgroups.
+    const uint32_t parts = a.k > 4096u ? a.k / 2048u : 1u;
     const uint32_t cus = (uint32_t)d.dev->compute_units, tiles = a.rows / 16u;
-    const uint32_t groups = tiles < cus ? (2u * tiles <= cus ? 2u * tiles : tiles) : cus;
+    if (cus < parts) return fail(d, ZHIP_E_GPU, "%s: %u compute units for %u parts of a row", F::name(), cus, parts);
+    const uint32_t most = cus / parts;
+    const uint32_t groups = tiles < most ? (2u * tiles <= most ? 2u * tiles : tiles) : most;
     const bool halves = tiles < groups;  // every workgroup takes eight outputs of one tile
     const uint32_t left = halves ? tiles : tiles % groups;
-    ResArgs q{a, (uint32_t)w_bytes, mask, bias_bits, halves ? 0u : tiles / groups, left, (halves || 2u * left <= groups) ? 1u : 0u};
-    const dim3 grid(groups);
-    if (a.k == 2048u) {
-        if (pair) hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, true, 1>), grid, dim3(THREADS), 0, d.stream, q);
-        else hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, false, 1>), grid, dim3(THREADS), 0, d.stream, q);
+    ResArgs q{a, (uint32_t)w_bytes, mask, bias_bits, halves ? 0u : tiles / groups, left, (halves || 2u * left <= groups) ? 1u : 0u, parts, nullptr};
+    const dim3 grid(groups * parts);
+    if (parts > 1u) {
+        const uint64_t bytes = (uint64_t)parts * (pair ? 2u : 1u) * 8u * a.rows * sizeof(float);
+        if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", F::name());
+        if (zhip_result r = d.work->reserve(d, bytes)) return r;
+        q.partial = reinterpret_cast<float *>(d.work->data);
+        if (pair) hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, true, 1, true>), grid, dim3(THREADS), 0, d.stream, q);
+        else hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, false, 1, true>), grid, dim3(THREADS), 0, d.stream, q);
+        if (zhip_result r = check_launch(d, F::name())) return r;
+        const dim3 sums((a.rows * a.m + 255u) / 256u);
+        if (pair) hipLaunchKernelGGL(matvec_kquant_mfma_parts_sum_kernel<true>, sums, dim3(256), 0, d.stream, a, q.partial, parts);
+        else hipLaunchKernelGGL(matvec_kquant_mfma_parts_sum_kernel<false>, sums, dim3(256), 0, d.stream, a, q.partial, parts);
+    } else if (a.k == 2048u) {
+        if (pair) hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, true, 1, false>), grid, dim3(THREADS), 0, d.stream, q);
+        else hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, false, 1, false>), grid, dim3(THREADS), 0, d.stream, q);
     } else {
-        if (pair) hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, true, 2>), grid, dim3(THREADS), 0, d.stream, q);
-        else hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, false, 2>), grid, dim3(THREADS), 0, d.stream, q);
+        if (pair) hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, true, 2, false>), grid, dim3(THREADS), 0, d.stream, q);
+        else hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, false, 2, false>), grid, dim3(THREADS), 0, d.stream, q);
     }
     return check_launch(d, F::name());
 }
