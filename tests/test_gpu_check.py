@@ -478,6 +478,10 @@ def test_quant_matvec_mfma_variant(ctx, t, pair, rows, n, k, prologue):
     (8, 4112, 1024, 0, 0, False),    # rows of 1024 weights: the kernel that moves a tile's 32 rows as one flat stretch
     (3, 4128, 1024, 5, 7, True),
     (4, 5, 1024, 1, 2, True),        # fewer rows than a unit of eight
+    # rows of more than 4096 weights: workgroups that share a tile, 2048 columns each
+    (8, 1296, 14336, 3, 7, True),    # seven parts, 81 tiles over 36 walkers
+    (3, 4096, 6144, 0, 0, False),    # three parts, 256 tiles over 85 walkers
+    (5, 48, 8192, 0, 0, False),      # four parts, fewer tiles than walkers
 ])
 def test_matvec_q8_0_mfma_variant(ctx, rows, n, k, col0, pad, accumulate):
     """The matrix-core variant of matvec_q8_0 (the id of a wave per sixteen rows): every
@@ -513,7 +517,8 @@ def test_matvec_q8_0_mfma_variant(ctx, rows, n, k, col0, pad, accumulate):
 
 
 @pytest.mark.parametrize("norm", [False, True])
-@pytest.mark.parametrize("rows,n,k", [(8, 4128, 4096), (3, 64, 2048), (5, 3072, 1024), (2, 4104, 1024)])
+@pytest.mark.parametrize("rows,n,k", [(8, 4128, 4096), (3, 64, 2048), (5, 3072, 1024), (2, 4104, 1024),
+                                      (6, 528, 8192)])  # rows in four parts (Q8_0; the others' pair steps over such rows run the default variant)
 @pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q6_k, TensorType.q3_k])
 def test_matvec_q8_0_mfma_variant_silu_pair(ctx, t, rows, n, k, norm):
     """The matrix-core variant of matvec_q8_0, matvec_q6_k and matvec_q3_k on the fused gate / up step (SILU_PAIR: gate rows,
@@ -589,6 +594,11 @@ def test_matvec_q8_0_mfma_variant_prologues(ctx, rows, n, k, prologue):
     (2, 64, 1024, 0, 0, False, None),          # one unit a tile
     (7, 8232, 1024, 0, 0, True, "norm"),
     (3, 96, 3072, 0, 0, False, None),          # k the kernel does not take: the default variant's
+    # rows of more than 4096 weights: workgroups that share a tile, 2048 columns each
+    (8, 1300, 14336, 3, 2, True, None),        # seven parts, 36 walkers: whole rounds, a tail, a ragged last unit
+    (4, 4096, 6144, 0, 0, False, None),        # three parts, at most four tokens
+    (5, 200, 8192, 0, 0, True, "act"),         # four parts, fewer rows than walkers
+    (2, 96, 14336, 0, 0, False, "norm"),       # with the RMSNorm prologue: the default variant's
 ])
 @pytest.mark.parametrize("t", [TensorType.q6_k, TensorType.q3_k])
 def test_matvec_q6_k_mfma_variant(ctx, t, rows, n, k, col0, pad, accumulate, prologue):
@@ -599,19 +609,20 @@ def test_matvec_q6_k_mfma_variant(ctx, t, rows, n, k, col0, pad, accumulate, pro
     to its lone launch."""
     c = ctx
     stride = col0 + n + pad
-    div, eps = 4 if prologue == "norm_act" else 0, 1e-6
+    div, eps = 4 if prologue in ("norm_act", "act") else 0, 1e-6
+    norm = prologue in ("norm", "norm_act")
     x = c.random(rows * k, 3).reshape(rows, k)
     x[0] *= np.float32(1e-4)
     nw = c.random(k, 1.5)
     raw, values = quant_rows(c, t, n, k)
     init = c.random(rows * stride, 2).reshape(rows, stride)
     xa, wa, na = c.upload(x), c.gpu_weights(t, raw, k), c.upload(nw)
-    x64 = np.stack([norm_row(r, nw if prologue else None, eps) for r in x])
+    x64 = np.stack([norm_row(r, nw if norm else None, eps) for r in x])
     if div:
         x64 = (x64 / div) * sigmoid64(x64 / div)
     prod = x64 @ values.astype(np.float64).T
     want = prod + (init[:, col0 : col0 + n] if accumulate else 0)
-    p = lambda: P.MatvecBf16(n=n, k=k, col0=col0, out_stride=stride, eps=eps, norm=prologue is not None, accumulate=accumulate)
+    p = lambda: P.MatvecBf16(n=n, k=k, col0=col0, out_stride=stride, eps=eps, norm=norm, accumulate=accumulate)
     variant = K.MatvecVariant(MFMA_VARIANT.wg, MFMA_VARIANT.lanes, MFMA_VARIANT.rows, div)
     pipeline = c.set.matvec(c.rec, K.weight_kernel("matvec", t), variant)
     grid_x = K.div_ceil(n, variant.group_rows())

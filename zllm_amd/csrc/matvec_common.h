@@ -74,4 +74,11 @@ __device__ __forceinline__ void stage_token(const MvArgs &a, uint32_t token, flo
     stage_token(a, token, dst, red, [](uint32_t i) { return i; });
 }
 
+// Matrix-core variants over rows of more than 4096 weights: `parts` workgroups share a tile, each
+// over 2048 of its columns, and leave their sums in `partial` ([part][gate, up][token of 8][output],
+// outputs a.rows apart); this launch adds a tile's parts in the order of their columns and applies
+// the SILU_PAIR / ACCUMULATE epilogue (matvec_mfma_resident.hip).
+constexpr uint32_t kMatvecMaxParts = 8;  // rows of up to 16384 weights
+zhip_result launch_matvec_parts_sum(const Dispatch &d, const char *name, const MvArgs &a, const float *partial, uint32_t parts);
+
 }  // namespace zhip

@@ -441,8 +441,6 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_resident_kernel(Re
     wait_loads<0>();  // nothing may still land in LDS once the workgroup is gone
 }
 
-constexpr uint32_t kMaxParts = 8;  // rows of up to 16384 weights
-
 // The outputs of a step over long rows: the parts' sums added in the order of their columns,
 // then the SILU_PAIR / ACCUMULATE epilogue. One thread an output.
 template <bool PAIR>
@@ -454,16 +452,16 @@ __global__ __launch_bounds__(256) void matvec_kquant_mfma_parts_sum_kernel(MvArg
     const size_t plane = (size_t)8u * a.rows;
     float *o = a.out + (size_t)t * a.out_stride + a.col0 + row;
     // Every load first: the parts were written by other workgroups and come from memory.
-    float first[kMaxParts], second[kMaxParts];
+    float first[kMatvecMaxParts], second[kMatvecMaxParts];
 #pragma unroll
-    for (uint32_t p = 0; p < kMaxParts; p++) {
+    for (uint32_t p = 0; p < kMatvecMaxParts; p++) {
         first[p] = p < parts ? src[per * p * plane] : 0.f;
         second[p] = (PAIR && p < parts) ? src[(per * p + 1u) * plane] : 0.f;
     }
     const float before = (a.flags & FLAG_ACCUMULATE) ? *o : 0.f;
     float sum = first[0], up = second[0];
 #pragma unroll
-    for (uint32_t p = 1; p < kMaxParts; p++) {
+    for (uint32_t p = 1; p < kMatvecMaxParts; p++) {
         if (p < parts) {
             sum += first[p];
             up += second[p];
@@ -475,12 +473,19 @@ __global__ __launch_bounds__(256) void matvec_kquant_mfma_parts_sum_kernel(MvArg
 
 }  // namespace
 
+zhip_result launch_matvec_parts_sum(const Dispatch &d, const char *name, const MvArgs &a, const float *partial, uint32_t parts) {
+    const dim3 sums((a.rows * a.m + 255u) / 256u);
+    if (a.flags & FLAG_SILU_PAIR) hipLaunchKernelGGL(matvec_kquant_mfma_parts_sum_kernel<true>, sums, dim3(256), 0, d.stream, a, partial, parts);
+    else hipLaunchKernelGGL(matvec_kquant_mfma_parts_sum_kernel<false>, sums, dim3(256), 0, d.stream, a, partial, parts);
+    return check_launch(d, name);
+}
+
 // Whether this kernel can run the (already validated) arguments: whole tiles, k split into
 // one or two blocks a wave, or rows of 6144 .. 16384 weights in parts of 2048 (without the
 // RMSNorm prologue).
 bool matvec_q4k_mfma_resident_accepts(const MvArgs &a) {
     const bool pair = a.flags & FLAG_SILU_PAIR;
-    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMaxParts && !(a.flags & FLAG_NORM);
+    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts && !(a.flags & FLAG_NORM);
     return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u || parts) && a.rows % 16u == 0 && (!pair || a.half % 16u == 0);
 }
 
@@ -509,9 +514,7 @@ static zhip_result launch_resident(const Dispatch &d, const MvArgs &a, uint64_t 
         if (pair) hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, true, 1, true>), grid, dim3(THREADS), 0, d.stream, q);
         else hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, false, 1, true>), grid, dim3(THREADS), 0, d.stream, q);
         if (zhip_result r = check_launch(d, F::name())) return r;
-        const dim3 sums((a.rows * a.m + 255u) / 256u);
-        if (pair) hipLaunchKernelGGL(matvec_kquant_mfma_parts_sum_kernel<true>, sums, dim3(256), 0, d.stream, a, q.partial, parts);
-        else hipLaunchKernelGGL(matvec_kquant_mfma_parts_sum_kernel<false>, sums, dim3(256), 0, d.stream, a, q.partial, parts);
+        return launch_matvec_parts_sum(d, F::name(), a, q.partial, parts);
     } else if (a.k == 2048u) {
         if (pair) hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, true, 1, false>), grid, dim3(THREADS), 0, d.stream, q);
         else hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, false, 1, false>), grid, dim3(THREADS), 0, d.stream, q);

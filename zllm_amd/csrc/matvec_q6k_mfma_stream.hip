@@ -1,5 +1,5 @@
 // matvec_q6_k and matvec_q3_k, matrix-core variant (MatvecVariant wg 512, lanes 64, rows 16) for steps of up to
-// eight tokens and k = 1024, 2048 or 4096: the weight stream is read once for all tokens of the step
+// eight tokens and k = 1024, 2048 or 4096 (longer rows in parts, at the end of this comment): the weight stream is read once for all tokens of the step
 // and the per-weight work is done once. Contract as the default variant's
 // (src/kernels/matvec_quant.wgsl.hbs with the decoder of src/kernels/quant/q6_k_dot.wgsl; block
 // formula src/ref/tensor.zig:118-140): out[t][col0 + j] (+)= sum over 16-weight sub-blocks of
@@ -53,6 +53,14 @@
 // one token on the default variant). Q8_0 on 151936 x 1024 at two / four / eight tokens:
 // 33.9 / 32.9 / 35.6 us (41.7 us with the rows read line by line, row by row, by the kernel that
 // takes k = 2048 and 4096; the default variant 33.6 / 44.1 / 79.7 us).
+//
+// Rows of 6144 .. 16384 weights (a multiple of 2048; the FFN-down shapes), Q6_K and Q3_K: the
+// operands of so many positions do not fit a workgroup's registers, so k / 2048 workgroups share
+// a walker's tiles, each over two units of every tile's rows and under its own per-token scales;
+// they store their sums per part and launch_matvec_parts_sum (matvec_mfma_resident.hip) adds
+// them in the order of their columns and applies the epilogue. Steps with the RMSNorm prologue
+// or the SILU_PAIR epilogue over such rows stay with the default variant. 4096 x 14336 at four /
+// eight tokens: Q6_K 19.1 / 20.3 us (default variant 27.1 / 51.8), Q3_K 16.1 / 17.3 us (26.2 / 49.3).
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -133,6 +141,10 @@ struct Q6Args {
     uint32_t by_die;     // workgroups renumbered die by die (the grid is a multiple of eight)
     uint32_t bias;       // 0x64646464: the bytes of two f16 1024.0 exponents, as a kernel argument
                          // so that the byte shuffles stay one instruction each
+    // Rows of more than 4096 weights: `parts` workgroups share a tile, each over 2048 of its
+    // columns, and leave their sums in `partial` ([part][token of 8][output]).
+    uint32_t parts;
+    float *partial;
 };
 
 __device__ __forceinline__ void lds_barrier() {
@@ -176,8 +188,11 @@ __device__ __forceinline__ qf16x8 weights_f16(qu32x2 q, uint32_t bias) {
 
 // NU: units of a tile (k = 1024 NU).
 // FEW: at most four tokens, whose eight rows then leave every lane four results instead of eight.
-template <class F, int NU, bool FEW>
+// LONG (NU = 2): k = 2048 q.parts; workgroup i multiplies columns 2048 (i % parts) .. (part
+// `kpart`) of the tiles that walker i / parts takes, and launch_matvec_parts_sum adds the parts.
+template <class F, int NU, bool FEW, bool LONG>
 __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Args q) {
+    static_assert(!LONG || NU == 2, "parts of a long row are 2048 columns");
     constexpr uint32_t ROW_UNIT = row_unit<F>(), UNIT = unit_bytes<F>();
     constexpr int LOADS = F::LOADS, SLOTS = F::SLOTS;
     const MvArgs &a = q.a;
@@ -194,8 +209,9 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     asm volatile("" : "+v"(bias));
 
     // The workgroup's tiles: b, b + G, ... and its share of the rows after the whole rounds.
-    const uint32_t G = gridDim.x;
-    const uint32_t b = q.by_die ? (blockIdx.x & 7u) * (G >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+    const uint32_t kpart = LONG ? blockIdx.x % q.parts : 0u, walker = LONG ? blockIdx.x / q.parts : blockIdx.x;
+    const uint32_t G = LONG ? gridDim.x / q.parts : gridDim.x;
+    const uint32_t b = q.by_die ? (walker & 7u) * (G >> 3) + (walker >> 3) : walker;
     const uint32_t tail_units = q.tail_base + (b < q.tail_rem ? 1u : 0u);
     const uint32_t tail_row = 32u * q.rounds * G + 8u * (b * q.tail_base + (b < q.tail_rem ? b : q.tail_rem));
     // With SILU_PAIR (src/kernels/matvec_quant.wgsl.hbs:110-125) an output tile is two weight
@@ -226,7 +242,7 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     auto issue = [&](uint32_t v, uint32_t slot) __attribute__((always_inline)) {
         const uint32_t p = v / NU, u = v % NU;
         const bool real = p < count && wave < F::LOADERS;
-        const uint32_t base = (real ? first_row(p) : 0u) * a.row_bytes + ROW_UNIT * u, rows = rows_of(p);
+        const uint32_t base = (real ? first_row(p) : 0u) * a.row_bytes + ROW_UNIT * (NU * kpart + u), rows = rows_of(p);
         // (a load against the empty buffer still lands zeros: the eighth wave's in a spare KB)
         const uint32_t dst = wave < F::LOADERS ? ring0 + slot * UNIT + 1024u * (LOADS * wave) : ring0 + SLOTS * UNIT + KEPT * 1024u + 64u;
 #pragma unroll
@@ -251,7 +267,8 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     // inputs' loads and this arithmetic (loads complete in order within a wave), the next three
     // once the inputs are in: all four at once would hold up the other waves' inputs in the
     // CU's one address pipeline (+0.7 us).
-    const bool norm = (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
+    // (the sum of squares of a long row is not any one workgroup's: such steps run other kernels)
+    const bool norm = !LONG && (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
     float *lds_max = lds_inverse + 16 + 256, *lds_ss = lds_max + 64;  // [wave][token], behind the spare KB
     // Operand row r of the matrix instruction is piece r / 8 of token 4 (r / 4 % 2) + r % 4 (rows
     // 16 .. 31 are zeros), so that a lane's results are its weight row times both pieces of four
@@ -271,7 +288,7 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
         const uint32_t t1 = lane >> 3, l8 = lane & 7u, t1c = t1 < a.m ? t1 : a.m - 1u;
         float4 r1[4 * NU], g1[4 * NU];
         const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.x, ((a.m - 1u) * a.xr + a.k) * 4u);
-        const uint32_t x1 = (t1 * a.xr + 128u * wave + 4u * l8) * 4u;
+        const uint32_t x1 = (t1 * a.xr + 1024u * NU * kpart + 128u * wave + 4u * l8) * 4u;
 #pragma unroll
         for (int u = 0; u < NU; u++)
 #pragma unroll
@@ -538,7 +555,8 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
             if (tk < a.m && row < out_rows(po) && j < a.rows) {
                 float *o = a.out + (size_t)tk * a.out_stride + a.col0 + j;
                 const float total = lds_kept[256u * (po % KEPT) + (tid & 255u)];
-                store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + total : total);
+                if (LONG) store_apart(q.partial + ((size_t)kpart * 8u + tk) * a.rows + j, total);
+                else store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + total : total);
             }
         }
     };
@@ -588,9 +606,9 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     }
 }
 
-template <class F, int NU, bool FEW>
+template <class F, int NU, bool FEW, bool LONG = false>
 zhip_result launch_blocks(const Dispatch &d, const Q6Args &q, dim3 grid) {
-    auto kernel = matvec_kquant_mfma_stream_kernel<F, NU, FEW>;
+    auto kernel = matvec_kquant_mfma_stream_kernel<F, NU, FEW, LONG>;
     constexpr uint32_t bytes = lds_bytes<F>();
     static bool configured = false;
     if (!configured) {
@@ -609,13 +627,26 @@ zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) 
     // 32-bit byte offsets, a tile past the last row.
     const uint64_t used = ((uint64_t)((a.flags & FLAG_SILU_PAIR) ? a.half : 0u) + a.rows) * a.row_bytes;
     if (used + 64ull * a.row_bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "%s: weights of 4 GiB or more", F::name());
+    // The workgroups that walk the tiles: one a CU, or (rows of more than 4096 weights) one for
+    // every `parts` CUs, each of them `parts` workgroups.
+    const uint32_t parts = a.k > 4096u ? a.k / 2048u : 1u;
     const uint32_t cus = (uint32_t)d.dev->compute_units;
-    const uint32_t units = (a.rows + 7u) / 8u;
-    const uint32_t groups = units < cus ? units : cus;
+    if (cus < parts) return fail(d, ZHIP_E_GPU, "%s: %u compute units for %u parts of a row", F::name(), cus, parts);
+    const uint32_t units = (a.rows + 7u) / 8u, most = cus / parts;
+    const uint32_t groups = units < most ? units : most;
     const uint32_t rounds = (a.rows / 32u) / groups;
     const uint32_t tail = (a.rows - 32u * rounds * groups + 7u) / 8u;
-    Q6Args q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, 0x64646464u};
-    const dim3 grid(groups);
+    Q6Args q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, 0x64646464u, parts, nullptr};
+    const dim3 grid(groups * parts);
+    if constexpr (!F::FLAT) {
+        if (parts > 1u) {
+            if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", F::name());
+            if (zhip_result r = d.work->reserve(d, (uint64_t)parts * 8u * a.rows * sizeof(float))) return r;
+            q.partial = reinterpret_cast<float *>(d.work->data);
+            if (zhip_result r = a.m <= 4u ? launch_blocks<F, 2, true, true>(d, q, grid) : launch_blocks<F, 2, false, true>(d, q, grid)) return r;
+            return launch_matvec_parts_sum(d, F::name(), a, q.partial, parts);
+        }
+    }
     if constexpr (F::FLAT) {  // (the unit is the whole row: k = 1024 only)
         return a.m <= 4u ? launch_blocks<F, 1, true>(d, q, grid) : launch_blocks<F, 1, false>(d, q, grid);
     } else {
@@ -624,8 +655,11 @@ zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) 
     }
 }
 
+// k of 1024, 2048 or 4096, or 6144 .. 16384 in parts of 2048 (without the RMSNorm prologue and
+// the SILU_PAIR epilogue).
 bool stream_accepts(const MvArgs &a, uint32_t block_bytes) {
-    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u) && a.rows >= 1 && a.xr % 4u == 0 &&
+    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts && !(a.flags & (FLAG_NORM | FLAG_SILU_PAIR));
+    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u || parts) && a.rows >= 1 && a.xr % 4u == 0 &&
            (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == a.k / 256u * block_bytes;
 }
 

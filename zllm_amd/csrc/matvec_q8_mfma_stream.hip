@@ -1,4 +1,5 @@
-// matvec_q8_0, matrix-core variant for steps of up to eight tokens and k = 2048 or 4096: the
+// matvec_q8_0, matrix-core variant for steps of up to eight tokens and k = 2048 or 4096 (longer
+// rows in parts, below): the
 // weight stream is read once for all tokens of the step and nothing but partial sums crosses
 // LDS. Contract as the other variants (src/kernels/matvec_quant.wgsl.hbs with the decoder of
 // src/kernels/quant/q8_0_dot.wgsl:5-14): out[t][col0 + j] (+)= sum over 32-weight blocks of
@@ -31,6 +32,11 @@
 // in the middle of a cache line and a wave's 128 bytes of it lie across two; 151936 x 1024 ran
 // at 42 us, 3.9 TB/s against 6.6 TB/s at k = 4096. Such rows go to the kernel that moves a
 // tile's rows as one stretch of whole lines, matvec_q6k_mfma_stream.hip.)
+// Rows of 6144 .. 16384 weights (a multiple of 2048): k / 2048 workgroups share a walker's tiles,
+// each over 2048 columns (eight blocks a wave) and under its own per-token scales; they store
+// their sums per part and launch_matvec_parts_sum (matvec_mfma_resident.hip) adds them in the
+// order of their columns and applies the epilogue. Not with the RMSNorm prologue. 4096 x 14336
+// at four / eight tokens: 18.9 / 19.2 us (default variant 26.5 / 50.7).
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -60,6 +66,10 @@ struct StreamArgs {
     uint32_t split;      // or (split) half of one, eight rows, for each of the first 2 * left
     uint32_t bias;       // 0x64646464: the bytes of two f16 1024.0 exponents, as a kernel argument
                          // so that the byte shuffles stay one instruction each
+    // Rows of more than 4096 weights: `parts` workgroups share a tile, each over 2048 of its
+    // columns, and leave their sums in `partial` ([part][gate, up][token of 8][output]).
+    uint32_t parts;
+    float *partial;
 };
 
 // A barrier that waits for this wave's LDS traffic only: the weight loads of the tile ahead
@@ -123,8 +133,11 @@ constexpr uint32_t PART_BYTES = 2u * WAVES * 128u * 4u, SCALE_BYTES = 576u;  // 
 template <int NS> constexpr uint32_t lds_bytes() { return PART_BYTES + SCALE_BYTES + WAVES * DEPTH * slot_bytes<NS>(); }
 static_assert(lds_bytes<16>() <= 160u * 1024u, "the rings must fit the CU's LDS");
 
-template <int NS>
+// LONG (NS = 8): k = 2048 q.parts; workgroup i multiplies columns 2048 (i % parts) .. (part
+// `kpart`) of the tiles that walker i / parts takes, and launch_matvec_parts_sum adds the parts.
+template <int NS, bool LONG>
 __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamArgs q) {
+    static_assert(!LONG || NS == 8, "parts of a long row are 2048 columns");
     const MvArgs &a = q.a;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     float *lds_part = reinterpret_cast<float *>(lds);                  // [tile parity][wave][2 lane + token of the lane's two]
@@ -150,10 +163,11 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
     // tiles, the gate rows and then the up rows `half` further down: tile p of the run is weight
     // tile p % per of output tile p / per.
     const uint32_t per = (a.flags & FLAG_SILU_PAIR) ? 2u : 1u;
-    const bool extra = blockIdx.x < (q.split ? 2u * q.left : q.left);
+    const uint32_t kpart = LONG ? blockIdx.x % q.parts : 0u, walker = LONG ? blockIdx.x / q.parts : blockIdx.x, walkers = LONG ? gridDim.x / q.parts : gridDim.x;
+    const bool extra = walker < (q.split ? 2u * q.left : q.left);
     const uint32_t count = per * (q.rounds + (extra ? 1u : 0u));
-    const uint32_t last_row = 16u * (q.rounds * gridDim.x + (q.split ? blockIdx.x >> 1 : blockIdx.x)) + (q.split ? 8u * (blockIdx.x & 1u) : 0u);
-    auto out0 = [&](uint32_t p) { return p / per < q.rounds ? 16u * (blockIdx.x + (p / per) * gridDim.x) : last_row; };  // first output of tile p
+    const uint32_t last_row = 16u * (q.rounds * walkers + (q.split ? walker >> 1 : walker)) + (q.split ? 8u * (walker & 1u) : 0u);
+    auto out0 = [&](uint32_t p) { return p / per < q.rounds ? 16u * (walker + (p / per) * walkers) : last_row; };  // first output of tile p
     auto first_row = [&](uint32_t p) { return out0(p) + ((p % per) ? a.half : 0u); };
     auto rows_of = [&](uint32_t p) { return (q.split && p / per >= q.rounds) ? 8u : 16u; };
     // A half tile's loads. Weights: load i brings rows (64 / CHUNKS) i .. of the half's k range,
@@ -168,10 +182,10 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
 #pragma unroll
     for (int i = 0; i < WLOADS; i++) {
         const uint32_t row = ROWS_PER_LOAD * i + lrow;
-        woff[i] = row * a.row_bytes + PARTS * LINE * wave + 16u * (lpos ^ line_key(row));
+        woff[i] = row * a.row_bytes + 2048u * kpart + PARTS * LINE * wave + 16u * (lpos ^ line_key(row));
     }
     constexpr uint32_t SWORDS = HB / 2;  // words of scales a row and half
-    const uint32_t soff = (lane / SWORDS) * a.row_bytes + a.k + 2u * NS * wave + 4u * (lane % SWORDS);
+    const uint32_t soff = (lane / SWORDS) * a.row_bytes + a.k + 128u * kpart + 2u * NS * wave + 4u * (lane % SWORDS);
     auto load_half = [&](uint32_t u, uint32_t slot) __attribute__((always_inline)) {
         // (past the run's last tile the loads still run, so that the waits count the same loads
         // every step, but against an empty buffer: zeros land and nothing is fetched)
@@ -196,14 +210,15 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
     const uint32_t tok = l16 >> 1, sub = l16 & 1u, tsrc = tok < a.m ? tok : a.m - 1u;
     float4 raw[NS];
     {
-        const float *xt = a.x + (size_t)tsrc * a.xr + NS * 32u * wave + 8u * g + 4u * sub;
+        const float *xt = a.x + (size_t)tsrc * a.xr + 2048u * kpart + NS * 32u * wave + 8u * g + 4u * sub;
 #pragma unroll
         for (int s = 0; s < NS; s++) raw[s] = *reinterpret_cast<const float4 *>(xt + 32 * s);
     }
     // A step's prologue (src/kernels/matvec_quant.wgsl.hbs:73-89) on the same registers, in the
     // default variant's arithmetic: RMSNorm times the norm weights (the wave ranges' sums of
     // squares meet in LDS, added in the order of the ranges) and / or silu(x / act_div).
-    const bool norm = (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
+    // (the sum of squares of a long row is not any one workgroup's: such steps run other kernels)
+    const bool norm = !LONG && (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
     float4 gw[NS];
     if (norm) {
         const float *gt = a.norm_w + NS * 32u * wave + 8u * g + 4u * sub;
@@ -332,7 +347,9 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
 #pragma unroll
             for (uint32_t wv = 1; wv < WAVES; wv++) sum += src[wv * 128u];
             sum *= lds_inverse[tk];
-            if (per == 2u && !(p & 1u)) {
+            if (LONG) {
+                if (tk < a.m && row < rows_of(p)) store_apart(q.partial + ((size_t)(per * kpart + (p % per)) * 8u + tk) * a.rows + out0(p) + row, sum);
+            } else if (per == 2u && !(p & 1u)) {
                 held = sum;  // the gate tile's result, until the up tile's arrives
             } else {
                 const float v = per == 2u ? silu_f(held) * sum : sum;
@@ -377,13 +394,15 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
 // Whether this kernel can run the (already validated) arguments: whole tiles, k split into 4, 8
 // or 16 blocks a wave.
 bool matvec_q8_mfma_stream_accepts(const MvArgs &a) {
-    return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u) && (!(a.flags & FLAG_SILU_PAIR) || a.half % 16u == 0) && a.rows % 16u == 0 &&
+    // (rows of 6144 .. 16384 weights in parts of 2048, without the RMSNorm prologue)
+    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts && !(a.flags & FLAG_NORM);
+    return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u || parts) && (!(a.flags & FLAG_SILU_PAIR) || a.half % 16u == 0) && a.rows % 16u == 0 &&
            a.xr % 4u == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0;
 }
 
-template <int NS>
+template <int NS, bool LONG = false>
 static zhip_result launch_blocks(const Dispatch &d, const StreamArgs &q, dim3 grid) {
-    auto kernel = matvec_q8_mfma_stream_kernel<NS>;
+    auto kernel = matvec_q8_mfma_stream_kernel<NS, LONG>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes<NS>()) != hipSuccess) {
@@ -400,12 +419,25 @@ zhip_result launch_matvec_q8_mfma_stream(const Dispatch &d, const MvArgs &a, uin
     // 32-bit byte offsets, a tile past the last row.
     const uint64_t reach = ((uint64_t)((a.flags & FLAG_SILU_PAIR) ? a.half : 0u) + a.rows + 16u) * a.row_bytes;
     if (w_bytes >= 0xfffffff0ull || reach >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "matvec_q8_0: operands of 4 GiB or more");
+    // The workgroups that walk the tiles: one a CU, or (rows of more than 4096 weights) one for
+    // every `parts` CUs, each of them `parts` workgroups.
+    const uint32_t parts = a.k > 4096u ? a.k / 2048u : 1u;
     const uint32_t cus = (uint32_t)d.dev->compute_units, tiles = a.rows / 16u;
-    const uint32_t groups = tiles < cus ? (2u * tiles <= cus ? 2u * tiles : tiles) : cus;
+    if (cus < parts) return fail(d, ZHIP_E_GPU, "matvec_q8_0: %u compute units for %u parts of a row", cus, parts);
+    const uint32_t most = cus / parts;
+    const uint32_t groups = tiles < most ? (2u * tiles <= most ? 2u * tiles : tiles) : most;
     const uint32_t left = tiles % groups;
-    StreamArgs q{a, (uint32_t)w_bytes, tiles / groups, left, (tiles < groups || 2u * left <= groups) ? 1u : 0u, 0x64646464u};
+    StreamArgs q{a, (uint32_t)w_bytes, tiles / groups, left, (tiles < groups || 2u * left <= groups) ? 1u : 0u, 0x64646464u, parts, nullptr};
     if (tiles < groups) { q.rounds = 0; q.left = tiles; }
-    const dim3 grid(groups);
+    const dim3 grid(groups * parts);
+    if (parts > 1u) {
+        const uint64_t bytes = (uint64_t)parts * ((a.flags & FLAG_SILU_PAIR) ? 2u : 1u) * 8u * a.rows * sizeof(float);
+        if (!d.work) return fail(d, ZHIP_E_GPU, "matvec_q8_0: no workspace");
+        if (zhip_result r = d.work->reserve(d, bytes)) return r;
+        q.partial = reinterpret_cast<float *>(d.work->data);
+        if (zhip_result r = launch_blocks<8, true>(d, q, grid)) return r;
+        return launch_matvec_parts_sum(d, "matvec_q8_0", a, q.partial, parts);
+    }
     return a.k == 2048u ? launch_blocks<8>(d, q, grid) : launch_blocks<16>(d, q, grid);
 }
 
