@@ -577,14 +577,17 @@ def bench_formats(env):
 
 def bench_down(env):
     """The FFN-down multiply of the same model (K = 14336, N = 4096: rows longer than a step's
-    tokens can share workgroup memory for) at one, two and four tokens, Q4_K and Q8_0."""
-    synth, oracle, TensorType = env["synth"], env["oracle"], env["TensorType"]
+    tokens can share workgroup memory for) at one, two, four and eight tokens, Q4_K and Q8_0, on
+    the default variant and (`_mc`, four and eight tokens) on the matrix-core variant id, where
+    the workgroups that share a tile take 2048 columns each."""
+    synth, oracle, K, TensorType = env["synth"], env["oracle"], env["K"], env["TensorType"]
     n, k = 4096, 14336
+    mc = K.MatvecVariant(wg=512, lanes=64, rows=16)
     res = {}
     for name, ot in (("q4_k", oracle.Q4_K), ("q8_0", oracle.Q8_0)):
         raw = synth.random_blocks(synth.rng(0xD0), name, n, k)
-        for m in (1, 2, 4):
-            res[f"{name}_m{m}"] = _multi_token(env, TensorType[name], ot, raw, n, k, m, None)
+        for m, variant in ((1, None), (2, None), (4, None), (8, None), (4, mc), (8, mc)):
+            res[f"{name}_m{m}" + ("_mc" if variant else "")] = _multi_token(env, TensorType[name], ot, raw, n, k, m, variant)
     return res
 
 
