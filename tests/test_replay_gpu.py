@@ -293,3 +293,63 @@ def test_a_parameter_block_written_by_a_kernel_of_the_step_is_not_replayed():
     finally:
         for d in devs:
             d.deinit()
+
+
+def test_rows_in_parts_are_replayed_with_their_sums():
+    """Verify steps on the matrix-core variant id whose down multiplies run over rows of 6144
+    weights: three workgroups share a tile and a launch of its own adds their sums out of the
+    context's workspace, so a recorded dispatch is two graph nodes. Every replay bit for bit
+    what the eager device gives, and the arithmetic right."""
+    hidden, ff, layers, m = 2048, 6144, 4, 4
+    g = synth.rng(0x9A7)
+    weights = [(synth.q4_k_rows(g, 2 * ff, hidden), synth.q4_k_rows(g, hidden, ff), synth.activations(g, 1, hidden).reshape(-1)) for _ in range(layers)]
+    mc = K.MatvecVariant(wg=512, lanes=64, rows=16)
+    devs = [Device.open(0), Device.open(0, Device.NO_REPLAY)]
+    try:
+        steps = []
+        for d in devs:
+            c = Ctx(d)
+            x = c.output(m * hidden)
+            b = K.Builder(c.rec, c.set)
+            ls, cur = [], x
+            for gate_up, down, norm in weights:
+                wg, wd = c.gpu_weights(TensorType.q4_k, gate_up, hidden), c.gpu_weights(TensorType.q4_k, down, ff)
+                act, nxt = c.output(m * ff), c.output(m * hidden)
+                ls.append(b.add_matvec(Kernel.matvec_q4_k, mc, P.MatvecBf16(n=ff, k=hidden, col0=0, out_stride=ff, eps=EPS, norm=True, silu_pair=True, half=ff),
+                                       [cur, wg, act, c.upload(norm)], K.Grid.rows_y(K.div_ceil(ff, mc.group_rows()))))
+                ls.append(b.add_matvec(Kernel.matvec_q4_k, mc, P.MatvecBf16(n=hidden, k=ff, col0=0, out_stride=hidden),
+                                       [act, wd, nxt, wd], K.Grid.rows_y(K.div_ceil(hidden, mc.group_rows()))))
+                cur = nxt
+            b.finish()
+            c.flush()
+
+            def step(xs, c=c, x=x, ls=ls, out=cur):
+                c.rec.write_buffer(x.buffer, 0, np.ascontiguousarray(xs, dtype=np.float32).reshape(-1).view(np.uint8))
+                for l in ls:
+                    l.record(c.rec, K.Extent(rows=m))
+                return c.read(out)[: m * hidden].copy()
+
+            steps.append((c, step))
+        (rc, rstep), (ec, estep) = steps
+        seen = []
+        for i in range(5):
+            xs = synth.activations(synth.rng(0xA00 + i), m, hidden)
+            got, want = rstep(xs), estep(xs)
+            assert np.array_equal(got, want), f"step {i}"
+            seen.append(got)
+            unrelated_work(rc, 0xB00 + i)
+        # The first step allocated the workspace, so the second was the first sight of the sequence
+        # with that allocation; the third was captured and replayed, as were the two after it.
+        assert rc.host.replayed_submits() == 3 and ec.host.replayed_submits() == 0
+        assert not np.array_equal(seen[0], seen[1])
+        cur = synth.activations(synth.rng(0xA00), m, hidden).astype(np.float64)
+        for gate_up, down, norm in weights:
+            cur = cur / np.sqrt(np.mean(cur * cur, axis=1, keepdims=True) + EPS) * norm
+            both = cur @ oracle.Matrix(oracle.Q4_K, gate_up, 2 * ff, hidden).rows().astype(np.float64).T
+            with np.errstate(over="ignore"):  # (a very negative gate: exp overflows to inf and the quotient is 0)
+                act = both[:, :ff] / (1 + np.exp(-both[:, :ff])) * both[:, ff:]
+            cur = act @ oracle.Matrix(oracle.Q4_K, down, hidden, ff).rows().astype(np.float64).T
+        assert rel_err(seen[0].reshape(m, hidden), cur) <= 1e-4
+    finally:
+        for d in devs:
+            d.deinit()
