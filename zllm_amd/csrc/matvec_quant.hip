@@ -625,7 +625,7 @@ template <class P, int MT, bool PAIR, int STG>
 __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
     const MvArgs &a = q.a;
     extern __shared__ float4 lds4[];
-    __shared__ float red[8];
+    __shared__ float red[16];  // [token of those loaded at once][wave]
     constexpr int NSUM = P::NSUM, RUN = 64 / NSUM;
     const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6;
     const uint32_t tasks = q.tasks;
@@ -755,6 +755,7 @@ __global__ __launch_bounds__(256) void matvec_quant_kernel(KArgs q) {
             }
 #pragma unroll
             for (int t = 0; t < TG; t++) {
+                if (first + t >= MT) continue;  // (a last group of fewer tokens than are loaded at once)
                 float4 *dst = lds4 + (size_t)(first + t) * tok_stride4;
 #pragma unroll
                 for (int j = 0; j < 4; j++) {
@@ -1534,7 +1535,8 @@ static zhip_result run_quant(const Dispatch &d, const KArgs &q, uint32_t lds, ui
 }
 
 // Launches the multiply for validated arguments: one pass per group of up to
-// four tokens.
+// four tokens (a pass of three has kernels of its own: in the four-token ones a quarter of the
+// multiply-adds would go to a token that is not there).
 template <class P>
 static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
     KArgs q{};
@@ -1549,7 +1551,7 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
     if (tok_lds > max_lds) return fail(d, ZHIP_E_BAD_COMMAND, "%s: k = %u does not fit workgroup memory", P::name(), a.k);
     for (uint32_t t0 = 0; t0 < a.m;) {
         uint32_t left = a.m - t0;
-        uint32_t mt = left >= 3u ? 4u : left;
+        uint32_t mt = left >= 4u ? 4u : left;
         // A step of exactly two tokens over rows of 65 .. 256 tasks keeps both tokens' slices in
         // registers like the one-token step (Q4_K 4096 x 14336: 16.5 us tile by tile).
         if (a.m == 2u && !pair && q.tasks > 64u && q.tasks <= 256u) {
@@ -1578,12 +1580,13 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
             const uint32_t blocks = batches < cus ? batches : cus;
             zhip_result r;
             if (mt == 2u) r = pair ? run_long<P, 2, true>(d, q, blocks) : run_long<P, 2, false>(d, q, blocks);
+            else if (mt == 3u) r = pair ? run_long<P, 3, true>(d, q, blocks) : run_long<P, 3, false>(d, q, blocks);
             else r = pair ? run_long<P, 4, true>(d, q, blocks) : run_long<P, 4, false>(d, q, blocks);
             if (r != ZHIP_OK) return r;
             t0 += q.mt;
             continue;
         }
-        while (mt > 1u && mt * tok_lds > 80u * 1024u - 64u) mt >>= 1;
+        while (mt > 1u && mt * tok_lds > 80u * 1024u - 64u) mt = mt == 3u ? 2u : mt >> 1;
         q.t0 = t0;
         q.mt = left < mt ? left : mt;
         const uint32_t lds = (uint32_t)(mt * tok_lds);
@@ -1652,6 +1655,11 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
         else if (mt == 2u) {
             if (small && P::STAGE2 != 2) r = pair ? run_quant<P, 2, true, 2>(d, q, lds, blocks) : run_quant<P, 2, false, 2>(d, q, lds, blocks);
             else r = pair ? run_quant<P, 2, true, P::STAGE2>(d, q, lds, blocks) : run_quant<P, 2, false, P::STAGE2>(d, q, lds, blocks);
+        } else if (mt == 3u) {
+            // (three tokens: the four-token pass's choices, at most three loaded at once)
+            constexpr int STAGE3 = P::STAGE4 > 3 ? 3 : P::STAGE4;
+            if (small && P::ALL4 && STAGE3 != 3) r = pair ? run_quant<P, 3, true, 3>(d, q, lds, blocks) : run_quant<P, 3, false, 3>(d, q, lds, blocks);
+            else r = pair ? run_quant<P, 3, true, STAGE3>(d, q, lds, blocks) : run_quant<P, 3, false, STAGE3>(d, q, lds, blocks);
         } else {
             if (small && P::ALL4 && P::STAGE4 != 4) r = pair ? run_quant<P, 4, true, 4>(d, q, lds, blocks) : run_quant<P, 4, false, 4>(d, q, lds, blocks);
             else r = pair ? run_quant<P, 4, true, P::STAGE4>(d, q, lds, blocks) : run_quant<P, 4, false, P::STAGE4>(d, q, lds, blocks);
