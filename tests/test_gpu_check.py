@@ -518,7 +518,7 @@ def test_matvec_q8_0_mfma_variant(ctx, rows, n, k, col0, pad, accumulate):
 
 @pytest.mark.parametrize("norm", [False, True])
 @pytest.mark.parametrize("rows,n,k", [(8, 4128, 4096), (3, 64, 2048), (5, 3072, 1024), (2, 4104, 1024),
-                                      (6, 528, 8192)])  # rows in four parts (Q8_0; the others' pair steps over such rows run the default variant)
+                                      (6, 528, 8192), (3, 1304, 6144)])  # rows in four and in three parts (1304 outputs: whole rounds and a ragged tail)
 @pytest.mark.parametrize("t", [TensorType.q8_0, TensorType.q6_k, TensorType.q3_k])
 def test_matvec_q8_0_mfma_variant_silu_pair(ctx, t, rows, n, k, norm):
     """The matrix-core variant of matvec_q8_0, matvec_q6_k and matvec_q3_k on the fused gate / up step (SILU_PAIR: gate rows,

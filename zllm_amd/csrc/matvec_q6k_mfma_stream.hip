@@ -59,7 +59,7 @@
 // a walker's tiles, each over two units of every tile's rows and under its own per-token scales;
 // they store their sums per part and launch_matvec_parts_sum (matvec_mfma_resident.hip) adds
 // them in the order of their columns and applies the epilogue. Steps with the RMSNorm prologue
-// or the SILU_PAIR epilogue over such rows stay with the default variant. 4096 x 14336 at four /
+// over such rows stay with the default variant. 4096 x 14336 at four /
 // eight tokens: Q6_K 19.1 / 20.3 us (default variant 27.1 / 51.8), Q3_K 16.1 / 17.3 us (26.2 / 49.3).
 #include <hip/hip_runtime.h>
 
@@ -142,7 +142,7 @@ struct Q6Args {
     uint32_t bias;       // 0x64646464: the bytes of two f16 1024.0 exponents, as a kernel argument
                          // so that the byte shuffles stay one instruction each
     // Rows of more than 4096 weights: `parts` workgroups share a tile, each over 2048 of its
-    // columns, and leave their sums in `partial` ([part][token of 8][output]).
+    // columns, and leave their sums in `partial` ([part][gate, up][token of 8][output]).
     uint32_t parts;
     float *partial;
 };
@@ -529,6 +529,9 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     };
     // (a wave sums tokens i and 4 + i, whose partial sums lie side by side: no two lanes on a bank)
     float held = 0.f;  // the gate tile's result, until the up tile's arrives
+    // What waits in lds_kept for the burst of stores: an output tile's results, or (LONG, where
+    // the epilogue is the sums' launch's) every weight tile's sums, the gate tile's and the up tile's.
+    const uint32_t kper = LONG ? 1u : per;  // weight tiles an entry stands for
     auto sum_up = [&](uint32_t p) __attribute__((always_inline)) {
         const uint32_t po = p / per;
         if ((tid >> 8) != (po & 1u)) return;  // (the same half of the workgroup for an output tile's two weight tiles)
@@ -542,20 +545,21 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
 #pragma unroll
         for (uint32_t wv = 1; wv < WAVES; wv++) total += of_wave(wv);
         total *= lds_inverse[tk];
-        if (per == 2u && !(p & 1u)) held = total;
-        else lds_kept[256u * (po % KEPT) + 32u * tk + row] = per == 2u ? silu_f(held) * total : total;
+        if (!LONG && per == 2u && !(p & 1u)) held = total;
+        else lds_kept[256u * ((p / kper) % KEPT) + 32u * tk + row] = (!LONG && per == 2u) ? silu_f(held) * total : total;
     };
-    // The outputs of output tiles first .. first + n - 1, from LDS to memory in one burst: 128
-    // contiguous bytes a token and tile.
+    // Entries first .. first + n - 1 from LDS to memory in one burst: 128 contiguous bytes a
+    // token and tile.
     auto store_kept = [&](uint32_t first, uint32_t n) __attribute__((always_inline)) {
         lds_barrier();
-        for (uint32_t po = first + (tid >> 8); po < first + n; po += 2u) {
+        for (uint32_t e = first + (tid >> 8); e < first + n; e += 2u) {
+            const uint32_t po = LONG ? e / per : e, which = LONG ? e % per : 0u;
             const uint32_t row = tid & 31u, tk = (tid >> 5) & 7u;
             const uint32_t j = out_row(po) + row;
             if (tk < a.m && row < out_rows(po) && j < a.rows) {
                 float *o = a.out + (size_t)tk * a.out_stride + a.col0 + j;
-                const float total = lds_kept[256u * (po % KEPT) + (tid & 255u)];
-                if (LONG) store_apart(q.partial + ((size_t)kpart * 8u + tk) * a.rows + j, total);
+                const float total = lds_kept[256u * (e % KEPT) + (tid & 255u)];
+                if (LONG) store_apart(q.partial + ((size_t)(per * kpart + which) * 8u + tk) * a.rows + j, total);
                 else store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + total : total);
             }
         }
@@ -579,7 +583,7 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
             sum_up(p - 1u);
             // (the next tile's sums are kept only behind a later barrier, which no thread passes
             // before it has stored what it stores here)
-            if (p % (per * KEPT) == 0u) store_kept(p / per - KEPT, KEPT);
+            if (p % (kper * KEPT) == 0u) store_kept(p / kper - KEPT, KEPT);
         }
         multiply(unit, cur, next);
         cur = next;
@@ -601,7 +605,7 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     if (count > 0u) {
         lds_barrier();
         sum_up(count - 1u);
-        const uint32_t last = count / per - 1u;  // the run's last output tile
+        const uint32_t last = count / kper - 1u;  // the run's last entry
         store_kept(last - last % KEPT, last % KEPT + 1u);
     }
 }
@@ -641,7 +645,7 @@ zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) 
     if constexpr (!F::FLAT) {
         if (parts > 1u) {
             if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", F::name());
-            if (zhip_result r = d.work->reserve(d, (uint64_t)parts * 8u * a.rows * sizeof(float))) return r;
+            if (zhip_result r = d.work->reserve(d, (uint64_t)parts * ((a.flags & FLAG_SILU_PAIR) ? 2u : 1u) * 8u * a.rows * sizeof(float))) return r;
             q.partial = reinterpret_cast<float *>(d.work->data);
             if (zhip_result r = a.m <= 4u ? launch_blocks<F, 2, true, true>(d, q, grid) : launch_blocks<F, 2, false, true>(d, q, grid)) return r;
             return launch_matvec_parts_sum(d, F::name(), a, q.partial, parts);
@@ -655,10 +659,9 @@ zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) 
     }
 }
 
-// k of 1024, 2048 or 4096, or 6144 .. 16384 in parts of 2048 (without the RMSNorm prologue and
-// the SILU_PAIR epilogue).
+// k of 1024, 2048 or 4096, or 6144 .. 16384 in parts of 2048 (without the RMSNorm prologue).
 bool stream_accepts(const MvArgs &a, uint32_t block_bytes) {
-    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts && !(a.flags & (FLAG_NORM | FLAG_SILU_PAIR));
+    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts && !(a.flags & FLAG_NORM);
     return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u || parts) && a.rows >= 1 && a.xr % 4u == 0 &&
            (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == a.k / 256u * block_bytes;
 }
