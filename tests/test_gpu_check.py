@@ -413,11 +413,12 @@ MFMA_VARIANT = K.MatvecVariant(wg=512, lanes=64, rows=16)
     (True, 8, 4128, 4096),    # gate and up tiles of 258 output tiles
     (True, 3, 64, 2048),      # one block a wave
     (False, 2, 48, 2048),
-    # rows of more than 4096 weights: workgroups that share a tile, 2048 columns each (steps
-    # with the RMSNorm prologue run the default variant)
+    # rows of more than 4096 weights: workgroups that share a tile, 2048 columns each (with the
+    # RMSNorm prologue the tokens' scales come from a launch of their own)
     (False, 8, 1296, 14336),  # seven parts, 81 tiles over 36 walkers: two rounds and nine tiles in halves
     (True, 4, 528, 8192),     # four parts, gate and up, fewer tiles than walkers
     (False, 5, 4096, 6144),   # three parts, 256 tiles over 85 walkers: one whole tile left over
+    (False, 3, 528, 28672),   # fourteen parts
 ])
 @pytest.mark.parametrize("prologue", ["plain", "norm", "norm_act"])
 @pytest.mark.parametrize("t", [TensorType.q4_k, TensorType.q5_k])
@@ -482,6 +483,7 @@ def test_quant_matvec_mfma_variant(ctx, t, pair, rows, n, k, prologue):
     (8, 1296, 14336, 3, 7, True),    # seven parts, 81 tiles over 36 walkers
     (3, 4096, 6144, 0, 0, False),    # three parts, 256 tiles over 85 walkers
     (5, 48, 8192, 0, 0, False),      # four parts, fewer tiles than walkers
+    (2, 272, 20480, 0, 0, False),    # ten parts
 ])
 def test_matvec_q8_0_mfma_variant(ctx, rows, n, k, col0, pad, accumulate):
     """The matrix-core variant of matvec_q8_0 (the id of a wave per sixteen rows): every
@@ -551,7 +553,7 @@ def test_matvec_q8_0_mfma_variant_silu_pair(ctx, t, rows, n, k, norm):
 
 
 @pytest.mark.parametrize("prologue", ["norm", "norm_act"])
-@pytest.mark.parametrize("rows,n,k", [(6, 4112, 4096), (3, 96, 2048), (2, 200, 1024), (4, 4128, 1024)])
+@pytest.mark.parametrize("rows,n,k", [(6, 4112, 4096), (3, 96, 2048), (2, 200, 1024), (4, 4128, 1024), (5, 1040, 14336)])
 def test_matvec_q8_0_mfma_variant_prologues(ctx, rows, n, k, prologue):
     """The matrix-core variant of matvec_q8_0 on steps with the RMSNorm and silu(x / act_div)
     prologues (src/kernels/matvec_quant.wgsl.hbs:73-89), which the streaming kernel computes
@@ -598,7 +600,8 @@ def test_matvec_q8_0_mfma_variant_prologues(ctx, rows, n, k, prologue):
     (8, 1300, 14336, 3, 2, True, None),        # seven parts, 36 walkers: whole rounds, a tail, a ragged last unit
     (4, 4096, 6144, 0, 0, False, None),        # three parts, at most four tokens
     (5, 200, 8192, 0, 0, True, "act"),         # four parts, fewer rows than walkers
-    (2, 96, 14336, 0, 0, False, "norm"),       # with the RMSNorm prologue: the default variant's
+    (2, 96, 14336, 0, 0, False, "norm"),       # with the RMSNorm prologue: the tokens' scales from a launch of their own
+    (3, 300, 28672, 0, 0, True, "norm_act"),   # fourteen parts
 ])
 @pytest.mark.parametrize("t", [TensorType.q6_k, TensorType.q3_k])
 def test_matvec_q6_k_mfma_variant(ctx, t, rows, n, k, col0, pad, accumulate, prologue):

@@ -78,7 +78,12 @@ __device__ __forceinline__ void stage_token(const MvArgs &a, uint32_t token, flo
 // over 2048 of its columns, and leave their sums in `partial` ([part][gate, up][token of 8][output],
 // outputs a.rows apart); this launch adds a tile's parts in the order of their columns and applies
 // the SILU_PAIR / ACCUMULATE epilogue (matvec_mfma_resident.hip).
-constexpr uint32_t kMatvecMaxParts = 8;  // rows of up to 16384 weights
+constexpr uint32_t kMatvecMaxParts = 16;  // rows of up to 32768 weights
 zhip_result launch_matvec_parts_sum(const Dispatch &d, const char *name, const MvArgs &a, const float *partial, uint32_t parts);
+// A step over such rows with the RMSNorm prologue: no workgroup sees a whole row, so a launch of
+// its own leaves each token's 1 / sqrt(mean(x^2) + eps) in scales[token] beforehand (the sum of
+// squares as stage_token takes it). The workspace's first kPartsScalesBytes hold them.
+constexpr uint32_t kPartsScalesBytes = 64;
+zhip_result launch_matvec_parts_scales(const Dispatch &d, const char *name, const MvArgs &a, float *scales);
 
 }  // namespace zhip

@@ -28,15 +28,18 @@
 // epilogue and store. Each lane reads its row's header and nibbles back from
 // the copy (chunks XOR-permuted by row against bank conflicts) and multiplies.
 //
-// Rows of 6144 .. 16384 weights (a multiple of 2048; the FFN-down shapes) do not fit a
+// Rows of 6144 .. 32768 weights (a multiple of 2048; the FFN-down shapes) do not fit a
 // workgroup's registers: `parts` = k / 2048 workgroups share a walker's tiles, workgroup b taking
 // columns 2048 (b % parts) .. of the tiles of walker b / parts (one block a wave, the tile's
 // sixteen pieces of nine or eleven lines a whole row apart), each under its own per-token
 // scales, and store their sums per part; a second launch adds a tile's parts in the order of
-// their columns and applies the epilogue. Steps with the RMSNorm prologue, whose sum of squares
-// is no single workgroup's, stay with the default variant. Measured on Q4_K 4096 x 14336 at
-// one to eight tokens: 14.3 - 14.8 us (12.1 + the sums' launch) against 10.3 / 14.3 / 21.7 /
-// 21.6 / 40.9 us at one / two / three / four / eight tokens on the default variant.
+// their columns and applies the epilogue. With the RMSNorm prologue, whose sum of squares is no
+// single workgroup's, a small launch in front leaves every token's scale in memory
+// (launch_matvec_parts_scales). Measured on Q4_K 4096 x 14336 at one to eight tokens: 14.3 -
+// 14.8 us (12.1 + the sums' launch) against 10.3 / 14.3 / 19.2 / 21.6 / 40.9 us at one / two /
+// three / four / eight tokens on the default variant; 8192 x 28672 34.3 - 36.4 us against
+// 46.4 / 69.7 / 133.8 us at one / four / eight; 28672 x 8192 with the RMSNorm prologue 37.7 -
+// 38.6 us against 26.7 / 83.7 / 169.0.
 //
 // Contract as the other variants (src/kernels/matvec_quant.wgsl.hbs); a token's
 // result does not depend on how many tokens share the launch.
@@ -93,6 +96,7 @@ struct ResArgs {
     // columns, and leave their sums in `partial` ([part][gate, up][token of 8][output]).
     uint32_t parts;
     float *partial;
+    const float *scales;  // with the RMSNorm prologue: each token's 1 / sqrt(mean(x^2) + eps)
 };
 
 __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_buffer(const void *base, uint32_t bytes) {
@@ -241,28 +245,35 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_resident_kernel(Re
     // A step's prologue (src/kernels/matvec_quant.wgsl.hbs:73-89) on the same registers, in the
     // default variant's arithmetic: RMSNorm times the norm weights (the wave ranges' sums of
     // squares meet in LDS, added in the order of the ranges) and / or silu(x / act_div).
-    // (the sum of squares of a long row is not any one workgroup's: such steps run other kernels)
-    const bool norm = !LONG && (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
+    // (the sum of squares of a long row is not any one workgroup's: it comes ready in q.scales)
+    const bool norm = (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
     float4 gw[NB * 8];
+    float ready = 0.f;  // (asked for before the first weights, like the inputs)
     if (norm) {
-        const float *gt = a.norm_w + NB * 256u * wave + 8u * g + 4u * sub;
+        const float *gt = a.norm_w + 2048u * kpart + NB * 256u * wave + 8u * g + 4u * sub;
 #pragma unroll
         for (int s = 0; s < NB * 8; s++) gw[s] = *reinterpret_cast<const float4 *>(gt + 32 * s);
+        if (LONG) ready = q.scales[tsrc];
     }
     load_tile(0, 0);
     if (norm) {
-        float ss = 0.f;
+        float rs;
+        if (LONG) {
+            rs = ready;
+        } else {
+            float ss = 0.f;
 #pragma unroll
-        for (int s = 0; s < NB * 8; s++) ss += raw[s].x * raw[s].x + raw[s].y * raw[s].y + raw[s].z * raw[s].z + raw[s].w * raw[s].w;
-        ss += __shfl_xor(ss, 1, 64);
-        ss += __shfl_xor(ss, 16, 64);
-        ss += __shfl_xor(ss, 32, 64);
-        if (g == 0u && sub == 0u) lds_ss[8u * wave + tok] = ss;
-        lds_barrier();
-        float total = lds_ss[tok];
+            for (int s = 0; s < NB * 8; s++) ss += raw[s].x * raw[s].x + raw[s].y * raw[s].y + raw[s].z * raw[s].z + raw[s].w * raw[s].w;
+            ss += __shfl_xor(ss, 1, 64);
+            ss += __shfl_xor(ss, 16, 64);
+            ss += __shfl_xor(ss, 32, 64);
+            if (g == 0u && sub == 0u) lds_ss[8u * wave + tok] = ss;
+            lds_barrier();
+            float total = lds_ss[tok];
 #pragma unroll
-        for (uint32_t wv = 1; wv < WAVES; wv++) total += lds_ss[8u * wv + tok];
-        const float rs = 1.0f / sqrtf(total / (float)a.k + a.eps);
+            for (uint32_t wv = 1; wv < WAVES; wv++) total += lds_ss[8u * wv + tok];
+            rs = 1.0f / sqrtf(total / (float)a.k + a.eps);
+        }
 #pragma unroll
         for (int s = 0; s < NB * 8; s++) {
             raw[s].x = raw[s].x * rs * gw[s].x; raw[s].y = raw[s].y * rs * gw[s].y;
@@ -473,6 +484,28 @@ __global__ __launch_bounds__(256) void matvec_kquant_mfma_parts_sum_kernel(MvArg
 
 }  // namespace
 
+// A token's 1 / sqrt(mean(x^2) + eps), its sum of squares taken as stage_token takes it: vector i
+// by thread i % 256, the four waves' sums in order.
+__global__ __launch_bounds__(256) void matvec_parts_scales_kernel(MvArgs a, float *scales) {
+    __shared__ float red[4];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, k4 = a.k / 4u;
+    const float4 *xrow = reinterpret_cast<const float4 *>(a.x + (size_t)blockIdx.x * a.xr);
+    float ss = 0.f;
+    for (uint32_t i = tid; i < k4; i += 256u) {
+        const float4 v = xrow[i];
+        ss += v.x * v.x + v.y * v.y + v.z * v.z + v.w * v.w;
+    }
+    ss = wave_sum(ss);
+    if (lane == 0u) red[wave] = ss;
+    __syncthreads();
+    if (tid == 0u) scales[blockIdx.x] = 1.0f / sqrtf(((red[0] + red[1]) + (red[2] + red[3])) / (float)a.k + a.eps);
+}
+
+zhip_result launch_matvec_parts_scales(const Dispatch &d, const char *name, const MvArgs &a, float *scales) {
+    hipLaunchKernelGGL(matvec_parts_scales_kernel, dim3(a.m), dim3(256), 0, d.stream, a, scales);
+    return check_launch(d, name);
+}
+
 zhip_result launch_matvec_parts_sum(const Dispatch &d, const char *name, const MvArgs &a, const float *partial, uint32_t parts) {
     const dim3 sums((a.rows * a.m + 255u) / 256u);
     if (a.flags & FLAG_SILU_PAIR) hipLaunchKernelGGL(matvec_kquant_mfma_parts_sum_kernel<true>, sums, dim3(256), 0, d.stream, a, partial, parts);
@@ -481,11 +514,10 @@ zhip_result launch_matvec_parts_sum(const Dispatch &d, const char *name, const M
 }
 
 // Whether this kernel can run the (already validated) arguments: whole tiles, k split into
-// one or two blocks a wave, or rows of 6144 .. 16384 weights in parts of 2048 (without the
-// RMSNorm prologue).
+// one or two blocks a wave, or rows of 6144 .. 32768 weights in parts of 2048.
 bool matvec_q4k_mfma_resident_accepts(const MvArgs &a) {
     const bool pair = a.flags & FLAG_SILU_PAIR;
-    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts && !(a.flags & FLAG_NORM);
+    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts;
     return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u || parts) && a.rows % 16u == 0 && (!pair || a.half % 16u == 0);
 }
 
@@ -504,13 +536,17 @@ static zhip_result launch_resident(const Dispatch &d, const MvArgs &a, uint64_t 
     const uint32_t groups = tiles < most ? (2u * tiles <= most ? 2u * tiles : tiles) : most;
     const bool halves = tiles < groups;  // every workgroup takes eight outputs of one tile
     const uint32_t left = halves ? tiles : tiles % groups;
-    ResArgs q{a, (uint32_t)w_bytes, mask, bias_bits, halves ? 0u : tiles / groups, left, (halves || 2u * left <= groups) ? 1u : 0u, parts, nullptr};
+    ResArgs q{a, (uint32_t)w_bytes, mask, bias_bits, halves ? 0u : tiles / groups, left, (halves || 2u * left <= groups) ? 1u : 0u, parts, nullptr, nullptr};
     const dim3 grid(groups * parts);
     if (parts > 1u) {
         const uint64_t bytes = (uint64_t)parts * (pair ? 2u : 1u) * 8u * a.rows * sizeof(float);
         if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", F::name());
-        if (zhip_result r = d.work->reserve(d, bytes)) return r;
-        q.partial = reinterpret_cast<float *>(d.work->data);
+        if (zhip_result r = d.work->reserve(d, kPartsScalesBytes + bytes)) return r;
+        q.partial = reinterpret_cast<float *>(d.work->data + kPartsScalesBytes);
+        if (a.flags & FLAG_NORM) {
+            q.scales = reinterpret_cast<const float *>(d.work->data);
+            if (zhip_result r = launch_matvec_parts_scales(d, F::name(), a, reinterpret_cast<float *>(d.work->data))) return r;
+        }
         if (pair) hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, true, 1, true>), grid, dim3(THREADS), 0, d.stream, q);
         else hipLaunchKernelGGL((matvec_kquant_mfma_resident_kernel<F, false, 1, true>), grid, dim3(THREADS), 0, d.stream, q);
         if (zhip_result r = check_launch(d, F::name())) return r;

@@ -54,13 +54,14 @@
 // 33.9 / 32.9 / 35.6 us (41.7 us with the rows read line by line, row by row, by the kernel that
 // takes k = 2048 and 4096; the default variant 33.6 / 44.1 / 79.7 us).
 //
-// Rows of 6144 .. 16384 weights (a multiple of 2048; the FFN-down shapes), Q6_K and Q3_K: the
+// Rows of 6144 .. 32768 weights (a multiple of 2048; the FFN-down shapes), Q6_K and Q3_K: the
 // operands of so many positions do not fit a workgroup's registers, so k / 2048 workgroups share
 // a walker's tiles, each over two units of every tile's rows and under its own per-token scales;
 // they store their sums per part and launch_matvec_parts_sum (matvec_mfma_resident.hip) adds
-// them in the order of their columns and applies the epilogue. Steps with the RMSNorm prologue
-// over such rows stay with the default variant. 4096 x 14336 at four /
-// eight tokens: Q6_K 19.1 / 20.3 us (default variant 27.1 / 51.8), Q3_K 16.1 / 17.3 us (26.2 / 49.3).
+// them in the order of their columns and applies the epilogue; with the RMSNorm prologue the
+// tokens' scales come ready from launch_matvec_parts_scales. 4096 x 14336 at four / eight
+// tokens: Q6_K 19.1 / 20.3 us (default variant 27.1 / 51.8), Q3_K 16.1 / 17.3 us (26.2 / 49.3);
+// Q6_K 8192 x 8192 with the RMSNorm prologue 23.9 / 25.0 us (36.1 / 78.5).
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -145,6 +146,7 @@ struct Q6Args {
     // columns, and leave their sums in `partial` ([part][gate, up][token of 8][output]).
     uint32_t parts;
     float *partial;
+    const float *scales;  // with the RMSNorm prologue: each token's 1 / sqrt(mean(x^2) + eps)
 };
 
 __device__ __forceinline__ void lds_barrier() {
@@ -267,8 +269,8 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     // inputs' loads and this arithmetic (loads complete in order within a wave), the next three
     // once the inputs are in: all four at once would hold up the other waves' inputs in the
     // CU's one address pipeline (+0.7 us).
-    // (the sum of squares of a long row is not any one workgroup's: such steps run other kernels)
-    const bool norm = !LONG && (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
+    // (the sum of squares of a long row is not any one workgroup's: it comes ready in q.scales)
+    const bool norm = (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
     float *lds_max = lds_inverse + 16 + 256, *lds_ss = lds_max + 64;  // [wave][token], behind the spare KB
     // Operand row r of the matrix instruction is piece r / 8 of token 4 (r / 4 % 2) + r % 4 (rows
     // 16 .. 31 are zeros), so that a lane's results are its weight row times both pieces of four
@@ -294,27 +296,34 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
 #pragma unroll
             for (int i = 0; i < 4; i++)
                 r1[4 * u + i] = __builtin_bit_cast(float4, __builtin_amdgcn_raw_buffer_load_b128(xbuf, t1 < a.m ? x1 + 4u * (1024u * u + 32u * i) : 0xfffffff0u, 0, 0));
+        float ready = 0.f;  // (asked for before the first weights, like the inputs)
         if (norm) {
-            const float *gp = a.norm_w + 128u * wave + 4u * l8;
+            const float *gp = a.norm_w + 1024u * NU * kpart + 128u * wave + 4u * l8;
 #pragma unroll
             for (int u = 0; u < NU; u++)
 #pragma unroll
                 for (int i = 0; i < 4; i++) g1[4 * u + i] = *reinterpret_cast<const float4 *>(gp + 1024 * u + 32 * i);
+            if (LONG) ready = q.scales[t1c];
         }
         issue(0, 0);
         if (norm) {
-            float ss = 0.f;
+            float rs;
+            if (LONG) {
+                rs = ready;
+            } else {
+                float ss = 0.f;
 #pragma unroll
-            for (int i = 0; i < 4 * NU; i++) ss += r1[i].x * r1[i].x + r1[i].y * r1[i].y + r1[i].z * r1[i].z + r1[i].w * r1[i].w;
-            ss += __shfl_xor(ss, 1, 64);
-            ss += __shfl_xor(ss, 2, 64);
-            ss += __shfl_xor(ss, 4, 64);
-            if (l8 == 0u) lds_ss[8u * wave + t1] = ss;
-            lds_barrier();
-            float total = lds_ss[t1];
+                for (int i = 0; i < 4 * NU; i++) ss += r1[i].x * r1[i].x + r1[i].y * r1[i].y + r1[i].z * r1[i].z + r1[i].w * r1[i].w;
+                ss += __shfl_xor(ss, 1, 64);
+                ss += __shfl_xor(ss, 2, 64);
+                ss += __shfl_xor(ss, 4, 64);
+                if (l8 == 0u) lds_ss[8u * wave + t1] = ss;
+                lds_barrier();
+                float total = lds_ss[t1];
 #pragma unroll
-            for (uint32_t wv = 1; wv < WAVES; wv++) total += lds_ss[8u * wv + t1];
-            const float rs = 1.0f / sqrtf(total / (float)a.k + a.eps);
+                for (uint32_t wv = 1; wv < WAVES; wv++) total += lds_ss[8u * wv + t1];
+                rs = 1.0f / sqrtf(total / (float)a.k + a.eps);
+            }
 #pragma unroll
             for (int i = 0; i < 4 * NU; i++) {
                 r1[i].x = r1[i].x * rs * g1[i].x; r1[i].y = r1[i].y * rs * g1[i].y;
@@ -640,13 +649,17 @@ zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) 
     const uint32_t groups = units < most ? units : most;
     const uint32_t rounds = (a.rows / 32u) / groups;
     const uint32_t tail = (a.rows - 32u * rounds * groups + 7u) / 8u;
-    Q6Args q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, 0x64646464u, parts, nullptr};
+    Q6Args q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, 0x64646464u, parts, nullptr, nullptr};
     const dim3 grid(groups * parts);
     if constexpr (!F::FLAT) {
         if (parts > 1u) {
             if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", F::name());
-            if (zhip_result r = d.work->reserve(d, (uint64_t)parts * ((a.flags & FLAG_SILU_PAIR) ? 2u : 1u) * 8u * a.rows * sizeof(float))) return r;
-            q.partial = reinterpret_cast<float *>(d.work->data);
+            if (zhip_result r = d.work->reserve(d, kPartsScalesBytes + (uint64_t)parts * ((a.flags & FLAG_SILU_PAIR) ? 2u : 1u) * 8u * a.rows * sizeof(float))) return r;
+            q.partial = reinterpret_cast<float *>(d.work->data + kPartsScalesBytes);
+            if (a.flags & FLAG_NORM) {
+                q.scales = reinterpret_cast<const float *>(d.work->data);
+                if (zhip_result r = launch_matvec_parts_scales(d, F::name(), a, reinterpret_cast<float *>(d.work->data))) return r;
+            }
             if (zhip_result r = a.m <= 4u ? launch_blocks<F, 2, true, true>(d, q, grid) : launch_blocks<F, 2, false, true>(d, q, grid)) return r;
             return launch_matvec_parts_sum(d, F::name(), a, q.partial, parts);
         }
@@ -659,9 +672,9 @@ zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) 
     }
 }
 
-// k of 1024, 2048 or 4096, or 6144 .. 16384 in parts of 2048 (without the RMSNorm prologue).
+// k of 1024, 2048 or 4096, or 6144 .. 32768 in parts of 2048.
 bool stream_accepts(const MvArgs &a, uint32_t block_bytes) {
-    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts && !(a.flags & FLAG_NORM);
+    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts;
     return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u || parts) && a.rows >= 1 && a.xr % 4u == 0 &&
            (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == a.k / 256u * block_bytes;
 }

@@ -32,11 +32,12 @@
 // in the middle of a cache line and a wave's 128 bytes of it lie across two; 151936 x 1024 ran
 // at 42 us, 3.9 TB/s against 6.6 TB/s at k = 4096. Such rows go to the kernel that moves a
 // tile's rows as one stretch of whole lines, matvec_q6k_mfma_stream.hip.)
-// Rows of 6144 .. 16384 weights (a multiple of 2048): k / 2048 workgroups share a walker's tiles,
+// Rows of 6144 .. 32768 weights (a multiple of 2048): k / 2048 workgroups share a walker's tiles,
 // each over 2048 columns (eight blocks a wave) and under its own per-token scales; they store
 // their sums per part and launch_matvec_parts_sum (matvec_mfma_resident.hip) adds them in the
-// order of their columns and applies the epilogue. Not with the RMSNorm prologue. 4096 x 14336
-// at four / eight tokens: 18.9 / 19.2 us (default variant 26.5 / 50.7).
+// order of their columns and applies the epilogue; with the RMSNorm prologue the tokens' scales
+// come ready from launch_matvec_parts_scales. 4096 x 14336 at four / eight tokens: 18.9 /
+// 19.2 us (default variant 26.5 / 50.7).
 #include <hip/hip_runtime.h>
 
 #include <type_traits>
@@ -70,6 +71,7 @@ struct StreamArgs {
     // columns, and leave their sums in `partial` ([part][gate, up][token of 8][output]).
     uint32_t parts;
     float *partial;
+    const float *scales;  // with the RMSNorm prologue: each token's 1 / sqrt(mean(x^2) + eps)
 };
 
 // A barrier that waits for this wave's LDS traffic only: the weight loads of the tile ahead
@@ -217,32 +219,39 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
     // A step's prologue (src/kernels/matvec_quant.wgsl.hbs:73-89) on the same registers, in the
     // default variant's arithmetic: RMSNorm times the norm weights (the wave ranges' sums of
     // squares meet in LDS, added in the order of the ranges) and / or silu(x / act_div).
-    // (the sum of squares of a long row is not any one workgroup's: such steps run other kernels)
-    const bool norm = !LONG && (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
+    // (the sum of squares of a long row is not any one workgroup's: it comes ready in q.scales)
+    const bool norm = (a.flags & FLAG_NORM) != 0, act = a.act_div > 0.f;
     float4 gw[NS];
+    float ready = 0.f;  // (asked for before the first weights, like the inputs)
     if (norm) {
-        const float *gt = a.norm_w + NS * 32u * wave + 8u * g + 4u * sub;
+        const float *gt = a.norm_w + 2048u * kpart + NS * 32u * wave + 8u * g + 4u * sub;
 #pragma unroll
         for (int s = 0; s < NS; s++) gw[s] = *reinterpret_cast<const float4 *>(gt + 32 * s);
+        if (LONG) ready = q.scales[tsrc];
     }
     // (One half tile of weights behind them for now: with more, the requests of the workgroups
     // that start first fill the memory system's queues and the inputs of the others arrive
     // after them, 4.5 us into the kernel instead of 1.7.)
     load_half(0, 0);
     if (norm) {
-        float ss = 0.f;
+        float rs;
+        if (LONG) {
+            rs = ready;
+        } else {
+            float ss = 0.f;
 #pragma unroll
-        for (int s = 0; s < NS; s++) ss += raw[s].x * raw[s].x + raw[s].y * raw[s].y + raw[s].z * raw[s].z + raw[s].w * raw[s].w;
-        ss += __shfl_xor(ss, 1, 64);
-        ss += __shfl_xor(ss, 16, 64);
-        ss += __shfl_xor(ss, 32, 64);
-        float *lds_ss = lds_inverse + 8;  // [wave][token]: the range's sum of squares
-        if (g == 0u && sub == 0u) lds_ss[8u * wave + tok] = ss;
-        lds_barrier();
-        float total = lds_ss[tok];
+            for (int s = 0; s < NS; s++) ss += raw[s].x * raw[s].x + raw[s].y * raw[s].y + raw[s].z * raw[s].z + raw[s].w * raw[s].w;
+            ss += __shfl_xor(ss, 1, 64);
+            ss += __shfl_xor(ss, 16, 64);
+            ss += __shfl_xor(ss, 32, 64);
+            float *lds_ss = lds_inverse + 8;  // [wave][token]: the range's sum of squares
+            if (g == 0u && sub == 0u) lds_ss[8u * wave + tok] = ss;
+            lds_barrier();
+            float total = lds_ss[tok];
 #pragma unroll
-        for (uint32_t wv = 1; wv < WAVES; wv++) total += lds_ss[8u * wv + tok];
-        const float rs = 1.0f / sqrtf(total / (float)a.k + a.eps);
+            for (uint32_t wv = 1; wv < WAVES; wv++) total += lds_ss[8u * wv + tok];
+            rs = 1.0f / sqrtf(total / (float)a.k + a.eps);
+        }
 #pragma unroll
         for (int s = 0; s < NS; s++) {
             raw[s].x = raw[s].x * rs * gw[s].x; raw[s].y = raw[s].y * rs * gw[s].y;
@@ -394,8 +403,8 @@ __global__ __launch_bounds__(THREADS) void matvec_q8_mfma_stream_kernel(StreamAr
 // Whether this kernel can run the (already validated) arguments: whole tiles, k split into 4, 8
 // or 16 blocks a wave.
 bool matvec_q8_mfma_stream_accepts(const MvArgs &a) {
-    // (rows of 6144 .. 16384 weights in parts of 2048, without the RMSNorm prologue)
-    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts && !(a.flags & FLAG_NORM);
+    // (rows of 6144 .. 32768 weights in parts of 2048)
+    const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts;
     return a.m >= 1 && a.m <= 8 && (a.k == 2048u || a.k == 4096u || parts) && (!(a.flags & FLAG_SILU_PAIR) || a.half % 16u == 0) && a.rows % 16u == 0 &&
            a.xr % 4u == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0;
 }
@@ -427,14 +436,18 @@ zhip_result launch_matvec_q8_mfma_stream(const Dispatch &d, const MvArgs &a, uin
     const uint32_t most = cus / parts;
     const uint32_t groups = tiles < most ? (2u * tiles <= most ? 2u * tiles : tiles) : most;
     const uint32_t left = tiles % groups;
-    StreamArgs q{a, (uint32_t)w_bytes, tiles / groups, left, (tiles < groups || 2u * left <= groups) ? 1u : 0u, 0x64646464u, parts, nullptr};
+    StreamArgs q{a, (uint32_t)w_bytes, tiles / groups, left, (tiles < groups || 2u * left <= groups) ? 1u : 0u, 0x64646464u, parts, nullptr, nullptr};
     if (tiles < groups) { q.rounds = 0; q.left = tiles; }
     const dim3 grid(groups * parts);
     if (parts > 1u) {
         const uint64_t bytes = (uint64_t)parts * ((a.flags & FLAG_SILU_PAIR) ? 2u : 1u) * 8u * a.rows * sizeof(float);
         if (!d.work) return fail(d, ZHIP_E_GPU, "matvec_q8_0: no workspace");
-        if (zhip_result r = d.work->reserve(d, bytes)) return r;
-        q.partial = reinterpret_cast<float *>(d.work->data);
+        if (zhip_result r = d.work->reserve(d, kPartsScalesBytes + bytes)) return r;
+        q.partial = reinterpret_cast<float *>(d.work->data + kPartsScalesBytes);
+        if (a.flags & FLAG_NORM) {
+            q.scales = reinterpret_cast<const float *>(d.work->data);
+            if (zhip_result r = launch_matvec_parts_scales(d, "matvec_q8_0", a, reinterpret_cast<float *>(d.work->data))) return r;
+        }
         if (zhip_result r = launch_blocks<8, true>(d, q, grid)) return r;
         return launch_matvec_parts_sum(d, "matvec_q8_0", a, q.partial, parts);
     }
