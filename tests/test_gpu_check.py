@@ -338,7 +338,11 @@ def test_quant_matvec_act_prologue(ctx, t, k):
     (TensorType.q8_0, 10240, True, 2, 19),
     (TensorType.q5_k, 16384, False, 4, 9),    # 256 tasks: four whole slices, a batch of rows with units past the end
     (TensorType.q3_k, 4352, False, 1, 3),     # 68 tasks: a second slice of four lanes, three rows
-    (TensorType.q6_k, 16640, False, 2, 21),   # 260 tasks: past the sliced kernel's four slices
+    (TensorType.q6_k, 16640, False, 2, 21),   # 260 tasks: past the sliced kernel's four slices, short of its five
+    (TensorType.q4_k, 25600, False, 2, 37),   # 400 tasks: seven slices, the last a quarter full
+    (TensorType.q8_0, 32768, False, 3, 20),   # eight slices, the longest row
+    (TensorType.q5_k, 20480, False, 2, 11),   # five slices
+    (TensorType.q3_k, 24576, False, 2, 9),    # six slices
     (TensorType.q4_k, 11008, False, 2, 30),   # two tokens over three slices: a workgroup of six waves
     (TensorType.q8_0, 8192, False, 2, 70),    # two tokens over two slices
     # Steps of exactly two tokens over short rows keep both tokens' inputs in registers:

@@ -1295,7 +1295,7 @@ static zhip_result run_long(const Dispatch &d, const KArgs &q, uint32_t blocks) 
     return check_launch(d, P::name());
 }
 
-// One-token steps over rows of 65 .. 256 tasks (k above 4096, up to 16384: the FFN-down shapes).
+// One-token steps over rows of 65 .. 512 tasks (k above 4096, up to 32768: the FFN-down shapes).
 // matvec_quant_kernel walks such a row with one wave, a lane taking a task of every 64-task
 // slice in turn with its inputs read from LDS each time. Here a slice is a wave's for the whole
 // launch, so the lane's 64 inputs stay in registers as in the short-row case: the waves of a
@@ -1311,14 +1311,15 @@ static zhip_result run_long(const Dispatch &d, const KArgs &q, uint32_t blocks) 
 // a task, loads zeros). What the outputs hold, for a step that accumulates, is asked for before
 // the round's loads: loads complete in order within a wave, so behind them it would wait for
 // rows of the next round.
-template <class P, int MT, bool PAIR, int R, int NW>
+// K4: the most vectors of four inputs a token has (4096: k <= 16384; 8192: k <= 32768).
+template <class P, int MT, bool PAIR, int R, int NW, int K4 = 4096>
 __global__ __launch_bounds__(64 * NW) void matvec_quant_slices_kernel(KArgs q) {
     const MvArgs &a = q.a;
     extern __shared__ float4 lds4[];  // the tokens in task order, padded per task; then the partial sums [parity][group][unit of the round][slice][row][token][lane]
     __shared__ float red[4 * MT];
     constexpr int NSUM = P::NSUM, RUN = 64 / NSUM, kRows = PAIR ? 2 : 1;
     constexpr uint32_t THREADS = 64u * NW;
-    constexpr int XV = (4096 + THREADS - 1) / THREADS;  // vectors of a token a thread stages (k <= 16384)
+    constexpr int XV = (K4 + THREADS - 1) / THREADS;  // vectors of a token a thread stages
     static_assert(R % 2 == 0, "the buffers alternate by name");
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(tid >> 6));
@@ -1497,10 +1498,10 @@ __global__ __launch_bounds__(64 * NW) void matvec_quant_slices_kernel(KArgs q) {
     }
 }
 
-template <class P, int MT, bool PAIR, int R, int NW>
+template <class P, int MT, bool PAIR, int R, int NW, int K4 = 4096>
 static zhip_result run_slices(const Dispatch &d, const KArgs &q, uint32_t lds, uint32_t blocks) {
-    if (!lds_opt_in<matvec_quant_slices_kernel<P, MT, PAIR, R, NW>, 160 * 1024 - 64>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", P::name(), lds);
-    hipLaunchKernelGGL((matvec_quant_slices_kernel<P, MT, PAIR, R, NW>), dim3(blocks), dim3(64 * NW), lds, d.stream, q);
+    if (!lds_opt_in<matvec_quant_slices_kernel<P, MT, PAIR, R, NW, K4>, 160 * 1024 - 64>()) return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", P::name(), lds);
+    hipLaunchKernelGGL((matvec_quant_slices_kernel<P, MT, PAIR, R, NW, K4>), dim3(blocks), dim3(64 * NW), lds, d.stream, q);
     return check_launch(d, P::name());
 }
 
@@ -1614,6 +1615,27 @@ static zhip_result launch_quant(const Dispatch &d, const MvArgs &a) {
             } else {
                 if (pair) r = two ? run_slices<P, 1, true, 2, 8>(d, q, lds1, blocks) : run_slices<P, 1, true, 4, 8>(d, q, lds1, blocks);
                 else r = two ? run_slices<P, 1, false, 2, 8>(d, q, lds1, blocks) : run_slices<P, 1, false, 4, 8>(d, q, lds1, blocks);
+            }
+            if (r != ZHIP_OK) return r;
+            t0 += q.mt;
+            continue;
+        }
+        // One token over rows of 288 .. 512 tasks (k up to 32768: the FFN-down multiplies of the
+        // widest models): five to eight slices, a wave each, one group a workgroup and CU, two
+        // units a round. Q4_K 8192 x 28672: 29.1 us against 46.4 through the general kernel;
+        // 5120 x 25600 22.2 against 32.3; 5120 x 20480 21.3 against 24.9 (Q6_K 25.4 against
+        // 31.1). Rows of 257 .. 287 tasks, whose fifth wave would be all but idle, stay with the
+        // general kernel (Q4_K 5120 x 17408: 19.5 us there, 20.5 here).
+        if (a.m == 1u && !pair && q.tasks >= 288u && q.tasks <= 512u) {
+            const uint32_t slices = (q.tasks + 63u) / 64u, cus = (uint32_t)d.dev->compute_units;
+            const uint32_t want = (a.rows + 1u) / 2u, blocks = want < cus ? want : cus;
+            const uint32_t lds1 = q.tasks * kTaskStride * 4u + 2u * slices * 2u * 256u;
+            zhip_result r;
+            switch (slices) {
+            case 5: r = run_slices<P, 1, false, 2, 5, 8192>(d, q, lds1, blocks); break;
+            case 6: r = run_slices<P, 1, false, 2, 6, 8192>(d, q, lds1, blocks); break;
+            case 7: r = run_slices<P, 1, false, 2, 7, 8192>(d, q, lds1, blocks); break;
+            default: r = run_slices<P, 1, false, 2, 8, 8192>(d, q, lds1, blocks); break;
             }
             if (r != ZHIP_OK) return r;
             t0 += q.mt;
