@@ -10,9 +10,9 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libzllm_hip.so")
 
-SOURCES = ["host.cpp", "matvec.hip", "matvec_quant.hip", "matvec_mfma_resident.hip", "matvec_q8_mfma_stream.hip", "matvec_bf16_mfma_stream.hip", "matvec_q6k_mfma_stream.hip", "matmul_f32.hip", "matmul_mfma.hip", "matmul_mfma_wide.hip", "matmul_q8_bf16.hip", "matmul_q8_bf16_wide.hip", "matmul_stream.hip", "matmul_int8.hip", "matmul_q8_i8.hip",
+SOURCES = ["host.cpp", "matvec.hip", "matvec_quant.hip", "matvec_quant_q8.hip", "matvec_quant_q3.hip", "matvec_quant_q4.hip", "matvec_quant_q5.hip", "matvec_quant_q6.hip", "matvec_mfma_resident.hip", "matvec_q8_mfma_stream.hip", "matvec_bf16_mfma_stream.hip", "matvec_q6k_mfma_stream.hip", "matmul_f32.hip", "matmul_mfma.hip", "matmul_mfma_wide.hip", "matmul_q8_bf16.hip", "matmul_q8_bf16_wide.hip", "matmul_stream.hip", "matmul_int8.hip", "matmul_q8_i8.hip",
            "quantize_q8.hip", "elementwise.hip", "no_alloc.hip"]
-HEADERS = ["common.h", "decode.h", "matvec_common.h", "matmul_q8_tiles.h", os.path.join("..", "..", "include", "zllm_hip.h")]
+HEADERS = ["common.h", "decode.h", "matvec_common.h", "matvec_quant.h", "matmul_q8_tiles.h", os.path.join("..", "..", "include", "zllm_hip.h")]
 
 # -packed-fp32-ops off: some packed-FP32 forms have given wrong results on the
 # target machines; ordinary float code must not be turned into them.

@@ -101,7 +101,7 @@ struct DecQ4_K {
     static constexpr int RUNS = 2;
     static constexpr int E = 32;
     static constexpr uint32_t BLOCK = 256;
-    static constexpr int CHUNK = 4;  // has its own multiply (matvec_quant.hip)
+    static constexpr int CHUNK = 4;  // has its own multiply (matvec_quant.h)
     static const char *name() { return "matvec_q4_k"; }
     static uint32_t row_bytes(uint32_t k) { return k / 256u * 144u; }
     __device__ static uint32_t xoff(uint32_t task, int h) {

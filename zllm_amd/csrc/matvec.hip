@@ -344,7 +344,7 @@ constexpr uint64_t kBf16StreamBytes = 16ull << 20;
 static bool bf16_stream_pays(const Dispatch &d, const MvArgs &a) {
     return d.dev->wide_decode && (uint64_t)a.rows * a.row_bytes >= kBf16StreamBytes;
 }
-// The tuned multiply (matvec_quant.hip): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
+// The tuned multiply (matvec_quant.h, a source file a format): type 3, 4, 5, 6 (K-quants) or 8 (Q8_0).
 zhip_result launch_matvec_quant(const Dispatch &d, const MvArgs &a, int type);
 
 template <class D, int MT>

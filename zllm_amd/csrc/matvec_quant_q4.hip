@@ -1,0 +1,8 @@
+// matvec_q4_k: the default decode kernels of matvec_quant.h for this format.
+#include "matvec_quant.h"
+
+namespace zhip {
+
+zhip_result launch_matvec_quant_q4(const Dispatch &d, const MvArgs &a) { return launch_quant<KQ4>(d, a); }
+
+}  // namespace zhip
