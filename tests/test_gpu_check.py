@@ -599,7 +599,9 @@ def test_matvec_q8_0_mfma_variant_prologues(ctx, rows, n, k, prologue):
     (4, 300, 4096, 5, 0, True, "norm_act"),
     (2, 64, 1024, 0, 0, False, None),          # one unit a tile
     (7, 8232, 1024, 0, 0, True, "norm"),
-    (3, 96, 3072, 0, 0, False, None),          # k the kernel does not take: the default variant's
+    (3, 96, 3072, 0, 0, False, None),          # three units a tile
+    (6, 1000, 3072, 3, 2, True, "norm"),
+    (2, 64, 5120, 0, 0, False, None),          # k the kernel does not take: the default variant's
     # rows of more than 4096 weights: workgroups that share a tile, 2048 columns each
     (8, 1300, 14336, 3, 2, True, None),        # seven parts, 36 walkers: whole rounds, a tail, a ragged last unit
     (4, 4096, 6144, 0, 0, False, None),        # three parts, at most four tokens

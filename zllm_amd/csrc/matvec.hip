@@ -323,7 +323,7 @@ bool matvec_bf16_mfma_stream_accepts(const MvArgs &a);
 zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes, bool f16);
 bool matvec_q5k_mfma_resident_accepts(const MvArgs &a);
 zhip_result launch_matvec_q5k_mfma_resident(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
-// matvec_q6_k on the matrix cores for k of 1024, 2048, 4096 or 6144 .. 32768 in parts (matvec_q6k_mfma_stream.hip).
+// matvec_q6_k on the matrix cores for k of 1024, 2048, 3072, 4096 or 6144 .. 32768 in parts (matvec_q6k_mfma_stream.hip).
 bool matvec_q6k_mfma_stream_accepts(const MvArgs &a);
 zhip_result launch_matvec_q6k_mfma_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes);
 bool matvec_q3k_mfma_stream_accepts(const MvArgs &a);
@@ -433,7 +433,7 @@ static zhip_result launch_matvec(const Dispatch &d, bool quant) {
     if (D::CHUNK == 3 && matrix_cores && matvec_q3k_mfma_stream_accepts(a)) return launch_matvec_q3k_mfma_stream(d, a, d.bind[2].size);
     // (matvec_q5_k: the Q4_K kernel for k of 2048, 4096 or 6144 .. 32768 in parts, with the fifth bits; other shapes run the default variant)
     if (D::CHUNK == 5 && matrix_cores && matvec_q5k_mfma_resident_accepts(a)) return launch_matvec_q5k_mfma_resident(d, a, d.bind[2].size);
-    // (matvec_q6_k and matvec_q3_k: k of 1024, 2048, 4096 or 6144 .. 32768 in parts; every workgroup builds the tokens' operands, prologue included)
+    // (matvec_q6_k and matvec_q3_k: k of 1024, 2048, 3072, 4096 or 6144 .. 32768 in parts; every workgroup builds the tokens' operands, prologue included)
     if (D::CHUNK == 6 && matrix_cores && matvec_q6k_mfma_stream_accepts(a)) return launch_matvec_q6k_mfma_stream(d, a, d.bind[2].size);
     // The kernels that keep the tokens' operands in registers (k of 2048 or 4096, longer rows in parts of 2048, and whole tiles) compute a step's prologue (RMSNorm, silu(x / act_div):
     // src/kernels/matvec_quant.wgsl.hbs:73-89) themselves: their operands are built from one

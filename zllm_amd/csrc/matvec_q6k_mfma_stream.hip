@@ -1,5 +1,5 @@
 // matvec_q6_k and matvec_q3_k, matrix-core variant (MatvecVariant wg 512, lanes 64, rows 16) for steps of up to
-// eight tokens and k = 1024, 2048 or 4096 (longer rows in parts, at the end of this comment): the weight stream is read once for all tokens of the step
+// eight tokens and k = 1024, 2048, 3072 or 4096 (longer rows in parts, at the end of this comment): the weight stream is read once for all tokens of the step
 // and the per-weight work is done once. Contract as the default variant's
 // (src/kernels/matvec_quant.wgsl.hbs with the decoder of src/kernels/quant/q6_k_dot.wgsl; block
 // formula src/ref/tensor.zig:118-140): out[t][col0 + j] (+)= sum over 16-weight sub-blocks of
@@ -604,10 +604,8 @@ __global__ __launch_bounds__(THREADS) void matvec_kquant_mfma_stream_kernel(Q6Ar
     for (uint32_t p = 0; p < count; p++) {
         step(p, std::integral_constant<int, 0>{});
         if constexpr (NU >= 2) step(p, std::integral_constant<int, 1>{});
-        if constexpr (NU >= 4) {
-            step(p, std::integral_constant<int, 2>{});
-            step(p, std::integral_constant<int, 3>{});
-        }
+        if constexpr (NU >= 3) step(p, std::integral_constant<int, 2>{});
+        if constexpr (NU >= 4) step(p, std::integral_constant<int, 3>{});
         hand_over(p);
     }
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // nothing may still land in LDS once the workgroup is gone
@@ -667,15 +665,18 @@ zhip_result launch_stream(const Dispatch &d, const MvArgs &a, uint64_t w_bytes) 
     if constexpr (F::FLAT) {  // (the unit is the whole row: k = 1024 only)
         return a.m <= 4u ? launch_blocks<F, 1, true>(d, q, grid) : launch_blocks<F, 1, false>(d, q, grid);
     } else {
-    if (a.m <= 4u) return a.k == 1024u ? launch_blocks<F, 1, true>(d, q, grid) : a.k == 2048u ? launch_blocks<F, 2, true>(d, q, grid) : launch_blocks<F, 4, true>(d, q, grid);
-    return a.k == 1024u ? launch_blocks<F, 1, false>(d, q, grid) : a.k == 2048u ? launch_blocks<F, 2, false>(d, q, grid) : launch_blocks<F, 4, false>(d, q, grid);
+    if (a.m <= 4u)
+        return a.k == 1024u ? launch_blocks<F, 1, true>(d, q, grid) : a.k == 2048u ? launch_blocks<F, 2, true>(d, q, grid)
+             : a.k == 3072u ? launch_blocks<F, 3, true>(d, q, grid) : launch_blocks<F, 4, true>(d, q, grid);
+    return a.k == 1024u ? launch_blocks<F, 1, false>(d, q, grid) : a.k == 2048u ? launch_blocks<F, 2, false>(d, q, grid)
+         : a.k == 3072u ? launch_blocks<F, 3, false>(d, q, grid) : launch_blocks<F, 4, false>(d, q, grid);
     }
 }
 
-// k of 1024, 2048 or 4096, or 6144 .. 32768 in parts of 2048.
+// k of 1024, 2048, 3072 or 4096, or 6144 .. 32768 in parts of 2048.
 bool stream_accepts(const MvArgs &a, uint32_t block_bytes) {
     const bool parts = a.k > 4096u && a.k % 2048u == 0 && a.k / 2048u <= kMatvecMaxParts;
-    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 4096u || parts) && a.rows >= 1 && a.xr % 4u == 0 &&
+    return a.m >= 1 && a.m <= 8 && (a.k == 1024u || a.k == 2048u || a.k == 3072u || a.k == 4096u || parts) && a.rows >= 1 && a.xr % 4u == 0 &&
            (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == a.k / 256u * block_bytes;
 }
 
