@@ -1411,6 +1411,37 @@ def test_matmul_int8_shapes(ctx, t, rows, n, k):
     assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32))
 
 
+@pytest.mark.parametrize("t,k", [(TensorType.q4_k, 1024), (TensorType.q5_k, 768), (TensorType.q6_k, 2560), (TensorType.q3_k, 512)])
+def test_matmul_kquant_int8_long_and_short_steps_keep_token_bits(ctx, t, k):
+    """The K formats' whole-k int8 multiply takes one kernel for long steps (a wave walks all of
+    k, part after part) and another for short ones (a tile's k in four parts, a wave each, met in
+    LDS): 512 tokens x 4096 outputs are 1024 tiles and a long step, chunks of 128 tokens and
+    fewer short ones; k of 2, 3, 4 and 10 blocks (parts of no, one or several blocks). The same
+    bits either way, and 1e-5 against float64 over the rounded activations
+    (src/kernels/check.zig:839-871)."""
+    c = ctx
+    rows, n, col0, stride = 512, 4096, 4, 4104
+    x = c.random(rows * k, 1).reshape(rows, k)
+    xs = oracle.round_like_llama(ORACLE_TYPE[t], x)
+    raw, values = quant_rows(c, t, n, k)
+    wa = c.gpu_weights(t, raw, k)
+    init = c.random(rows * stride, 0.5).reshape(rows, stride)
+
+    def run(first, count):
+        out = c.upload(init[first : first + count])
+        launch_int8(c, t, quantize_x(c, t, c.upload(x[first : first + count]), count, k), wa, out, count, n, k, 1, None, col0=col0, stride=stride)
+        return c.read(out).reshape(count, stride)
+
+    got = run(0, rows)
+    want = init[:, col0 : col0 + n] + xs.astype(np.float64) @ values.astype(np.float64).T
+    assert rel_err(got[:, col0 : col0 + n], want) <= 1e-5
+    mask = np.ones(stride, dtype=bool)
+    mask[col0 : col0 + n] = False
+    assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32)), "columns outside the chunk were written"
+    for first, count in ((0, 1), (1, 63), (64, 128), (192, 33), (225, 287)):
+        assert got[first : first + count].tobytes() == run(first, count).tobytes(), "token chunking changed bits"
+
+
 def test_matmul_q8_0_int8_whole_steps_keep_token_bits(ctx):
     """matmul_q8_0 with k a multiple of 128, unsliced, takes the kernel whose scale products
     run on the matrix cores, in 128- or 64-token tiles: a token's sums are the same bits

@@ -16,6 +16,11 @@
 // slices need no special paths. Every output is summed over k in increasing
 // order by a sequence of operations that does not depend on its position in
 // the tile: token chunking cannot change bits.
+//
+// The K formats over whole, unsliced k (what a planner's prefill step is) have kernels of their
+// own further down: 32 x 32 x 32 matrix instructions on 32-token tiles, k summed in four parts
+// that one wave walks one after the other (long steps) or four waves side by side (short
+// steps, whose few tiles would otherwise leave a CU one wave that walks all of k).
 #include <hip/hip_runtime.h>
 
 #include "common.h"
@@ -592,13 +597,103 @@ struct W8Q3 {
 };
 
 constexpr uint32_t WT = 32, WN = 64;  // tokens and rows of a workgroup of the wide kernel
-// LDS of a workgroup: two token buffers (32 lines of 256 bytes and 256 bytes of token scales)
-// and one slot of blocks per wave: a wave reads its rows' blocks into registers at the start of a
-// step and then asks for the next step's into the same slot, which nobody else reads.
+// The sum over k is taken in KP parts, steps KP' steps / KP .. of part KP', each added up in the
+// order of its steps, and the parts as ((p0 + p1) + p2) + p3. A workgroup of the kernel for long
+// steps walks all of k, part after part; the kernel for short steps (SPLIT), whose few
+// tiles would leave the chip to one wave a CU walking sixteen blocks one after the other, gives a
+// 32 x 32 tile four waves, a part each, which meet in LDS. The same operations on every output
+// either way: how a prompt is cut into steps does not change a token's bits.
+constexpr uint32_t KP = 4;
+// LDS: two token buffers (32 lines of 256 bytes and 256 bytes of token scales) and one slot of
+// blocks per wave: a wave reads its rows' blocks into registers at the start of a step and then
+// asks for the next step's into the same slot, which nobody else reads. The two waves of a
+// workgroup for long steps (32 rows each) share the token buffers; a wave of the SPLIT kernel
+// has its own (its steps are not the other waves').
 template <class P> constexpr uint32_t wide_wslot() { return ((32u * (P::BLOCK / 16u) + 63u) / 64u) * 1024u; }
 constexpr uint32_t WIDE_TOKENS = WT * 256u + 256u;
-template <class P> constexpr uint32_t wide_lds() { return 2u * WIDE_TOKENS + 2u * wide_wslot<P>(); }
+// (27 KB a workgroup of the kernel for long steps: five of them a CU, which is what bounds its
+// waves a SIMD; a buffer more would cost the fifth and a tenth of the kernel's speed)
+template <class P, bool SPLIT> constexpr uint32_t wide_lds() { return SPLIT ? KP * (2u * WIDE_TOKENS + wide_wslot<P>()) : 2u * WIDE_TOKENS + 2u * wide_wslot<P>(); }
 
+// One step's multiply: the block `cur` of the lane's row times the 32 tokens of the step in
+// `base`, into `acc` (the lane's sixteen results are tokens 8 j + 4 h + i, j < 4, i < 4, of its row).
+// A block's units are summed in integers (a unit's exact sum times its scale, one 24-bit
+// multiply-add a result; Q4_K / Q5_K minimums by one more matrix instruction a unit whose second
+// operand is the unit's minimum in all 32 positions, accumulated by the matrix cores), and the
+// block's f32 scales are applied once.
+template <class P, bool HALVES>
+__device__ __forceinline__ void wide_multiply(const typename P::Raw &cur, const uint8_t *base, uint32_t a_line, uint32_t a_key, uint32_t h, float (&acc)[16]) {
+    constexpr uint32_t DX_AT = WT * 256u;
+    i32x16 isum = {}, msum = {};
+    const i32x16 zero = {};
+    // The eight 6-bit scales and minimums of a Q4_K / Q5_K block as bytes of four words
+    // (src/ref/tensor.zig:94-98), unpacked four at a time.
+    uint32_t sc4[2] = {0u, 0u}, mn4[2] = {0u, 0u};
+    if constexpr (!HALVES) {
+        sc4[0] = cur.h.y & 0x3f3f3f3fu;
+        mn4[0] = cur.h.z & 0x3f3f3f3fu;
+        sc4[1] = (cur.h.w & 0x0f0f0f0fu) | ((cur.h.y >> 2) & 0x30303030u);
+        mn4[1] = ((cur.h.w >> 4) & 0x0f0f0f0fu) | ((cur.h.z >> 2) & 0x30303030u);
+    }
+#pragma unroll
+    for (uint32_t u = 0; u < 8; u++) {
+        if constexpr (HALVES) {
+            iu32x2 w8[2];
+            int sc[2];
+            P::unit(cur, u, h, w8, sc);
+#pragma unroll
+            for (uint32_t half = 0; half < 2; half++) {
+                const long af = *reinterpret_cast<const long *>(base + a_line + 16u * ((2u * u + half) ^ a_key) + 8u * h);
+                const i32x16 is = __builtin_amdgcn_mfma_i32_32x32x16_i8(af, as_operand(w8[half]), zero, 0, 0, 0);
+#pragma unroll
+                for (int e = 0; e < 16; e++) isum[e] = __mul24(sc[half], is[e]) + isum[e];
+            }
+        } else {
+            const int scale = (int)((sc4[u >> 2] >> (8u * (u & 3u))) & 0xffu);
+            const iu32x4 w16 = P::unit(cur, u);
+            const uint32_t m4 = __builtin_amdgcn_perm(0u, mn4[u >> 2], 0x01010101u * (u & 3u));  // the unit's minimum in every byte
+            const i32x4 af = *reinterpret_cast<const i32x4 *>(base + a_line + 16u * ((2u * u + h) ^ a_key));
+            const i32x16 is = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, w16), zero, 0, 0, 0);
+            msum = __builtin_amdgcn_mfma_i32_32x32x32_i8(af, __builtin_bit_cast(i32x4, iu32x4{m4, m4, m4, m4}), msum, 0, 0, 0);
+#pragma unroll
+            for (int e = 0; e < 16; e++) isum[e] = __mul24(scale, is[e]) + isum[e];
+        }
+    }
+    float d, dmin = 0.f;
+    if constexpr (HALVES) {
+        d = P::scale(cur);
+    } else {
+        d = half_bits_to_float(cur.h.x & 0xffffu);
+        dmin = half_bits_to_float(cur.h.x >> 16);
+    }
+#pragma unroll
+    for (uint32_t jj = 0; jj < 4; jj++) {
+        const if32x4 dxv = *reinterpret_cast<const if32x4 *>(base + DX_AT + 4u * (8u * jj + 4u * h));
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+            const int e = 4 * jj + i;
+            float part = d * (float)isum[e];
+            if (!HALVES) part = fmaf(-dmin, (float)msum[e], part);
+            acc[e] = fmaf(dxv[i], part, acc[e]);
+        }
+    }
+}
+
+// The lane's sixteen sums to their outputs.
+__device__ __forceinline__ void wide_store(const I8Args &a, uint32_t j, uint32_t t0, uint32_t h, const float (&total)[16]) {
+    if (j >= a.n) return;
+    float *out = a.out + a.col0 + j;
+#pragma unroll
+    for (uint32_t e = 0; e < 16; e++) {
+        const uint32_t t = t0 + 8u * (e >> 2) + 4u * h + (e & 3u);
+        if (t >= a.rows) continue;
+        float *o = out + (size_t)t * a.out_stride;
+        *o = a.accumulate ? *o + total[e] : total[e];
+    }
+}
+
+// Long steps: 32 tokens x 64 rows a workgroup, a wave 32 rows over all of k. (The step's multiply
+// is written out here, the same operations as wide_multiply.)
 template <class P, bool HALVES>
 __global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds_wide[];
@@ -642,10 +737,24 @@ __global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
     for (int e = 0; e < 16; e++) acc[e] = 0.f;
     const uint32_t a_line = lrow * 256u, a_key = lrow & 15u;
 
+    // At a part's last step the part's sums join the total of the parts before it.
+    float total[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) total[e] = 0.f;
+    uint32_t part = 0;
+    auto close = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) {
+            total[e] = part == 0u ? acc[e] : total[e] + acc[e];
+            acc[e] = 0.f;
+        }
+        part++;
+    };
     fetch_tokens(0, 0);
     fetch_weights(0);
     sync_after_loads();
     for (uint32_t s = 0; s < steps; s++) {
+        while (s >= (part + 1u) * steps / KP) close();
         const uint32_t buf = s & 1u;
         const uint8_t *base = lds_wide + buf * WIDE_TOKENS;
         typename P::Raw cur;
@@ -717,6 +826,7 @@ __global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
         }
         sync_after_loads();
     }
+    while (part < KP) close();
     const uint32_t j = n0 + 32u * wave + lrow;
     if (j >= a.n) return;
     float *out = a.out + a.col0 + j;
@@ -725,25 +835,117 @@ __global__ __launch_bounds__(128) void matmul_kquant_i8_wide_kernel(I8Args a) {
         const uint32_t t = t0 + 8u * (e >> 2) + 4u * h + (e & 3u);
         if (t >= a.rows) continue;
         float *o = out + (size_t)t * a.out_stride;
-        *o = a.accumulate ? *o + acc[e] : acc[e];
+        *o = a.accumulate ? *o + total[e] : total[e];
     }
 }
 
+// Short steps: 32 tokens x 32 rows a workgroup of KP waves, wave p over part p of k. A wave has
+// token buffers and a weight slot of its own and waits for nobody until the parts meet: waves
+// 1 .. 3 leave their sums in LDS (their token buffers, done with) and wave 0 adds.
 template <class P, bool HALVES>
-zhip_result launch_kquant_wide(const Dispatch &d, const char *name, const I8Args &a) {
-    constexpr uint32_t bytes = wide_lds<P>();
-    auto kernel = matmul_kquant_i8_wide_kernel<P, HALVES>;
+__global__ __launch_bounds__(64 * KP) void matmul_kquant_i8_split_kernel(I8Args a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds_wide[];
+    constexpr uint32_t CPR = P::BLOCK / 16u, WLOADS = (32u * CPR + 63u) / 64u, WSLOT = wide_wslot<P>(), WAVE_LDS = 2u * WIDE_TOKENS + WSLOT;
+    constexpr uint32_t DX_AT = WT * 256u;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, lrow = lane & 31u, h = lane >> 5;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t n0 = blockIdx.x * 32u, t0 = blockIdx.y * WT;
+    const uint32_t steps = a.k / 256u;
+    const __amdgpu_buffer_rsrc_t xbuf = make_buffer(a.qx, a.qx_bytes), wbuf = make_buffer(a.w, a.w_bytes), dbuf = make_buffer(a.dx, a.dx_bytes);
+    uint8_t *tokens = lds_wide + wave * WAVE_LDS, *slot = tokens + 2u * WIDE_TOKENS;
+
+    // Loads of a step: the 32 tokens (load i brings tokens 4 i .. + 3, lane l token l / 16 of them
+    // and the chunk that belongs at position l % 16), their scales, the 32 rows' blocks.
+    uint32_t xoff[8], woff[WLOADS];
+#pragma unroll
+    for (uint32_t i = 0; i < 8; i++) {
+        const uint32_t t = 4u * i + (lane >> 4);
+        xoff[i] = (t0 + t) * a.k + 16u * ((lane & 15u) ^ (t & 15u));
+    }
+#pragma unroll
+    for (uint32_t i = 0; i < WLOADS; i++) {
+        const uint32_t c = 64u * i + lane;
+        woff[i] = c < 32u * CPR ? (n0 + c / CPR) * a.row_bytes + 16u * (c % CPR) : 0xfffffff0u - a.row_bytes;
+    }
+    const uint32_t doff = lane < 32u ? (t0 + lane) * (a.k / 256u) * 4u : 0xfffffff0u - a.k;
+    auto fetch = [&](uint32_t s) __attribute__((always_inline)) {
+        uint8_t *base = tokens + (s & 1u) * WIDE_TOKENS;
+#pragma unroll
+        for (uint32_t i = 0; i < 8; i++) load_lds_b128(xbuf, base + 1024u * i, xoff[i], 256u * s);
+        load_lds_b32(dbuf, base + DX_AT, doff + 4u * s);
+#pragma unroll
+        for (uint32_t i = 0; i < WLOADS; i++) load_lds_b128(wbuf, slot + 1024u * i, woff[i], s * P::BLOCK);
+    };
+
+    float acc[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) acc[e] = 0.f;
+    const uint32_t a_line = lrow * 256u, a_key = lrow & 15u;
+    const uint32_t first = wave * steps / KP, last = (wave + 1u) * steps / KP;
+    if (first < last) {
+        fetch(first);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        for (uint32_t s = first; s < last; s++) {
+            const uint8_t *base = tokens + (s & 1u) * WIDE_TOKENS;
+            typename P::Raw cur;
+            P::load(slot + lrow * P::BLOCK, h, cur);
+            // The next step's loads go out once this wave's reads of the slot (and, a step ago,
+            // of the other token buffer) have returned; the compiler, which sees no dependency
+            // between the two, must not move the loads up.
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+            if (s + 1u < last) fetch(s + 1u);
+            wide_multiply<P, HALVES>(cur, base, a_line, a_key, h, acc);
+            asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" ::: "memory");
+        }
+    }
+    float *mine = reinterpret_cast<float *>(tokens) + lane;
+    if (wave != 0u) {
+#pragma unroll
+        for (int e = 0; e < 16; e++) mine[64 * e] = acc[e];
+    }
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (wave != 0u) return;
+    float total[16];
+#pragma unroll
+    for (int e = 0; e < 16; e++) {
+        const float *theirs = reinterpret_cast<const float *>(lds_wide) + 64 * e + lane;
+        total[e] = ((acc[e] + theirs[1u * WAVE_LDS / 4u]) + theirs[2u * WAVE_LDS / 4u]) + theirs[3u * WAVE_LDS / 4u];
+    }
+    wide_store(a, n0 + lrow, t0, h, total);
+}
+
+template <class P, bool HALVES, bool SPLIT>
+zhip_result launch_kquant_wide_as(const Dispatch &d, const char *name, const I8Args &a) {
+    constexpr uint32_t bytes = wide_lds<P, SPLIT>();
+    const void *kernel;
+    if constexpr (SPLIT) kernel = reinterpret_cast<const void *>(matmul_kquant_i8_split_kernel<P, HALVES>);
+    else kernel = reinterpret_cast<const void *>(matmul_kquant_i8_wide_kernel<P, HALVES>);
     static bool configured = false;
     if (!configured) {
-        if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
+        if (hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes) != hipSuccess) {
             (void)hipGetLastError();
             return fail(d, ZHIP_E_GPU, "%s: cannot reserve %u bytes of LDS", name, bytes);
         }
         configured = true;
     }
-    const dim3 grid((a.n + WN - 1u) / WN, (a.rows + WT - 1u) / WT);
-    hipLaunchKernelGGL(kernel, grid, dim3(128), bytes, d.stream, a);
+    const dim3 grid((a.n + (SPLIT ? 32u : WN) - 1u) / (SPLIT ? 32u : WN), (a.rows + WT - 1u) / WT);
+    if constexpr (SPLIT) hipLaunchKernelGGL((matmul_kquant_i8_split_kernel<P, HALVES>), grid, dim3(64u * KP), bytes, d.stream, a);
+    else hipLaunchKernelGGL((matmul_kquant_i8_wide_kernel<P, HALVES>), grid, dim3(128u), bytes, d.stream, a);
     return check_launch(d, name);
+}
+
+// Steps whose 32-token x 64-row tiles are fewer than two a CU (three where a wave's walk is 32
+// blocks or more) take the kernel that gives a tile's k to four waves. Measured, Q4_K, the
+// multiply alone, weights from HBM: 64 x 4096 x 4096 21.2 -> 9.3 us, 128 tokens 21.3 -> 16.1,
+// 256 tokens 30.4 against 29.8 (left as it is), 64 x 14336 x 4096 65.4 -> 21.5, 256 tokens
+// 96.1 -> 75.4, 384 tokens 96.9 against 111.3 (left).
+template <class P, bool HALVES>
+zhip_result launch_kquant_wide(const Dispatch &d, const char *name, const I8Args &a) {
+    const uint64_t tiles = (uint64_t)((a.n + WN - 1u) / WN) * ((a.rows + WT - 1u) / WT);
+    const bool split = tiles < (a.k >= 32u * 256u ? 3ull : 2ull) * (uint64_t)d.dev->compute_units;
+    return split ? launch_kquant_wide_as<P, HALVES, true>(d, name, a) : launch_kquant_wide_as<P, HALVES, false>(d, name, a);
 }
 
 // The K-format kernel's weight buffers are dynamic LDS (with the static token buffers a
