@@ -746,21 +746,24 @@ def bench_prefill_grid(env):
     src/sched/sched.zig:77-91, src/plan/plan.zig:129) on the three shapes of a layer: keys
     `m<tokens>_k<k>_n<n>`, each with the bf16 matrix-core rung on packed bf16 activations
     ("bf16": us, fraction of the 2.5 PFLOP/s peak) and the reference's default path, quantize_q8
-    + matmul_q8_0 on the int8 matrix cores ("int8": us, fraction of the 5 POP/s peak). Checked
-    on every 8th token."""
+    + matmul_q8_0 on the int8 matrix cores ("int8": us, fraction of the 5 POP/s peak), and the
+    same default path over Q4_K weights of the shape, the format of most of a Q4_K_M file
+    ("q4_k": us). Checked on every 8th token."""
     synth, oracle, K, TensorType = env["synth"], env["oracle"], env["K"], env["TensorType"]
     res = {}
     for k, n in ((4096, 14336), (14336, 4096), (4096, 4096)):
         raw = synth.q8_0_rows(synth.rng(0x9D + n), n, k)
+        raw4 = synth.q4_k_rows(synth.rng(0x9E + n), n, k)
         for rows in (64, 128, 256, 512):
             if env.get("grid") and f"m{rows}_k{k}_n{n}" not in env["grid"]:
                 continue
             flops = 2 * rows * n * k
             t, err, _ = _prefill_q8(env, rows, k, n, K.Prefill.bf16_mfma_xbf16, check_stride=8)
             ti, erri = _prefill_int8(env, TensorType.q8_0, oracle.Q8_0, raw, rows, k, n, check_stride=8)
+            t4, err4 = _prefill_int8(env, TensorType.q4_k, oracle.Q4_K, raw4, rows, k, n, check_stride=8)
             res[f"m{rows}_k{k}_n{n}"] = {"bf16": [round(t * 1e6, 2), round(flops / t / 1e12 / MFMA_BF16_PEAK_TFLOPS, 3)],
                                          "int8": [round(ti * 1e6, 2), round(flops / ti / 1e12 / MFMA_INT8_PEAK_TOPS, 3)],
-                                         "err": [sig2(err), sig2(erri)]}
+                                         "q4_k": round(t4 * 1e6, 2), "err": [sig2(err), sig2(erri), sig2(err4)]}
     return res
 
 
