@@ -21,7 +21,7 @@
 //    replaces the conversion.
 // Two full-rate vector operations per output and unit remain.
 //
-// Tiling as in matmul_q8_bf16.hip: a workgroup computes 128 (or 64) tokens x 64 matrix rows;
+// Tiling as in matmul_q8_bf16.hip: a workgroup computes 128 (or 64, or 32) tokens x 64 matrix rows;
 // wave w multiplies rows 32 (w % 2) .. + 31 by all the tile's tokens over unit w / 2 of every
 // step, lane l holding row (token) l % 32 and bytes 16 (l / 32) .. + 15 of the unit. Operands
 // arrive straight in LDS (range-checked buffers: what lies past a binding reads as zero) three
@@ -49,7 +49,9 @@ constexpr int BN = 64, BK = 128, WAVES = 8, THREADS = 64 * WAVES;
 // of row scales ([8 rows][4 f16], the rest filler) and 256 bytes of token scales ([16 tokens][4 f32]).
 template <int TT> constexpr int abuf_bytes() { return 32 * TT * 128; }
 constexpr int WBUF = BN * 128, SBUF = WAVES * 256, DBUF = WAVES * 256;
-template <int TT> constexpr int buf_bytes() { return abuf_bytes<TT>() + WBUF + SBUF + DBUF; }
+// (and, with 32-token tiles, a spare KB where the loads of the four waves that have no token
+// lines to bring land their nothing)
+template <int TT> constexpr int buf_bytes() { return abuf_bytes<TT>() + WBUF + SBUF + DBUF + (TT == 1 ? 1024 : 0); }
 // Three buffers, or the exchange of the four units' sums that reuses them (8 waves x 3 inboxes x TT KB).
 template <int TT> constexpr int lds_bytes() { return 3 * buf_bytes<TT>() > 8 * 3 * TT * 1024 ? 3 * buf_bytes<TT>() : 8 * 3 * TT * 1024; }
 static_assert(lds_bytes<4>() <= 160 * 1024, "the buffers must fit the CU's LDS");
@@ -93,14 +95,14 @@ __device__ __forceinline__ uint32_t line_key(uint32_t row) { return (row & 7u) ^
 template <int TT>
 struct Frags {
     i32x4 w, tok[TT];  // the row's and each tile's token's sixteen bytes of the unit
-    float dw, dx[TT / 2];  // the row's scale; the scale of the lane's token in tile 2 pair + lane / 32
+    float dw, dx[(TT + 1) / 2];  // the row's scale; the scale of the lane's token in tile 2 pair + lane / 32
 };
 
 template <int TT>
 __global__ __launch_bounds__(THREADS) void matmul_q8_i8_kernel(Q8I8Args a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int BM = 32 * TT, ABUF = abuf_bytes<TT>(), BUF = buf_bytes<TT>();
-    constexpr int XL = TT / 2;            // token-line loads a wave issues per step
+    constexpr int XL = (TT + 1) / 2;      // token-line loads a wave issues per step (32-token tiles: four of the waves bring nothing)
     constexpr int PER_STEP = XL + 3;
     const uint32_t tid = threadIdx.x, lane = tid & 63u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -115,7 +117,7 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_i8_kernel(Q8I8Args a) {
 #pragma unroll
     for (int i = 0; i < XL; i++) {
         const uint32_t row = 8u * (wave + 8u * i) + (lane >> 3);
-        xoff[i] = (t0 + row) * a.k + 16u * ((lane & 7u) ^ line_key(row));
+        xoff[i] = row < (uint32_t)BM ? (t0 + row) * a.k + 16u * ((lane & 7u) ^ line_key(row)) : 0xF0000000u;
     }
     const uint32_t wrow = 8u * wave + (lane >> 3);
     const uint32_t woff = (j0 + wrow) * a.row_bytes + 16u * ((lane & 7u) ^ line_key(wrow));
@@ -125,7 +127,8 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_i8_kernel(Q8I8Args a) {
     auto fetch = [&](uint32_t buf, uint32_t step) __attribute__((always_inline)) {
         const uint32_t base = lds0 + buf * BUF;
 #pragma unroll
-        for (int i = 0; i < XL; i++) load_lds_b128(xbuf, base + 1024u * (wave + 8u * i), xoff[i], 128u * step);
+        for (int i = 0; i < XL; i++)
+            load_lds_b128(xbuf, base + (8u * (wave + 8u * i) < (uint32_t)BM ? 1024u * (wave + 8u * i) : (uint32_t)(ABUF + WBUF + SBUF + DBUF)), xoff[i], 128u * step);
         load_lds_b128(wbuf, base + ABUF + 1024u * wave, woff, 128u * step);
         load_lds_b32(wbuf, base + ABUF + WBUF + 256u * wave, soff, 8u * step);
         load_lds_b32(dbuf, base + ABUF + WBUF + SBUF + 256u * wave, doff, 16u * step);
@@ -185,10 +188,20 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_i8_kernel(Q8I8Args a) {
         const i32x16 zero_i = magic;
         const f32x32 zero_f = {};
         i32x16 sums[TT];
-        f32x32 scale[TT / 2];
+        f32x32 scale[(TT + 1) / 2];
         sums[0] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w, f.tok[0], zero_i, 0, 0, 0);
         scale[0] = __builtin_amdgcn_mfma_f32_32x32x1f32(f.dw, f.dx[0], zero_f, 0, 0, 0);
-        sums[1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w, f.tok[1], zero_i, 0, 0, 0);
+        if constexpr (TT == 1) {
+            // One tile: its scaling follows the next step's matrix instructions.
+            read_tile(nxt_buf, 0);
+            read_scales(nxt_buf, 0);
+            read_rows(nxt_buf);
+            scale_into(acc[0], sums_left, scale_left);
+            sums_left = sums[0];
+            scale_left = low(scale[0]);
+            return;
+        }
+        sums[TT - 1 < 1 ? 0 : 1] = __builtin_amdgcn_mfma_i32_32x32x32_i8(f.w, f.tok[TT - 1 < 1 ? 0 : 1], zero_i, 0, 0, 0);
         read_tile(nxt_buf, 0);
         read_tile(nxt_buf, 1);
         read_scales(nxt_buf, 0);
@@ -217,7 +230,7 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_i8_kernel(Q8I8Args a) {
         } else {
             read_rows(nxt_buf);
             scale_into(acc[0], sums[0], low(scale[0]));
-            sums_left = sums[1];
+            sums_left = sums[TT - 1 < 1 ? 0 : 1];
             scale_left = high(scale[0]);
             __builtin_amdgcn_sched_group_barrier(0x100, 2, 0);
             __builtin_amdgcn_sched_group_barrier(0x002, 32, 0);
@@ -233,7 +246,7 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_i8_kernel(Q8I8Args a) {
 #pragma unroll
     for (int tt = 0; tt < TT; tt++) read_tile(0, tt);
 #pragma unroll
-    for (int pair = 0; pair < TT / 2; pair++) read_scales(0, pair);
+    for (int pair = 0; pair < (TT + 1) / 2; pair++) read_scales(0, pair);
     read_rows(0);
     sync_keeping_loads<PER_STEP>();      // step 1 has landed; buffer 0 has been read
 
@@ -259,10 +272,11 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_i8_kernel(Q8I8Args a) {
 
     // The four units of a tile meet in LDS: the wave of unit q keeps token tile q % TT (with
     // 64-token tiles, units q and q + 2 each keep half of tile q % 2: parts 2 (q / 2) and + 1 of the
-    // lane's four groups of sums) and hands the rest to their owners.
+    // lane's four groups of sums; with 32-token tiles unit q keeps part q) and hands the rest to
+    // their owners.
     f32x4 *inbox = reinterpret_cast<f32x4 *>(lds);
     constexpr int PARTS = TT;
-    auto owner_of = [](int tt, int part) { return TT == 4 ? tt : tt + 2 * (part / 2); };
+    auto owner_of = [](int tt, int part) { return TT == 4 ? tt : TT == 2 ? tt + 2 * (part / 2) : part; };
     auto slot = [&](uint32_t owner, uint32_t from, int part) {
         return (((owner * 2u + wn) * 3u + ((from + 3u - owner) & 3u)) * PARTS + part) * 64u + lane;
     };
@@ -273,7 +287,7 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_i8_kernel(Q8I8Args a) {
 #pragma unroll
             for (int p = 0; p < 4; p++) {
                 if (owner_of(tt, p) == Q) continue;
-                inbox[slot(owner_of(tt, p), Q, TT == 4 ? p : p % 2)] = f32x4{acc[tt][4 * p], acc[tt][4 * p + 1], acc[tt][4 * p + 2], acc[tt][4 * p + 3]};
+                inbox[slot(owner_of(tt, p), Q, TT == 4 ? p : TT == 2 ? p % 2 : 0)] = f32x4{acc[tt][4 * p], acc[tt][4 * p + 1], acc[tt][4 * p + 2], acc[tt][4 * p + 3]};
             }
     };
     const bool aligned = ((a.out_stride | a.col0) & 3u) == 0u && (reinterpret_cast<uintptr_t>(a.out) & 15u) == 0u;
@@ -285,7 +299,7 @@ __global__ __launch_bounds__(THREADS) void matmul_q8_i8_kernel(Q8I8Args a) {
         const uint32_t t = t0 + 32u * tile + lrow;
 #pragma unroll
         for (int i = 0; i < PARTS; i++) {
-            constexpr int first = TT == 4 ? 0 : 2 * (Q / 2);
+            constexpr int first = TT == 4 ? 0 : TT == 2 ? 2 * (Q / 2) : Q;
             const int p = first + i;
             f32x4 part[4];
 #pragma unroll
@@ -353,10 +367,12 @@ zhip_result launch_matmul_q8_i8(const Dispatch &d, const char *name, const uint8
     a.qx = qx; a.w = w; a.dx = dx; a.out = out;
     a.rows = rows; a.n = n; a.k = k; a.col0 = col0; a.out_stride = out_stride; a.accumulate = accumulate;
     a.row_bytes = row_bytes; a.qx_bytes = qx_bytes; a.w_bytes = w_bytes; a.dx_bytes = dx_bytes;
-    // 128-token tiles unless those leave half of the CUs idle: then 64-token tiles on twice the CUs.
-    const uint64_t tall = (uint64_t)((rows + 127u) / 128u) * ((n + BN - 1) / BN);
-    if (rows > 64u && 2u * tall > (uint64_t)d.dev->compute_units) return launch_tile<4>(d, name, a);
-    return launch_tile<2>(d, name, a);
+    // 128-token tiles unless those leave half of the CUs idle: then 64-token tiles on twice the
+    // CUs, then 32-token tiles.
+    const uint64_t columns = (n + BN - 1) / BN, cus = (uint64_t)d.dev->compute_units;
+    if (rows > 64u && 2u * ((rows + 127u) / 128u) * columns > cus) return launch_tile<4>(d, name, a);
+    if (rows > 32u && 2u * ((rows + 63u) / 64u) * columns > cus) return launch_tile<2>(d, name, a);
+    return launch_tile<1>(d, name, a);
 }
 
 }  // namespace zhip
