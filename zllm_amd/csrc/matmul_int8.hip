@@ -936,15 +936,16 @@ zhip_result launch_kquant_wide_as(const Dispatch &d, const char *name, const I8A
     return check_launch(d, name);
 }
 
-// Steps whose 32-token x 64-row tiles are fewer than two a CU (three where a wave's walk is 32
+// Steps whose 32-token x 64-row tiles are fewer than 1.75 a CU (three where a wave's walk is 32
 // blocks or more) take the kernel that gives a tile's k to four waves. Measured, Q4_K, the
 // multiply alone, weights from HBM: 64 x 4096 x 4096 21.2 -> 9.3 us, 128 tokens 21.3 -> 16.1,
 // 256 tokens 30.4 against 29.8 (left as it is), 64 x 14336 x 4096 65.4 -> 21.5, 256 tokens
-// 96.1 -> 75.4, 384 tokens 96.9 against 111.3 (left).
+// 96.1 -> 75.4, 384 tokens 96.9 against 111.3 (left); 192 x 4096 x 4096 (1.5 tiles a CU)
+// 30.6 -> 23.0, 64 x 4096 x 14336 (1.75) 28.5 against 31.8 (left).
 template <class P, bool HALVES>
 zhip_result launch_kquant_wide(const Dispatch &d, const char *name, const I8Args &a) {
     const uint64_t tiles = (uint64_t)((a.n + WN - 1u) / WN) * ((a.rows + WT - 1u) / WT);
-    const bool split = tiles < (a.k >= 32u * 256u ? 3ull : 2ull) * (uint64_t)d.dev->compute_units;
+    const bool split = 4u * tiles < (a.k >= 32u * 256u ? 12ull : 7ull) * (uint64_t)d.dev->compute_units;
     return split ? launch_kquant_wide_as<P, HALVES, true>(d, name, a) : launch_kquant_wide_as<P, HALVES, false>(d, name, a);
 }
 
