@@ -1,5 +1,5 @@
-"""Seeded random shapes through the decode multiply's matrix-core variant id and through the
-prefill rungs: the edges the fixed cases of test_gpu_check.py do not name (row counts below a
+"""Seeded random shapes through the decode multiply's matrix-core variant id, the prefill rungs
+and the int8 prefill: the edges the fixed cases of test_gpu_check.py do not name (row counts below a
 tile, rows in any number of parts, ragged token counts, column offsets and padded strides).
 Each case against float64 over the oracle's decoded weights (1e-5 of the output's scale, the
 reference's gpu-check tolerance, src/kernels/check.zig:205-222), nothing outside the outputs
@@ -138,3 +138,53 @@ def test_prefill_rungs_random_shapes(ctx, seed):
             assert got[a:b].tobytes() == run(a, b - a).tobytes(), (what, "token chunking changed bits", a, b)
         release(c, wa)
     c.set.select_prefill(c.rec, K.Prefill.scalar_f32)
+
+
+@pytest.mark.parametrize("seed", [21, 22])
+def test_int8_prefill_random_shapes(ctx, seed):
+    """Thirty cases a seed of the reference's default prefill, quantize_q8 + matmul_<type> over
+    whole k, every format: 1 .. 512 tokens, 1 .. 8000 outputs, k of 1 .. 36 blocks of 256 (the
+    K formats' four parts of k with no, one or several blocks each; steps short and long enough
+    for either of their kernels and for each of the Q8_0 kernel's tile heights). 1e-5 against
+    float64 over the rounded activations (src/kernels/check.zig:839-871); then the same tokens
+    in up to four steps cut at random, bit for bit."""
+    c = ctx
+    rng = np.random.default_rng(seed)
+    for case in range(30):
+        t = list(ORACLE_TYPE)[rng.integers(5)]
+        k = int(rng.choice([256, 512, 768, 1024, 1280, 2048, 4096, 9216]))
+        n = int(rng.choice([1, 31, 64, 100, 1000, 2830, 4096, 8000]))
+        rows = int(rng.choice([1, 5, 31, 32, 33, 64, 65, 100, 128, 129, 300, 512]))
+        col0, pad, acc = int(rng.choice([0, 0, 3, 4])), int(rng.choice([0, 4, 5])), int(rng.integers(2))
+        what = f"case {case}: {t.name} rows={rows} n={n} k={k} col0={col0} pad={pad} accumulate={acc}"
+        g = synth.rng(int(rng.integers(1 << 30)))
+        raw = synth.random_blocks(g, t.name, n, k)
+        vals = oracle.dequantize(ORACLE_TYPE[t], raw, n * k).reshape(n, k).astype(np.float64)
+        x = synth.activations(g, rows, k)
+        xs = oracle.round_like_llama(ORACLE_TYPE[t], x).astype(np.float64)
+        stride = col0 + n + pad
+        init = synth.activations(g, rows, stride)
+        wa = c.gpu_weights(t, raw, k)
+        block = K.act_block(t)
+
+        def run(first, count):
+            out, xa = c.upload(init[first : first + count]), c.upload(x[first : first + count])
+            qx, dx = c.output(count * k // 4), c.output(count * k // block)
+            l = c.launcher()
+            l.launch(Kernel.quantize_q8, P.QuantizeQ8(k=k, block=block), [xa, qx, dx, xa], (K.div_ceil(k, 256), count, 1))
+            l.launch(K.weight_kernel("matmul", t), P.MatmulQuant(rows=count, n=n, k=k, col0=col0, out_stride=stride, accumulate=acc, k_slice=k),
+                     [qx, wa, out, dx], (K.div_ceil(n, K.matmul_quant_tile_n), K.div_ceil(count, K.matmul_quant_tile_t), 1))
+            r = c.read(out).reshape(count, stride).copy()
+            release(c, out, xa, qx, dx)
+            return r
+
+        got = run(0, rows)
+        want = (init[:, col0 : col0 + n] if acc else 0) + xs @ vals.T
+        assert rel_err(got[:, col0 : col0 + n], want) <= 1e-5, what
+        mask = np.ones(stride, dtype=bool)
+        mask[col0 : col0 + n] = False
+        assert np.array_equal(got[:, mask].view(np.uint32), init[:, mask].view(np.uint32)), what
+        cuts = sorted(set([0, rows] + [int(v) for v in rng.integers(0, rows + 1, size=3)]))
+        for a, b in zip(cuts[:-1], cuts[1:]):
+            assert got[a:b].tobytes() == run(a, b - a).tobytes(), (what, "token chunking changed bits", a, b)
+        release(c, wa)
