@@ -125,7 +125,9 @@ def bf16_tokens_case(c, m, n, k, col0=0, pad=0, accumulate=False, norm=False, x=
     (19, 2052, 4096, 8, 0, True, False),
     (3, 100, 1024, 0, 0, False, False),        # a small matrix: the general kernel
     (5, 1100, 9728, 0, 0, False, False),       # rows longer than 4096: stretches of columns, each launch adding to the one before
-    (6, 800, 14336, 3, 5, True, False),        # ... onto what the output already holds
+    (6, 800, 14336, 3, 5, True, False),        # ... onto what the output already holds (four equal stretches: one launch, and one for their sums)
+    (19, 1100, 8192, 8, 0, True, True),        # two equal stretches, three groups of tokens, the prologue
+    (5, 1000, 12288, 0, 0, False, False),      # three equal stretches
     (5, 1000, 8704, 0, 0, False, True),        # with the RMSNorm prologue: the tokens are normalised and split once for all the stretches
     (3, 1100, 9728, 0, 0, False, False),       # the same rows at fewer tokens (the general kernel: passes of as many tokens as fit workgroup memory)
     (2, 800, 14336, 3, 5, True, False),

@@ -72,6 +72,11 @@ struct StreamArgs {
     uint32_t plane_first;   // the launch's first position
     uint32_t t0;            // the launch's first token in the planes
     const float *inverse;   // F16 kernels: one over each token's scale
+    // Rows of more than 4096 weights in equal stretches of columns (LONG kernels): `parts`
+    // workgroups share a tile, a stretch each, and leave their sums in `partial`
+    // ([part][token of 8][output], outputs a.rows apart).
+    uint32_t parts;
+    float *partial;
 };
 
 // A barrier that waits for this wave's LDS traffic only: the weight loads of the pieces ahead
@@ -133,9 +138,12 @@ __device__ __forceinline__ uint32_t upper_halves(uint32_t lo, uint32_t hi) { ret
 // times 2^11, after a power of two has put its largest magnitude at 2^14 (an input keeps 22
 // bits); the planes come from matvec_f16_split_kernel, and a token's sums are multiplied by one
 // over its scale.
-template <int NP, bool SPLIT, bool F16>
+// LONG: k = 512 NP q.parts; workgroup i multiplies stretch i % parts (`kpart`) of the tiles that
+// walker i / parts takes, and launch_matvec_parts_sum adds the stretches' sums.
+template <int NP, bool SPLIT, bool F16, bool LONG>
 __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(StreamArgs q) {
     static_assert(SPLIT || !F16, "f16 tokens are always split beforehand");
+    static_assert(SPLIT || !LONG, "the stretches of a long row read the tokens from the planes");
     constexpr uint32_t PIECES = F16 ? 2u : 3u;
     const MvArgs &a = q.a;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
@@ -153,8 +161,9 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
     // hardware deals workgroups out to the chip's eight dies in turn; b numbers them so that a
     // die's workgroups take neighbouring tiles (one die then reads a contiguous eighth of every
     // round's stretch of the matrix: 55 us against 58 us for four tokens over 151936 x 1024).
-    const uint32_t G = gridDim.x;
-    const uint32_t b = q.by_die ? (blockIdx.x & 7u) * (G >> 3) + (blockIdx.x >> 3) : blockIdx.x;
+    const uint32_t kpart = LONG ? blockIdx.x % q.parts : 0u, walker = LONG ? blockIdx.x / q.parts : blockIdx.x;
+    const uint32_t G = LONG ? gridDim.x / q.parts : gridDim.x;
+    const uint32_t b = q.by_die ? (walker & 7u) * (G >> 3) + (walker >> 3) : walker;
     const uint32_t tail_units = q.tail_base + (b < q.tail_rem ? 1u : 0u);
     const uint32_t tail_row = 32u * q.rounds * G + 8u * (b * q.tail_base + (b < q.tail_rem ? b : q.tail_rem));
     const uint32_t count = q.rounds + (tail_units ? 1u : 0u);
@@ -167,7 +176,7 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
     auto line_key = [](uint32_t row) { return (row >> 1) & 7u; };
     uint32_t woff[LOADS];
 #pragma unroll
-    for (int j = 0; j < LOADS; j++) woff[j] = (8u * j + (lane >> 3)) * a.row_bytes + 128u * NP * wave + 16u * ((lane & 7u) ^ line_key(8u * j + (lane >> 3)));
+    for (int j = 0; j < LOADS; j++) woff[j] = (8u * j + (lane >> 3)) * a.row_bytes + 1024u * NP * kpart + 128u * NP * wave + 16u * ((lane & 7u) ^ line_key(8u * j + (lane >> 3)));
     uint32_t load_tile = 0, load_piece = 0, load_slot = 0;
     auto issue = [&]() __attribute__((always_inline)) {
         // (past the run's last piece the loads still run, so that the waits count the same loads
@@ -202,7 +211,7 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
         // Every step's operand is sixteen bytes of a plane; the lanes of absent tokens and of
         // the zero rows ask past the buffer's end and get zeros.
         const __amdgpu_buffer_rsrc_t pbuf = make_buffer(q.planes, PIECES * q.plane_tokens * q.plane_k * 2u);
-        const uint32_t at = live ? ((piece * q.plane_tokens + q.t0 + tok) * q.plane_k + q.plane_first + 64u * NP * wave + 8u * kap) * 2u : 0xfffffff0u;
+        const uint32_t at = live ? ((piece * q.plane_tokens + q.t0 + tok) * q.plane_k + q.plane_first + 512u * NP * kpart + 64u * NP * wave + 8u * kap) * 2u : 0xfffffff0u;
 #pragma unroll
         for (int s = 0; s < 4 * NP; s++) xf[s] = __builtin_bit_cast(hu32x4, __builtin_amdgcn_raw_buffer_load_b128(pbuf, live ? at + 32u * s : at, 0, 0));
         issue();
@@ -271,7 +280,8 @@ __global__ __launch_bounds__(THREADS) void matvec_bf16_mfma_stream_kernel(Stream
             if (tk < a.m && row < rows_of(p) && j < a.rows) {
                 float *o = a.out + (size_t)tk * a.out_stride + a.col0 + j;
                 const float total = lds_kept[256u * (p % KEPT) + (tid & 255u)];
-                store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + total : total);
+                if (LONG) store_apart(q.partial + ((size_t)kpart * 8u + tk) * a.rows + j, total);
+                else store_apart(o, (a.flags & FLAG_ACCUMULATE) ? *o + total : total);
             }
         }
     };
@@ -373,9 +383,9 @@ __global__ __launch_bounds__(256) void matvec_f16_split_kernel(MvArgs a, uint2 *
     }
 }
 
-template <int NP, bool SPLIT, bool F16>
+template <int NP, bool SPLIT, bool F16, bool LONG = false>
 zhip_result launch_blocks(const Dispatch &d, const StreamArgs &q, dim3 grid) {
-    auto kernel = matvec_bf16_mfma_stream_kernel<NP, SPLIT, F16>;
+    auto kernel = matvec_bf16_mfma_stream_kernel<NP, SPLIT, F16, LONG>;
     static bool configured = false;
     if (!configured) {
         if (hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, LDS_BYTES) != hipSuccess) {
@@ -392,22 +402,23 @@ zhip_result launch_blocks(const Dispatch &d, const StreamArgs &q, dim3 grid) {
 
 // Whether this kernel can run the (already validated) arguments: k split into whole lines a
 // wave, no pair.
-// (rows of more than 4096 weights are taken in stretches of columns, a launch each; up to 16384: the split launch stages a token in 64 KB of LDS)
+// (rows of more than 4096 weights are taken in stretches of columns: equal ones in one launch, workgroups sharing a
+// tile, with a launch for their sums; unequal ones a launch each; up to 16384: the split launch stages a token in 64 KB of LDS)
 bool matvec_bf16_mfma_stream_accepts(const MvArgs &a) {
     return a.m >= 1 && a.k >= 1024u && a.k <= 16384u && a.k % 512u == 0 && !(a.flags & FLAG_SILU_PAIR) && a.act_div == 0.f && a.rows >= 1 &&
            a.xr % 4u == 0 && (reinterpret_cast<uintptr_t>(a.x) & 15u) == 0 && (reinterpret_cast<uintptr_t>(a.w) & 15u) == 0 && a.row_bytes == 2u * a.k;
 }
 
-template <bool SPLIT, bool F16>
+template <bool SPLIT, bool F16, bool LONG = false>
 static zhip_result launch_for_k(const Dispatch &d, const StreamArgs &q, dim3 grid) {
     switch (q.a.k / 512u) {
-    case 2: return launch_blocks<2, SPLIT, F16>(d, q, grid);
-    case 3: return launch_blocks<3, SPLIT, F16>(d, q, grid);
-    case 4: return launch_blocks<4, SPLIT, F16>(d, q, grid);
-    case 5: return launch_blocks<5, SPLIT, F16>(d, q, grid);
-    case 6: return launch_blocks<6, SPLIT, F16>(d, q, grid);
-    case 7: return launch_blocks<7, SPLIT, F16>(d, q, grid);
-    default: return launch_blocks<8, SPLIT, F16>(d, q, grid);
+    case 2: return launch_blocks<2, SPLIT, F16, LONG>(d, q, grid);
+    case 3: return launch_blocks<3, SPLIT, F16, LONG>(d, q, grid);
+    case 4: return launch_blocks<4, SPLIT, F16, LONG>(d, q, grid);
+    case 5: return launch_blocks<5, SPLIT, F16, LONG>(d, q, grid);
+    case 6: return launch_blocks<6, SPLIT, F16, LONG>(d, q, grid);
+    case 7: return launch_blocks<7, SPLIT, F16, LONG>(d, q, grid);
+    default: return launch_blocks<8, SPLIT, F16, LONG>(d, q, grid);
     }
 }
 
@@ -422,18 +433,26 @@ zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, u
     const uint32_t groups = units < cus ? units : cus;
     const uint32_t rounds = (a.rows / 32u) / groups;
     const uint32_t tail = (a.rows - 32u * rounds * groups + 7u) / 8u;
-    StreamArgs q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, nullptr, 0u, 0u, 0u, 0u, nullptr};
+    StreamArgs q{a, (uint32_t)(used < w_bytes ? used : w_bytes), rounds, tail / groups, tail % groups, groups % 8u == 0 ? 1u : 0u, nullptr, 0u, 0u, 0u, 0u, nullptr, 1u, nullptr};
     // The tokens are split (and normalised) by a launch of their own where that is cheaper than
     // every workgroup splitting them again, and wherever the step carries the RMSNorm prologue
     // (the workgroups computing the norm themselves at k = 1024 measured the same: 151936 x 1024
     // at 2 / 4 / 8 tokens 53.3 / 54.1 / 56.3 us against 54.2 / 54.2 / 55.5 us this way). f16
     // tokens, which need their scales first, always.
     const bool split = f16 || (a.flags & FLAG_NORM) || a.k >= 2048u;
+    // Rows of more than 4096 weights (the FFN-down shapes; the general kernel takes them token by
+    // token) go in stretches of up to 4096 columns. Stretches of equal length (14336 = 4 x 3584,
+    // 8192 = 2 x 4096 ...) go out as one launch: `launches` workgroups share a walker's tiles, a
+    // stretch each, and a second launch adds the stretches' sums in their order and applies the
+    // epilogue (their sums wait in the workspace, behind the tokens' planes).
+    const uint32_t pieces = a.k / 512u, launches = (a.k + 4095u) / 4096u;
+    const bool together = launches > 1u && pieces % launches == 0u && split && launches <= kMatvecMaxParts && cus >= launches;
+    const uint64_t planes_bytes = (((f16 ? 4ull : 6ull) * a.m * a.k + 4ull * a.m + 64u) + 255u) & ~255ull;
     if (split) {
         const uint64_t bytes = (f16 ? 4ull : 6ull) * a.m * a.k;
         if (!d.work) return fail(d, ZHIP_E_GPU, "%s: no workspace", name);
         if (bytes >= 0xfffffff0ull) return fail(d, ZHIP_E_BAD_COMMAND, "%s: a step of %u tokens", name, a.m);
-        if (zhip_result r = d.work->reserve(d, bytes + 4ull * a.m + 64u)) return r;
+        if (zhip_result r = d.work->reserve(d, planes_bytes + (together ? (uint64_t)launches * 8u * a.rows * sizeof(float) : 0ull))) return r;
         float *inverse = reinterpret_cast<float *>(d.work->data + bytes);
         if (f16) hipLaunchKernelGGL(matvec_f16_split_kernel, dim3(a.m), dim3(256), a.k * 4u, d.stream, a, reinterpret_cast<uint2 *>(d.work->data), inverse);
         else hipLaunchKernelGGL(matvec_bf16_split_kernel, dim3(a.m), dim3(256), a.k * 4u, d.stream, a, reinterpret_cast<uint2 *>(d.work->data));
@@ -446,10 +465,29 @@ zhip_result launch_matvec_bf16_mfma_stream(const Dispatch &d, const MvArgs &a, u
         q.a.norm_w = nullptr;
     }
     const dim3 grid(groups);
-    // Rows of more than 4096 weights (the FFN-down shapes; the general kernel takes them token by
-    // token): stretches of up to 4096 columns, each a launch that adds to the one before; the
-    // tokens are split once, prologue included, for all of them.
-    const uint32_t pieces = a.k / 512u, launches = (a.k + 4095u) / 4096u;
+    // Stretches of unequal length: each a launch that adds to the one before; the tokens are
+    // split once, prologue included, for all of them.
+    if (together) {
+        const uint32_t most = cus / launches, walkers = units < most ? units : most;
+        const uint32_t lrounds = (a.rows / 32u) / walkers, ltail = (a.rows - 32u * lrounds * walkers + 7u) / 8u;
+        q.rounds = lrounds; q.tail_base = ltail / walkers; q.tail_rem = ltail % walkers; q.by_die = walkers % 8u == 0 ? 1u : 0u;
+        q.parts = launches;
+        q.partial = reinterpret_cast<float *>(d.work->data + planes_bytes);
+        q.a.k = 512u * (pieces / launches);
+        q.plane_first = 0;
+        for (uint32_t t0 = 0; t0 < a.m; t0 += 8u) {
+            q.a.x = a.x + (size_t)t0 * a.xr;
+            q.a.out = a.out + (size_t)t0 * a.out_stride;
+            q.a.m = a.m - t0 < 8u ? a.m - t0 : 8u;
+            q.a.flags = a.flags & ~FLAG_NORM;
+            q.t0 = t0;
+            if (zhip_result r = f16 ? launch_for_k<true, true, true>(d, q, dim3(walkers * launches)) : launch_for_k<true, false, true>(d, q, dim3(walkers * launches))) return r;
+            MvArgs sum = q.a;
+            sum.k = a.k;
+            if (zhip_result r = launch_matvec_parts_sum(d, name, sum, q.partial, launches)) return r;
+        }
+        return ZHIP_OK;
+    }
     for (uint32_t t0 = 0; t0 < a.m; t0 += 8u) {
         uint32_t first = 0;
         for (uint32_t c = 0; c < launches; c++) {
